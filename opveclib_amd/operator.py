@@ -1,0 +1,537 @@
+"""
+Operator front-end: the ``@operator`` decorator, lazy operator handles, gradient registration, the operator-DAG
+builder and the ``evaluate``/``profile`` entry points that run a DAG of operators on the GPU.
+
+Behavioural counterpart of the reference's opveclib/operator.py:128-806 and 2099-2335.  ``evaluate`` and ``profile``
+keep their signatures; the only supported ``target_language`` is ``'hip'``: every operator of the (optionally fused)
+DAG is turned into a HIP kernel for gfx950, compiled with hipcc, loaded through the C-ABI launcher and enqueued on the
+current PyTorch HIP stream.  There is no CPU execution path in this package.
+"""
+
+import dis
+import hashlib
+import inspect
+from collections import namedtuple
+
+import numpy as np
+
+from . import language as lang
+from .expression import TensorType, ExpressionDAG, input, OutputTensor
+from .local import version, logger
+
+
+class _TensorParam(object):
+    """Placeholder kept for API familiarity; the launcher's parameter struct lives in ``opveclib_amd.launcher``."""
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# lazy handles
+# ----------------------------------------------------------------------------------------------------------------------
+_INFIX = (('add', '__add__', '__radd__'), ('sub', '__sub__', '__rsub__'), ('mul', '__mul__', '__rmul__'),
+          ('div', '__truediv__', '__rtruediv__'), ('mod', '__mod__', '__rmod__'))
+_COMPARE = (('eq', '__eq__'), ('ne', '__ne__'), ('lt', '__lt__'), ('le', '__le__'), ('gt', '__gt__'),
+            ('ge', '__ge__'))
+
+
+class OperatorOutput(object):
+    """
+    An un-evaluated output tensor of an operator, used for building lazily evaluated DAGs of operators
+    (operator.py:134-221).  Infix arithmetic dispatches to the element-wise operators that
+    ``opveclib_amd.stdops`` registers with :meth:`register_magic_method`.
+    """
+
+    # raise operator priority so that numpy does not try to use its own operator
+    __array_priority__ = 1
+    _builtin_ops = {}
+
+    @staticmethod
+    def register_magic_method(key, value):
+        OperatorOutput._builtin_ops[key] = value
+
+    def __init__(self, parent, index):
+        if not isinstance(parent, _Operator):
+            raise TypeError('parent must be an Operator')
+        if not isinstance(index, int):
+            raise TypeError('index must be an int')
+
+        self.parent = parent
+        self.index = index
+        self.tensor_type = parent.output_types[index]
+        self.shape = self.tensor_type.shape
+        self.dtype = self.tensor_type.dtype
+        self.size = self.tensor_type.size
+        self.rank = self.tensor_type.rank
+
+    def __neg__(self):
+        return OperatorOutput._builtin_ops['neg'](self)
+
+    def __bool__(self):
+        raise SyntaxError('Cannot resolve operator values at interpretation time.')
+
+    __hash__ = None
+
+
+class _Operator(object):
+    """
+    One application of an operator function to concrete input types: its expression DAG, output types, inputs
+    and (optionally) its gradient DAG (operator.py:232-334).  Indexing yields :class:`OperatorOutput` handles.
+    """
+
+    __array_priority__ = 1
+
+    def __init__(self, dag, output_types, inputs, grad_dag, from_gradient, name):
+        self.inputs = inputs
+        self.expression_dag = dag
+        self.output_types = output_types
+        self.name = name
+        self.grad_dag = grad_dag
+        self.from_gradient = from_gradient
+        logger.debug('Operator created: ' + str(dag.name))
+
+    def __getitem__(self, item):
+        if not isinstance(item, int):
+            raise TypeError('index must be an int')
+        if item < 0 or item >= len(self.output_types):
+            raise IndexError('operator ' + str(self.name) + ' has ' + str(len(self.output_types)) + ' outputs')
+        return OperatorOutput(self, item)
+
+    def __len__(self):
+        return len(self.output_types)
+
+    def check_binary(self):
+        if len(self.output_types) != 1:
+            raise SyntaxError('Cannot use binary infix operators on multi-output operators. '
+                              'Explicitly index an output.')
+
+    def __neg__(self):
+        self.check_binary()
+        return -self[0]
+
+    __hash__ = None
+
+
+def _install_infix():
+    def out_forward(key):
+        return lambda self, other: OperatorOutput._builtin_ops[key](self, other)
+
+    def out_reverse(key):
+        return lambda self, other: OperatorOutput._builtin_ops[key](other, self)
+
+    def op_forward(dunder):
+        def method(self, other):
+            self.check_binary()
+            return getattr(self[0], dunder)(other)
+        return method
+
+    for key, fwd, rev in _INFIX:
+        setattr(OperatorOutput, fwd, out_forward(key))
+        setattr(OperatorOutput, rev, out_reverse(key))
+        setattr(_Operator, fwd, op_forward(fwd))
+        setattr(_Operator, rev, op_forward(rev))
+    for key, dunder in _COMPARE:
+        setattr(OperatorOutput, dunder, out_forward(key))
+        setattr(_Operator, dunder, op_forward(dunder))
+    OperatorOutput.__div__ = OperatorOutput.__truediv__
+    OperatorOutput.__rdiv__ = OperatorOutput.__rtruediv__
+
+
+_install_infix()
+
+
+class _GradientPlaceholder(object):
+    """Stands for an operator input or an upstream gradient while a gradient function is traced."""
+
+    def __init__(self, shape, dtype):
+        self.tensor_type = TensorType(shape, dtype)
+        self.rank = self.tensor_type.rank
+        self.shape = shape
+        self.dtype = dtype
+
+
+def _resolve_output(x):
+    """
+    Convert single-output Operators to an OperatorOutput (operator.py:337-354).
+
+    :raises ValueError: When argument is a multi-output Operator
+    :raises TypeError: When argument is neither an Operator nor an OperatorOutput
+    """
+    if isinstance(x, _Operator):
+        if len(x.output_types) != 1:
+            raise ValueError('Only a single-output Operator can be used as an input to another operator. '
+                             'Index a specific output from multi-output Operators.')
+        return x[0]
+    if not isinstance(x, OperatorOutput):
+        raise TypeError('Only operator outputs can be used to build an op dag. Received a ' + str(type(x)))
+    return x
+
+
+def _op_hash(op):
+    """Content name of an operator: 'f' + sha224(serialised DAG + library version) (operator.py:357-358)."""
+    return 'f' + hashlib.sha224(op.SerializeToString() + version.encode('utf-8')).hexdigest()
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# tracing
+# ----------------------------------------------------------------------------------------------------------------------
+def _as_list(x):
+    try:
+        len(x)
+    except TypeError:
+        return [x]
+    return list(x)
+
+
+def _with_full_inputs(found_dag, full_inputs):
+    """
+    A traced gradient DAG may use only some of its possible inputs, in any order.  Return a copy of its proto whose
+    ``dag_input_types`` list all of ``full_inputs`` in order and whose leaf references are renumbered to match
+    (operator.py:526-553).
+    """
+    remap = {}
+    for found_index, found_input in enumerate(found_dag.inputs):
+        for full_index, candidate in enumerate(full_inputs):
+            if candidate is found_input:
+                remap[found_index] = full_index
+                break
+        else:
+            raise ValueError('Gradient DAG depends on a tensor that is not one of its declared inputs.')
+
+    reordered = lang.OperatorDAG()
+    reordered.CopyFrom(found_dag.proto_dag)
+    del reordered.dag_input_types[:]
+    for placeholder in full_inputs:
+        reordered.dag_input_types.add().CopyFrom(placeholder.tensor_type.as_proto())
+    for ref in reordered.references:
+        for input_ref in ref.input_refs:
+            if input_ref.is_leaf:
+                input_ref.dag_input_index = remap[input_ref.dag_input_index]
+    return reordered
+
+
+class _OpGenerator(object):
+    """The callable that ``@operator()`` returns: calling it traces the function for the given input types."""
+
+    def __init__(self, op_function, forbid_none_valued_constants, name):
+        self.op_function = op_function
+        self.forbid_none_valued_constants = forbid_none_valued_constants
+        self.name = op_function.__name__ if name is None else name
+        self.grad_function = None
+
+    def __str__(self):
+        return self.op_function.__name__
+
+    def __call__(self, *inputs, **defined_constants):
+        # ops applied inside a gradient graph do not get gradient DAGs of their own
+        from_gradient = False
+        for inp in inputs:
+            if getattr(inp, 'from_gradient', False) or isinstance(inp, _GradientPlaceholder):
+                from_gradient = True
+            elif isinstance(inp, OperatorOutput) and inp.parent.from_gradient:
+                from_gradient = True
+
+        spec = inspect.getfullargspec(self.op_function)
+        if spec.defaults is None:
+            input_names = spec.args
+            constants = dict(defined_constants)
+        else:
+            input_names = spec.args[:-len(spec.defaults)]
+            constants = dict(zip(spec.args[-len(spec.defaults):], spec.defaults))
+            constants.update(defined_constants)
+
+        if self.forbid_none_valued_constants:
+            for key in constants.keys():
+                if constants[key] is None:
+                    raise ValueError(self.name + ' argument ' + key + ' is None, which implies an unset constant.\n'
+                                     '  If a None constant is meaningful for this operator, the operator should be '
+                                     'defined with the appropriate decorator flag.')
+
+        input_types = []
+        for inp_n, inp in enumerate(inputs):
+            try:
+                inp = _resolve_output(inp)
+            except TypeError:
+                pass
+            try:
+                input_types.append(TensorType.like(inp))
+            except AttributeError:
+                raise TypeError('Unexpectedly received a ' + inp.__class__.__name__ +
+                                ' instead of a tensor at argument position ' +
+                                str(inp_n + 1) + ' in the call to ' + self.name + '.  '
+                                'Should this argument be passed as a constant (keyword argument) instead?')
+
+        num_inputs = len(input_types)
+        if len(input_names) != num_inputs and spec.varargs is None:
+            err_msg = '\n'
+            err_msg += self.name + ' function signature expects ' + str(len(input_names)) + \
+                ' input tensor argument(s):\n' + str(input_names) + '\n'
+            err_msg += 'but was supplied with ' + str(num_inputs) + '.\n'
+            if len(input_names) > num_inputs:
+                remaining_names = input_names[num_inputs - len(input_names):]
+                err_msg += 'Should ' + str(remaining_names) + ' be passed to constructor as constant?'
+            raise TypeError(err_msg)
+
+        ExpressionDAG.clear()
+        input_exprs = [input(cur_type) for cur_type in input_types]
+
+        # interpret function to build up ExpressionDAG
+        output_exprs = self.op_function(*input_exprs, **constants)
+        if output_exprs is None:
+            raise ValueError('No outputs returned from op function')
+        output_exprs = _as_list(output_exprs)
+
+        if len(output_exprs) != ExpressionDAG.num_outputs:
+            raise ValueError('Defined ' + str(ExpressionDAG.num_outputs) + ' outputs, but returned ' +
+                             str(len(output_exprs)) +
+                             '. Number of defined outputs must equal number of returned outputs.')
+
+        # outputs are numbered by return position, not by declaration order, and their declarations are permuted
+        # so that they appear in the DAG in that order too
+        output_types = []
+        slots = []
+        for index, expr in enumerate(output_exprs):
+            if type(expr) is not OutputTensor:
+                raise TypeError('User functions must only return outputs. Instead got:\n' + str(expr))
+            slots.append(ExpressionDAG.expr_index(expr))
+            output_types.append(TensorType.like(expr))
+        for index, expr in enumerate(output_exprs):
+            expr.proto_expr.io_index = index
+        for slot, expr in zip(sorted(slots), output_exprs):
+            ExpressionDAG.replace(slot, expr)
+
+        expression_dag = ExpressionDAG.as_proto()
+        ExpressionDAG.clear()
+        expression_dag.name = self.name
+
+        grad_dag = None
+        if self.grad_function is not None and not from_gradient:
+            grad_inputs = [_GradientPlaceholder(t.shape, t.dtype) for t in input_types + output_types]
+            grad_outputs = _as_list(self.grad_function(*grad_inputs, **constants))
+
+            # a None among the gradient outputs means "no gradient defined": no gradient DAG at all
+            if not any(g is None for g in grad_outputs):
+                for grad_output_index, grad_output in enumerate(grad_outputs):
+                    if isinstance(grad_output, _Operator) and len(grad_output.output_types) != 1:
+                        raise TypeError('A multi-output operator was returned from a gradient function, '
+                                        'but the meaning of this is ambiguous: explicitly index each '
+                                        'output from operator: ' + str(grad_output.name))
+                    cur_input_type = input_types[grad_output_index]
+                    cur_grad_output_type = TensorType.like(_resolve_output(grad_output))
+                    if cur_input_type != cur_grad_output_type:
+                        raise TypeError('Gradient output index ' + str(grad_output_index) + ', with TensorType: ' +
+                                        str(cur_grad_output_type) + ' is inconsistent with operator input index ' +
+                                        str(grad_output_index) + ', with TensorType: ' + str(cur_input_type))
+                grad_dag = _with_full_inputs(_build_op_dag(*grad_outputs), grad_inputs)
+
+        return _Operator(expression_dag, output_types, inputs, grad_dag, from_gradient, self.name)
+
+    def add_grad(self, grad_function):
+        if self.grad_function is not None:
+            raise ValueError('Gradient function is already defined for operator ' + str(self.name) + '.')
+        self.grad_function = grad_function
+
+
+def _check_variable_rebinding(op_function):
+    """
+    A name bound to ``variable(...)`` must afterwards only be updated with ``<<=``; a plain re-assignment would
+    silently rebind the Python name instead of emitting an assignment into the operator
+    (operator.py:566-641, pinned by test_operator.py:246-278).  Raises SyntaxError at decoration time.
+    """
+    co = op_function.__code__
+    variable_names = set()
+    line_instrs = []
+    cur_line = None
+    prev = None
+    for instr in dis.get_instructions(co):
+        if instr.starts_line is not None:
+            cur_line = instr.starts_line
+            line_instrs = []
+        if instr.opname == 'STORE_FAST':
+            binds_variable = any(i.opname in ('LOAD_GLOBAL', 'LOAD_ATTR', 'LOAD_METHOD') and i.argval == 'variable'
+                                 for i in line_instrs)
+            via_lshift = prev is not None and (
+                prev.opname == 'INPLACE_LSHIFT' or (prev.opname == 'BINARY_OP' and prev.argrepr == '<<='))
+            if instr.argval in variable_names and not via_lshift:
+                raise SyntaxError('Cannot reassign to symbol "' + instr.argval + '" in operator "' + co.co_name +
+                                  '" because it refers to an OVL variable. Use the <<= operator'
+                                  ' to assign to OVL variables. \n' +
+                                  '  File "' + co.co_filename + '", line ' + str(cur_line))
+            if binds_variable:
+                variable_names.add(instr.argval)
+        line_instrs.append(instr)
+        prev = instr
+
+
+def operator(forbid_none_valued_constants=True, name=None):
+    """
+    Decorator that turns a worker function into an operator (operator.py:564-648).  Positional parameters of the
+    function are tensors, keyword / defaulted parameters are compile-time constants.
+    """
+    def wrapper(op_function):
+        _check_variable_rebinding(op_function)
+        op = _OpGenerator(op_function, forbid_none_valued_constants, name)
+        op.__name__ = op_function.__name__
+        op.__doc__ = op_function.__doc__
+        return op
+
+    return wrapper
+
+
+def gradient(op_function):
+    """
+    Decorator that registers the gradient of ``op_function`` (operator.py:651-673).  The gradient function receives
+    the operator's inputs followed by the gradients of its outputs (plus the same constants) and returns one
+    gradient per input; it may itself be an ``@operator()`` or a plain function composing operators.
+    """
+    if not isinstance(op_function, _OpGenerator):
+        raise TypeError('gradient decorator argument must be a function decorated as an operator')
+
+    def wrapper(grad_function):
+        if isinstance(grad_function, _OpGenerator):
+            def resolved(*args, **defaults):
+                op = grad_function(*args, **defaults)
+                return [op[output_index] for output_index in range(len(op.output_types))]
+        else:
+            resolved = grad_function
+
+        op_function.add_grad(resolved)
+        resolved.__name__ = grad_function.__name__
+        resolved.__doc__ = grad_function.__doc__
+        return resolved
+
+    return wrapper
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# operator DAG
+# ----------------------------------------------------------------------------------------------------------------------
+_OperatorDAG = namedtuple('_OperatorDAG', ['proto_dag', 'inputs', 'operators', 'grad_dags'])
+
+
+def _build_op_dag(*outputs):
+    """
+    Collect every operator the requested outputs depend on (operator.py:679-806).  Operators are ordered by their
+    depth in the DAG (ties keep discovery order), tensors that do not come from an operator become DAG inputs
+    (deduplicated by identity, in discovery order).
+
+    :param outputs: operator outputs (or single-output operators) from which to build the dag
+    :return: an _OperatorDAG(proto_dag, inputs, operators, grad_dags)
+    """
+    ops = []            # discovery order
+    slot_of = {}        # id(op) -> index in ops
+    depth = []
+    wiring = []         # per op: list of (parent_slot, parent_output, dag_input_index)
+    dag_inputs = []
+    dag_input_slot = {}
+
+    def visit(node):
+        if not isinstance(node, _Operator):
+            raise TypeError()
+        if id(node) in slot_of:
+            return slot_of[id(node)]
+        slot = len(ops)
+        slot_of[id(node)] = slot
+        ops.append(node)
+        depth.append(None)
+        wiring.append(None)
+
+        edges = []
+        deepest_parent = -1
+        for cur_input in node.inputs:
+            try:
+                resolved = _resolve_output(cur_input)
+            except TypeError:
+                key = id(cur_input)
+                if key not in dag_input_slot:
+                    dag_input_slot[key] = len(dag_inputs)
+                    dag_inputs.append(cur_input)
+                edges.append((None, None, dag_input_slot[key]))
+            else:
+                parent_slot = visit(resolved.parent)
+                deepest_parent = max(deepest_parent, depth[parent_slot])
+                edges.append((parent_slot, resolved.index, None))
+        wiring[slot] = edges
+        depth[slot] = deepest_parent + 1
+        return slot
+
+    requested = []
+    for dag_output in outputs:
+        cur_output = _resolve_output(dag_output)
+        requested.append((visit(cur_output.parent), cur_output.index))
+
+    order = sorted(range(len(ops)), key=lambda slot: (depth[slot], slot))
+    position = dict((slot, new) for new, slot in enumerate(order))
+    sorted_ops = [ops[slot] for slot in order]
+
+    op_dag = lang.OperatorDAG()
+    for op in sorted_ops:
+        op_dag.operators.add().CopyFrom(op.expression_dag)
+    for dag_input in dag_inputs:
+        op_dag.dag_input_types.add().CopyFrom(TensorType.like(dag_input).as_proto())
+    for slot in order:
+        ref_list = op_dag.references.add()
+        for parent_slot, parent_output, dag_input_index in wiring[slot]:
+            proto_ref = ref_list.input_refs.add()
+            if parent_slot is None:
+                proto_ref.is_leaf = True
+                proto_ref.dag_input_index = dag_input_index
+            else:
+                proto_ref.op_index = position[parent_slot]
+                proto_ref.op_output_index = parent_output
+    for parent_slot, parent_output in requested:
+        proto_ref = op_dag.dag_outputs.add()
+        proto_ref.op_index = position[parent_slot]
+        proto_ref.op_output_index = parent_output
+
+    grad_dags = [op.grad_dag for op in sorted_ops]
+    return _OperatorDAG(proto_dag=op_dag, inputs=dag_inputs, operators=sorted_ops, grad_dags=grad_dags)
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# evaluation
+# ----------------------------------------------------------------------------------------------------------------------
+def _normalise_output_list(output_list):
+    if isinstance(output_list, (_Operator, OperatorOutput)):
+        if isinstance(output_list, _Operator):
+            return [output_list[i] for i in range(len(output_list.output_types))]
+        return [output_list]
+    return list(output_list)
+
+
+def evaluate(output_list, target_language='hip', opt_level=3):
+    """
+    Evaluate a collection of OVL operator outputs on the GPU (operator.py:2099-2117).
+
+    :param output_list: an operator, an operator output, or a list of either
+    :param target_language: must be 'hip'
+    :param opt_level: operators are fused when opt_level >= 3
+    :return: one array for a single requested output, otherwise a list in request order.  Arrays are numpy arrays
+        when every DAG input was a numpy array, otherwise torch tensors on the inputs' device.
+    """
+    evaluated_outputs = profile(output_list, target_language=target_language,
+                                profiling_iterations=1, opt_level=opt_level)[0]
+    if len(evaluated_outputs) == 1:
+        return evaluated_outputs[0]
+    return evaluated_outputs
+
+
+def profile(output_list, target_language='hip', profiling_iterations=1, opt_level=3):
+    """
+    Evaluate a collection of OVL operator outputs and time every generated operator (operator.py:2120-2335).
+
+    :param profiling_iterations: number of timed launches per operator, a positive int
+    :return: (outputs, {operator hash name: float64[profiling_iterations] milliseconds})
+    """
+    if target_language != 'hip':
+        raise ValueError('Unsupported target_language: ' + str(target_language) +
+                         '. This package generates HIP kernels for gfx950 only (target_language=\'hip\').')
+    if not isinstance(profiling_iterations, int) or profiling_iterations < 1:
+        raise ValueError('profiling_iterations must be a positive int')
+
+    from .fusion import _merge_op_dag
+    from . import runtime
+
+    op_dag = _build_op_dag(*_normalise_output_list(output_list))
+    dag = op_dag.proto_dag
+    if opt_level >= 3:
+        dag, _ = _merge_op_dag(dag, None)
+    return runtime.run_op_dag(dag, op_dag.inputs, profiling_iterations)
