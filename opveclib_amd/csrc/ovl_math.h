@@ -1,0 +1,279 @@
+// float32 transcendental functions for generated operators: exp, log, expm1, tanh.
+//
+// Generated operators must reproduce, on the GPU, what the reference's generated C++ computes with the host C
+// library (opveclib/expression.py:1430-1456 maps EXP/LOG/TANH on float32 to expf/logf/tanhf).  Differences of one
+// unit in the last place between two correct math libraries are amplified without bound by later cancellation
+// (x - y with x close to y), so these routines follow the algorithms of the C library that the reference path runs
+// on (GNU libc 2.35, x86-64, processors with FMA):
+//
+//   expf, logf   table driven, evaluated in double precision (Arm Optimized Routines' single precision exp/log:
+//                exp(x) = 2^(k/32) * P3(r) with a 32 entry table of 2^(i/32); log(x) = log(c_i) + k*ln2 + P3(z/c_i - 1)
+//                with a 16 entry table of (1/c_i, log c_i)).  The x86-64 build of the library selects a variant
+//                compiled with fused multiply-add; the places where a multiply feeds an add are therefore fused
+//                here too (fma), everywhere else products are rounded separately.
+//   expm1f       FreeBSD msun / fdlibm single precision expm1: argument reduction by k*ln2 (two part ln2), a
+//                degree 5 rational correction in float arithmetic, scaling by 2^k through the exponent field.
+//   tanhf        fdlibm single precision tanh on top of expm1f: -t/(t+2) with t = expm1f(-2|x|) for |x| < 1,
+//                1 - 2/(t+2) with t = expm1f(2|x|) for 1 <= |x| < 22, +-1 beyond.
+//
+// The file compiles as plain C++ for the host as well (no HIP headers needed), which is how the routines are checked
+// against the host C library over all 2^32 float arguments.  All arithmetic must be compiled without contraction
+// (-ffp-contract=off); fused operations are spelled out with __builtin_fma.
+#ifndef OVL_MATH_H_
+#define OVL_MATH_H_
+
+#include <stdint.h>
+
+#if defined(__HIPCC__)
+#define OVL_HD __device__ __forceinline__
+#define OVL_TABLE static __device__ const
+#else
+#define OVL_HD static inline
+#define OVL_TABLE static const
+#endif
+
+// Every multiply-add site can be switched between fused (bit set) and separately rounded (bit clear); the default
+// mask is the combination that reproduces the host C library bit for bit.
+#ifndef OVL_MATH_FMA_SITES
+#define OVL_MATH_FMA_SITES 0xffffffffu
+#endif
+#define OVL_MADD(site, a, b, c) \
+    (((OVL_MATH_FMA_SITES >> (site)) & 1u) ? __builtin_fma((a), (b), (c)) : ((a) * (b) + (c)))
+
+namespace ovl_math {
+
+OVL_HD uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }
+OVL_HD float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+OVL_HD uint64_t as_u64(double f) { return __builtin_bit_cast(uint64_t, f); }
+OVL_HD double as_f64(uint64_t u) { return __builtin_bit_cast(double, u); }
+
+// ---------------------------------------------------------------------------------------------------------------------
+// expf
+// ---------------------------------------------------------------------------------------------------------------------
+#define OVL_EXP2F_TABLE_BITS 5
+#define OVL_EXP2F_N (1 << OVL_EXP2F_TABLE_BITS)
+
+// tab[i] = bits(2^(i/32)) - (i << 47): adding k << 47 puts k/32's integer part into the exponent field
+#define OVL_EXP2F_TABLE { \
+    0x3ff0000000000000ull, 0x3fefd9b0d3158574ull, 0x3fefb5586cf9890full, 0x3fef9301d0125b51ull, \
+    0x3fef72b83c7d517bull, 0x3fef54873168b9aaull, 0x3fef387a6e756238ull, 0x3fef1e9df51fdee1ull, \
+    0x3fef06fe0a31b715ull, 0x3feef1a7373aa9cbull, 0x3feedea64c123422ull, 0x3feece086061892dull, \
+    0x3feebfdad5362a27ull, 0x3feeb42b569d4f82ull, 0x3feeab07dd485429ull, 0x3feea47eb03a5585ull, \
+    0x3feea09e667f3bcdull, 0x3fee9f75e8ec5f74ull, 0x3feea11473eb0187ull, 0x3feea589994cce13ull, \
+    0x3feeace5422aa0dbull, 0x3feeb737b0cdc5e5ull, 0x3feec49182a3f090ull, 0x3feed503b23e255dull, \
+    0x3feee89f995ad3adull, 0x3feeff76f2fb5e47ull, 0x3fef199bdd85529cull, 0x3fef3720dcef9069ull, \
+    0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull }
+
+OVL_TABLE uint64_t exp2f_tab[OVL_EXP2F_N] = OVL_EXP2F_TABLE;
+
+OVL_HD uint32_t top12(float x) { return as_u32(x) >> 20; }
+
+OVL_HD float expf_(float x) {
+    const double InvLn2N = 0x1.71547652b82fep+0 * OVL_EXP2F_N;
+    const double Shift = 0x1.8p+52;
+    const double C0 = 0x1.c6af84b912394p-5 / OVL_EXP2F_N / OVL_EXP2F_N / OVL_EXP2F_N;
+    const double C1 = 0x1.ebfce50fac4f3p-3 / OVL_EXP2F_N / OVL_EXP2F_N;
+    const double C2 = 0x1.62e42ff0c52d6p-1 / OVL_EXP2F_N;
+
+    double xd = (double)x;
+    uint32_t abstop = top12(x) & 0x7ff;
+    if (abstop >= top12(88.0f)) {
+        // |x| >= 88 or x is nan
+        if (as_u32(x) == as_u32(-__builtin_inff())) return 0.0f;
+        if (abstop >= top12(__builtin_inff())) return x + x;
+        if (x > 0x1.62e42ep6f) return __builtin_inff();     // overflow
+        if (x < -0x1.9fe368p6f) return 0.0f;                // underflow
+    }
+    // x*N/Ln2 = k + r with r in [-1/2, 1/2] and int k
+    double kd = OVL_MADD(0, InvLn2N, xd, Shift);
+    uint64_t ki = as_u64(kd);
+    kd -= Shift;
+    double r = OVL_MADD(1, InvLn2N, xd, -kd);
+    // exp(x) = 2^(k/N) * 2^(r/N) ~= s * (C0*r^3 + C1*r^2 + C2*r + 1)
+    uint64_t t = exp2f_tab[ki % OVL_EXP2F_N];
+    t += ki << (52 - OVL_EXP2F_TABLE_BITS);
+    double s = as_f64(t);
+    double z2 = OVL_MADD(2, C0, r, C1);
+    double r2 = r * r;
+    double y = OVL_MADD(3, C2, r, 1.0);
+    y = OVL_MADD(4, z2, r2, y);
+    y = y * s;
+    return (float)y;
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// logf
+// ---------------------------------------------------------------------------------------------------------------------
+#define OVL_LOGF_TABLE_BITS 4
+#define OVL_LOGF_N (1 << OVL_LOGF_TABLE_BITS)
+
+struct logf_entry { double invc, logc; };
+
+#define OVL_LOGF_TABLE { \
+    { 0x1.661ec79f8f3bep+0, -0x1.57bf7808caadep-2 }, \
+    { 0x1.571ed4aaf883dp+0, -0x1.2bef0a7c06ddbp-2 }, \
+    { 0x1.49539f0f010bp+0, -0x1.01eae7f513a67p-2 }, \
+    { 0x1.3c995b0b80385p+0, -0x1.b31d8a68224e9p-3 }, \
+    { 0x1.30d190c8864a5p+0, -0x1.6574f0ac07758p-3 }, \
+    { 0x1.25e227b0b8eap+0, -0x1.1aa2bc79c81p-3 }, \
+    { 0x1.1bb4a4a1a343fp+0, -0x1.a4e76ce8c0e5ep-4 }, \
+    { 0x1.12358f08ae5bap+0, -0x1.1973c5a611cccp-4 }, \
+    { 0x1.0953f419900a7p+0, -0x1.252f438e10c1ep-5 }, \
+    { 0x1p+0, 0x0p+0 }, \
+    { 0x1.e608cfd9a47acp-1, 0x1.aa5aa5df25984p-5 }, \
+    { 0x1.ca4b31f026aap-1, 0x1.c5e53aa362eb4p-4 }, \
+    { 0x1.b2036576afce6p-1, 0x1.526e57720db08p-3 }, \
+    { 0x1.9c2d163a1aa2dp-1, 0x1.bc2860d22477p-3 }, \
+    { 0x1.886e6037841edp-1, 0x1.1058bc8a07ee1p-2 }, \
+    { 0x1.767dcf5534862p-1, 0x1.4043057b6ee09p-2 } }
+
+OVL_TABLE logf_entry logf_tab[OVL_LOGF_N] = OVL_LOGF_TABLE;
+
+OVL_HD float logf_(float x) {
+    const double Ln2 = 0x1.62e42fefa39efp-1;
+    const double A0 = -0x1.00ea348b88334p-2, A1 = 0x1.5575b0be00b6ap-2, A2 = -0x1.ffffef20a4123p-2;
+    const uint32_t Off = 0x3f330000;
+
+    uint32_t ix = as_u32(x);
+    if (ix == 0x3f800000) return 0.0f;
+    if (ix - 0x00800000 >= 0x7f800000 - 0x00800000) {
+        // x < 0x1p-126 or inf or nan
+        if (ix * 2 == 0) return -__builtin_inff();
+        if (ix == 0x7f800000) return x;
+        if ((ix & 0x80000000) || ix * 2 >= 0xff000000) return __builtin_nanf("");
+        // x is subnormal, normalize it
+        ix = as_u32(x * 0x1p23f);
+        ix -= 23u << 23;
+    }
+    // x = 2^k z; z in [Off, 2*Off) is exact; the range is split into N subintervals, c is near the centre of z's
+    uint32_t tmp = ix - Off;
+    int i = (tmp >> (23 - OVL_LOGF_TABLE_BITS)) % OVL_LOGF_N;
+    int k = (int32_t)tmp >> 23;
+    uint32_t iz = ix - (tmp & (0x1ffu << 23));
+    double invc = logf_tab[i].invc;
+    double logc = logf_tab[i].logc;
+    double z = (double)as_f32(iz);
+    // log(x) = log1p(z/c-1) + log(c) + k*Ln2
+    double r = OVL_MADD(8, z, invc, -1.0);
+    double y0 = OVL_MADD(9, (double)k, Ln2, logc);
+    double r2 = r * r;
+    double y = OVL_MADD(10, A1, r, A2);
+    y = OVL_MADD(11, A0, r2, y);
+    y = OVL_MADD(12, y, r2, y0 + r);
+    return (float)y;
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// expm1f and tanhf (float arithmetic throughout)
+// ---------------------------------------------------------------------------------------------------------------------
+OVL_HD float expm1f_(float x) {
+    const float one = 1.0f, huge = 1.0e+30f, tiny = 1.0e-30f;
+    const float o_threshold = 8.8721679688e+01f;    // 0x42b17180
+    const float ln2_hi = 6.9313812256e-01f;         // 0x3f317180
+    const float ln2_lo = 9.0580006145e-06f;         // 0x3717f7d1
+    const float invln2 = 1.4426950216e+00f;         // 0x3fb8aa3b
+    const float Q1 = -3.3333335072e-02f;            // 0xbd088889
+    const float Q2 = 1.5873016091e-03f;             // 0x3ad00d01
+    const float Q3 = -7.9365076090e-05f;            // 0xb8a670cd
+    const float Q4 = 4.0082177293e-06f;             // 0x36867e54
+    const float Q5 = -2.0109921195e-07f;            // 0xb457edbb
+
+    float y, hi, lo, c = 0.0f, t, e, hxs, hfx, r1;
+    int32_t k;
+    uint32_t hx = as_u32(x);
+    uint32_t xsb = hx & 0x80000000u;    // sign bit of x
+    hx &= 0x7fffffffu;                  // bits of |x|
+
+    // filter out huge and non-finite argument
+    if (hx >= 0x4195b844u) {            // |x| >= 27*ln2
+        if (hx >= 0x42b17218u) {        // |x| >= 88.721...
+            if (hx > 0x7f800000u) return x + x;                         // NaN
+            if (hx == 0x7f800000u) return (xsb == 0) ? x : -1.0f;       // exp(+-inf) - 1 = {inf, -1}
+            if (x > o_threshold) return huge * huge;                    // overflow
+        }
+        if (xsb != 0) return tiny - one;                                // x < -27*ln2: -1 (inexact)
+    }
+
+    // argument reduction
+    if (hx > 0x3eb17218u) {             // |x| > 0.5 ln2
+        if (hx < 0x3F851592u) {         // and |x| < 1.5 ln2
+            if (xsb == 0) { hi = x - ln2_hi; lo = ln2_lo; k = 1; }
+            else { hi = x + ln2_hi; lo = -ln2_lo; k = -1; }
+        } else {
+            k = (int32_t)(invln2 * x + ((xsb == 0) ? 0.5f : -0.5f));
+            t = (float)k;
+            hi = x - t * ln2_hi;        // t*ln2_hi is exact here
+            lo = t * ln2_lo;
+        }
+        x = hi - lo;
+        c = (hi - x) - lo;
+    } else if (hx < 0x33000000u) {      // |x| < 2**-25: return x
+        t = huge + x;
+        return x - (t - (huge + x));
+    } else {
+        k = 0;
+    }
+
+    // x is now in primary range
+    hfx = 0.5f * x;
+    hxs = x * hfx;
+    r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
+    t = 3.0f - r1 * hfx;
+    e = hxs * ((r1 - t) / (6.0f - x * t));
+    if (k == 0) return x - (x * e - hxs);       // c is 0
+    e = (x * (e - c) - c);
+    e -= hxs;
+    if (k == -1) return 0.5f * (x - e) - 0.5f;
+    if (k == 1) {
+        if (x < -0.25f) return -2.0f * (e - (x + 0.5f));
+        return one + 2.0f * (x - e);
+    }
+    if (k <= -2 || k > 56) {            // suffice to return exp(x)-1
+        y = one - (e - x);
+        y = as_f32(as_u32(y) + ((uint32_t)k << 23));    // add k to y's exponent
+        return y - one;
+    }
+    if (k < 23) {
+        t = as_f32(0x3f800000u - (0x1000000u >> k));    // t = 1 - 2^-k
+        y = t - (e - x);
+        y = as_f32(as_u32(y) + ((uint32_t)k << 23));
+    } else {
+        t = as_f32((uint32_t)(0x7f - k) << 23);          // 2^-k
+        y = x - (e + t);
+        y += one;
+        y = as_f32(as_u32(y) + ((uint32_t)k << 23));
+    }
+    return y;
+}
+
+OVL_HD float tanhf_(float x) {
+    const float one = 1.0f, two = 2.0f, tiny = 1.0e-30f;
+    float t, z;
+    uint32_t jx = as_u32(x);
+    uint32_t ix = jx & 0x7fffffffu;
+    bool negative = (jx & 0x80000000u) != 0;
+
+    if (ix >= 0x7f800000u) {            // inf or NaN
+        if (!negative) return one / x + one;    // tanh(+inf) = +1, tanh(NaN) = NaN
+        return one / x - one;
+    }
+    if (ix < 0x41b00000u) {             // |x| < 22
+        if (ix == 0) return x;          // +-0
+        if (ix < 0x24000000u) return x * (one + x);     // |x| < 2**-55
+        // |x| >= 1: z = 1 - 2/(t+2) with t = expm1(2|x|);  |x| < 1: z = -t/(t+2) with t = expm1(-2|x|).
+        // Both cases share one expm1 evaluation and one division; each lane performs exactly the operations of
+        // its own case.
+        float ax = as_f32(ix);
+        bool big = ix >= 0x3f800000u;
+        t = expm1f_(big ? two * ax : -two * ax);
+        float q = (big ? two : -t) / (t + two);
+        z = big ? one - q : q;
+    } else {                            // |x| >= 22: +-1 (inexact)
+        z = one - tiny;
+    }
+    return negative ? -z : z;
+}
+
+}  // namespace ovl_math
+
+#endif  // OVL_MATH_H_

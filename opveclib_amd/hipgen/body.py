@@ -1,0 +1,196 @@
+"""
+Emission of the per-worker body of an operator as HIP device code.
+
+One statement per expression in DAG order, the same sequence of typed operations that the reference's generator
+emits for the CPU and CUDA targets (opveclib/expression.py: every ``gen_c``, statement forms listed at
+1293-1306, 1351-1352, 1386-1387, 1422-1423, 1479-1481, 1739-1742, 1794-1795, 1881-1882, 1904-1905, 1996-2006,
+2064-2183), so a worker performs the same arithmetic in the same order.  Kernel templates customise how tensor
+reads and stores are realised through the ``read_hook`` / ``store_hook`` callbacks (vector register lanes, LDS
+tiles, plain global accesses).
+"""
+
+from .. import language as lang
+
+CTYPE = {
+    lang.FLOAT32: 'float', lang.FLOAT64: 'double',
+    lang.INT8: 'int8_t', lang.INT16: 'int16_t', lang.INT32: 'int32_t', lang.INT64: 'long long',
+    lang.UINT8: 'uint8_t', lang.UINT16: 'uint16_t', lang.UINT32: 'uint32_t', lang.UINT64: 'uint64_t'}
+
+# device math entry points (ovl_* are defined in csrc/ovl_device.h)
+UNARY = {
+    lang.ACOS: {lang.FLOAT32: 'acosf', lang.FLOAT64: 'acos'},
+    lang.ASIN: {lang.FLOAT32: 'asinf', lang.FLOAT64: 'asin'},
+    lang.ATAN: {lang.FLOAT32: 'atanf', lang.FLOAT64: 'atan'},
+    lang.COS: {lang.FLOAT32: 'cosf', lang.FLOAT64: 'cos'},
+    lang.COSH: {lang.FLOAT32: 'coshf', lang.FLOAT64: 'cosh'},
+    lang.SIN: {lang.FLOAT32: 'sinf', lang.FLOAT64: 'sin'},
+    lang.SINH: {lang.FLOAT32: 'sinhf', lang.FLOAT64: 'sinh'},
+    lang.TAN: {lang.FLOAT32: 'tanf', lang.FLOAT64: 'tan'},
+    lang.TANH: {lang.FLOAT32: 'ovl_tanhf', lang.FLOAT64: 'tanh'},
+    lang.EXP: {lang.FLOAT32: 'ovl_expf', lang.FLOAT64: 'exp'},
+    lang.LOG: {lang.FLOAT32: 'ovl_logf', lang.FLOAT64: 'log'},
+    lang.LOG10: {lang.FLOAT32: 'log10f', lang.FLOAT64: 'log10'},
+    lang.SQRT: {lang.FLOAT32: 'sqrtf', lang.FLOAT64: 'sqrt'},
+    lang.CEIL: {lang.FLOAT32: 'ceilf', lang.FLOAT64: 'ceil'},
+    lang.FLOOR: {lang.FLOAT32: 'floorf', lang.FLOAT64: 'floor'},
+    lang.ABS: {lang.FLOAT32: 'fabsf', lang.FLOAT64: 'fabs', lang.INT8: 'ovl_abs_8', lang.INT16: 'ovl_abs_16',
+               lang.INT32: 'abs', lang.INT64: 'llabs'},
+    lang.ISINF: {lang.FLOAT32: 'isinf', lang.FLOAT64: 'isinf'},
+    lang.ISFINITE: {lang.FLOAT32: 'isfinite', lang.FLOAT64: 'isfinite'},
+    lang.ISNAN: {lang.FLOAT32: 'isnan', lang.FLOAT64: 'isnan'},
+}
+_NEGATABLE = (lang.FLOAT32, lang.FLOAT64, lang.INT8, lang.INT16, lang.INT32, lang.INT64)
+UNARY[lang.NEGATE] = dict((t, '-') for t in _NEGATABLE)
+UNARY[lang.NOT] = dict((t, '!') for t in CTYPE)
+
+INFIX = {lang.ADD: '+', lang.SUBTRACT: '-', lang.MULTIPLY: '*', lang.DIVIDE: '/', lang.MODULO: '%',
+         lang.EQUAL: '==', lang.NOTEQUAL: '!=', lang.LESS: '<', lang.LESS_EQ: '<=', lang.GREATER: '>',
+         lang.GREATER_EQ: '>=', lang.AND: '&&', lang.OR: '||'}
+
+LIMITS = {lang.MIN_VALUE: {lang.FLOAT32: 'FLT_MIN', lang.FLOAT64: 'DBL_MIN'},
+          lang.MAX_VALUE: {lang.FLOAT32: 'FLT_MAX', lang.FLOAT64: 'DBL_MAX'},
+          lang.EPSILON: {lang.FLOAT32: 'FLT_EPSILON', lang.FLOAT64: 'DBL_EPSILON'}}
+
+
+def literal(value, dtype=None):
+    """
+    Text of a numeric literal.  Floating point literals are written as C double literals exactly like Python prints
+    them, so the conversion to the destination type happens in the compiled code, as it does for the reference's
+    generated text (a ``float e = 1.0001;`` statement rounds the double literal to float).
+    """
+    if isinstance(value, float):
+        if value != value:
+            return '__builtin_nan("")'
+        if value == float('inf'):
+            return '__builtin_inf()'
+        if value == float('-inf'):
+            return '(-__builtin_inf())'
+        return repr(float(value))
+    value = int(value)
+    if dtype == lang.UINT64 or value > 2 ** 63 - 1:
+        return str(value) + 'ull'
+    if value < -2 ** 31 or value > 2 ** 31 - 1:
+        return str(value) + 'll'
+    return str(value)
+
+
+def binary_text(code, dtype, a, b):
+    if code == lang.MIN:
+        return '(((' + a + ')<(' + b + '))?(' + a + '):(' + b + '))'
+    if code == lang.MAX:
+        return '(((' + a + ')>(' + b + '))?(' + a + '):(' + b + '))'
+    if code == lang.POW:
+        return ('powf(' if dtype == lang.FLOAT32 else 'pow(') + a + ',' + b + ')'
+    if code == lang.ATAN2:
+        return ('atan2f(' if dtype == lang.FLOAT32 else 'atan2(') + a + ',' + b + ')'
+    if code == lang.MODULO and dtype == lang.FLOAT32:
+        return 'fmodf(' + a + ',' + b + ')'
+    if code == lang.MODULO and dtype == lang.FLOAT64:
+        return 'fmod(' + a + ',' + b + ')'
+    return '(' + a + ' ' + INFIX[code] + ' ' + b + ')'
+
+
+class BodyEmitter(object):
+    """
+    Walks the DAG and produces the statement list of one worker.
+
+    :param info: the analysed DAG (:class:`analysis.DagInfo`)
+    :param position_exprs: list of C expressions, one per workgroup dimension, giving this worker's position
+    :param read_hook: ``f(node, tensor_node, index_name) -> C expression or None``; None selects the plain global
+        read ``in<k>[index]``
+    :param store_hook: ``f(node, tensor_node, index_name, value_name) -> C statement or None``; None selects the
+        plain global store ``out<k>[index] = value;``
+    """
+
+    def __init__(self, info, position_exprs, read_hook=None, store_hook=None, suffix=''):
+        self.info = info
+        self.position_exprs = position_exprs
+        self.read_hook = read_hook
+        self.store_hook = store_hook
+        self.suffix = suffix
+
+    def tensor_name(self, node):
+        if node.code == lang.INPUT:
+            return 'in' + str(node.io_index)
+        if node.code == lang.OUTPUT:
+            return 'out' + str(node.io_index)
+        if node.code == lang.POSITION:
+            return 'position'
+        return 'e' + str(node.idx) + self.suffix
+
+    def emit(self):
+        info = self.info
+        names = {}
+        stmts = []
+        indent = 0
+
+        def put(text):
+            stmts.append('    ' * indent + text)
+
+        for node in info.nodes:
+            code = node.code
+            ops = node.ops
+            name = 'e' + str(node.idx) + self.suffix
+            if code in (lang.INPUT, lang.OUTPUT):
+                name = self.tensor_name(node)
+            elif code == lang.POSITION:
+                name = 'position'
+                put('const uint32_t position[' + str(len(self.position_exprs)) + '] = {' +
+                    ', '.join(self.position_exprs) + '};')
+            elif code == lang.CONST_SCALAR:
+                name = literal(node.data[0], node.dtype)
+            elif code == lang.CONST_TENSOR:
+                name = '{' + ', '.join(literal(v, node.dtype) for v in node.data) + '}'
+            elif code in LIMITS:
+                name = LIMITS[code][node.dtype]
+            elif code in (lang.VARIABLE, lang.CAST):
+                put(CTYPE[node.dtype] + ' ' + name + ' = ' + names[ops[0]] + ';')
+            elif code == lang.TENSOR:
+                put(CTYPE[node.dtype] + ' ' + name + '[' + str(node.size) + '] = ' + names[ops[0]] + ';')
+            elif code == lang.ASSIGN_VARIABLE:
+                put(names[ops[0]] + ' = ' + names[ops[1]] + ';')
+            elif code == lang.ASSIGN_TENSOR:
+                tensor = info.nodes[ops[0]]
+                text = None
+                if tensor.code == lang.OUTPUT and self.store_hook is not None:
+                    text = self.store_hook(node, tensor, names[ops[1]], names[ops[2]])
+                if text is None:
+                    text = names[ops[0]] + '[' + names[ops[1]] + '] = ' + names[ops[2]] + ';'
+                if text:
+                    put(text)
+            elif code == lang.READ_TENSOR:
+                tensor = info.nodes[ops[0]]
+                text = None
+                if tensor.code == lang.INPUT and self.read_hook is not None:
+                    text = self.read_hook(node, tensor, names[ops[1]])
+                if text is None:
+                    text = names[ops[0]] + '[' + names[ops[1]] + ']'
+                put(CTYPE[node.dtype] + ' ' + name + ' = ' + text + ';')
+            elif code == lang.RANGE:
+                i, start, stop, step = (names[o] for o in ops)
+                put('for(' + i + ' = ' + start + '; ((' + i + ' < ' + stop + ')&&(' + step + '>0)) || ((' +
+                    i + ' > ' + stop + ')&&(' + step + '<0)); ' + i + '+=' + step + '){')
+                indent += 1
+            elif code in (lang.ENDRANGE, lang.ENDIF):
+                indent -= 1
+                put('}')
+            elif code == lang.IF:
+                put('if(' + names[ops[0]] + '){')
+                indent += 1
+            elif code == lang.ELSEIF:
+                indent -= 1
+                put('} else if(' + names[ops[0]] + '){')
+                indent += 1
+            elif code == lang.ELSE:
+                indent -= 1
+                put('} else {')
+                indent += 1
+            elif code in UNARY:
+                put(CTYPE[node.dtype] + ' ' + name + ' = ' + UNARY[code][node.dtype] + '(' + names[ops[0]] + ');')
+            elif code in INFIX or code in (lang.MIN, lang.MAX, lang.POW, lang.ATAN2):
+                put(CTYPE[node.dtype] + ' ' + name + ' = ' +
+                    binary_text(code, node.dtype, names[ops[0]], names[ops[1]]) + ';')
+            else:
+                raise NotImplementedError('expression code ' + str(code))
+            names[node.idx] = name
+        return stmts

@@ -1,0 +1,212 @@
+"""
+The map kernel template: one thread processes VEC consecutive workers along the last workgroup dimension.
+
+Replaces the reference's one-thread-per-worker CUDA template (opveclib/expression.py:595-609, launched with 32
+threads per block, expression.py:696-698 and operator.py:30).  For gfx950 the template
+
+* gives each thread VEC workers that are neighbours along the last workgroup dimension, so that every tensor access
+  whose flat index is ``base(outer position) + last position + constant`` becomes one aligned vector load or store of
+  up to 16 bytes per thread, fully coalesced across the 64 lanes of a wavefront;
+* hoists those loads to the top of the thread's iteration (all loads in flight before the arithmetic starts) and
+  buffers the stores in registers until the end of the iteration;
+* runs a grid-stride loop with 256-thread workgroups (four wavefronts), sized to a multiple of the CU count;
+* keeps every other access (gathers, scatters, accesses inside loops or behind non-exhaustive conditions) as the
+  scalar access the worker function asked for.
+
+With VEC = 1 it is the fully general fallback for any DAG.
+"""
+
+from .. import language as lang
+from .analysis import ITEMSIZE
+from .body import BodyEmitter, CTYPE
+
+BLOCK = 256
+
+
+class Access(object):
+    """A group of identical tensor accesses (same tensor, same affine index) realised as one vector."""
+
+    def __init__(self, tensor, aff, reg):
+        self.tensor = tensor
+        self.aff = aff
+        self.reg = reg
+
+
+def _index_expr(aff, pos_names, wide):
+    """C expression of an affine index in the position variables of lane 0."""
+    ctype = 'uint64_t' if wide else 'uint32_t'
+    terms = []
+    if aff.const != 0 or not aff.coeffs:
+        terms.append('(' + ctype + ')' + str(aff.const) + ('ull' if wide else 'u'))
+    for (kind, k), c in sorted(aff.coeffs.items()):
+        assert kind == 'p'
+        term = '(' + ctype + ')' + pos_names[k]
+        if c != 1:
+            term = term + ' * (' + ctype + ')' + str(c) + ('ull' if wide else 'u')
+        terms.append(term)
+    return ' + '.join(terms)
+
+
+def choose_vec(info):
+    """Largest power-of-two vector width (elements) usable for this DAG, and the accesses it vectorises."""
+    last = len(info.workgroup_shape) - 1
+    extent = info.workgroup_shape[last]
+    accesses = info.tensor_accesses()
+    widest = 1
+    for _, tensor, _ in accesses:
+        widest = max(widest, ITEMSIZE[tensor.dtype])
+    vec = max(1, 16 // widest)
+    while vec > 1:
+        if extent % vec == 0 and any(_is_vector_access(info, node, tensor, aff, vec)
+                                     for node, tensor, aff in accesses):
+            break
+        vec //= 2
+    return vec
+
+
+def _is_vector_access(info, node, tensor, aff, vec):
+    if aff is None or not aff.only_position():
+        return False
+    last = len(info.workgroup_shape) - 1
+    if aff.coeff(('p', last)) != 1:
+        return False
+    if aff.const % vec != 0:
+        return False
+    for sym, c in aff.coeffs.items():
+        if sym != ('p', last) and c % vec != 0:
+            return False
+    if aff.lo < 0 or aff.hi >= tensor.size:
+        return False            # cannot prove every lane in bounds for every worker
+    if info.in_loop[node.idx]:
+        return False
+    return True
+
+
+def generate(info, kernel_name, vec=None):
+    """
+    :return: (kernel source text, launch description dict) for the map template.
+    """
+    rank = len(info.workgroup_shape)
+    last = rank - 1
+    if vec is None:
+        vec = choose_vec(info)
+    if info.workgroup_shape[last] % vec != 0:
+        raise ValueError('vector width does not divide the last workgroup dimension')
+
+    accesses = info.tensor_accesses()
+    loads = {}      # (input node idx, signature) -> Access
+    stores = {}     # (output node idx, signature) -> Access
+    store_keys = []
+    for node, tensor, aff in accesses:
+        if vec > 1 and _is_vector_access(info, node, tensor, aff, vec):
+            key = (tensor.idx, aff.signature())
+            if node.code == lang.READ_TENSOR:
+                if key not in loads:
+                    loads[key] = Access(tensor, aff, 'ld%d' % len(loads))
+            else:
+                store_keys.append(key)
+    certain = info.definitely_stores(store_keys)
+    for node, tensor, aff in accesses:
+        if node.code == lang.ASSIGN_TENSOR and aff is not None:
+            key = (tensor.idx, aff.signature())
+            if key in certain and key not in stores and vec > 1 and _is_vector_access(info, node, tensor, aff, vec):
+                stores[key] = Access(tensor, aff, 'st%d' % len(stores))
+
+    def read_hook(node, tensor, index_name):
+        aff = info.affine[node.ops[1]]
+        if aff is not None:
+            acc = loads.get((tensor.idx, aff.signature()))
+            if acc is not None and not info.in_loop[node.idx]:
+                return acc.reg + '[lane]'
+        return None
+
+    def store_hook(node, tensor, index_name, value_name):
+        aff = info.affine[node.ops[1]]
+        if aff is not None:
+            acc = stores.get((tensor.idx, aff.signature()))
+            if acc is not None and not info.in_loop[node.idx]:
+                return acc.reg + '[lane] = ' + value_name + ';'
+        return None
+
+    pos_names = ['p%d' % k for k in range(rank)]
+    lane_position = list(pos_names)
+    lane_position[last] = pos_names[last] + ' + lane' if vec > 1 else pos_names[last]
+    body = BodyEmitter(info, lane_position, read_hook, store_hook).emit()
+
+    num_vectors = info.num_workers // vec
+    args = []
+    for i in range(len(info.inputs)):
+        args.append('const ' + CTYPE[info.inputs[i].dtype] + '* __restrict__ in' + str(i))
+    for i in range(len(info.outputs)):
+        args.append(CTYPE[info.outputs[i].dtype] + '* __restrict__ out' + str(i))
+
+    src = []
+    vec_types = {}
+    for acc in list(loads.values()) + list(stores.values()):
+        ctype = CTYPE[acc.tensor.dtype]
+        vec_types[ctype] = 'ovl_' + ctype.replace(' ', '_') + 'x' + str(vec)
+    for ctype, vname in sorted(vec_types.items()):
+        src.append('typedef ' + ctype + ' ' + vname + ' __attribute__((ext_vector_type(' + str(vec) + ')));')
+    src.append('')
+    src.append('extern "C" __global__ void __launch_bounds__(%d)' % BLOCK)
+    src.append(kernel_name + '(' + ', '.join(args) + ') {')
+    src.append('    const uint32_t num_vectors = %du;' % num_vectors)
+    src.append('    const uint32_t stride = gridDim.x * %du;' % BLOCK)
+    src.append('    for (uint32_t v = blockIdx.x * %du + threadIdx.x; v < num_vectors; v += stride) {' % BLOCK)
+    src.append('        const uint32_t worker0 = v * %du;' % vec)
+    # position of the first of this thread's workers
+    block = 1
+    blocks = [1] * rank
+    for k in range(rank - 2, -1, -1):
+        block *= info.workgroup_shape[k + 1]
+        blocks[k] = block
+    for k in range(rank):
+        expr = 'worker0'
+        if k > 0:
+            expr = '(worker0 % ' + str(blocks[k - 1]) + 'u)'
+        src.append('        const uint32_t %s = %s / %du;' % (pos_names[k], expr, blocks[k]))
+
+    for acc in loads.values():
+        vname = vec_types[CTYPE[acc.tensor.dtype]]
+        wide = acc.aff.hi >= 2 ** 32
+        src.append('        const %s %s = *reinterpret_cast<const %s*>(in%d + (%s));' % (
+            vname, acc.reg, vname, acc.tensor.io_index, _index_expr(acc.aff, pos_names, wide)))
+    for acc in stores.values():
+        src.append('        %s %s;' % (vec_types[CTYPE[acc.tensor.dtype]], acc.reg))
+
+    if vec > 1:
+        src.append('        #pragma unroll')
+        src.append('        for (uint32_t lane = 0; lane < %du; ++lane) {' % vec)
+        pad = '            '
+    else:
+        src.append('        {')
+        pad = '            '
+    for stmt in body:
+        src.append(pad + stmt)
+    src.append('        }')
+    for acc in stores.values():
+        vname = vec_types[CTYPE[acc.tensor.dtype]]
+        wide = acc.aff.hi >= 2 ** 32
+        src.append('        *reinterpret_cast<%s*>(out%d + (%s)) = %s;' % (
+            vname, acc.tensor.io_index, _index_expr(acc.aff, pos_names, wide), acc.reg))
+    src.append('    }')
+    src.append('}')
+
+    align = {}
+    for acc in loads.values():
+        key = ('in', acc.tensor.io_index)
+        align[key] = max(align.get(key, 1), vec * ITEMSIZE[acc.tensor.dtype])
+    for acc in stores.values():
+        key = ('out', acc.tensor.io_index)
+        align[key] = max(align.get(key, 1), vec * ITEMSIZE[acc.tensor.dtype])
+
+    launch = {
+        'template': 'map',
+        'vec': vec,
+        'block': BLOCK,
+        'blocks_needed': (num_vectors + BLOCK - 1) // BLOCK,
+        'align': align,
+        'vector_loads': len(loads),
+        'vector_stores': len(stores),
+    }
+    return '\n'.join(src) + '\n', launch

@@ -507,8 +507,7 @@ def evaluate(output_list, target_language='hip', opt_level=3):
     :return: one array for a single requested output, otherwise a list in request order.  Arrays are numpy arrays
         when every DAG input was a numpy array, otherwise torch tensors on the inputs' device.
     """
-    evaluated_outputs = profile(output_list, target_language=target_language,
-                                profiling_iterations=1, opt_level=opt_level)[0]
+    evaluated_outputs = _run(output_list, target_language, 1, opt_level, timed=False)[0]
     if len(evaluated_outputs) == 1:
         return evaluated_outputs[0]
     return evaluated_outputs
@@ -521,6 +520,10 @@ def profile(output_list, target_language='hip', profiling_iterations=1, opt_leve
     :param profiling_iterations: number of timed launches per operator, a positive int
     :return: (outputs, {operator hash name: float64[profiling_iterations] milliseconds})
     """
+    return _run(output_list, target_language, profiling_iterations, opt_level, timed=True)
+
+
+def _run(output_list, target_language, profiling_iterations, opt_level, timed):
     if target_language != 'hip':
         raise ValueError('Unsupported target_language: ' + str(target_language) +
                          '. This package generates HIP kernels for gfx950 only (target_language=\'hip\').')
@@ -534,4 +537,4 @@ def profile(output_list, target_language='hip', profiling_iterations=1, opt_leve
     dag = op_dag.proto_dag
     if opt_level >= 3:
         dag, _ = _merge_op_dag(dag, None)
-    return runtime.run_op_dag(dag, op_dag.inputs, profiling_iterations)
+    return runtime.run_op_dag(dag, op_dag.inputs, profiling_iterations, timed=timed)
