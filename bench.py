@@ -1,0 +1,286 @@
+#!/usr/bin/env python
+"""
+Benchmark of the generated-operator hot path on one MI355X.
+
+Headline workload ("chain8"): the fused element-wise chain of eight OVL operators
+(add, mul by scalar 1.0001, tanh, sigmoid, log1p, expm1, sub, abs) over two float32 [8192, 8192] inputs drawn
+uniformly from [-1, 1] (numpy default_rng(2)); the optimizer fuses the eight operators into one kernel.  One step is
+one launch of the fused kernel on inputs that are already resident in HBM.  The metric is the achieved HBM bandwidth
+in GB/s counted on algorithmic bytes (each input element read once, each output element written once:
+3 * 2^26 * 4 + 4 bytes per launch).
+
+The JSON line also carries
+  roofline      algorithmic bytes / average kernel duration (HIP events recorded around every launch on the launch
+                stream) against the 8 TB/s HBM peak,
+  cpu_baseline  the CPU oracle (the reference-shaped generated C++ compiled with the reference's flags) timed on this
+                machine's host cores on a row slice of the same workload,
+  others        time, bandwidth and roofline fraction of the remaining configurations (shift+expm1+log1p, cumsum,
+                cumprod, LSTM cell forward and gradient, gather+transposed scatter).
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+_ROOT = os.path.dirname(os.path.abspath(__file__))
+if _ROOT not in sys.path:
+    sys.path.insert(0, _ROOT)
+
+import numpy as np
+
+HBM_PEAK_GBPS = 8000.0
+
+# HBM bytes per launch of the chain8 kernel from rocprofv3 counters (FETCH_SIZE + WRITE_SIZE, scaled by the same
+# counters' reading for a copy kernel of known size); None until measured.  Source: profiles/chain8_*.txt
+CHAIN8_TRAFFIC_BYTES = None
+
+
+class Spec(object):
+    """Shape and dtype of a tensor, enough to trace an operator without allocating the tensor."""
+
+    def __init__(self, shape, dtype=np.float32):
+        self.shape = list(shape)
+        self.dtype = np.dtype(dtype).type
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# workloads
+# ----------------------------------------------------------------------------------------------------------------------
+def chain8_outputs(a, b, s):
+    from tests.cases import chain8
+    return [chain8(a, b, s)[-1][0]]
+
+
+def c1_outputs(x):
+    from opveclib_amd.examples import shift_cyclic, expm1, log1p
+    return [log1p(expm1(shift_cyclic(x)))[0]]
+
+
+def cumsum_outputs(x):
+    from opveclib_amd.examples import cumsum
+    return [cumsum(x, axis=1)[0]]
+
+
+def cumprod_outputs(x):
+    from opveclib_amd.examples import cumprod
+    return [cumprod(x, axis=1)[0]]
+
+
+def lstm_outputs(concat, c):
+    from opveclib_amd.lstm import lstm
+    op = lstm(concat, c, forget_bias=1.0)
+    return [op[0], op[1]]
+
+
+def lstm_grad_outputs(concat, c, dc, dh):
+    from opveclib_amd.lstm import lstm_grad
+    op = lstm_grad(concat, c, dc, dh, forget_bias=1.0)
+    return [op[0], op[1]]
+
+
+def gather_outputs(a, b_flat):
+    from opveclib_amd.examples import gather_transpose
+    return [gather_transpose(a, b_flat, alpha=0.5, stride=7919)[0]]
+
+
+def all_workload_outputs():
+    """Operator outputs of every benchmark workload at full size, built from shape specs (used to compile ahead)."""
+    f32, f64 = np.float32, np.float64
+    yield chain8_outputs(Spec((8192, 8192)), Spec((8192, 8192)), Spec((1,)))
+    yield chain8_outputs(Spec((2048, 8192)), Spec((2048, 8192)), Spec((1,)))
+    yield c1_outputs(Spec((1 << 20,)))
+    yield cumsum_outputs(Spec((4096, 16384), f32))
+    yield cumprod_outputs(Spec((4096, 16384), f32))
+    yield cumsum_outputs(Spec((1024, 16384), f64))
+    yield cumprod_outputs(Spec((1024, 16384), f64))
+    yield lstm_outputs(Spec((4096, 4096)), Spec((4096, 1024)))
+    yield lstm_grad_outputs(Spec((4096, 4096)), Spec((4096, 1024)), Spec((4096, 1024)), Spec((4096, 1024)))
+    yield gather_outputs(Spec((16384, 16384)), Spec((16384 * 16384,)))
+
+
+def uniform(rng, lo, hi, shape, dtype=np.float32):
+    return (lo + (hi - lo) * rng.random(shape, dtype=dtype)).astype(dtype)
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# measurement
+# ----------------------------------------------------------------------------------------------------------------------
+class Prepared(object):
+    """A fused operator DAG with its device tensors, ready to be launched repeatedly."""
+
+    def __init__(self, outputs):
+        import torch
+        from opveclib_amd import runtime
+        from opveclib_amd.operator import _build_op_dag
+        from opveclib_amd.fusion import _merge_op_dag
+        op_dag = _build_op_dag(*outputs)
+        self.dag, _ = _merge_op_dag(op_dag.proto_dag, None)
+        self.device = torch.device('cuda', 0)
+        self.leaves = [x if isinstance(x, torch.Tensor) else torch.from_numpy(np.ascontiguousarray(x)).to(self.device)
+                       for x in op_dag.inputs]
+        self.ops = [runtime.load_operator(op) for op in self.dag.operators]
+        self.buffers = []
+        self.steps = []
+        for op_index, compiled in enumerate(self.ops):
+            ins = []
+            for ref in self.dag.references[op_index].input_refs:
+                ins.append(self.leaves[ref.dag_input_index] if ref.is_leaf
+                           else self.buffers[ref.op_index][ref.op_output_index])
+            compiled.check_inputs(ins)
+            outs = compiled.allocate_outputs(self.device)
+            self.buffers.append(outs)
+            self.steps.append((compiled, compiled.params(ins, compiled.input_types), len(ins),
+                               compiled.params(outs, compiled.output_types), len(outs)))
+        self.algorithmic_bytes = sum(c.gen.algorithmic_bytes for c in self.ops)
+        self.kernels = [c.lib.info for c in self.ops]
+
+    def launch(self, stream):
+        for compiled, in_params, n_in, out_params, n_out in self.steps:
+            compiled.lib.launch(in_params, n_in, out_params, n_out, stream)
+
+    def results(self):
+        return [self.buffers[ref.op_index][ref.op_output_index] for ref in self.dag.dag_outputs]
+
+
+def measure(prepared, steps, warmup):
+    """Returns (ms per step from the host clock around the timed region, mean ms per launch from HIP events)."""
+    import torch
+    stream_obj = torch.cuda.current_stream()
+    stream = stream_obj.cuda_stream
+    for _ in range(warmup):
+        prepared.launch(stream)
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        starts[i].record(stream_obj)
+        prepared.launch(stream)
+        stops[i].record(stream_obj)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    per_launch = [s.elapsed_time(e) for s, e in zip(starts, stops)]
+    return (t1 - t0) * 1e3 / steps, float(np.mean(per_launch)), float(np.min(per_launch))
+
+
+def side_workload(name, outputs, steps, warmup):
+    prepared = Prepared(outputs)
+    wall_ms, event_ms, min_ms = measure(prepared, steps, warmup)
+    gbps = prepared.algorithmic_bytes / (event_ms * 1e-3) / 1e9
+    return {'workload': name, 'us': round(event_ms * 1e3, 2), 'min_us': round(min_ms * 1e3, 2),
+            'GB/s': round(gbps, 1), 'frac': round(gbps / HBM_PEAK_GBPS, 4),
+            'algorithmic_bytes': prepared.algorithmic_bytes,
+            'kernels': [k['kernel'] for k in prepared.kernels]}
+
+
+def cpu_baseline(seed_arrays, rows, iters=3):
+    """The CPU oracle on the first ``rows`` rows of the chain8 inputs, all host threads, best of ``iters``."""
+    import oracle
+    a, b, s = seed_arrays
+    outs = chain8_outputs(np.ascontiguousarray(a[:rows]), np.ascontiguousarray(b[:rows]), s)
+    threads = oracle.hardware_threads()
+    _, times = oracle.profile(outs, profiling_iterations=iters, opt_level=3, num_threads=threads)
+    ms = min(min(t) for t in times.values()) if len(times) == 1 else sum(min(t) for t in times.values())
+    nbytes = 3 * rows * a.shape[1] * 4 + 4
+    return {'value': round(nbytes / (ms * 1e-3) / 1e9, 3), 'unit': 'GB/s', 'cores': threads, 'kind': 'port',
+            'ms': round(ms, 2),
+            'sample': 'first %d of %d rows of the chain8 inputs; reference-shaped fused C++ (g++, no -O flag as in '
+                      'the reference), std::thread block split, thread create/join inside the timed region, '
+                      'best of %d' % (rows, a.shape[0], iters)}, outs
+
+
+def main():
+    parser = argparse.ArgumentParser()
+    parser.add_argument('--gpus', type=int, default=1)
+    parser.add_argument('--steps', type=int, default=50)
+    parser.add_argument('--warmup', type=int, default=5)
+    parser.add_argument('--no-others', action='store_true', help='skip the secondary configurations')
+    parser.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline')
+    args = parser.parse_args()
+    if args.gpus != 1:
+        sys.exit('bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)' % args.gpus)
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit('bench.py needs a HIP device')
+    import opveclib_amd  # noqa: F401
+
+    rng = np.random.default_rng(2)
+    shape = (8192, 8192)
+    a = uniform(rng, -1, 1, shape)
+    b = uniform(rng, -1, 1, shape)
+    s = np.array([1.0001], np.float32)
+
+    chain = Prepared(chain8_outputs(a, b, s))
+    assert len(chain.ops) == 1, 'the 8-op chain must fuse into one kernel'
+    wall_ms, event_ms, min_ms = measure(chain, args.steps, args.warmup)
+    nbytes = chain.algorithmic_bytes
+    value = nbytes / (wall_ms * 1e-3) / 1e9
+    achieved = nbytes / (event_ms * 1e-3) / 1e9
+
+    result = {
+        'metric': 'achieved HBM bandwidth on the fused 8-op chain (algorithmic bytes / time)',
+        'value': round(value, 1), 'unit': 'GB/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+        'ms_per_step': round(wall_ms, 4), 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
+        'dtype': 'f32', 'data': 'synthetic',
+        'config': {'workload': 'chain8: add, mul 1.0001, tanh, sigmoid, log1p, expm1, sub, abs fused into one kernel; '
+                               'A, B float32 [8192, 8192] uniform[-1, 1], numpy default_rng(2)',
+                   'algorithmic_bytes': nbytes, 'kernel': chain.kernels[0]['kernel'],
+                   'pct_of_hbm_peak': round(100.0 * value / HBM_PEAK_GBPS, 2)},
+        'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
+                     'frac': round(achieved / HBM_PEAK_GBPS, 4), 'traffic': CHAIN8_TRAFFIC_BYTES,
+                     'kernel_us': round(event_ms * 1e3, 2), 'kernel_min_us': round(min_ms * 1e3, 2)},
+    }
+
+    if not args.no_cpu:
+        rows = 2048
+        base, cpu_outs = cpu_baseline((a, b, s), rows)
+        result['cpu_baseline'] = base
+        # the GPU result on the same rows must equal the oracle's bit for bit
+        import oracle
+        ref = oracle.evaluate(cpu_outs, opt_level=0)
+        got = chain.results()[0][:rows].cpu().numpy()
+        result['parity'] = {'rows_checked': rows, 'bit_exact': bool(np.array_equal(got, ref))}
+    else:
+        result['cpu_baseline'] = None
+
+    if not args.no_others:
+        others = []
+        steps = max(5, min(args.steps, 20))
+        g = np.random.default_rng(0)
+        others.append(side_workload('c1 shift_cyclic -> expm1 -> log1p, f32[2^20]',
+                                    c1_outputs(uniform(g, -0.9, 0.9, 1 << 20)), steps, args.warmup))
+        del chain
+        torch.cuda.empty_cache()
+        g = np.random.default_rng(3)
+        xs = g.standard_normal((4096, 16384), dtype=np.float32)
+        others.append(side_workload('c3 cumsum f32[4096,16384] last axis', cumsum_outputs(xs), steps, args.warmup))
+        xp = uniform(g, 0.99, 1.01, (4096, 16384))
+        others.append(side_workload('c3 cumprod f32[4096,16384] last axis', cumprod_outputs(xp), steps, args.warmup))
+        xd = g.standard_normal((1024, 16384))
+        others.append(side_workload('c3 cumsum f64[1024,16384] last axis', cumsum_outputs(xd), steps, args.warmup))
+        g = np.random.default_rng(4)
+        concat = g.standard_normal((4096, 4096), dtype=np.float32)
+        c = g.standard_normal((4096, 1024), dtype=np.float32)
+        dh = g.standard_normal((4096, 1024), dtype=np.float32)
+        dc = g.standard_normal((4096, 1024), dtype=np.float32)
+        others.append(side_workload('c4 lstm cell forward [4096, 4x1024]', lstm_outputs(concat, c), steps,
+                                    args.warmup))
+        others.append(side_workload('c4 lstm cell gradient [4096, 4x1024]',
+                                    lstm_grad_outputs(concat, c, dc, dh), steps, args.warmup))
+        torch.cuda.empty_cache()
+        g5 = torch.Generator(device='cuda')
+        g5.manual_seed(5)
+        a5 = torch.randn((16384, 16384), device='cuda', generator=g5)
+        b5 = torch.randn((16384 * 16384,), device='cuda', generator=g5)
+        others.append(side_workload('c5 gather + transposed scatter f32[16384,16384]', gather_outputs(a5, b5),
+                                    max(3, steps // 4), 2))
+        result['others'] = others
+
+    print(json.dumps(result))
+
+
+if __name__ == '__main__':
+    main()

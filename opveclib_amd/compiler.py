@@ -70,18 +70,20 @@ def build_library(source):
     name = library_name(source)
     so_path = os.path.join(directory, name)
     src_path = so_path[:-3] + '.hip'
-    with _lock:
-        if os.path.exists(so_path):
-            return so_path
-        logger.debug('Compiling HIP operator ' + name)
-        with open(src_path, 'w') as f:
-            f.write(source)
-        tmp_path = so_path + '.tmp.%d' % os.getpid()
-        cmd = [local.hipcc] + list(HIPCC_FLAGS) + ['-I' + local.csrc_directory, src_path, '-o', tmp_path]
-        try:
-            subprocess.check_output(cmd, stderr=subprocess.STDOUT, universal_newlines=True)
-        except subprocess.CalledProcessError as exception:
-            logger.error('hipcc error: ' + exception.output)
-            raise RuntimeError('hipcc failed for ' + src_path + ':\n' + exception.output)
-        os.replace(tmp_path, so_path)
+    # Concurrent builders of the same library each compile into a private temporary file and rename it into place;
+    # the rename is atomic, so readers only ever see complete libraries.
+    logger.debug('Compiling HIP operator ' + name)
+    tag = '.tmp.%d.%d' % (os.getpid(), threading.get_ident())
+    tmp_src = src_path + tag
+    with open(tmp_src, 'w') as f:
+        f.write(source)
+    os.replace(tmp_src, src_path)
+    tmp_path = so_path + tag
+    cmd = [local.hipcc] + list(HIPCC_FLAGS) + ['-I' + local.csrc_directory, src_path, '-o', tmp_path]
+    try:
+        subprocess.check_output(cmd, stderr=subprocess.STDOUT, universal_newlines=True)
+    except subprocess.CalledProcessError as exception:
+        logger.error('hipcc error: ' + exception.output)
+        raise RuntimeError('hipcc failed for ' + src_path + ':\n' + exception.output)
+    os.replace(tmp_path, so_path)
     return so_path

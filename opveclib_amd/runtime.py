@@ -118,14 +118,17 @@ def _require_gpu():
 
 
 def _to_device(x, torch, device):
-    """Contiguous device tensor for a DAG input; returns (tensor, came_from_host_array)."""
+    """Contiguous, 16-byte aligned device tensor for a DAG input; returns (tensor, came_from_host_array)."""
     if isinstance(x, np.ndarray):
         return torch.from_numpy(np.ascontiguousarray(x)).to(device), True
     if isinstance(x, torch.Tensor):
         t = x.detach()
         if t.device.type != 'cuda':
             t = t.to(device)
-        return t.contiguous(), False
+        t = t.contiguous()
+        if t.data_ptr() % 16 != 0:
+            t = t.clone()       # a view into the middle of an allocation: vector loads need an aligned base
+        return t, False
     return torch.from_numpy(np.ascontiguousarray(np.asarray(x))).to(device), True
 
 

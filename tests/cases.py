@@ -1,0 +1,594 @@
+"""
+The shared table of parity cases.
+
+Every case builds a small DAG of operators from seeded inputs.  The GPU tests evaluate each case through the HIP
+path and compare it with the CPU oracle; the repository build step walks the same table to compile every HIP
+operator (and every oracle operator) ahead of time, so that a GPU run only loads binaries.
+"""
+
+import numpy as np
+
+import opveclib_amd as ovl
+from opveclib_amd import stdops
+from opveclib_amd.examples import (shift_cyclic, cumsum, cumprod, accumulate, expm1, log1p, absolute,
+                                   gather_transpose)
+from opveclib_amd.lstm import lstm, lstm_grad
+
+
+class Case(object):
+    """
+    :param name: test id
+    :param build: function(rng) -> list of operator outputs
+    :param max_ulp: 0 demands bit-exact equality with the oracle; otherwise the largest allowed distance in units in
+        the last place (float32) and, for float64 outputs, ``rel`` bounds the relative error instead
+    """
+
+    def __init__(self, name, build, max_ulp=0, rel=0.0, seed=0):
+        self.name = name
+        self.build = build
+        self.max_ulp = max_ulp
+        self.rel = rel
+        self.seed = seed
+
+    def outputs(self):
+        return self.build(np.random.default_rng(self.seed))
+
+    def __repr__(self):
+        return self.name
+
+
+def uniform(rng, lo, hi, shape, dtype=np.float32):
+    return (lo + (hi - lo) * rng.random(shape, dtype=dtype)).astype(dtype)
+
+
+def all_outputs(op):
+    """Every output of an operator application (gradient-decorated operators already return such a list)."""
+    if isinstance(op, (list, tuple)):
+        return list(op)
+    return [op[i] for i in range(len(op.output_types))]
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# the five benchmark configurations, at sizes the oracle finishes in well under a second
+# ----------------------------------------------------------------------------------------------------------------------
+def chain8(a, b, s):
+    """The fused 8-op chain: add, mul by scalar, tanh, sigmoid, log1p, expm1, sub, abs; returns every stage."""
+    t1 = stdops.add(a, b)
+    t2 = stdops.mul(t1, s)
+    t3 = stdops.tanh(t2)
+    t4 = stdops.sigmoid(t3)
+    t5 = log1p(t4)
+    t6 = expm1(t5)
+    t7 = stdops.sub(t6, b)
+    y = absolute(t7)
+    return [t1, t2, t3, t4, t5, t6, t7, y]
+
+
+def c1_shift_expm1_log1p(rng, n=1 << 14):
+    x = uniform(rng, -0.9, 0.9, n)
+    return [log1p(expm1(shift_cyclic(x)))[0]]
+
+
+def c1_shift_only(rng, n=1 << 14):
+    x = uniform(rng, -0.9, 0.9, n)
+    return [shift_cyclic(x)[0]]
+
+
+def c2_chain(rng, shape=(96, 256)):
+    a = uniform(rng, -1, 1, shape)
+    b = uniform(rng, -1, 1, shape)
+    s = np.array([1.0001], np.float32)
+    return [chain8(a, b, s)[-1][0]]
+
+
+def c2_chain_stages(rng, shape=(96, 256)):
+    a = uniform(rng, -1, 1, shape)
+    b = uniform(rng, -1, 1, shape)
+    s = np.array([1.0001], np.float32)
+    return [t[0] for t in chain8(a, b, s)]
+
+
+def c3_cumsum_f32(rng, shape=(48, 1024)):
+    return [cumsum(rng.standard_normal(shape, dtype=np.float32), axis=1)[0]]
+
+
+def c3_cumprod_f32(rng, shape=(48, 1024)):
+    return [cumprod(uniform(rng, 0.99, 1.01, shape), axis=1)[0]]
+
+
+def c3_cumsum_f64(rng, shape=(24, 1024)):
+    return [cumsum(rng.standard_normal(shape), axis=1)[0]]
+
+
+def c3_cumprod_f64(rng, shape=(24, 1024)):
+    return [cumprod(uniform(rng, 0.99, 1.01, shape, np.float64), axis=1)[0]]
+
+
+def c4_lstm(rng, batch=32, units=128):
+    concat = rng.standard_normal((batch, 4 * units), dtype=np.float32)
+    c = rng.standard_normal((batch, units), dtype=np.float32)
+    return all_outputs(lstm(concat, c, forget_bias=1.0))
+
+
+def c4_lstm_grad(rng, batch=32, units=128):
+    concat = rng.standard_normal((batch, 4 * units), dtype=np.float32)
+    c = rng.standard_normal((batch, units), dtype=np.float32)
+    dc = rng.standard_normal((batch, units), dtype=np.float32)
+    dh = rng.standard_normal((batch, units), dtype=np.float32)
+    return all_outputs(lstm_grad(concat, c, dc, dh, forget_bias=1.0))
+
+
+def c5_gather_transpose(rng, shape=(192, 320)):
+    a = rng.standard_normal(shape, dtype=np.float32)
+    b = rng.standard_normal(shape, dtype=np.float32)
+    return [gather_transpose(a, b.reshape(-1), alpha=0.5, stride=7919)[0]]
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# scalar math coverage (the reference's test_unary_math.py / test_binary_math.py inputs)
+# ----------------------------------------------------------------------------------------------------------------------
+def _unary_op(fcn):
+    @ovl.operator()
+    def unary(input0):
+        out = ovl.output_like(input0)
+        pos = ovl.position_in(input0.shape)
+        out[pos] = fcn(input0[pos])
+        return out
+    return unary
+
+
+def _binary_op(fcn):
+    @ovl.operator()
+    def binary_math(op_input0, op_input1):
+        out = ovl.output_like(op_input0)
+        pos = ovl.position_in(op_input0.shape)
+        out[pos] = fcn(op_input0[pos], op_input1[pos])
+        return out
+    return binary_math
+
+
+UNARY_FLOAT = [
+    ('arccos', ovl.arccos, np.arccos, 'one'), ('arcsin', ovl.arcsin, np.arcsin, 'one'),
+    ('arctan', ovl.arctan, np.arctan, 'atan'), ('cos', ovl.cos, np.cos, 'any'), ('cosh', ovl.cosh, np.cosh, 'any'),
+    ('sin', ovl.sin, np.sin, 'any'), ('sinh', ovl.sinh, np.sinh, 'any'), ('tan', ovl.tan, np.tan, 'any'),
+    ('tanh', ovl.tanh, np.tanh, 'any'), ('exp', ovl.exp, np.exp, 'any'), ('log', ovl.log, np.log, 'pos'),
+    ('log10', ovl.log10, np.log10, 'pos'), ('sqrt', ovl.sqrt, np.sqrt, 'pos'), ('ceil', ovl.ceil, np.ceil, 'any'),
+    ('floor', ovl.floor, np.floor, 'any'), ('absolute', ovl.absolute, np.absolute, 'any'),
+    ('negate', lambda x: -x, lambda x: -x, 'any')]
+
+#: float32 functions whose device implementation reproduces the host C library bit for bit
+EXACT_F32 = ('tanh', 'exp', 'log', 'sqrt', 'ceil', 'floor', 'absolute', 'negate')
+
+
+def unary_input(kind, dtype, length=100):
+    """Inputs of the reference's unary tests (test_unary_math.py:113-117): RandomState(1), 100 elements."""
+    rng = np.random.RandomState(1)
+    rand = rng.uniform(-10, 10, length).astype(dtype)
+    rand_pos = np.abs(rand) + np.finfo(dtype).eps
+    rand_one = rng.uniform(-1.0 + np.finfo(dtype).eps, 1 - np.finfo(dtype).eps, length).astype(dtype)
+    return {'any': rand, 'pos': rand_pos, 'one': rand_one, 'atan': (3.14 / 2 * rand_one).astype(dtype)}[kind]
+
+
+def _unary_case(name, fcn, kind, dtype):
+    def build(rng):
+        return [_unary_op(fcn)(unary_input(kind, dtype))[0]]
+    exact = dtype == np.float32 and name in EXACT_F32 or name in ('sqrt', 'ceil', 'floor', 'absolute', 'negate')
+    return Case('unary_%s_%s' % (name, np.dtype(dtype).name), build,
+                max_ulp=0 if exact else 2, rel=0 if exact else 1e-12)
+
+
+BINARY_ALL = [
+    ('add', lambda a, b: a + b), ('sub', lambda a, b: a - b), ('mul', lambda a, b: a * b),
+    ('div', lambda a, b: a / b), ('mod', lambda a, b: a % b),
+    ('eq', lambda a, b: a == b), ('ne', lambda a, b: a != b),
+    ('or', lambda a, b: ovl.logical_or(a, b)), ('and', lambda a, b: ovl.logical_and(a, b)),
+    ('lt', lambda a, b: a < b), ('le', lambda a, b: a <= b), ('gt', lambda a, b: a > b), ('ge', lambda a, b: a >= b),
+    ('min', lambda a, b: ovl.minimum(a, b)), ('max', lambda a, b: ovl.maximum(a, b))]
+BINARY_FLOAT = [('pow', lambda a, b: ovl.power(a, b)), ('atan2', lambda a, b: ovl.arctan2(a, b))]
+
+ALL_DTYPES = [np.float32, np.float64, np.int8, np.int16, np.int32, np.int64,
+              np.uint8, np.uint16, np.uint32, np.uint64]
+
+
+def binary_inputs(name, dtype, length=10):
+    """Inputs of the reference's binary tests (test_binary_math.py:57-72): RandomState(1), 10 elements."""
+    rng = np.random.RandomState(1)
+
+    def cast(arg):
+        if np.dtype(dtype).kind == 'u':
+            return np.abs(arg).astype(dtype)
+        return arg.astype(dtype)
+
+    x = cast(rng.uniform(-10, 10, length))
+    y = cast(rng.uniform(-10, 10, length))
+    y_nonzero = (y + np.equal(y, 0)).astype(dtype)
+    x_binary = cast(rng.uniform(0, 1, length) > 0.5)
+    y_binary = cast(rng.uniform(0, 1, length) > 0.5)
+    if name in ('div', 'mod'):
+        return x, y_nonzero
+    if name in ('eq', 'ne', 'or', 'and'):
+        return x_binary, y_binary
+    if name == 'pow':
+        return np.abs(x), y
+    return x, y
+
+
+def _binary_case(name, fcn, dtype):
+    def build(rng):
+        a, b = binary_inputs(name, dtype)
+        return [_binary_op(fcn)(a, b)[0]]
+    approx = name in ('pow', 'atan2')
+    return Case('binary_%s_%s' % (name, np.dtype(dtype).name), build,
+                max_ulp=2 if approx else 0, rel=1e-12 if approx else 0)
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# control flow, indexing and multi-output operators from the reference's tests
+# ----------------------------------------------------------------------------------------------------------------------
+@ovl.operator()
+def clip(arg, threshold1=None, threshold2=None):
+    pos = ovl.position_in(arg.shape)
+    clipped = ovl.output_like(arg)
+    x = arg[pos]
+    with ovl.if_(x < threshold1):
+        clipped[pos] = threshold1
+    with ovl.elif_(x > threshold2):
+        clipped[pos] = threshold2
+    with ovl.else_():
+        clipped[pos] = x
+    return clipped
+
+
+@ovl.operator()
+def set_limits(arg):
+    pos = ovl.position_in(arg.shape)
+    limits = ovl.output([arg.shape[0], 3], arg.dtype)
+    t = arg.dtype
+    limits[pos, 0] = ovl.min_value(t)
+    limits[pos, 1] = ovl.max_value(t)
+    limits[pos, 2] = ovl.epsilon(t)
+    return limits
+
+
+@ovl.operator()
+def fill_range(input0):
+    assert len(input0.shape) == 1
+    ovl.position_in([1])
+    num_elements = input0.shape[0]
+    out_right = ovl.output(input0.shape, input0.dtype)
+    out_left = ovl.output(input0.shape, input0.dtype)
+    for i in ovl.arange(num_elements):
+        out_right[i] = input0[i] * ovl.cast(i, input0.dtype)
+    for i in ovl.arange(num_elements - 1, -1, -1):
+        out_left[i] = input0[i] * ovl.cast(i, input0.dtype)
+    return out_right, out_left
+
+
+@ovl.operator()
+def dot(input0, input1):
+    num_vectors = input0.shape[0]
+    dot_out = ovl.output(num_vectors, input0.dtype)
+    pos = ovl.position_in(num_vectors)[0]
+    accum = ovl.variable(0.0, ovl.float64)
+    num_elements = ovl.variable(input0.shape[1], ovl.uint32)
+    for i in ovl.arange(num_elements):
+        accum <<= accum + input0[pos, i] * input1[pos, i]
+    dot_out[pos] = accum
+    return dot_out
+
+
+@ovl.operator()
+def multi_op(input0, input1, input2):
+    pos = ovl.position_in(input0.shape)
+    output0 = ovl.output_like(input0)
+    output1 = ovl.output_like(input0)
+    output2 = ovl.output_like(input0)
+    a = input0[pos]
+    b = input1[pos]
+    c = input2[pos]
+    d = a + b
+    output0[pos] = d
+    output1[pos] = d * c
+    output2[pos] = d + c
+    return output0, output1, output2
+
+
+@ovl.operator()
+def reorder(input0):
+    pos = ovl.position_in(input0.shape)
+    output3 = ovl.output_like(input0)
+    output0 = ovl.output_like(input0)
+    output2 = ovl.output_like(input0)
+    output1 = ovl.output_like(input0)
+    inp = input0[pos]
+    output0[pos] = 2 * inp
+    output1[pos] = 3 * inp
+    output2[pos] = 4 * inp
+    output3[pos] = 5 * inp
+    return output0, output1, output2, output3
+
+
+@ovl.operator()
+def pad(in0, n=None):
+    rows_in, cols_in = in0.shape
+    rows = rows_in + 2 * n
+    cols = cols_in + 2 * n
+    out = ovl.output([rows, cols], in0.dtype)
+    pos = ovl.position_in([rows, cols])
+    i_row = pos[0]
+    i_col = pos[1]
+    row_in = ovl.variable(i_row, dtype=pos.dtype)
+    col_in = ovl.variable(i_col, dtype=pos.dtype)
+    with ovl.if_(row_in < n):
+        row_in <<= 0
+    with ovl.elif_(row_in >= (rows_in + n)):
+        row_in <<= rows_in - 1
+    with ovl.else_():
+        row_in <<= row_in - n
+    with ovl.if_(col_in < n):
+        col_in <<= 0
+    with ovl.elif_(col_in >= (cols_in + n)):
+        col_in <<= cols_in - 1
+    with ovl.else_():
+        col_in <<= col_in - n
+    out[i_row, i_col] = in0[row_in, col_in]
+    return out
+
+
+@ovl.operator()
+def crop(in0, n=None):
+    rows = in0.shape[0] - 2 * n
+    cols = in0.shape[1] - 2 * n
+    pos = ovl.position_in([rows, cols])
+    i_row = pos[0]
+    i_col = pos[1]
+    out = ovl.output([rows, cols], in0.dtype)
+    out[i_row, i_col] = in0[n + i_row, n + i_col]
+    return out
+
+
+@ovl.operator()
+def local_window_sum(x, width=None):
+    """Worker-local tensor: gather ``width`` neighbours into a local array, then sum it back to front."""
+    n = x.shape[0]
+    out = ovl.output_like(x)
+    pos = ovl.position_in(n)[0]
+    window = ovl.zeros(width, x.dtype)
+    for k in ovl.arange(width):
+        window[k] = x[(pos + ovl.cast(k, ovl.uint32)) % n]
+    acc = ovl.variable(0, x.dtype)
+    for k in ovl.arange(width - 1, -1, -1):
+        acc <<= acc + window[k]
+    out[pos] = acc
+    return out
+
+
+def _simple(name, fcn, max_ulp=0, rel=0.0):
+    return Case(name, fcn, max_ulp=max_ulp, rel=rel)
+
+
+def _stdops_lstm(rng):
+    batches, vec_len = 4, 24
+    concat_arg = rng.standard_normal((batches, 4 * vec_len), dtype=np.float32)
+    c = rng.standard_normal((batches, vec_len), dtype=np.float32)
+    i, j, f, o = all_outputs(stdops.split(concat_arg, split_dim=1, num_split=4))
+    new_c = stdops.mul(c, stdops.sigmoid(f)) + stdops.sigmoid(i) * stdops.tanh(j)
+    new_h = stdops.tanh(new_c) * stdops.sigmoid(o)
+    return [new_c[0], new_h[0]]
+
+
+def _broadcast(rng):
+    a = rng.standard_normal((6, 20), dtype=np.float32)
+    s = np.array([[2.5]], np.float32)
+    return [stdops.mul(a, s)[0], stdops.sub(s, a)[0], stdops.div(a, s)[0], stdops.mod(a, s)[0],
+            stdops.less(a, s)[0], stdops.equal(a, a)[0]]
+
+
+def _concat_ragged(rng):
+    a = rng.standard_normal((3, 4))
+    b = rng.standard_normal((3, 7))
+    c = rng.standard_normal((3, 1))
+    return [stdops.concat(a, b, c, concat_dim=1)[0]]
+
+
+def _split_concat(rng):
+    a = rng.standard_normal((8, 12), dtype=np.float32)
+    parts = all_outputs(stdops.split(a, split_dim=1, num_split=3))
+    return [stdops.concat(parts[2], parts[0], parts[1], concat_dim=0)[0]]
+
+
+def _int_accumulate(rng):
+    b = np.arange(1, 16).reshape(3, 5)
+    return [cumsum(b, axis=0)[0], cumprod(b, axis=0)[0], cumsum(np.arange(1, 6))[0]]
+
+
+def _accumulate_axes(rng):
+    a = rng.random((5, 6, 7))
+    outs = []
+    for axis in range(3):
+        outs.append(cumsum(a, axis=axis)[0])
+        outs.append(cumprod(a, axis=axis)[0])
+    return outs
+
+
+def _accumulate_max(rng):
+    a = rng.standard_normal((9, 130), dtype=np.float32)
+    return [accumulate(a, inner_fcn=lambda acc, x: ovl.maximum(acc, x), axis=1)[0]]
+
+
+def _edge_expm1_log1p(rng):
+    a = np.array([1e-10, -1e-10, 0.0, np.inf], dtype=np.float64)
+    b = np.array([1e-99, -1e-99, 0.0, np.inf], dtype=np.float64)
+    a32 = np.array([1e-10, -1e-10, 0.0, np.inf, -np.inf, 88.0, -104.0, 1e-38, -0.0], dtype=np.float32)
+    return [expm1(a)[0], log1p(b)[0], expm1(a32)[0], log1p(np.abs(a32))[0]]
+
+
+def _odd_sizes(rng):
+    # sizes that are not multiples of the vector width, rank 1 and rank 3
+    a = rng.standard_normal(1001, dtype=np.float32)
+    b = rng.standard_normal((3, 5, 7), dtype=np.float32)
+    return [stdops.tanh(a)[0], stdops.add(b, b)[0], shift_cyclic(a)[0], shift_cyclic(np.array([3.0], np.float32))[0]]
+
+
+CASES = [
+    Case('c1_shift', c1_shift_only),
+    Case('c1_shift_expm1_log1p', c1_shift_expm1_log1p),
+    Case('c2_chain', c2_chain, seed=2),
+    Case('c2_chain_stages', c2_chain_stages, seed=2),
+    Case('c3_cumsum_f32', c3_cumsum_f32, seed=3),
+    Case('c3_cumprod_f32', c3_cumprod_f32, seed=3),
+    Case('c3_cumsum_f64', c3_cumsum_f64, seed=3),
+    Case('c3_cumprod_f64', c3_cumprod_f64, seed=3),
+    Case('c4_lstm', c4_lstm, seed=4),
+    Case('c4_lstm_grad', c4_lstm_grad, seed=4),
+    Case('c5_gather_transpose', c5_gather_transpose, seed=5),
+    _simple('clip', lambda rng: [clip(rng.random(1000), threshold1=0.1, threshold2=0.9)[0]]),
+    _simple('limits_f32', lambda rng: [set_limits(np.array([0], np.float32))[0]]),
+    _simple('limits_f64', lambda rng: [set_limits(np.array([0], np.float64))[0]]),
+    _simple('arange', lambda rng: all_outputs(fill_range(np.random.RandomState(1).uniform(-1, 1, 10)))),
+    _simple('dot', lambda rng: [dot(np.random.RandomState(1).uniform(-1, 1, (100, 10)),
+                                    np.random.RandomState(2).uniform(-1, 1, (100, 10)))[0]]),
+    _simple('multi_output', lambda rng: all_outputs(multi_op(rng.random(5), rng.random(5), rng.random(5)))),
+    _simple('reorder', lambda rng: all_outputs(reorder(rng.random(5)))),
+    _simple('pad_crop', lambda rng: [crop(pad(rng.random((3, 5)), n=2), n=2)[0]]),
+    _simple('local_tensor', lambda rng: [local_window_sum(rng.standard_normal(37, dtype=np.float32), width=5)[0]]),
+    _simple('stdops_lstm', _stdops_lstm),
+    _simple('broadcast', _broadcast),
+    _simple('concat_ragged', _concat_ragged),
+    _simple('split_concat', _split_concat),
+    _simple('int_accumulate', _int_accumulate),
+    _simple('accumulate_axes', _accumulate_axes),
+    _simple('accumulate_max', _accumulate_max),
+    _simple('edge_expm1_log1p', _edge_expm1_log1p, max_ulp=2, rel=1e-12),
+    _simple('odd_sizes', _odd_sizes),
+]
+for _name, _fcn, _np, _kind in UNARY_FLOAT:
+    for _dt in (np.float32, np.float64):
+        CASES.append(_unary_case(_name, _fcn, _kind, _dt))
+for _name, _fcn in BINARY_ALL:
+    for _dt in ALL_DTYPES:
+        CASES.append(_binary_case(_name, _fcn, _dt))
+for _name, _fcn in BINARY_FLOAT:
+    for _dt in (np.float32, np.float64):
+        CASES.append(_binary_case(_name, _fcn, _dt))
+for _dt in (np.float32, np.float64, np.int8, np.int16, np.int32, np.int64):
+    CASES.append(Case('abs_%s' % np.dtype(_dt).name,
+                      (lambda dt: lambda rng: [_unary_op(ovl.absolute)(
+                          (np.random.RandomState(1).uniform(-100, 100, 100)).astype(dt))[0]])(_dt)))
+for _dt in ALL_DTYPES:
+    CASES.append(Case('not_%s' % np.dtype(_dt).name,
+                      (lambda dt: lambda rng: [_unary_op(ovl.logical_not)(
+                          np.random.RandomState(1).randint(0, 2, 100).astype(dt))[0]])(_dt)))
+for _dt in (np.float32, np.float64):
+    for _pname, _p in (('isinf', ovl.isinf), ('isfinite', ovl.isfinite), ('isnan', ovl.isnan)):
+        CASES.append(Case('%s_%s' % (_pname, np.dtype(_dt).name),
+                          (lambda dt, p: lambda rng: [_unary_op(p)(
+                              np.array([1.5, 0, np.nan, np.inf, -np.inf]).astype(dt))[0]])(_dt, _p)))
+
+CASE_BY_NAME = dict((c.name, c) for c in CASES)
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# comparison helpers
+# ----------------------------------------------------------------------------------------------------------------------
+def ulp_distance(a, b):
+    """Element-wise distance in representable values between two float arrays of one dtype (NaN == NaN)."""
+    a = np.ascontiguousarray(a)
+    b = np.ascontiguousarray(b)
+    assert a.dtype == b.dtype and a.shape == b.shape
+    if a.dtype == np.float32:
+        ia = a.view(np.int32).astype(np.int64)
+        ib = b.view(np.int32).astype(np.int64)
+        bias = np.int64(0x80000000)
+    else:
+        ia = a.view(np.int64).astype(np.float64)
+        ib = b.view(np.int64).astype(np.float64)
+        bias = np.float64(2.0 ** 63)
+    ia = np.where(ia < 0, -(ia + bias), ia)
+    ib = np.where(ib < 0, -(ib + bias), ib)
+    dist = np.abs(ia - ib)
+    both_nan = np.isnan(a) & np.isnan(b)
+    return np.where(both_nan, 0, dist)
+
+
+def assert_matches(case, got, ref, what=''):
+    assert got.dtype == ref.dtype, '%s %s: dtype %s vs %s' % (case.name, what, got.dtype, ref.dtype)
+    assert got.shape == ref.shape, '%s %s: shape %s vs %s' % (case.name, what, got.shape, ref.shape)
+    if case.max_ulp == 0 or ref.dtype.kind in 'iu':
+        if ref.dtype.kind == 'f':
+            equal = (got == ref) | (np.isnan(got) & np.isnan(ref))
+            # bit-exact apart from the NaN payload: also the sign of zero must agree
+            equal &= np.signbit(got) == np.signbit(ref)
+        else:
+            equal = got == ref
+        assert equal.all(), '%s %s: %d of %d elements differ (bit-exact expected)' % (
+            case.name, what, int((~equal).sum()), equal.size)
+    elif ref.dtype == np.float64:
+        finite = np.isfinite(ref)
+        assert np.array_equal(got[~finite], ref[~finite], equal_nan=True), case.name + ' non-finite values differ'
+        denom = np.maximum(np.abs(ref[finite]), np.finfo(np.float64).tiny)
+        err = np.abs(got[finite] - ref[finite]) / denom
+        assert err.size == 0 or err.max() <= case.rel, '%s %s: relative error %g > %g' % (
+            case.name, what, err.max(), case.rel)
+    else:
+        dist = ulp_distance(got, ref)
+        assert dist.max() <= case.max_ulp, '%s %s: %g ulp > %d' % (case.name, what, dist.max(), case.max_ulp)
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# ahead-of-time compilation and the smoke check
+# ----------------------------------------------------------------------------------------------------------------------
+def _operators_of(outputs, opt_level):
+    from opveclib_amd.operator import _build_op_dag
+    from opveclib_amd.fusion import _merge_op_dag
+    dag = _build_op_dag(*outputs).proto_dag
+    if opt_level >= 3:
+        dag, _ = _merge_op_dag(dag, None)
+    return list(dag.operators)
+
+
+def prebuild_all(cases=None, workers=8, with_oracle=True):
+    """Compile the HIP library (and the oracle library) of every operator used by the cases and the benchmark."""
+    from concurrent.futures import ThreadPoolExecutor
+    from opveclib_amd import compiler, runtime
+    import oracle
+    import bench
+
+    ops = {}
+    oracle_ops = {}
+    for case in (cases or CASES):
+        outs = case.outputs()
+        for level in (0, 3):
+            for op in _operators_of(outs, level):
+                ops[op.SerializeToString()] = op
+        for op in _operators_of(outs, 0):
+            oracle_ops[op.SerializeToString()] = op
+    for outs in bench.all_workload_outputs():
+        for op in _operators_of(outs, 3):
+            ops[op.SerializeToString()] = op
+
+    compiler.prebuild_mode = True
+    try:
+        with ThreadPoolExecutor(max_workers=workers) as pool:
+            list(pool.map(runtime.build_operator, ops.values()))
+            if with_oracle:
+                list(pool.map(oracle.compile_op, oracle_ops.values()))
+    finally:
+        compiler.prebuild_mode = False
+    return len(ops), len(oracle_ops)
+
+
+def run_case_on_gpu(case, opt_level):
+    import oracle
+    outs = case.outputs()
+    ref = oracle.profile(outs, 1, 0)[0]
+    got = ovl.evaluate(outs, target_language='hip', opt_level=opt_level)
+    got = got if isinstance(got, list) else [got]
+    assert len(got) == len(ref)
+    for n, (g, r) in enumerate(zip(got, ref)):
+        assert_matches(case, g, r, 'output %d opt_level %d' % (n, opt_level))
+
+
+def smoke_check():
+    for name in ('c2_chain', 'c4_lstm', 'c1_shift'):
+        run_case_on_gpu(CASE_BY_NAME[name], 3)

@@ -1,0 +1,76 @@
+"""The C-ABI launcher library: it loads, exports every function its header declares, and reports errors by code."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from opveclib_amd import launcher
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, 'include', 'ovl_launch.h')
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
+    return sorted(set(re.findall(r'\b(ovl_[a-z_0-9]+)\s*\(', text)) - {'ovl_entry_fn'})
+
+
+def test_header_and_binding_agree():
+    assert declared_functions() == sorted(launcher.EXPORTED_SYMBOLS)
+
+
+def test_every_declared_symbol_is_exported(launcher_library):
+    raw = ctypes.CDLL(launcher.library_path)
+    for name in declared_functions():
+        assert hasattr(raw, name), name
+    assert launcher_library.ovl_abi_version() == 1
+
+
+def test_struct_layout_matches_header():
+    # { void* data; int32_t dtype; uint64_t len; } on LP64: 8 + 4 (+4 padding) + 8
+    assert ctypes.sizeof(launcher.OvlTensor) == 24
+    assert launcher.OvlTensor.data.offset == 0
+    assert launcher.OvlTensor.dtype.offset == 8
+    assert launcher.OvlTensor.len.offset == 16
+
+
+def test_dtype_sizes_and_messages(launcher_library):
+    L = launcher_library
+    sizes = {1: 2, 2: 4, 3: 8, 4: 1, 5: 2, 6: 4, 7: 8, 8: 1, 9: 2, 10: 4, 11: 8, 0: 0, 12: 0, 99: 0}
+    for code, size in sizes.items():
+        assert L.ovl_dtype_size(code) == size
+    assert L.ovl_strerror(0) == b'success'
+    for code in range(1, 7):
+        assert len(L.ovl_strerror(code)) > 0
+    assert b'unknown' in L.ovl_strerror(1234)
+
+
+def test_error_codes_without_a_gpu(launcher_library, tmp_path):
+    L = launcher_library
+    handle = ctypes.c_void_p()
+    assert L.ovl_lib_open(b'/nonexistent/operator.so', ctypes.byref(handle)) == launcher.OVL_EOPEN
+    assert b'/nonexistent/operator.so' in L.ovl_last_error()
+    assert L.ovl_lib_open(None, ctypes.byref(handle)) == launcher.OVL_EINVAL
+    assert L.ovl_lib_close(None) == launcher.OVL_EINVAL
+
+    # any shared object opens; a missing entry point is reported, not called
+    assert L.ovl_lib_open(launcher.library_path.encode(), ctypes.byref(handle)) == launcher.OVL_OK
+    fn = launcher.ENTRY_FN()
+    assert L.ovl_lib_sym(handle, b'no_such_operator_generic_hip', ctypes.byref(fn)) == launcher.OVL_ESYMBOL
+    assert L.ovl_launch(handle, b'no_such_operator_generic_hip', None, 0, None, 0, None) == launcher.OVL_ESYMBOL
+    assert L.ovl_lib_close(handle) == launcher.OVL_OK
+
+    null_fn = launcher.ENTRY_FN()
+    assert L.ovl_launch_fn(null_fn, None, 0, None, 0, None) == launcher.OVL_EINVAL
+    assert L.ovl_time(null_fn, None, 0, None, 0, None, 0, None) == launcher.OVL_EINVAL
+    with pytest.raises(launcher.LauncherError):
+        launcher.check(launcher.OVL_EOPEN)
+
+
+def test_missing_launcher_is_a_loud_error(monkeypatch):
+    monkeypatch.setattr(launcher, '_lib', None)
+    monkeypatch.setattr(launcher, 'library_path', '/nonexistent/libovl_launch.so')
+    with pytest.raises(RuntimeError):
+        launcher.library()

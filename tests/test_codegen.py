@@ -1,0 +1,127 @@
+"""HIP code generator: access analysis, template selection and that the generated sources compile for gfx950."""
+import numpy as np
+import pytest
+
+import opveclib_amd as ovl
+from opveclib_amd import hipgen, runtime, stdops, compiler
+from opveclib_amd.hipgen.analysis import DagInfo
+from opveclib_amd.hipgen import map_kernel
+from opveclib_amd.operator import _build_op_dag
+from opveclib_amd.fusion import _merge_op_dag
+from opveclib_amd.examples import shift_cyclic, cumsum, gather_transpose, expm1
+from opveclib_amd.lstm import lstm, lstm_grad
+from tests import cases
+
+
+def fused(outputs):
+    dag, _ = _merge_op_dag(_build_op_dag(*outputs).proto_dag, None)
+    return dag
+
+
+def test_affine_forms_of_tensor_accesses():
+    concat = np.zeros((8, 4 * 16), np.float32)
+    c = np.zeros((8, 16), np.float32)
+    info = DagInfo(lstm(concat, c, forget_bias=1.0).expression_dag)
+    reads = [(t.io_index, a.signature()) for n, t, a in info.tensor_accesses() if n.code == ovl.language.READ_TENSOR]
+    p0, p1 = ('p', 0), ('p', 1)
+    assert reads == [(0, (((p0, 64), (p1, 1)), 0)), (0, (((p0, 64), (p1, 1)), 16)),
+                     (0, (((p0, 64), (p1, 1)), 32)), (0, (((p0, 64), (p1, 1)), 48)),
+                     (1, (((p0, 16), (p1, 1)), 0))]
+    for _, tensor, aff in info.tensor_accesses():
+        assert 0 <= aff.lo and aff.hi < tensor.size
+
+
+def test_modulo_that_cannot_wrap_is_dropped_and_one_that_can_is_not():
+    a = np.zeros((16, 32), np.float32)
+    info = DagInfo(gather_transpose(a, a.reshape(-1), alpha=0.5, stride=3).expression_dag)
+    by_tensor = {}
+    for node, tensor, aff in info.tensor_accesses():
+        by_tensor.setdefault((node.code, tensor.io_index), []).append(aff)
+    gather = by_tensor[(ovl.language.READ_TENSOR, 1)][0]
+    assert gather is not None and gather.signature() == (((('p', 0), 3), (('p', 1), 1)), 0)   # (i*3+j) % 512 == i*3+j
+    scatter = by_tensor[(ovl.language.ASSIGN_TENSOR, 0)][0]
+    assert scatter.signature() == (((('p', 0), 1), (('p', 1), 16)), 0)                        # out[j, i]
+
+    info = DagInfo(shift_cyclic(np.zeros(64, np.float32)).expression_dag)
+    store = [aff for node, _, aff in info.tensor_accesses() if node.code == ovl.language.ASSIGN_TENSOR][0]
+    assert store is None                                                                     # (p+1) % n wraps
+
+
+def test_unsigned_wraparound_is_not_affine():
+    info = DagInfo(cases.pad(np.zeros((3, 5)), n=2).expression_dag)
+    read = [aff for node, _, aff in info.tensor_accesses() if node.code == ovl.language.READ_TENSOR][0]
+    assert read is None             # the row/column come from reassigned variables
+
+
+def test_vector_width_selection():
+    f32 = np.zeros((8, 64), np.float32)
+    assert map_kernel.choose_vec(DagInfo(stdops.add(f32, f32).expression_dag)) == 4
+    f64 = np.zeros((8, 64), np.float64)
+    assert map_kernel.choose_vec(DagInfo(stdops.add(f64, f64).expression_dag)) == 2
+    i8 = np.zeros((8, 64), np.int8)
+    assert map_kernel.choose_vec(DagInfo(stdops.add(i8, i8).expression_dag)) == 16
+    odd = np.zeros((8, 63), np.float32)
+    assert map_kernel.choose_vec(DagInfo(stdops.add(odd, odd).expression_dag)) == 1
+    two = np.zeros((8, 62), np.float32)
+    assert map_kernel.choose_vec(DagInfo(stdops.add(two, two).expression_dag)) == 2
+    # accumulate along the last axis: workers are rows, nothing is contiguous across workers
+    assert map_kernel.choose_vec(DagInfo(cumsum(f32, axis=1).expression_dag)) == 1
+
+
+def test_chain8_kernel_shape():
+    a = np.zeros((64, 256), np.float32)
+    s = np.array([1.0001], np.float32)
+    dag = fused([cases.chain8(a, a.copy(), s)[-1][0]])
+    gen = hipgen.generate(dag.operators[0], 'f' + '0' * 56)
+    assert gen.launch['template'] == 'map' and gen.launch['vec'] == 4
+    assert gen.launch['vector_loads'] == 2          # A and B once each, although B is used twice
+    assert gen.launch['vector_stores'] == 1         # stores under if/elif/else chains still become one vector store
+    assert gen.algorithmic_bytes == 3 * a.size * 4 + 4
+    assert gen.entry == 'f' + '0' * 56 + '_generic_hip'
+    assert 'ovl_tanhf' in gen.source and 'ovl_expf' in gen.source and 'ovl_logf' in gen.source
+
+
+def test_conditional_store_without_else_stays_scalar():
+    @ovl.operator()
+    def maybe(x):
+        out = ovl.output_like(x)
+        pos = ovl.position_in(x.shape)
+        with ovl.if_(x[pos] > 0):
+            out[pos] = x[pos]
+        return out
+    gen = hipgen.generate(maybe(np.zeros((4, 64), np.float32)).expression_dag, 'f' + '1' * 56)
+    assert gen.launch['vector_loads'] == 1 and gen.launch['vector_stores'] == 0
+
+
+@pytest.mark.parametrize('name', ['c1_shift', 'c2_chain', 'c3_cumsum_f64', 'c4_lstm_grad', 'c5_gather_transpose',
+                                  'local_tensor', 'concat_ragged', 'dot', 'binary_mod_int8', 'unary_tan_float64'])
+def test_generated_sources_compile(name):
+    outs = cases.CASE_BY_NAME[name].outputs()
+    for op in fused(outs).operators:
+        gen, so_path = runtime.build_operator(op)
+        assert so_path.endswith('_generic_hip.so')
+        assert compiler.find_library(gen.source) == so_path
+
+
+def test_entry_point_validates_before_touching_the_gpu(launcher_library):
+    """Argument checks of a generated entry point run on the host, so they can be exercised without a device."""
+    import ctypes
+    from opveclib_amd import launcher
+    a = np.zeros(64, np.float32)
+    gen, so_path = runtime.build_operator(stdops.add(a, a).expression_dag)
+    lib = launcher.OperatorLibrary(so_path, gen.entry, gen.info_symbol)
+    assert lib.info['template'] == 'map' and lib.info['algorithmic_bytes'] == 3 * 64 * 4
+    good = launcher.tensor_array([(4096, 2, 64), (8192, 2, 64)])
+    out = launcher.tensor_array([(12288, 2, 64)])
+    L = launcher_library
+    assert L.ovl_launch_fn(lib.fn, good, 1, out, 1, None) == launcher.OVL_EARGS         # wrong input count
+    assert L.ovl_launch_fn(lib.fn, good, 2, out, 0, None) == launcher.OVL_EARGS         # wrong output count
+    bad_len = launcher.tensor_array([(4096, 2, 63), (8192, 2, 64)])
+    assert L.ovl_launch_fn(lib.fn, bad_len, 2, out, 1, None) == launcher.OVL_EARGS
+    bad_type = launcher.tensor_array([(4096, 3, 64), (8192, 2, 64)])
+    assert L.ovl_launch_fn(lib.fn, bad_type, 2, out, 1, None) == launcher.OVL_EARGS
+    misaligned = launcher.tensor_array([(4100, 2, 64), (8192, 2, 64)])
+    assert L.ovl_launch_fn(lib.fn, misaligned, 2, out, 1, None) == launcher.OVL_EALIGN
+    with pytest.raises(launcher.LauncherError) as err:
+        lib.launch(bad_len, 2, out, 1, None)
+    assert err.value.code == launcher.OVL_EARGS

@@ -1,0 +1,488 @@
+"""
+Operator front-end: tracing semantics, the operator-DAG builder, gradient capture and the fusion optimizer.
+Behaviours pinned by the reference in opveclib/test/test_operator.py:30-278 and test_operator_merge.py:186-393;
+numerical checks run on the CPU oracle.
+"""
+import numpy as np
+import pytest
+
+import opveclib_amd as ovl
+import oracle
+from opveclib_amd import language as lang
+from opveclib_amd import stdops
+from opveclib_amd.operator import _build_op_dag, _Operator, OperatorOutput, _op_hash
+from opveclib_amd.fusion import _MergeRef, _get_merge_refs_for_op_dag, _group_merge_refs, _merge_op_dag
+from opveclib_amd.examples import expm1, log1p, cumsum
+from tests import cases
+
+
+def index_by_id(items, item):
+    for n, cur in enumerate(items):
+        if cur is item:
+            return n
+    raise ValueError('not found')
+
+
+@ovl.operator()
+def add_one(x, y):
+    assert x.shape == y.shape
+    a = ovl.output_like(x)
+    b = ovl.output_like(y)
+    pos = ovl.position_in(a.shape)
+    a[pos] = x[pos] + 1
+    b[pos] = y[pos] + 1
+    return a, b
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# DAG builder
+# ----------------------------------------------------------------------------------------------------------------------
+def test_dag_builder_simple():
+    in0 = np.random.random(10)
+    in1 = np.random.random(10)
+    a1, b1 = add_one(in0, in1)
+    a2, b2 = add_one(a1, b1)
+    op_dag = _build_op_dag(a2, b2)
+    dag, inputs, operators = op_dag.proto_dag, op_dag.inputs, op_dag.operators
+
+    first = index_by_id(operators, a1.parent)
+    refs = dag.references[first].input_refs
+    assert refs[0].is_leaf is True and inputs[refs[0].dag_input_index] is in0
+    assert refs[1].is_leaf is True and inputs[refs[1].dag_input_index] is in1
+    second = index_by_id(operators, a2.parent)
+    assert second > first
+    refs = dag.references[second].input_refs
+    assert refs[0].is_leaf is False and refs[0].op_index == first and refs[0].op_output_index == 0
+    assert refs[1].op_index == first and refs[1].op_output_index == 1
+    assert [(o.op_index, o.op_output_index) for o in dag.dag_outputs] == [(second, 0), (second, 1)]
+
+    r1, s1, r2, s2 = oracle.evaluate([a1, b1, a2, b2])
+    assert np.all(r1 == in0 + 1) and np.all(s1 == in1 + 1) and np.all(r2 == in0 + 2) and np.all(s2 == in1 + 2)
+
+
+def test_dag_builder_complex():
+    in0, in1, in2 = np.random.random(10), np.random.random(10), np.random.random(10)
+    a, b = add_one(in0, in1)
+    c, d = add_one(a, in1)
+    e, f = add_one(in1, b)
+    g, h = add_one(f, a)
+    i, j = add_one(e, in2)
+
+    op_dag = _build_op_dag(i, h)
+    dag, inputs, operators = op_dag.proto_dag, op_dag.inputs, op_dag.operators
+    with pytest.raises(ValueError):
+        index_by_id(operators, c.parent)        # nothing requested depends on c or d
+
+    first = index_by_id(operators, a.parent)
+    second = index_by_id(operators, e.parent)
+    third = index_by_id(operators, g.parent)
+    fourth = index_by_id(operators, i.parent)
+    assert first < second < third and fourth > second
+    r = dag.references[second].input_refs
+    assert r[0].is_leaf is True and inputs[r[0].dag_input_index] is in1
+    assert r[1].is_leaf is False and (r[1].op_index, r[1].op_output_index) == (first, 1)
+    r = dag.references[third].input_refs
+    assert (r[0].op_index, r[0].op_output_index) == (second, 1)
+    assert (r[1].op_index, r[1].op_output_index) == (first, 0)
+    r = dag.references[fourth].input_refs
+    assert (r[0].op_index, r[0].op_output_index) == (second, 0)
+    assert r[1].is_leaf is True and inputs[r[1].dag_input_index] is in2
+    # in1 feeds two operators but is one DAG input
+    assert sum(1 for x in inputs if x is in1) == 1
+    assert len(dag.dag_input_types) == len(inputs)
+
+
+def test_only_operator_outputs_build_a_dag():
+    with pytest.raises(TypeError):
+        _build_op_dag(np.zeros(3))
+    multi = add_one(np.zeros(3), np.zeros(3))
+    with pytest.raises(ValueError):
+        _build_op_dag(multi)                    # ambiguous: index an output
+    with pytest.raises(IndexError):
+        multi[2]
+    assert isinstance(multi, _Operator) and isinstance(multi[1], OperatorOutput)
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# tracing semantics
+# ----------------------------------------------------------------------------------------------------------------------
+def test_outputs_are_numbered_in_return_order():
+    a = np.random.random(5)
+    op = cases.reorder(a)
+    outs = [e for e in op.expression_dag.expressions if e.code == lang.OUTPUT]
+    assert [e.io_index for e in outs] == [0, 1, 2, 3]       # declarations are permuted into return order
+    o0, o1, o2, o3 = oracle.evaluate(cases.all_outputs(op))
+    assert np.array_equal(o0, 2 * a) and np.array_equal(o1, 3 * a)
+    assert np.array_equal(o2, 4 * a) and np.array_equal(o3, 5 * a)
+
+
+def test_output_count_and_type_errors():
+    a = np.random.random(5)
+
+    @ovl.operator()
+    def too_few(input0):
+        pos = ovl.position_in(input0.shape)
+        o0 = ovl.output_like(input0)
+        o1 = ovl.output_like(input0)
+        o0[pos] = input0[pos]
+        o1[pos] = input0[pos]
+        return o0
+
+    @ovl.operator()
+    def no_outputs(input0):
+        pos = ovl.position_in(input0.shape)
+        o0 = ovl.output_like(input0)
+        o0[pos] = 2 * input0[pos]
+
+    @ovl.operator()
+    def bad_return(input0):
+        pos = ovl.position_in(input0.shape)
+        value = input0[pos]
+        o0 = ovl.output_like(input0)
+        o0[pos] = 2 * value
+        return value
+
+    with pytest.raises(ValueError):
+        too_few(a)
+    with pytest.raises(ValueError):
+        no_outputs(a)
+    with pytest.raises(TypeError):
+        bad_return(a)
+
+
+def test_variable_rebinding_is_a_syntax_error():
+    with pytest.raises(SyntaxError):
+        @ovl.operator()
+        def bad(data_in):
+            out = ovl.output_like(data_in)
+            pos = ovl.position_in(data_in)
+            a = ovl.variable(0, dtype=data_in.dtype)
+            a = 2
+            out[pos] = a
+            return out
+
+    with pytest.raises(SyntaxError):
+        @ovl.operator()
+        def bad2(data_in):
+            out = ovl.output_like(data_in)
+            pos = ovl.position_in(data_in)
+            a = ovl.variable(0, dtype=data_in.dtype)
+            a = a + data_in[pos]
+            out[pos] = a
+            return out
+
+    @ovl.operator()
+    def good(data_in):
+        out = ovl.output_like(data_in)
+        pos = ovl.position_in(data_in.shape)
+        a = ovl.variable(0, dtype=data_in.dtype)
+        a <<= a + data_in[pos]
+        b = 3
+        b = 4
+        out[pos] = a * b
+        return out
+    x = np.arange(4.0)
+    assert np.array_equal(oracle.evaluate(good(x)), 4 * x)
+
+
+def test_constants_and_argument_errors():
+    @ovl.operator()
+    def scale(x, factor=None):
+        out = ovl.output_like(x)
+        pos = ovl.position_in(x.shape)
+        out[pos] = x[pos] * factor
+        return out
+
+    x = np.arange(4.0)
+    with pytest.raises(ValueError):
+        scale(x)                            # factor left as None
+    with pytest.raises(TypeError):
+        scale(x, x, factor=1.0)             # too many tensors
+    with pytest.raises(TypeError):
+        scale(3.0, factor=2.0)              # a number is not a tensor
+    assert np.array_equal(oracle.evaluate(scale(x, factor=2.5)), 2.5 * x)
+    assert scale(x, factor=2.0).expression_dag != scale(x, factor=3.0).expression_dag
+    assert _op_hash(scale(x, factor=2.0).expression_dag) == _op_hash(scale(x, factor=2.0).expression_dag)
+
+    @ovl.operator(forbid_none_valued_constants=False)
+    def optional(x, flag=None):
+        out = ovl.output_like(x)
+        pos = ovl.position_in(x.shape)
+        out[pos] = x[pos] if flag is None else x[pos] + flag
+        return out
+    assert np.array_equal(oracle.evaluate(optional(x)), x)
+
+
+def test_infix_operators_on_lazy_outputs():
+    a = np.random.default_rng(0).standard_normal(7)
+    b = np.random.default_rng(1).standard_normal(7)
+    expr = (stdops.add(a, b) - a) * stdops.neg(b) / stdops.add(a, a)
+    assert np.array_equal(oracle.evaluate(expr), ((a + b) - a) * (-b) / (a + a))
+    with pytest.raises(SyntaxError):
+        add_one(a, b) + a                   # multi-output operators need an explicit index
+    with pytest.raises(SyntaxError):
+        bool(stdops.add(a, b)[0])
+
+
+def test_evaluate_rejects_other_targets():
+    with pytest.raises(ValueError):
+        ovl.evaluate(stdops.add(np.zeros(3), np.zeros(3)), target_language='cpp')
+    with pytest.raises(ValueError):
+        ovl.profile(stdops.add(np.zeros(3), np.zeros(3)), 'hip', 0, 3)
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# gradients
+# ----------------------------------------------------------------------------------------------------------------------
+def test_gradient_dag_capture():
+    x = np.random.default_rng(0).standard_normal((3, 4))
+    y = np.random.default_rng(1).standard_normal((3, 4))
+    op = stdops.mul(x, y)
+    grad = op.grad_dag
+    assert grad is not None
+    # gradient DAG inputs: the operator's inputs, then one gradient per output
+    assert len(grad.dag_input_types) == 3
+    assert len(grad.dag_outputs) == 2
+    assert [op_.name for op_ in grad.operators] == ['mul_grad']
+    # neg_grad ignores its first argument but the signature still lists it
+    neg_op = stdops.neg(x)
+    assert len(neg_op.grad_dag.dag_input_types) == 2
+    leaf = [r.dag_input_index for r in neg_op.grad_dag.references[0].input_refs]
+    assert leaf == [0, 1]
+    # operators applied while tracing a gradient do not carry gradient DAGs of their own
+    split_op = stdops.split(np.zeros((2, 6)), split_dim=1, num_split=3)
+    assert split_op.grad_dag is not None and [o.name for o in split_op.grad_dag.operators] == ['concat']
+    with pytest.raises(TypeError):
+        ovl.gradient(lambda x: x)
+    with pytest.raises(ValueError):
+        ovl.gradient(stdops.mul)(lambda *a: None)       # already has a gradient
+
+
+def test_gradient_dag_evaluates():
+    # rebuild operators from a captured gradient DAG and run them: d(x*y) = (y*g, x*g)
+    rng = np.random.default_rng(2)
+    x, y, g = rng.standard_normal((3, 4)), rng.standard_normal((3, 4)), rng.standard_normal((3, 4))
+    dx, dy = oracle.evaluate(stdops.mul_grad(x, y, g))
+    assert np.array_equal(dx, y * g) and np.array_equal(dy, x * g)
+    dx, dy = oracle.evaluate(stdops.div_grad(x, y, g))
+    assert np.allclose(dx, g / y) and np.allclose(dy, -x / (y * y) * g)
+    ds = oracle.evaluate(stdops.sigmoid_grad(x, g))
+    sg = 1 / (1 + np.exp(-x))
+    assert np.allclose(ds, sg * (1 - sg) * g)
+    assert np.allclose(oracle.evaluate(stdops.tanh_grad(x, g)), (1 - np.tanh(x) ** 2) * g)
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# fusion
+# ----------------------------------------------------------------------------------------------------------------------
+@ovl.operator()
+def t_add(in0, in1):
+    assert in0.shape == in1.shape
+    i = ovl.position_in(in0.shape)
+    s = ovl.output(in0.shape, in0.dtype)
+    s[i] = in0[i] + in1[i]
+    return s
+
+
+@ovl.operator()
+def t_mul(in0, in1):
+    i = ovl.position_in(in0.shape)
+    p = ovl.output(in0.shape, in0.dtype)
+    p[i] = in0[i] * in1[i]
+    return p
+
+
+@ovl.operator()
+def t_split(in0):
+    assert in0.shape[0] == 4
+    n_col = in0.shape[1]
+    i_col = ovl.position_in(n_col)
+    rows = [ovl.output(n_col, in0.dtype) for _ in range(4)]
+    for r in range(4):
+        rows[r][i_col] = in0[r, i_col]
+    return rows
+
+
+@ovl.operator()
+def t_concatenate(op0, op1, op2):
+    n_col = op0.shape[0]
+    i_col = ovl.position_in(n_col)
+    concat = ovl.output([3, n_col], op0.dtype)
+    concat[0, i_col] = op0[i_col]
+    concat[1, i_col] = op1[i_col]
+    concat[2, i_col] = op2[i_col]
+    return concat
+
+
+@ovl.operator()
+def t_cum_sum_rows(in0):
+    n_row, n_col = in0.shape
+    i_col = ovl.position_in(n_col)
+    accum = ovl.variable(0, in0.dtype)
+    out = ovl.output_like(in0)
+    for i_row in ovl.arange(n_row):
+        accum <<= accum + in0[i_row, i_col]
+        out[i_row, i_col] = accum
+    return out
+
+
+@ovl.operator()
+def t_cum_sum_cols(in0):
+    n_row, n_col = in0.shape
+    i_row = ovl.position_in(n_row)
+    accum = ovl.variable(0, in0.dtype)
+    out = ovl.output_like(in0)
+    for i_col in ovl.arange(n_col):
+        accum <<= accum + in0[i_row, i_col]
+        out[i_row, i_col] = accum
+    return out
+
+
+@ovl.operator()
+def t_mat_mul(in0, in1):
+    n_row, n_work = in0.shape
+    n_col = in1.shape[1]
+    pos = ovl.position_in([n_row, n_col])
+    out = ovl.output([n_row, n_col], in0.dtype)
+    accum = ovl.variable(0, dtype=in0.dtype)
+    for k in ovl.arange(n_work):
+        accum <<= accum + in0[pos[0], k] * in1[k, pos[1]]
+    out[pos[0], pos[1]] = accum
+    return out
+
+
+def same_refs(expected, found):
+    return len(expected) == len(found) and all(any(e.same(f) for f in found) for e in expected)
+
+
+def out_expr(op, k):
+    """Index of the OUTPUT expression number k in the operator's expression list."""
+    return [n for n, e in enumerate(op.parent.expression_dag.expressions)
+            if e.code == lang.OUTPUT and e.io_index == k][0]
+
+
+def test_merge_refs_split_concatenate():
+    in0 = np.random.random([4, 5])
+    row0, row1, row2, row3 = cases.all_outputs(t_split(in0))    # op 0
+    sum0 = t_add(row0, row1)                                    # op 1
+    sum1 = t_add(row2, row3)                                    # op 2
+    prod0 = t_mul(sum0, sum1)                                   # op 3
+    out0 = t_concatenate(sum0, prod0, sum1)                     # op 4
+    op_dag = _build_op_dag(out0)
+    ops = op_dag.operators
+    assert [index_by_id(ops, o.parent) for o in (row0, sum0[0], sum1[0], prod0[0], out0[0])] == [0, 1, 2, 3, 4]
+    s_out = out_expr(sum0[0], 0)
+    p_out = out_expr(prod0[0], 0)
+    # to_in_expr_index is the INPUT expression of the argument the edge feeds: arguments 0, 1, 2 are expressions 0, 1, 2
+    expected = [
+        _MergeRef(4, 0, 0, 1, s_out, 0), _MergeRef(4, 1, 1, 3, p_out, 0), _MergeRef(4, 2, 2, 2, s_out, 0),
+        _MergeRef(3, 0, 0, 1, s_out, 0), _MergeRef(3, 1, 1, 2, s_out, 0),
+        _MergeRef(2, 0, 0, 0, out_expr(row2, 2), 2), _MergeRef(2, 1, 1, 0, out_expr(row3, 3), 3),
+        _MergeRef(1, 0, 0, 0, out_expr(row0, 0), 0), _MergeRef(1, 1, 1, 0, out_expr(row1, 1), 1)]
+    found = _get_merge_refs_for_op_dag(op_dag.proto_dag)
+    assert same_refs(expected, found)
+    # only consumers fed by a single producer can be grouped: the two adds (from the split)
+    assert sorted(_group_merge_refs(op_dag.proto_dag, found)) == [(1, 0), (2, 0)]
+
+
+def test_merge_refs_multiple_outputs():
+    in0 = np.random.random([4, 4])
+    mmm0 = t_mat_mul(in0, in0)                                  # op 0
+    s0, s1, s2, s3 = cases.all_outputs(t_split(mmm0))           # op 1
+    sum0 = t_add(s0, s1)                                        # op 2
+    sum1 = t_add(s2, s3)                                        # op 3
+    op_dag = _build_op_dag(sum0, sum1)
+    expected = [
+        _MergeRef(3, 0, 0, 1, out_expr(s2, 2), 2), _MergeRef(3, 1, 1, 1, out_expr(s3, 3), 3),
+        _MergeRef(2, 0, 0, 1, out_expr(s0, 0), 0), _MergeRef(2, 1, 1, 1, out_expr(s1, 1), 1)]
+    assert same_refs(expected, _get_merge_refs_for_op_dag(op_dag.proto_dag))
+
+
+def test_no_merge_cases():
+    # a tensor written and read at loop-dependent indices cannot live in a scalar
+    nested = t_cum_sum_rows(t_cum_sum_rows(np.random.random([3, 5])))
+    assert _get_merge_refs_for_op_dag(_build_op_dag(nested).proto_dag) == []
+    # different workgroup shapes
+    c_col = t_cum_sum_cols(t_cum_sum_rows(np.random.random([3, 5])))
+    assert _get_merge_refs_for_op_dag(_build_op_dag(c_col).proto_dag) == []
+    # same workgroup shape, different access pattern
+    c_sym = t_cum_sum_cols(t_cum_sum_rows(np.random.random([3, 3])))
+    assert _get_merge_refs_for_op_dag(_build_op_dag(c_sym).proto_dag) == []
+    mm = t_cum_sum_cols(t_mat_mul(np.random.random([3, 5]), np.random.random([5, 2])))
+    assert _get_merge_refs_for_op_dag(_build_op_dag(mm).proto_dag) == []
+    a = np.random.random([3, 5])
+    cropped = cases.crop(cases.pad(a, n=2), n=2)
+    assert _get_merge_refs_for_op_dag(_build_op_dag(cropped).proto_dag) == []
+    assert np.allclose(a, oracle.evaluate(cropped, opt_level=3))
+    # broadcast across the edge: shapes differ
+    s = stdops.mul(stdops.add(np.ones((1,)), np.ones((1,))), np.ones((4,)))
+    assert _get_merge_refs_for_op_dag(_build_op_dag(s).proto_dag) == []
+    # the shift writes at (p+1) mod n, the consumer reads at p
+    from opveclib_amd.examples import shift_cyclic
+    sh = expm1(shift_cyclic(np.zeros(8, np.float32)))
+    assert _get_merge_refs_for_op_dag(_build_op_dag(sh).proto_dag) == []
+
+
+def fused_equals_unfused(outputs, expected_ops=None):
+    outputs = outputs if isinstance(outputs, list) else [outputs]
+    unfused = oracle.profile(outputs, 1, 0)[0]
+    fused = oracle.profile(outputs, 1, 3)[0]
+    for u, f in zip(unfused, fused):
+        assert np.array_equal(u, f, equal_nan=True)
+    if expected_ops is not None:
+        merged, _ = _merge_op_dag(_build_op_dag(*outputs).proto_dag, None)
+        assert len(merged.operators) == expected_ops, [o.name for o in merged.operators]
+    return unfused
+
+
+def test_fusion_preserves_results_bitwise():
+    rng = np.random.default_rng(3)
+    in0, in1, in2, in3 = (rng.random(5) for _ in range(4))
+    sum0 = t_add(in0, in1)
+    sum1 = t_add(sum0, in2)
+    fused_equals_unfused(sum1, expected_ops=1)
+    fused_equals_unfused([sum0, sum1], expected_ops=1)          # sum0 stays an output of the merged operator
+
+    m = rng.random([4, 5])
+    row0, row1, row2, row3 = cases.all_outputs(t_split(m))
+    s0 = t_add(row0, row1)
+    s1 = t_add(row2, row3)
+    p0 = t_mul(s0, s1)
+    fused_equals_unfused(t_concatenate(s0, p0, s1))
+
+    t0 = t_add(in1, in2)
+    fused_equals_unfused([t_add(in0, t0), t_add(in3, t0)])      # add tree: shared producer
+
+    fused_equals_unfused(cases._stdops_lstm(np.random.default_rng(4)), expected_ops=1)
+
+
+def test_chain8_fuses_into_one_operator():
+    rng = np.random.default_rng(2)
+    a = cases.uniform(rng, -1, 1, (8, 32))
+    b = cases.uniform(rng, -1, 1, (8, 32))
+    s = np.array([1.0001], np.float32)
+    stages = cases.chain8(a, b, s)
+    fused_equals_unfused(stages[-1], expected_ops=1)
+    merged, _ = _merge_op_dag(_build_op_dag(stages[-1]).proto_dag, None)
+    op = merged.operators[0]
+    assert op.name == 'add_mul_tanh_sigmoid_log1p_expm1_sub_absolute'
+    # A, B and the scalar: B is read by add and by sub but is a single argument
+    assert sum(1 for e in op.expressions if e.code == lang.INPUT) == 3
+    assert sum(1 for e in op.expressions if e.code == lang.OUTPUT) == 1
+    assert [(r.is_leaf, r.dag_input_index) for r in merged.references[0].input_refs] == \
+        [(True, 0), (True, 1), (True, 2)]
+    # requesting intermediate stages keeps them as outputs of the one fused operator
+    fused_equals_unfused([t[0] for t in stages], expected_ops=1)
+
+
+def test_multi_store_producers_fuse():
+    x = np.array([1e-10, -1e-10, 0.0, np.inf, 0.5, -0.5, 30.0], dtype=np.float64)
+    fused_equals_unfused(log1p(expm1(x)), expected_ops=1)
+    fused_equals_unfused(expm1(log1p(np.abs(x))), expected_ops=1)
+
+
+def test_merge_is_memoised():
+    a = np.zeros(4)
+    dag = _build_op_dag(t_add(t_add(a, a), a)).proto_dag
+    first = _merge_op_dag(dag, None)
+    assert _merge_op_dag(dag, None) is first

@@ -1,0 +1,115 @@
+"""GPU behaviour of the runtime and the launcher boundary: tensor kinds, timing, poisoning, error reporting."""
+import ctypes
+
+import numpy as np
+import pytest
+
+import opveclib_amd as ovl
+import oracle
+from opveclib_amd import runtime, launcher, stdops
+from opveclib_amd.examples import shift_cyclic, expm1
+from tests import cases
+
+pytestmark = pytest.mark.gpu
+
+
+def test_numpy_in_numpy_out_and_torch_in_torch_out():
+    import torch
+    rng = np.random.default_rng(0)
+    a = rng.standard_normal((16, 64), dtype=np.float32)
+    b = rng.standard_normal((16, 64), dtype=np.float32)
+    out = ovl.evaluate(stdops.add(a, b))
+    assert isinstance(out, np.ndarray) and np.array_equal(out, a + b)
+    ta, tb = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    tout = ovl.evaluate(stdops.add(ta, tb))
+    assert isinstance(tout, torch.Tensor) and tout.is_cuda
+    assert np.array_equal(tout.cpu().numpy(), a + b)
+    mixed = ovl.evaluate(stdops.add(ta, b))
+    assert isinstance(mixed, torch.Tensor)
+    # several outputs come back as a list in request order
+    s, d = ovl.evaluate([stdops.add(a, b), stdops.sub(a, b)])
+    assert np.array_equal(s, a + b) and np.array_equal(d, a - b)
+
+
+def test_views_and_non_contiguous_inputs():
+    import torch
+    base = torch.arange(4 * 70, dtype=torch.float32, device='cuda').reshape(4, 70)
+    shifted = base[:, 1:65]                 # non-contiguous rows
+    offset = base.reshape(-1)[1:257]        # contiguous but not 16-byte aligned
+    assert offset.data_ptr() % 16 != 0
+    out = ovl.evaluate(stdops.add(shifted, shifted))
+    assert torch.equal(out, shifted + shifted)
+    out = ovl.evaluate(stdops.add(offset, offset))
+    assert torch.equal(out, offset + offset)
+
+
+def test_profile_returns_times_per_operator():
+    a = np.random.default_rng(1).standard_normal(1 << 14).astype(np.float32)
+    outs, times = ovl.profile(expm1(shift_cyclic(a)), 'hip', 4, 3)
+    assert len(outs) == 1 and len(times) == 2           # the shift cannot fuse with its consumer
+    for name, ms in times.items():
+        assert name.startswith('f') and ms.shape == (4,) and ms.dtype == np.float64
+        assert np.all(ms > 0) and np.all(ms < 100)
+    ref = oracle.evaluate(expm1(shift_cyclic(a)))
+    assert np.array_equal(outs[0], ref)
+    _, fused_times = ovl.profile(stdops.mul(stdops.add(a, a), a), 'hip', 1, 3)
+    assert len(fused_times) == 1
+    _, unfused_times = ovl.profile(stdops.mul(stdops.add(a, a), a), 'hip', 1, 0)
+    assert len(unfused_times) == 2          # times are keyed by operator hash: two distinct operators
+
+
+def test_poison_marks_unwritten_elements():
+    import torch
+
+    @ovl.operator()
+    def write_evens(x):
+        out = ovl.output_like(x)
+        pos = ovl.position_in(x.shape)
+        with ovl.if_(pos[0] % 2 == 0):
+            out[pos] = x[pos]
+        return out
+
+    runtime.poison_outputs = True
+    try:
+        x = torch.ones(64, dtype=torch.float32, device='cuda')
+        out = ovl.evaluate(write_evens(x)).cpu().numpy()
+    finally:
+        runtime.poison_outputs = False
+    assert np.all(out[0::2] == 1.0)
+    assert np.all(out[1::2].view(np.uint32) == 0xFEFEFEFE)
+
+
+def test_launcher_reports_argument_errors_on_device():
+    import torch
+    a = torch.zeros(256, dtype=torch.float32, device='cuda')
+    compiled = runtime.load_operator(stdops.add(a, a).expression_dag)
+    stream = torch.cuda.current_stream().cuda_stream
+    out = torch.empty(256, dtype=torch.float32, device='cuda')
+    wrong = torch.zeros(256, dtype=torch.float64, device='cuda')
+    with pytest.raises(TypeError):
+        compiled.check_inputs([a, wrong])
+    params_in = launcher.tensor_array([(a.data_ptr(), 2, 256), (wrong.data_ptr(), 3, 256)])
+    params_out = launcher.tensor_array([(out.data_ptr(), 2, 256)])
+    with pytest.raises(launcher.LauncherError) as err:
+        compiled.lib.launch(params_in, 2, params_out, 1, stream)
+    assert err.value.code == launcher.OVL_EARGS
+    # ovl_launch by symbol name gives the same result as the resolved entry point
+    good_in = launcher.tensor_array([(a.data_ptr(), 2, 256), (a.data_ptr(), 2, 256)])
+    L = launcher.library()
+    assert L.ovl_launch(compiled.lib.handle, compiled.gen.entry.encode(), good_in, 2, params_out, 1, stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out, a + a)
+    times = (ctypes.c_double * 3)()
+    assert L.ovl_time(compiled.lib.fn, good_in, 2, params_out, 1, stream, 3, times) == 0
+    assert all(t > 0 for t in times)
+
+
+def test_launch_is_asynchronous_on_the_callers_stream():
+    import torch
+    side = torch.cuda.Stream()
+    a = torch.full((1 << 20,), 2.0, dtype=torch.float32, device='cuda')
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        out = ovl.evaluate(stdops.mul(stdops.add(a, a), a))
+    side.synchronize()
+    assert torch.all(out == 8.0)

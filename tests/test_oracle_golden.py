@@ -1,0 +1,280 @@
+"""
+Pins the CPU oracle (reference-shaped generated C++ + std::thread driver) against the golden vectors and known
+answers that the reference's own tests and documentation hold, and against closed forms.
+
+Each check is chosen so that a plausible mistake in the tracer, the emitter or the driver fails it: wrong index
+stride or order (shift, accumulate tables, gather/transposed scatter), wrong branch hoisting (expm1/log1p edge
+vectors, clip), wrong constant casting (limits, integer division/modulo semantics), wrong block split between host
+threads (every test runs with several thread counts).
+"""
+import numpy as np
+import pytest
+
+import opveclib_amd as ovl
+import oracle
+from opveclib_amd.examples import shift_cyclic, cumsum, cumprod, expm1, log1p, absolute, gather_transpose
+from opveclib_amd.lstm import lstm, lstm_grad
+from opveclib_amd import stdops
+from tests import cases
+
+
+def test_readme_shift_cyclic():
+    # README.rst:63-74: [0, 1, 2, 3, 4] -> [4, 0, 1, 2, 3]
+    a = np.array([0, 1, 2, 3, 4], dtype=np.float32)
+    for threads in (1, 3, 5, 8):
+        out = oracle.evaluate(shift_cyclic(a), num_threads=threads)
+        assert out.dtype == np.float32
+        assert out.tolist() == [4.0, 0.0, 1.0, 2.0, 3.0]
+    x = np.random.default_rng(0).standard_normal(1 << 12).astype(np.float32)
+    assert np.array_equal(oracle.evaluate(shift_cyclic(x)), np.roll(x, 1))
+
+
+def test_accumulate_doctest_tables():
+    # examples/test_accumulate.py:99-109 and 133-143
+    a = np.arange(1, 6)
+    assert oracle.evaluate(cumsum(a)).tolist() == [1, 3, 6, 10, 15]
+    assert oracle.evaluate(cumprod(a)).tolist() == [1, 2, 6, 24, 120]
+    b = np.arange(1, 16).reshape(3, 5)
+    assert oracle.evaluate(cumsum(b, axis=0)).tolist() == [[1, 2, 3, 4, 5], [7, 9, 11, 13, 15], [18, 21, 24, 27, 30]]
+    assert oracle.evaluate(cumprod(b, axis=0)).tolist() == [[1, 2, 3, 4, 5], [6, 14, 24, 36, 50],
+                                                            [66, 168, 312, 504, 750]]
+
+
+def test_accumulate_all_axes_bit_exact_with_numpy():
+    # examples/test_accumulate.py:158-166; numpy's accumulate is strictly sequential, so equality is exact
+    a = np.random.default_rng(1).random((5, 5, 5))
+    for axis in range(3):
+        assert np.array_equal(oracle.evaluate(cumsum(a, axis=axis)), np.cumsum(a, axis=axis))
+        assert np.array_equal(oracle.evaluate(cumprod(a, axis=axis)), np.cumprod(a, axis=axis))
+    f = np.random.default_rng(2).standard_normal((7, 300)).astype(np.float32)
+    assert np.array_equal(oracle.evaluate(cumsum(f, axis=1)), np.cumsum(f, axis=1, dtype=np.float32))
+
+
+def test_expm1_log1p_edge_vectors():
+    # examples/test_expm1.py:88-93 and test_log1p.py:87-92
+    a = np.array([1e-10, -1e-10, 0.0, np.inf], dtype=np.float64)
+    assert np.allclose(np.expm1(a), oracle.evaluate(expm1(a)), rtol=0, atol=1e-20)
+    # the naive formula is visibly wrong on the same vector (test_expm1.py:37-47)
+    assert not np.allclose(np.exp(a[:2]) - 1, np.expm1(a[:2]), rtol=1e-9, atol=0)
+    b = np.array([1e-99, -1e-99, 0.0, np.inf], dtype=np.float64)
+    assert np.allclose(np.log1p(b), oracle.evaluate(log1p(b)), rtol=0, atol=1e-20)
+    x = np.linspace(-0.9, 0.9, 1001)
+    assert np.allclose(oracle.evaluate(log1p(x)), np.log1p(x), rtol=1e-14, atol=0)
+    assert np.allclose(oracle.evaluate(expm1(x)), np.expm1(x), rtol=1e-14, atol=0)
+
+
+def test_clip_exact():
+    # test/test_clip.py:41-46
+    a = np.random.default_rng(3).random(1000)
+    out = oracle.evaluate(cases.clip(a, threshold1=0.1, threshold2=0.9))
+    assert np.all(np.equal(out, np.clip(a, 0.1, 0.9)))
+
+
+def test_limits_exact():
+    # test/test_limits.py:34-39
+    for t in (np.float32, np.float64):
+        out = oracle.evaluate(cases.set_limits(np.array([0]).astype(t)))
+        assert np.all(np.equal(out, np.array([[np.finfo(t).tiny, np.finfo(t).max, np.finfo(t).eps]])))
+
+
+def test_arange_both_directions():
+    # test/test_arange.py:42-52
+    x = np.random.RandomState(1).uniform(-1, 1, 10)
+    right, left = oracle.evaluate(cases.all_outputs(cases.fill_range(x)))
+    ref = x * np.arange(10)
+    assert np.all(right == ref)
+    assert np.all(left == ref)
+
+
+def test_dot_product():
+    # test/test_dot_product.py:40-47
+    rng = np.random.RandomState(1)
+    x = rng.uniform(-1, 1, (100, 10))
+    y = rng.uniform(-1, 1, (100, 10))
+    assert np.allclose(oracle.evaluate(cases.dot(x, y)), np.sum(x * y, axis=1))
+
+
+def test_multiple_outputs_and_reordering():
+    # test/test_multiple_outputs.py:47-54 and test_operator.py:154-182
+    rng = np.random.default_rng(4)
+    a, b, c = rng.random(5), rng.random(5), rng.random(5)
+    o = oracle.evaluate(cases.all_outputs(cases.multi_op(a, b, c)))
+    assert np.array_equal(o[0], a + b) and np.array_equal(o[1], (a + b) * c) and np.array_equal(o[2], a + b + c)
+    o0, o1, o2, o3 = oracle.evaluate(cases.all_outputs(cases.reorder(a)))
+    assert np.array_equal(o0, 2 * a) and np.array_equal(o1, 3 * a)
+    assert np.array_equal(o2, 4 * a) and np.array_equal(o3, 5 * a)
+
+
+def test_pad_crop_round_trip():
+    # test/test_operator_merge.py:262-268
+    a = np.random.default_rng(5).random((3, 5))
+    assert np.array_equal(oracle.evaluate(cases.crop(cases.pad(a, n=2), n=2)), a)
+    padded = oracle.evaluate(cases.pad(a, n=2))
+    assert np.array_equal(padded, np.pad(a, 2, mode='edge'))
+
+
+@pytest.mark.parametrize('dtype', [np.float32, np.float64])
+def test_unary_math_against_numpy(dtype):
+    # test/test_unary_math.py:110-161; the oracle calls the host libm, numpy calls its own routines: allclose
+    for name, fcn, np_fcn, kind in cases.UNARY_FLOAT:
+        x = cases.unary_input(kind, dtype)
+        out = oracle.evaluate(cases._unary_op(fcn)(x))
+        assert out.dtype == dtype
+        assert np.allclose(out, np_fcn(x)), name
+
+
+@pytest.mark.parametrize('dtype', cases.ALL_DTYPES)
+def test_binary_math_against_numpy(dtype):
+    # test/test_binary_math.py:40-105 with C semantics for integer division and modulo (78-90)
+    def truncated_division(a, b):
+        if np.dtype(dtype).kind == 'i':
+            return np.trunc(np.true_divide(a, b)).astype(dtype)
+        if np.dtype(dtype).kind == 'u':
+            return (a // b).astype(dtype)
+        return np.true_divide(a, b).astype(dtype)
+
+    def truncated_mod(a, b):
+        if np.dtype(dtype).kind == 'f':
+            return np.fmod(a, b)
+        return (a - b * np.trunc(np.true_divide(a, b)).astype(dtype)).astype(dtype)
+
+    expected = {
+        'add': lambda a, b: a + b, 'sub': lambda a, b: a - b, 'mul': lambda a, b: a * b,
+        'div': truncated_division, 'mod': truncated_mod,
+        'eq': np.equal, 'ne': np.not_equal, 'or': np.logical_or, 'and': np.logical_and,
+        'lt': np.less, 'le': np.less_equal, 'gt': np.greater, 'ge': np.greater_equal,
+        'min': np.minimum, 'max': np.maximum, 'pow': np.power, 'atan2': np.arctan2}
+    table = list(cases.BINARY_ALL)
+    if np.dtype(dtype).kind == 'f':
+        table += cases.BINARY_FLOAT
+    for name, fcn in table:
+        a, b = cases.binary_inputs(name, dtype)
+        out = oracle.evaluate(cases._binary_op(fcn)(a, b))
+        assert out.dtype == dtype, name
+        with np.errstate(over='ignore'):
+            ref = expected[name](a, b)
+        assert np.allclose(out, ref.astype(dtype)), name
+
+
+def test_predicates_and_not():
+    x = np.array([1.5, 0, np.nan, np.inf, -np.inf])
+    for t in (np.float32, np.float64):
+        xt = x.astype(t)
+        assert np.array_equal(oracle.evaluate(cases._unary_op(ovl.isinf)(xt)), np.isinf(xt).astype(t))
+        assert np.array_equal(oracle.evaluate(cases._unary_op(ovl.isfinite)(xt)), np.isfinite(xt).astype(t))
+        assert np.array_equal(oracle.evaluate(cases._unary_op(ovl.isnan)(xt)), np.isnan(xt).astype(t))
+    bits = np.random.RandomState(1).randint(0, 2, 100)
+    for t in cases.ALL_DTYPES:
+        out = oracle.evaluate(cases._unary_op(ovl.logical_not)(bits.astype(t)))
+        assert np.array_equal(out, np.logical_not(bits).astype(t))
+
+
+def test_stdops_broadcast_and_exact_arithmetic():
+    # stdops/test_math.py:23-89: infix operators on operator outputs vs numpy with exact equality
+    rng = np.random.default_rng(6)
+    a = rng.standard_normal((6, 20)).astype(np.float32)
+    b = rng.standard_normal((6, 20)).astype(np.float32)
+    s = np.array([[2.5]], np.float32)
+    got = oracle.evaluate([stdops.add(a, b)[0], stdops.mul(a, s)[0], stdops.sub(s, a)[0], stdops.div(a, s)[0],
+                           stdops.mod(a, s)[0], stdops.less(a, s)[0], stdops.equal(a, a)[0], stdops.neg(a)[0]])
+    ref = [a + b, a * s, s - a, a / s, np.fmod(a, s), (a < s).astype(np.float32), np.ones_like(a), -a]
+    for g, r in zip(got, ref):
+        assert np.array_equal(g, r)
+    lazy = stdops.add(a, b) * stdops.sub(a, b) - a
+    assert np.array_equal(oracle.evaluate(lazy), (a + b) * (a - b) - a)
+
+
+def test_concat_split():
+    rng = np.random.default_rng(7)
+    a, b, c = rng.standard_normal((3, 4)), rng.standard_normal((3, 7)), rng.standard_normal((3, 1))
+    assert np.array_equal(oracle.evaluate(stdops.concat(a, b, c, concat_dim=1)), np.concatenate([a, b, c], axis=1))
+    x = rng.standard_normal((8, 12)).astype(np.float32)
+    parts = oracle.evaluate(cases.all_outputs(stdops.split(x, split_dim=1, num_split=3)))
+    for p, r in zip(parts, np.split(x, 3, axis=1)):
+        assert np.array_equal(p, r)
+    same = oracle.evaluate(stdops.concat(x, x, concat_dim=0))
+    assert np.array_equal(same, np.concatenate([x, x], axis=0))
+
+
+def test_gather_transpose_brute_force():
+    rng = np.random.default_rng(5)
+    a = rng.standard_normal((24, 40), dtype=np.float32)
+    b = rng.standard_normal((24, 40), dtype=np.float32)
+    out = oracle.evaluate(gather_transpose(a, b.reshape(-1), alpha=0.5, stride=7919))
+    ref = np.empty((40, 24), np.float32)
+    flat = b.reshape(-1)
+    for i in range(24):
+        for j in range(40):
+            ref[j, i] = np.float32(0.5) * a[i, j] + flat[(i * 7919 + j) % flat.size]
+    assert np.array_equal(out, ref)
+
+
+def test_lstm_against_float64_closed_form_and_autograd():
+    # lstm/lstm.py:32-105; gradient cross-checked with torch.autograd on the CPU in float64
+    import torch
+    rng = np.random.default_rng(4)
+    batch, units = 6, 16
+    concat = rng.standard_normal((batch, 4 * units), dtype=np.float32)
+    c = rng.standard_normal((batch, units), dtype=np.float32)
+    dc = rng.standard_normal((batch, units), dtype=np.float32)
+    dh = rng.standard_normal((batch, units), dtype=np.float32)
+    new_c, new_h = oracle.evaluate(cases.all_outputs(lstm(concat, c, forget_bias=1.0)))
+    d_concat, d_c = oracle.evaluate(cases.all_outputs(lstm_grad(concat, c, dc, dh, forget_bias=1.0)))
+
+    tc = torch.tensor(concat, dtype=torch.float64, requires_grad=True)
+    tcp = torch.tensor(c, dtype=torch.float64, requires_grad=True)
+    i, j, f, o = torch.split(tc, units, dim=1)
+    ref_c = tcp * torch.sigmoid(f + 1.0) + torch.sigmoid(i) * torch.tanh(j)
+    ref_h = torch.tanh(ref_c) * torch.sigmoid(o)
+    assert np.allclose(new_c, ref_c.detach().numpy(), rtol=1e-5, atol=1e-6)
+    assert np.allclose(new_h, ref_h.detach().numpy(), rtol=1e-5, atol=1e-6)
+    loss = (ref_c * torch.tensor(dc, dtype=torch.float64)).sum() + (ref_h * torch.tensor(dh, dtype=torch.float64)).sum()
+    loss.backward()
+    assert np.allclose(d_concat, tc.grad.numpy(), rtol=1e-4, atol=1e-5)
+    assert np.allclose(d_c, tcp.grad.numpy(), rtol=1e-4, atol=1e-5)
+
+
+def test_stdops_lstm_equals_fused_lstm():
+    # test_operator_merge.py:311-321: the stdops composition computes the hand-fused cell (forget_bias 0)
+    rng = np.random.default_rng(8)
+    batch, units = 2, 5
+    concat = rng.standard_normal((batch, 4 * units), dtype=np.float32)
+    c = rng.standard_normal((batch, units), dtype=np.float32)
+    i, j, f, o = cases.all_outputs(stdops.split(concat, split_dim=1, num_split=4))
+    new_c = stdops.mul(c, stdops.sigmoid(f)) + stdops.sigmoid(i) * stdops.tanh(j)
+    new_h = stdops.tanh(new_c) * stdops.sigmoid(o)
+    a = oracle.evaluate([new_c, new_h])
+    b = oracle.evaluate(cases.all_outputs(lstm(concat, c, forget_bias=0.0)))
+    assert np.allclose(a[0], b[0], rtol=1e-6, atol=1e-7)
+    assert np.allclose(a[1], b[1], rtol=1e-6, atol=1e-7)
+
+
+def test_chain8_against_numpy():
+    rng = np.random.default_rng(2)
+    a = cases.uniform(rng, -1, 1, (16, 64))
+    b = cases.uniform(rng, -1, 1, (16, 64))
+    s = np.array([1.0001], np.float32)
+    y = oracle.evaluate(cases.chain8(a, b, s)[-1])
+    a64, b64 = a.astype(np.float64), b.astype(np.float64)
+    ref = np.abs(np.expm1(np.log1p(1 / (1 + np.exp(-np.tanh((a64 + b64) * np.float64(np.float32(1.0001))))))) - b64)
+    assert np.allclose(y, ref, rtol=0, atol=5e-7)
+
+
+def test_driver_reports_argument_errors():
+    import ctypes
+    a = np.zeros(8, np.float32)
+    so_path, entry = oracle.compile_op(shift_cyclic(a).expression_dag)
+    lib = oracle.driver()
+    out = np.zeros(8, np.float32)
+    good_in = (oracle.OvlTensor * 1)(oracle.OvlTensor(a.ctypes.data, 2, 8))
+    good_out = (oracle.OvlTensor * 1)(oracle.OvlTensor(out.ctypes.data, 2, 8))
+    assert lib.ovl_cpu_run(so_path.encode(), entry.encode(), good_in, 1, good_out, 1, 2, None, 1) == 0
+    # 0xFE poisoning happened before the run and every element was overwritten
+    assert np.array_equal(out, np.roll(a, 1))
+    bad_len = (oracle.OvlTensor * 1)(oracle.OvlTensor(a.ctypes.data, 2, 7))
+    assert lib.ovl_cpu_run(so_path.encode(), entry.encode(), bad_len, 1, good_out, 1, 2, None, 1) == 1
+    bad_type = (oracle.OvlTensor * 1)(oracle.OvlTensor(a.ctypes.data, 3, 8))
+    assert lib.ovl_cpu_run(so_path.encode(), entry.encode(), bad_type, 1, good_out, 1, 2, None, 1) == 1
+    assert lib.ovl_cpu_run(so_path.encode(), entry.encode(), good_in, 2, good_out, 1, 2, None, 1) == 1
+    assert lib.ovl_cpu_run(so_path.encode(), b'no_such_symbol', good_in, 1, good_out, 1, 2, None, 1) == 3
+    assert lib.ovl_cpu_run(b'/nonexistent/lib.so', entry.encode(), good_in, 1, good_out, 1, 2, None, 1) == 2
