@@ -32,9 +32,16 @@ __device__ __forceinline__ int8_t ovl_abs_8(int8_t x) { return (x < 0) ? -x : x;
 __device__ __forceinline__ int16_t ovl_abs_16(int16_t x) { return (x < 0) ? -x : x; }
 
 // float32 transcendental entry points used by generated code: bit-compatible with the host C library's
-// expf/logf/tanhf (see ovl_math.h)
-__device__ __forceinline__ float ovl_expf(float x) { return ovl_math::expf_(x); }
-__device__ __forceinline__ float ovl_logf(float x) { return ovl_math::logf_(x); }
-__device__ __forceinline__ float ovl_tanhf(float x) { return ovl_math::tanhf_(x); }
+// expf/logf/tanhf (see ovl_math.h).  ovl_exp_tab / ovl_log_tab name the lookup tables in scope: kernels that call
+// exp or log declare them with OVL_DECLARE_MATH_TABLES at their top, pointing at copies in LDS.
+#define ovl_expf(x) ovl_math::expf_((x), ovl_exp_tab)
+#define ovl_logf(x) ovl_math::logf_((x), ovl_log_tab)
+#define ovl_tanhf(x) ovl_math::tanhf_(x)
+
+#define OVL_DECLARE_MATH_TABLES()                                              \
+    __shared__ ovl_math::lds_tables ovl_lds_tables;                            \
+    ovl_math::load_tables(ovl_lds_tables);                                     \
+    const uint64_t* const ovl_exp_tab = ovl_lds_tables.exp2f;                  \
+    const ovl_math::logf_entry* const ovl_log_tab = ovl_lds_tables.logf
 
 #endif  // OVL_DEVICE_H_

@@ -68,7 +68,7 @@ OVL_TABLE uint64_t exp2f_tab[OVL_EXP2F_N] = OVL_EXP2F_TABLE;
 
 OVL_HD uint32_t top12(float x) { return as_u32(x) >> 20; }
 
-OVL_HD float expf_(float x) {
+OVL_HD float expf_(float x, const uint64_t* tab = exp2f_tab) {
     const double InvLn2N = 0x1.71547652b82fep+0 * OVL_EXP2F_N;
     const double Shift = 0x1.8p+52;
     const double C0 = 0x1.c6af84b912394p-5 / OVL_EXP2F_N / OVL_EXP2F_N / OVL_EXP2F_N;
@@ -90,7 +90,7 @@ OVL_HD float expf_(float x) {
     kd -= Shift;
     double r = OVL_MADD(1, InvLn2N, xd, -kd);
     // exp(x) = 2^(k/N) * 2^(r/N) ~= s * (C0*r^3 + C1*r^2 + C2*r + 1)
-    uint64_t t = exp2f_tab[ki % OVL_EXP2F_N];
+    uint64_t t = tab[ki % OVL_EXP2F_N];
     t += ki << (52 - OVL_EXP2F_TABLE_BITS);
     double s = as_f64(t);
     double z2 = OVL_MADD(2, C0, r, C1);
@@ -129,7 +129,23 @@ struct logf_entry { double invc, logc; };
 
 OVL_TABLE logf_entry logf_tab[OVL_LOGF_N] = OVL_LOGF_TABLE;
 
-OVL_HD float logf_(float x) {
+#if defined(__HIPCC__)
+// Copies of both lookup tables in LDS.  Table lookups are per-lane gathers; served from LDS they cost a few cycles,
+// while gathers from global memory occupy the vector memory pipeline that the kernel needs for streaming its tensors.
+struct lds_tables {
+    uint64_t exp2f[OVL_EXP2F_N];
+    logf_entry logf[OVL_LOGF_N];
+};
+
+// Must be called by every thread of the workgroup before any divergent control flow.
+__device__ __forceinline__ void load_tables(lds_tables& t) {
+    if (threadIdx.x < OVL_EXP2F_N) t.exp2f[threadIdx.x] = exp2f_tab[threadIdx.x];
+    if (threadIdx.x < OVL_LOGF_N) t.logf[threadIdx.x] = logf_tab[threadIdx.x];
+    __syncthreads();
+}
+#endif
+
+OVL_HD float logf_(float x, const logf_entry* tab = logf_tab) {
     const double Ln2 = 0x1.62e42fefa39efp-1;
     const double A0 = -0x1.00ea348b88334p-2, A1 = 0x1.5575b0be00b6ap-2, A2 = -0x1.ffffef20a4123p-2;
     const uint32_t Off = 0x3f330000;
@@ -150,8 +166,8 @@ OVL_HD float logf_(float x) {
     int i = (tmp >> (23 - OVL_LOGF_TABLE_BITS)) % OVL_LOGF_N;
     int k = (int32_t)tmp >> 23;
     uint32_t iz = ix - (tmp & (0x1ffu << 23));
-    double invc = logf_tab[i].invc;
-    double logc = logf_tab[i].logc;
+    double invc = tab[i].invc;
+    double logc = tab[i].logc;
     double z = (double)as_f32(iz);
     // log(x) = log1p(z/c-1) + log(c) + k*Ln2
     double r = OVL_MADD(8, z, invc, -1.0);
@@ -246,31 +262,70 @@ OVL_HD float expm1f_(float x) {
     return y;
 }
 
+// tanh in terms of expm1, arranged as straight-line code.  For 2^-55 <= |x| < 22 fdlibm evaluates
+//     |x| >= 1:  1 - 2/(t+2)  with t = expm1( 2|x|),     |x| < 1:  -t/(t+2)  with t = expm1(-2|x|),
+// so expm1 only ever sees arguments in (-2, -2^-54] or [2, 44).  On that domain its overflow/infinity filter does
+// nothing, its |a| < 2^-25 shortcut returns what the k = 0 path returns, and k = 1 cannot occur; what remains is one
+// argument reduction, one polynomial and five short result formulas.  All of them are evaluated and the lane's own
+// one is selected, which costs less on a wavefront than branching five ways; every selected value is produced by
+// exactly the operations fdlibm performs for that case, so results are unchanged (checked against the host C
+// library over all 2^32 arguments).
 OVL_HD float tanhf_(float x) {
     const float one = 1.0f, two = 2.0f, tiny = 1.0e-30f;
-    float t, z;
+    const float ln2_hi = 6.9313812256e-01f, ln2_lo = 9.0580006145e-06f, invln2 = 1.4426950216e+00f;
+    const float Q1 = -3.3333335072e-02f, Q2 = 1.5873016091e-03f, Q3 = -7.9365076090e-05f;
+    const float Q4 = 4.0082177293e-06f, Q5 = -2.0109921195e-07f;
+
     uint32_t jx = as_u32(x);
     uint32_t ix = jx & 0x7fffffffu;
     bool negative = (jx & 0x80000000u) != 0;
 
-    if (ix >= 0x7f800000u) {            // inf or NaN
-        if (!negative) return one / x + one;    // tanh(+inf) = +1, tanh(NaN) = NaN
-        return one / x - one;
+    if (ix >= 0x41b00000u || ix < 0x24000000u) {    // |x| >= 22 (or inf, NaN), |x| < 2**-55 (or zero)
+        if (ix >= 0x7f800000u) return negative ? one / x - one : one / x + one;
+        if (ix >= 0x41b00000u) return negative ? -(one - tiny) : (one - tiny);
+        if (ix == 0) return x;
+        return x * (one + x);
     }
-    if (ix < 0x41b00000u) {             // |x| < 22
-        if (ix == 0) return x;          // +-0
-        if (ix < 0x24000000u) return x * (one + x);     // |x| < 2**-55
-        // |x| >= 1: z = 1 - 2/(t+2) with t = expm1(2|x|);  |x| < 1: z = -t/(t+2) with t = expm1(-2|x|).
-        // Both cases share one expm1 evaluation and one division; each lane performs exactly the operations of
-        // its own case.
-        float ax = as_f32(ix);
-        bool big = ix >= 0x3f800000u;
-        t = expm1f_(big ? two * ax : -two * ax);
-        float q = (big ? two : -t) / (t + two);
-        z = big ? one - q : q;
-    } else {                            // |x| >= 22: +-1 (inexact)
-        z = one - tiny;
-    }
+
+    float ax = as_f32(ix);
+    bool big = ix >= 0x3f800000u;                   // |x| >= 1
+    float a = big ? two * ax : -two * ax;           // argument of expm1
+    uint32_t ha = as_u32(two * ax);                 // bits of |a|
+
+    // argument reduction a = k*ln2 + xr (+ correction c); k = 0 leaves a untouched
+    int32_t kg = (int32_t)(invln2 * a + (big ? 0.5f : -0.5f));
+    int32_t k = (ha > 0x3eb17218u) ? ((ha < 0x3F851592u) ? -1 : kg) : 0;
+    float t = (float)k;
+    float hi = a - t * ln2_hi;
+    float lo = t * ln2_lo;
+    float xr = hi - lo;
+    float c = (hi - xr) - lo;
+
+    float hfx = 0.5f * xr;
+    float hxs = xr * hfx;
+    float r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
+    float t3 = 3.0f - r1 * hfx;
+    float e = hxs * ((r1 - t3) / (6.0f - xr * t3));
+
+    float res0 = xr - (xr * e - hxs);               // k == 0
+    float e2 = xr * (e - c) - c;
+    e2 -= hxs;
+    float d = e2 - xr;
+    float resm1 = 0.5f * (-d) - 0.5f;               // k == -1: 0.5*(xr-e2) - 0.5
+    // k <= -2 or k > 56: (1 - d) * 2^k - 1;  3 <= k < 23: ((1 - 2^-k) - d) * 2^k;  23 <= k <= 56: ((xr-(e2+2^-k))+1) * 2^k
+    bool tail_a = (k <= -2) || (k > 56);
+    bool tail_b = (k >= 0) && (k < 23);
+    uint32_t ks = (uint32_t)k & 31u;
+    float base = tail_b ? as_f32(0x3f800000u - (0x1000000u >> ks)) : one;
+    float y = base - d;
+    float yc = (xr - (e2 + as_f32((uint32_t)(0x7f - k) << 23))) + one;
+    y = (tail_a || tail_b) ? y : yc;
+    y = as_f32(as_u32(y) + ((uint32_t)k << 23));    // add k to y's exponent
+    float resk = tail_a ? y - one : y;
+    float em1 = (k == 0) ? res0 : ((k == -1) ? resm1 : resk);
+
+    float q = (big ? two : -em1) / (em1 + two);
+    float z = big ? one - q : q;
     return negative ? -z : z;
 }
 

@@ -310,6 +310,10 @@ class DagInfo(object):
         return None
 
     # -- queries ---------------------------------------------------------------------------------------------------
+    def uses_math_tables(self):
+        """True when the body calls the table-driven float32 exp or log."""
+        return any(n.code in (lang.EXP, lang.LOG) and n.dtype == lang.FLOAT32 for n in self.nodes)
+
     def tensor_accesses(self):
         """[(node, tensor node, affine or None)] for reads of inputs and stores to outputs, in program order."""
         found = []
