@@ -119,15 +119,22 @@ class BodyEmitter(object):
         return 'e' + str(node.idx) + self.suffix
 
     def emit(self):
+        """All statements of the worker, in order."""
+        return [text for _, text in self.emit_tagged()]
+
+    def emit_tagged(self):
+        """[(index of the expression that produced it, statement text)] in program order."""
         info = self.info
         names = {}
         stmts = []
         indent = 0
+        current = [0]
 
         def put(text):
-            stmts.append('    ' * indent + text)
+            stmts.append((current[0], '    ' * indent + text))
 
         for node in info.nodes:
+            current[0] = node.idx
             code = node.code
             ops = node.ops
             name = 'e' + str(node.idx) + self.suffix

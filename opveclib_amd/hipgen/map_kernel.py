@@ -85,6 +85,19 @@ def _is_vector_access(info, node, tensor, aff, vec):
     return True
 
 
+def contiguous_unaligned(info, node, tensor, aff, vec):
+    """Unit stride along the last workgroup dimension, but the vector's first element may sit at any element
+    offset (e.g. a gather row that starts at i*7919): one 128-bit load with element alignment instead of VEC loads."""
+    if aff is None or not aff.only_position() or info.in_loop[node.idx]:
+        return False
+    last = len(info.workgroup_shape) - 1
+    if aff.coeff(('p', last)) != 1:
+        return False
+    if aff.lo < 0 or aff.hi >= tensor.size:
+        return False
+    return not _is_vector_access(info, node, tensor, aff, vec)
+
+
 def generate(info, kernel_name, vec=None):
     """
     :return: (kernel source text, launch description dict) for the map template.
@@ -98,6 +111,7 @@ def generate(info, kernel_name, vec=None):
 
     accesses = info.tensor_accesses()
     loads = {}      # (input node idx, signature) -> Access
+    unaligned = {}  # same, for loads that are contiguous but only element aligned
     stores = {}     # (output node idx, signature) -> Access
     store_keys = []
     for node, tensor, aff in accesses:
@@ -108,6 +122,10 @@ def generate(info, kernel_name, vec=None):
                     loads[key] = Access(tensor, aff, 'ld%d' % len(loads))
             else:
                 store_keys.append(key)
+        elif vec > 1 and node.code == lang.READ_TENSOR and contiguous_unaligned(info, node, tensor, aff, vec):
+            key = (tensor.idx, aff.signature())
+            if key not in unaligned:
+                unaligned[key] = Access(tensor, aff, 'lu%d' % len(unaligned))
     certain = info.definitely_stores(store_keys)
     for node, tensor, aff in accesses:
         if node.code == lang.ASSIGN_TENSOR and aff is not None:
@@ -118,7 +136,7 @@ def generate(info, kernel_name, vec=None):
     def read_hook(node, tensor, index_name):
         aff = info.affine[node.ops[1]]
         if aff is not None:
-            acc = loads.get((tensor.idx, aff.signature()))
+            acc = loads.get((tensor.idx, aff.signature())) or unaligned.get((tensor.idx, aff.signature()))
             if acc is not None and not info.in_loop[node.idx]:
                 return acc.reg + '[lane]'
         return None
@@ -145,11 +163,13 @@ def generate(info, kernel_name, vec=None):
 
     src = []
     vec_types = {}
-    for acc in list(loads.values()) + list(stores.values()):
+    for acc in list(loads.values()) + list(stores.values()) + list(unaligned.values()):
         ctype = CTYPE[acc.tensor.dtype]
-        vec_types[ctype] = 'ovl_' + ctype.replace(' ', '_') + 'x' + str(vec)
-    for ctype, vname in sorted(vec_types.items()):
+        vec_types[ctype] = ('ovl_' + ctype.replace(' ', '_') + 'x' + str(vec), ITEMSIZE[acc.tensor.dtype])
+    for ctype, (vname, itemsize) in sorted(vec_types.items()):
         src.append('typedef ' + ctype + ' ' + vname + ' __attribute__((ext_vector_type(' + str(vec) + ')));')
+        src.append('typedef ' + vname + ' ' + vname + '_u __attribute__((aligned(' + str(itemsize) + ')));')
+    vec_types = dict((k, v[0]) for k, v in vec_types.items())
     src.append('')
     src.append('extern "C" __global__ void __launch_bounds__(%d)' % BLOCK)
     src.append(kernel_name + '(' + ', '.join(args) + ') {')
@@ -175,6 +195,11 @@ def generate(info, kernel_name, vec=None):
         vname = vec_types[CTYPE[acc.tensor.dtype]]
         wide = acc.aff.hi >= 2 ** 32
         src.append('        const %s %s = __builtin_nontemporal_load(reinterpret_cast<const %s*>(in%d + (%s)));' % (
+            vname, acc.reg, vname, acc.tensor.io_index, _index_expr(acc.aff, pos_names, wide)))
+    for acc in unaligned.values():
+        vname = vec_types[CTYPE[acc.tensor.dtype]]
+        wide = acc.aff.hi >= 2 ** 32
+        src.append('        const %s %s = *reinterpret_cast<const %s_u*>(in%d + (%s));' % (
             vname, acc.reg, vname, acc.tensor.io_index, _index_expr(acc.aff, pos_names, wide)))
     for acc in stores.values():
         src.append('        %s %s;' % (vec_types[CTYPE[acc.tensor.dtype]], acc.reg))
@@ -211,7 +236,7 @@ def generate(info, kernel_name, vec=None):
         'block': BLOCK,
         'blocks_needed': (num_vectors + BLOCK - 1) // BLOCK,
         'align': align,
-        'vector_loads': len(loads),
+        'vector_loads': len(loads) + len(unaligned),
         'vector_stores': len(stores),
     }
     return '\n'.join(src) + '\n', launch

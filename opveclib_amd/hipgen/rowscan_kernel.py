@@ -1,0 +1,289 @@
+"""
+The row-scan kernel template: operators that walk the last axis of a tensor with a loop-carried accumulator
+(``accumulate`` / ``cumsum`` / ``cumprod`` of the reference's opveclib/examples/test_accumulate.py:22-147 along the last
+axis).
+
+The worker function is a strictly sequential recurrence per row (``acc = f(acc, x[row, i]); out[row, i] = acc`` for
+i = 1 .. L-1), so the order of the floating point operations is part of the result and must be kept: lane = row.  In
+the one-worker-per-thread template neighbouring lanes then read addresses a whole row apart.  Here a 256-thread
+workgroup owns ``ROWS`` consecutive rows and streams them through LDS in chunks of ``CHUNK`` columns with three
+rotating buffers:
+
+  * wavefronts 1-3 move data: 128-bit coalesced loads of chunk k+1 from global memory into LDS, and 128-bit
+    coalesced stores of the finished chunk k-1 from LDS to global memory;
+  * wavefront 0 scans chunk k in place in LDS: lane r walks row r left to right, four (float32) or two (float64)
+    columns per 128-bit LDS access, running the operator's own loop body for every column in order.
+
+One workgroup barrier separates the chunks.  The arithmetic each row sees is exactly the worker's sequential
+recurrence, so results equal the generic template's (and numpy's accumulate) bit for bit; all global traffic is
+coalesced and every element is read and written once.
+"""
+
+from .. import language as lang
+from .analysis import ITEMSIZE
+from .body import BodyEmitter, CTYPE
+
+BLOCK = 256
+WAVE = 64
+MOVERS = BLOCK - WAVE
+LDS_BUDGET = 128 * 1024
+NUM_CU = 256
+
+
+class ScanPlan(object):
+    def __init__(self, loop_item, counter, length, rows, x, out, vec, rows_per_block, chunk):
+        self.loop_item = loop_item
+        self.counter = counter
+        self.length = length
+        self.rows = rows
+        self.x = x
+        self.out = out
+        self.vec = vec
+        self.rows_per_block = rows_per_block
+        self.chunk = chunk
+
+
+def plan(info, rows_per_block=None, chunk=None):
+    """A ScanPlan when the DAG is a last-axis row scan this template can run, else None."""
+    forced_rows, forced_chunk = rows_per_block, chunk
+    if len(info.inputs) != 1 or len(info.outputs) != 1:
+        return None
+    loops = [item for item in info.tree if item.kind == 'loop']
+    if len(loops) != 1 or any(item.kind == 'if' for item in info.tree):
+        return None
+    loop = loops[0]
+    range_node = info.nodes[loop.node]
+    counter = range_node.ops[0]
+    if counter not in info.loop_counters:
+        return None
+    start, stop, step = (info._literal_int(o) for o in range_node.ops[1:])
+    if start != 1 or step != 1 or stop is None or stop < 2:
+        return None
+    length = stop
+    if any(inner.kind != 'stmt' for inner in loop.body):
+        return None                 # nested loops or conditionals inside the scan body: use the generic template
+
+    rows = info.num_workers
+    # row base = worker_index * length, expressed in the position components
+    rank = len(info.workgroup_shape)
+    stride = 1
+    wg_stride = [1] * rank
+    for k in range(rank - 2, -1, -1):
+        stride *= info.workgroup_shape[k + 1]
+        wg_stride[k] = stride
+    base = dict((('p', k), length * wg_stride[k]) for k in range(rank) if info.workgroup_shape[k] > 1)
+    in_loop = dict(base)
+    in_loop[('v', counter)] = 1
+    sig_first = (tuple(sorted(base.items())), 0)
+    sig_loop = (tuple(sorted(in_loop.items())), 0)
+
+    x = out = None
+    for node, tensor, aff in info.tensor_accesses():
+        if aff is None:
+            return None
+        expect = sig_loop if info.in_loop[node.idx] else sig_first
+        if aff.signature() != expect:
+            return None
+        if node.code == lang.READ_TENSOR:
+            if x is not None and x is not tensor:
+                return None
+            x = tensor
+        else:
+            if out is not None and out is not tensor:
+                return None
+            out = tensor
+    if x is None or out is None or x.dtype != out.dtype:
+        return None
+    if x.size != rows * length or out.size != rows * length:
+        return None
+    itemsize = ITEMSIZE[x.dtype]
+    if itemsize not in (4, 8) or x.dtype not in CTYPE:
+        return None
+    vec = 16 // itemsize
+
+    rows_per_block = forced_rows or max(1, min(WAVE, (rows + NUM_CU - 1) // NUM_CU))
+    chunk = None
+    for cand in ((forced_chunk,) if forced_chunk else (1024, 512, 256, 128, 64)):
+        if length % cand == 0 and 3 * rows_per_block * (cand + vec) * itemsize <= LDS_BUDGET:
+            chunk = cand
+            break
+    if chunk is None:
+        return None
+    return ScanPlan(loop, counter, length, rows, x, out, vec, rows_per_block, chunk)
+
+
+def generate(info, kernel_name, rows_per_block=None, chunk=None):
+    p = plan(info, rows_per_block, chunk)
+    assert p is not None
+    ctype = CTYPE[p.x.dtype]
+    vec, chunk, rpb = p.vec, p.chunk, p.rows_per_block
+    row_stride = chunk + vec        # keeps 128-bit alignment; lanes of the scanning wavefront fall in different banks
+    num_chunks = p.length // chunk
+    vectors_per_row = chunk // vec
+    tile_vectors = rpb * vectors_per_row
+
+    # position of a row: the workgroup is the tensor shape without the scanned axis
+    rank = len(info.workgroup_shape)
+    pos_exprs = []
+    stride = 1
+    strides = [1] * rank
+    for k in range(rank - 2, -1, -1):
+        stride *= info.workgroup_shape[k + 1]
+        strides[k] = stride
+    for k in range(rank):
+        expr = 'row'
+        if k > 0:
+            expr = '(row % ' + str(strides[k - 1]) + 'u)'
+        pos_exprs.append(expr + ' / ' + str(strides[k]) + 'u')
+
+    emitter = BodyEmitter(info, pos_exprs,
+                          read_hook=lambda node, tensor, idx: 'OVL_SCAN_IN',
+                          store_hook=lambda node, tensor, idx, value: 'OVL_SCAN_OUT(' + value + ');')
+    tagged = emitter.emit_tagged()
+    range_idx = p.loop_item.node
+    end_idx = max(i for i, _ in tagged)         # ENDRANGE is the last statement of a plan-conforming DAG
+    prologue = [t for i, t in tagged if i < range_idx]
+    body = [t.strip() for i, t in tagged if range_idx < i < end_idx]
+    counter_name = 'e' + str(p.counter)
+    counter_type = CTYPE[info.nodes[p.counter].dtype]
+
+    src = []
+    vname = 'ovl_scan_vec'
+    src.append('typedef %s %s __attribute__((ext_vector_type(%d)));' % (ctype, vname, vec))
+    src.append('')
+    src.append('extern "C" __global__ void __launch_bounds__(%d)' % BLOCK)
+    src.append('%s(const %s* __restrict__ in%d, %s* __restrict__ out%d) {' % (
+        kernel_name, ctype, p.x.io_index, ctype, p.out.io_index))
+    src.append('    __shared__ __attribute__((aligned(16))) %s tile[3][%d][%d];' % (ctype, rpb, row_stride))
+    src.append('    const uint32_t row0 = blockIdx.x * %du;' % rpb)
+    src.append('    const uint32_t lane = threadIdx.x %% %du;' % WAVE)
+    src.append('    const %s* __restrict__ gin = in%d;' % (ctype, p.x.io_index))
+    src.append('    %s* __restrict__ gout = out%d;' % (ctype, p.out.io_index))
+    src.append('')
+    vpt = (tile_vectors + MOVERS - 1) // MOVERS      # vectors each mover thread handles per chunk
+    src.append('    // Movers (threads 64..255): every thread owns up to %d vectors of each chunk.  A vector that does not exist' % vpt)
+    src.append('    // (past the tile or past the last row) is redirected to the thread\'s first vector for loading and skipped')
+    src.append('    // when writing, so the loops are branch free and all loads of a chunk are in flight together.')
+    src.append('    struct MoverRegs { %s v[%d]; };' % (vname, vpt))
+    src.append('    auto slot = [&](uint32_t m, uint32_t i, uint32_t& r, uint32_t& cv) -> bool {')
+    src.append('        const uint32_t v = m + i * %du;' % MOVERS)
+    src.append('        r = v / %du; cv = (v %% %du) * %du;' % (vectors_per_row, vectors_per_row, vec))
+    src.append('        return v < %du && row0 + r < %du;' % (tile_vectors, p.rows))
+    src.append('    };')
+    src.append('    auto issue_loads = [&](uint32_t k, uint32_t m, MoverRegs& regs) {')
+    src.append('        #pragma unroll')
+    src.append('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
+    src.append('            uint32_t r, cv;')
+    src.append('            if (!slot(m, i, r, cv)) { r = 0; cv = 0; }')
+    src.append('            const uint32_t gr = (row0 + r < %du) ? row0 + r : %du;' % (p.rows, p.rows - 1))
+    src.append('            const uint64_t g = (uint64_t)gr * %dull + k * %du + cv;' % (p.length, chunk))
+    src.append('            regs.v[i] = __builtin_nontemporal_load(reinterpret_cast<const %s*>(gin + g));' % vname)
+    src.append('        }')
+    src.append('    };')
+    src.append('    auto write_lds = [&](uint32_t k, uint32_t m, const MoverRegs& regs) {')
+    src.append('        #pragma unroll')
+    src.append('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
+    src.append('            uint32_t r, cv;')
+    src.append('            if (slot(m, i, r, cv)) *reinterpret_cast<%s*>(&tile[k %% 3u][r][cv]) = regs.v[i];' % vname)
+    src.append('        }')
+    src.append('    };')
+    src.append('    auto store_chunk = [&](uint32_t k, uint32_t m) {')
+    src.append('        MoverRegs regs;')
+    src.append('        #pragma unroll')
+    src.append('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
+    src.append('            uint32_t r, cv;')
+    src.append('            if (!slot(m, i, r, cv)) { r = 0; cv = 0; }')
+    src.append('            regs.v[i] = *reinterpret_cast<const %s*>(&tile[k %% 3u][r][cv]);' % vname)
+    src.append('        }')
+    src.append('        #pragma unroll')
+    src.append('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
+    src.append('            uint32_t r, cv;')
+    src.append('            if (slot(m, i, r, cv)) {')
+    src.append('                const uint64_t g = (uint64_t)(row0 + r) * %dull + k * %du + cv;' % (p.length, chunk))
+    src.append('                __builtin_nontemporal_store(regs.v[i], reinterpret_cast<%s*>(gout + g));' % vname)
+    src.append('            }')
+    src.append('        }')
+    src.append('    };')
+    src.append('')
+    src.append('    if (threadIdx.x >= %du) {' % WAVE)
+    src.append('        const uint32_t m = threadIdx.x - %du;' % WAVE)
+    src.append('        // Two register sets keep two chunks of loads in flight: while chunk k is being scanned, chunk k+1 is')
+    src.append('        // written to LDS from the set requested two iterations ago, and chunk k+3 is requested into that set.')
+    src.append('        MoverRegs set_a, set_b;')
+    src.append('        issue_loads(0u, m, set_a);')
+    src.append('        write_lds(0u, m, set_a);')
+    if num_chunks > 1:
+        src.append('        issue_loads(1u, m, set_b);')
+    if num_chunks > 2:
+        src.append('        issue_loads(2u, m, set_a);')
+    src.append('        __syncthreads();')
+    src.append('        auto step = [&](uint32_t k, MoverRegs& regs) {')
+    src.append('            if (k + 1u < %du) write_lds(k + 1u, m, regs);' % num_chunks)
+    src.append('            if (k + 3u < %du) issue_loads(k + 3u, m, regs);' % num_chunks)
+    src.append('            if (k >= 1u) store_chunk(k - 1u, m);')
+    src.append('            __syncthreads();')
+    src.append('        };')
+    src.append('        #pragma unroll 1')
+    src.append('        for (uint32_t k = 0; k + 1u < %du; k += 2u) {' % num_chunks)
+    src.append('            step(k, set_b);             // chunks 1, 3, 5, ... travel through set_b')
+    src.append('            step(k + 1u, set_a);        // chunks 2, 4, 6, ... travel through set_a')
+    src.append('        }')
+    if num_chunks % 2 == 1:
+        src.append('        step(%du, set_b);' % (num_chunks - 1))
+    src.append('        store_chunk(%du, m);' % (num_chunks - 1))
+    src.append('    } else {')
+    src.append('        // The scanning wavefront: lane r owns row row0 + r.  Surplus lanes shadow the last row of the tile: they')
+    src.append('        // compute and write the same values to the same LDS words as its owner, which keeps the loop branch free')
+    src.append('        // (masking them off instead was measured to be slower).')
+    src.append('        const uint32_t r = lane < %du ? lane : %du;' % (rpb, rpb - 1))
+    src.append('        const uint32_t row = (row0 + r < %du) ? row0 + r : %du;' % (p.rows, p.rows - 1))
+    src.append('        __syncthreads();')
+    src.append('        %s* rowp = &tile[0][r][0];' % ctype)
+    src.append('        %s xv = *reinterpret_cast<const %s*>(rowp);' % (vname, vname))
+    src.append('        // first column: the statements the worker runs before its loop')
+    src.append('#define OVL_SCAN_IN xv[0]')
+    src.append('#define OVL_SCAN_OUT(value) xv[0] = (value)')
+    for stmt in prologue:
+        src.append('        ' + stmt)
+    src.append('#undef OVL_SCAN_IN')
+    src.append('#undef OVL_SCAN_OUT')
+    src.append('#define OVL_SCAN_IN xv[u]')
+    src.append('#define OVL_SCAN_OUT(value) xv[u] = (value)')
+    src.append('#define OVL_SCAN_STEP(column) { %s = (%s)(column); %s }' % (
+        counter_name, counter_type, ' '.join(body)))
+    src.append('        #pragma unroll')
+    src.append('        for (uint32_t u = 1; u < %du; ++u) OVL_SCAN_STEP(u)' % vec)
+    src.append('        *reinterpret_cast<%s*>(rowp) = xv;' % vname)
+    src.append('        for (uint32_t k = 0; k < %du; ++k) {' % num_chunks)
+    src.append('            rowp = &tile[k % 3u][r][0];')
+    src.append('            uint32_t c = (k == 0u) ? %du : 0u;' % vec)
+    src.append('            // the next vector is read from LDS while the current one is being accumulated')
+    src.append('            %s next = *reinterpret_cast<const %s*>(rowp + c);' % (vname, vname))
+    src.append('            #pragma unroll 8')
+    src.append('            for (; c < %du; c += %du) {' % (chunk, vec))
+    src.append('                xv = next;')
+    src.append('                next = *reinterpret_cast<const %s*>(rowp + (c + %du < %du ? c + %du : c));' % (
+        vname, vec, chunk, vec))
+    src.append('                #pragma unroll')
+    src.append('                for (uint32_t u = 0; u < %du; ++u) OVL_SCAN_STEP(k * %du + c + u)' % (vec, chunk))
+    src.append('                *reinterpret_cast<%s*>(rowp + c) = xv;' % vname)
+    src.append('            }')
+    src.append('            __syncthreads();')
+    src.append('        }')
+    src.append('#undef OVL_SCAN_STEP')
+    src.append('#undef OVL_SCAN_IN')
+    src.append('#undef OVL_SCAN_OUT')
+    src.append('    }')
+    src.append('}')
+
+    blocks = (p.rows + rpb - 1) // rpb
+    launch = {
+        'template': 'rowscan',
+        'vec': vec,
+        'block': BLOCK,
+        'blocks_needed': blocks,
+        'align': {('in', p.x.io_index): 16, ('out', p.out.io_index): 16},
+        'vector_loads': 1,
+        'vector_stores': 1,
+    }
+    return '\n'.join(src) + '\n', launch

@@ -1,0 +1,226 @@
+"""
+The tile kernel template: a rank-2 workgroup whose operator stores one or more outputs transposed.
+
+A worker at (i, j) that writes ``out[j, i]`` makes neighbouring workers along j (the lanes of a wavefront in the
+one-worker-per-thread template of the reference, opveclib/expression.py:602-608) store to addresses a whole output
+row apart: every lane of every store instruction touches a different cache line.  This template gives one 256-thread
+workgroup a TILE x TILE block of workers:
+
+  phase 1  threads walk the tile row by row, VEC consecutive j per thread, exactly like the map kernel (aligned or
+           dword-aligned 128-bit loads along j, register-buffered 128-bit stores for outputs that are contiguous along
+           j); values of transposed outputs are written into an LDS tile at [j][i] (row length TILE+1 words, so that
+           both the column-wise writes and the row-wise reads spread over all LDS banks);
+  phase 2  after a barrier the threads walk the LDS tile the other way, VEC consecutive i per thread, and store
+           128-bit vectors that are contiguous along i, so a wavefront writes 256-byte runs of the output rows.
+
+The worker body is the same statement sequence as in every other template; only where a store lands changes.
+"""
+
+from .. import language as lang
+from .analysis import ITEMSIZE
+from .body import BodyEmitter, CTYPE
+from .map_kernel import Access, _index_expr, _is_vector_access, contiguous_unaligned
+
+BLOCK = 256
+TILE = 64
+
+
+def _is_transposed_store(info, node, tensor, aff, vec):
+    """out[.., p_last*C + p0 + c]: unit stride along workgroup dimension 0, vector aligned."""
+    if aff is None or not aff.only_position() or info.in_loop[node.idx]:
+        return False
+    if aff.coeff(('p', 0)) != 1:
+        return False
+    c_last = aff.coeff(('p', 1))
+    if c_last == 0 or c_last % vec != 0 or aff.const % vec != 0:
+        return False
+    if aff.lo < 0 or aff.hi >= tensor.size:
+        return False
+    return True
+
+
+def applicable(info):
+    """Vector width if the tile template fits this DAG, else None."""
+    if len(info.workgroup_shape) != 2:
+        return None
+    rows, cols = info.workgroup_shape
+    accesses = info.tensor_accesses()
+    widest = 1
+    for _, tensor, _ in accesses:
+        widest = max(widest, ITEMSIZE[tensor.dtype])
+    vec = max(1, 16 // widest)
+    if vec < 2 or rows % vec != 0 or cols % vec != 0:
+        return None
+    stores = [(n, t, a) for n, t, a in accesses if n.code == lang.ASSIGN_TENSOR]
+    keys = [(t.idx, a.signature()) for n, t, a in stores if _is_transposed_store(info, n, t, a, vec)]
+    if not keys:
+        return None
+    certain = info.definitely_stores(keys)
+    if not certain:
+        return None
+    # all transposed outputs share one element width so one tile geometry serves them all
+    return vec
+
+
+def generate(info, kernel_name):
+    vec = applicable(info)
+    assert vec is not None
+    rows, cols = info.workgroup_shape
+    accesses = info.tensor_accesses()
+
+    loads = {}
+    unaligned = {}
+    stores = {}
+    tstores = {}
+    store_keys = []
+    tkeys = []
+    for node, tensor, aff in accesses:
+        if node.code == lang.READ_TENSOR:
+            if _is_vector_access(info, node, tensor, aff, vec):
+                key = (tensor.idx, aff.signature())
+                loads.setdefault(key, Access(tensor, aff, 'ld%d' % len(loads)))
+            elif contiguous_unaligned(info, node, tensor, aff, vec):
+                key = (tensor.idx, aff.signature())
+                unaligned.setdefault(key, Access(tensor, aff, 'lu%d' % len(unaligned)))
+        else:
+            if _is_vector_access(info, node, tensor, aff, vec):
+                store_keys.append((tensor.idx, aff.signature()))
+            elif _is_transposed_store(info, node, tensor, aff, vec):
+                tkeys.append((tensor.idx, aff.signature()))
+    certain = info.definitely_stores(store_keys + tkeys)
+    for node, tensor, aff in accesses:
+        if node.code != lang.ASSIGN_TENSOR or aff is None:
+            continue
+        key = (tensor.idx, aff.signature())
+        if key not in certain:
+            continue
+        if key in store_keys and key not in stores:
+            stores[key] = Access(tensor, aff, 'st%d' % len(stores))
+        elif key in tkeys and key not in tstores:
+            tstores[key] = Access(tensor, aff, 'tile%d' % len(tstores))
+
+    def read_hook(node, tensor, index_name):
+        aff = info.affine[node.ops[1]]
+        if aff is not None and not info.in_loop[node.idx]:
+            acc = loads.get((tensor.idx, aff.signature())) or unaligned.get((tensor.idx, aff.signature()))
+            if acc is not None:
+                return acc.reg + '[lane]'
+        return None
+
+    def store_hook(node, tensor, index_name, value_name):
+        aff = info.affine[node.ops[1]]
+        if aff is not None and not info.in_loop[node.idx]:
+            key = (tensor.idx, aff.signature())
+            if key in stores:
+                return stores[key].reg + '[lane] = ' + value_name + ';'
+            if key in tstores:
+                return tstores[key].reg + '[tj + lane][ti] = ' + value_name + ';'
+        return None
+
+    body = BodyEmitter(info, ['p0', 'p1 + lane'], read_hook, store_hook).emit()
+
+    threads_per_row = TILE // vec
+    rows_per_pass = BLOCK // threads_per_row
+    tiles_i = (rows + TILE - 1) // TILE
+    tiles_j = (cols + TILE - 1) // TILE
+
+    args = []
+    for i in range(len(info.inputs)):
+        args.append('const ' + CTYPE[info.inputs[i].dtype] + '* __restrict__ in' + str(i))
+    for i in range(len(info.outputs)):
+        args.append(CTYPE[info.outputs[i].dtype] + '* __restrict__ out' + str(i))
+
+    src = []
+    vec_types = {}
+    for acc in list(loads.values()) + list(stores.values()) + list(tstores.values()) + list(unaligned.values()):
+        ctype = CTYPE[acc.tensor.dtype]
+        vec_types[ctype] = ('ovl_' + ctype.replace(' ', '_') + 'x' + str(vec), ITEMSIZE[acc.tensor.dtype])
+    for ctype, (vname, itemsize) in sorted(vec_types.items()):
+        src.append('typedef ' + ctype + ' ' + vname + ' __attribute__((ext_vector_type(' + str(vec) + ')));')
+        src.append('typedef ' + vname + ' ' + vname + '_u __attribute__((aligned(' + str(itemsize) + ')));')
+    vec_types = dict((k, v[0]) for k, v in vec_types.items())
+    src.append('')
+    src.append('extern "C" __global__ void __launch_bounds__(%d)' % BLOCK)
+    src.append(kernel_name + '(' + ', '.join(args) + ') {')
+    if info.uses_math_tables():
+        src.append('    OVL_DECLARE_MATH_TABLES();')
+    for acc in tstores.values():
+        src.append('    __shared__ %s %s[%d][%d];' % (CTYPE[acc.tensor.dtype], acc.reg, TILE, TILE + 1))
+    src.append('    const uint32_t num_tiles = %du;' % (tiles_i * tiles_j))
+    src.append('    for (uint32_t tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {')
+    src.append('        const uint32_t i0 = (tile / %du) * %du;' % (tiles_j, TILE))
+    src.append('        const uint32_t j0 = (tile %% %du) * %du;' % (tiles_j, TILE))
+    src.append('        const uint32_t tj = (threadIdx.x %% %du) * %du;' % (threads_per_row, vec))
+    src.append('        #pragma unroll 1')
+    src.append('        for (uint32_t ti = threadIdx.x / %du; ti < %du; ti += %du) {' % (
+        threads_per_row, TILE, rows_per_pass))
+    src.append('            const uint32_t p0 = i0 + ti;')
+    src.append('            const uint32_t p1 = j0 + tj;')
+    src.append('            if (p0 < %du && p1 < %du) {' % (rows, cols))
+    pos_names = ['p0', 'p1']
+    for acc in loads.values():
+        vname = vec_types[CTYPE[acc.tensor.dtype]]
+        wide = acc.aff.hi >= 2 ** 32
+        src.append('                const %s %s = __builtin_nontemporal_load(reinterpret_cast<const %s*>(in%d + (%s)));'
+                   % (vname, acc.reg, vname, acc.tensor.io_index, _index_expr(acc.aff, pos_names, wide)))
+    for acc in unaligned.values():
+        vname = vec_types[CTYPE[acc.tensor.dtype]]
+        wide = acc.aff.hi >= 2 ** 32
+        src.append('                const %s %s = *reinterpret_cast<const %s_u*>(in%d + (%s));' % (
+            vname, acc.reg, vname, acc.tensor.io_index, _index_expr(acc.aff, pos_names, wide)))
+    for acc in stores.values():
+        src.append('                %s %s;' % (vec_types[CTYPE[acc.tensor.dtype]], acc.reg))
+    src.append('                #pragma unroll')
+    src.append('                for (uint32_t lane = 0; lane < %du; ++lane) {' % vec)
+    for stmt in body:
+        src.append('                    ' + stmt)
+    src.append('                }')
+    for acc in stores.values():
+        vname = vec_types[CTYPE[acc.tensor.dtype]]
+        wide = acc.aff.hi >= 2 ** 32
+        src.append('                __builtin_nontemporal_store(%s, reinterpret_cast<%s*>(out%d + (%s)));' % (
+            acc.reg, vname, acc.tensor.io_index, _index_expr(acc.aff, pos_names, wide)))
+    src.append('            }')
+    src.append('        }')
+    src.append('        __syncthreads();')
+    # phase 2: rows of the LDS tile are runs along i
+    src.append('        const uint32_t oi = (threadIdx.x %% %du) * %du;' % (threads_per_row, vec))
+    src.append('        #pragma unroll 1')
+    src.append('        for (uint32_t oj = threadIdx.x / %du; oj < %du; oj += %du) {' % (
+        threads_per_row, TILE, rows_per_pass))
+    src.append('            const uint32_t p0 = i0 + oi;')
+    src.append('            const uint32_t p1 = j0 + oj;')
+    src.append('            if (p0 < %du && p1 < %du) {' % (rows, cols))
+    for acc in tstores.values():
+        vname = vec_types[CTYPE[acc.tensor.dtype]]
+        wide = acc.aff.hi >= 2 ** 32
+        src.append('                %s v_%s;' % (vname, acc.reg))
+        src.append('                #pragma unroll')
+        src.append('                for (uint32_t lane = 0; lane < %du; ++lane) v_%s[lane] = %s[oj][oi + lane];' % (
+            vec, acc.reg, acc.reg))
+        src.append('                __builtin_nontemporal_store(v_%s, reinterpret_cast<%s*>(out%d + (%s)));' % (
+            acc.reg, vname, acc.tensor.io_index, _index_expr(acc.aff, pos_names, wide)))
+    src.append('            }')
+    src.append('        }')
+    src.append('        __syncthreads();')
+    src.append('    }')
+    src.append('}')
+
+    align = {}
+    for acc in loads.values():
+        key = ('in', acc.tensor.io_index)
+        align[key] = max(align.get(key, 1), vec * ITEMSIZE[acc.tensor.dtype])
+    for acc in list(stores.values()) + list(tstores.values()):
+        key = ('out', acc.tensor.io_index)
+        align[key] = max(align.get(key, 1), vec * ITEMSIZE[acc.tensor.dtype])
+
+    launch = {
+        'template': 'transpose',
+        'vec': vec,
+        'block': BLOCK,
+        'blocks_needed': tiles_i * tiles_j,
+        'align': align,
+        'vector_loads': len(loads) + len(unaligned),
+        'vector_stores': len(stores) + len(tstores),
+    }
+    return '\n'.join(src) + '\n', launch

@@ -104,6 +104,18 @@ def c3_cumprod_f64(rng, shape=(24, 1024)):
     return [cumprod(uniform(rng, 0.99, 1.01, shape, np.float64), axis=1)[0]]
 
 
+def c3_rowscan_shapes(rng):
+    """Row-scan template corner cases: partial last workgroup, several rows per workgroup, rank 3, int32, max."""
+    outs = [cumsum(rng.standard_normal((515, 64), dtype=np.float32), axis=1)[0],
+            cumprod(uniform(rng, 0.9, 1.1, (259, 128), np.float64), axis=1)[0],
+            cumsum(rng.standard_normal((4, 70, 128), dtype=np.float32), axis=2)[0],
+            cumsum(rng.integers(-1000, 1000, size=(20, 192)).astype(np.int32), axis=1)[0],
+            accumulate(rng.standard_normal((7, 256), dtype=np.float32),
+                       inner_fcn=lambda acc, x: ovl.maximum(acc, x), axis=1)[0],
+            cumsum(rng.standard_normal(4096, dtype=np.float32))[0]]
+    return outs
+
+
 def c4_lstm(rng, batch=32, units=128):
     concat = rng.standard_normal((batch, 4 * units), dtype=np.float32)
     c = rng.standard_normal((batch, units), dtype=np.float32)
@@ -118,10 +130,17 @@ def c4_lstm_grad(rng, batch=32, units=128):
     return all_outputs(lstm_grad(concat, c, dc, dh, forget_bias=1.0))
 
 
-def c5_gather_transpose(rng, shape=(192, 320)):
-    a = rng.standard_normal(shape, dtype=np.float32)
-    b = rng.standard_normal(shape, dtype=np.float32)
-    return [gather_transpose(a, b.reshape(-1), alpha=0.5, stride=7919)[0]]
+def c5_gather_transpose(rng, shape=(192, 320), stride=7919, dtype=np.float32):
+    a = rng.standard_normal(shape, dtype=dtype)
+    b = rng.standard_normal(shape, dtype=dtype)
+    return [gather_transpose(a, b.reshape(-1), alpha=0.5, stride=stride)[0]]
+
+
+def c5_variants(rng):
+    """Gather index that provably never wraps (dword-aligned vector loads), ragged tile edges, float64 tiles."""
+    return (c5_gather_transpose(rng, (192, 320), stride=3) + c5_gather_transpose(rng, (68, 100), stride=5) +
+            c5_gather_transpose(rng, (130, 66), stride=7, dtype=np.float64) +
+            c5_gather_transpose(rng, (6, 10), stride=1))
 
 
 # ----------------------------------------------------------------------------------------------------------------------
@@ -439,9 +458,11 @@ CASES = [
     Case('c3_cumprod_f32', c3_cumprod_f32, seed=3),
     Case('c3_cumsum_f64', c3_cumsum_f64, seed=3),
     Case('c3_cumprod_f64', c3_cumprod_f64, seed=3),
+    Case('c3_rowscan_shapes', c3_rowscan_shapes, seed=3),
     Case('c4_lstm', c4_lstm, seed=4),
     Case('c4_lstm_grad', c4_lstm_grad, seed=4),
     Case('c5_gather_transpose', c5_gather_transpose, seed=5),
+    Case('c5_variants', c5_variants, seed=5),
     _simple('clip', lambda rng: [clip(rng.random(1000), threshold1=0.1, threshold2=0.9)[0]]),
     _simple('limits_f32', lambda rng: [set_limits(np.array([0], np.float32))[0]]),
     _simple('limits_f64', lambda rng: [set_limits(np.array([0], np.float64))[0]]),

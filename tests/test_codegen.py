@@ -68,6 +68,34 @@ def test_vector_width_selection():
     assert map_kernel.choose_vec(DagInfo(cumsum(f32, axis=1).expression_dag)) == 1
 
 
+def test_template_selection():
+    def template(op, options=None):
+        dag = op.expression_dag if hasattr(op, 'expression_dag') else op
+        return hipgen.generate(dag, 'f' + '4' * 56, options).launch
+
+    f32 = np.zeros((8, 64), np.float32)
+    assert template(stdops.add(f32, f32))['template'] == 'map'
+    # last-axis accumulation with a chunkable row length: the order-preserving row scan
+    scan = template(cumsum(np.zeros((48, 1024), np.float32), axis=1))
+    assert scan['template'] == 'rowscan' and scan['blocks_needed'] == 48
+    assert template(cumsum(np.zeros((1024, 16384), np.float64), axis=1))['blocks_needed'] == 256
+    assert template(cumsum(np.zeros((48, 1024), np.float32), axis=1), {'template': 'map'})['template'] == 'map'
+    # rows that are not a multiple of 64 long, other axes, and loop bodies with branches use the general template
+    assert template(cumsum(np.zeros((48, 1000), np.float32), axis=1))['template'] == 'map'
+    assert template(cumsum(np.zeros((48, 1024), np.float32), axis=0))['template'] == 'map'
+    assert template(cases.dot(np.zeros((16, 64)), np.zeros((16, 64))))['template'] == 'map'
+    # transposed store of a rank-2 workgroup: LDS tiles; the gather is one dword-aligned 128-bit load per thread
+    tr = template(gather_transpose(np.zeros((192, 320), np.float32), np.zeros(192 * 320, np.float32),
+                                   alpha=0.5, stride=3))
+    assert tr['template'] == 'transpose' and tr['vector_loads'] == 2 and tr['vector_stores'] == 1
+    assert tr['blocks_needed'] == 3 * 5
+    wraps = template(gather_transpose(np.zeros((192, 320), np.float32), np.zeros(192 * 320, np.float32),
+                                      alpha=0.5, stride=7919))
+    assert wraps['template'] == 'transpose' and wraps['vector_loads'] == 1        # the gather index may wrap: scalar
+    odd = template(gather_transpose(np.zeros((6, 9), np.float32), np.zeros(54, np.float32), alpha=0.5, stride=1))
+    assert odd['template'] == 'map'
+
+
 def test_chain8_kernel_shape():
     a = np.zeros((64, 256), np.float32)
     s = np.array([1.0001], np.float32)
