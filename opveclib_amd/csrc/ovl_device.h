@@ -31,6 +31,27 @@ typedef struct ovl_tensor {
 __device__ __forceinline__ int8_t ovl_abs_8(int8_t x) { return (x < 0) ? -x : x; }
 __device__ __forceinline__ int16_t ovl_abs_16(int16_t x) { return (x < 0) ? -x : x; }
 
+// Lane-to-lane moves inside a wavefront (data-parallel-primitive modifiers of the vector ALU).
+//   OVL_DPP_ROW_SHR1: lane i of every 16-lane row receives the value of lane i-1; lane 0 of the row keeps `old`
+//   OVL_DPP_ROW_ROR1: lane i receives lane i-1, lane 0 of the row receives lane 15
+#define OVL_DPP_ROW_SHR1 0x111
+#define OVL_DPP_ROW_ROR1 0x121
+template <int CTRL, typename T>
+__device__ __forceinline__ T ovl_dpp_move(T old, T src) {
+    if constexpr (sizeof(T) == 8) {
+        const uint64_t o = __builtin_bit_cast(uint64_t, old), s = __builtin_bit_cast(uint64_t, src);
+        const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp((int)(uint32_t)o, (int)(uint32_t)s, CTRL, 0xf, 0xf, false);
+        const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp((int)(uint32_t)(o >> 32), (int)(uint32_t)(s >> 32),
+                                                                  CTRL, 0xf, 0xf, false);
+        return __builtin_bit_cast(T, ((uint64_t)hi << 32) | lo);
+    } else if constexpr (sizeof(T) == 4) {
+        return __builtin_bit_cast(T, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old),
+                                                                 __builtin_bit_cast(int, src), CTRL, 0xf, 0xf, false));
+    } else {
+        return (T)__builtin_amdgcn_update_dpp((int)old, (int)src, CTRL, 0xf, 0xf, false);
+    }
+}
+
 // float32 transcendental entry points used by generated code: bit-compatible with the host C library's
 // expf/logf/tanhf (see ovl_math.h).  ovl_exp_tab / ovl_log_tab name the lookup tables in scope: kernels that call
 // exp or log declare them with OVL_DECLARE_MATH_TABLES at their top, pointing at copies in LDS.

@@ -287,3 +287,208 @@ def generate(info, kernel_name, rows_per_block=None, chunk=None):
         'vector_stores': 1,
     }
     return '\n'.join(src) + '\n', launch
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# The lane-skewed variant: no LDS, no barriers.
+#
+# Sixteen neighbouring lanes share one row; lane i of the group holds VEC consecutive columns of the current group of
+# 16*VEC columns, loaded and stored as one 128-bit access, so a wavefront reads and writes 256-byte runs of four rows.
+# The recurrence still runs strictly left to right: in phase p (p = 0..15) every lane runs the loop body over its own
+# VEC columns starting from the carried state it currently holds, then hands its final state to its right neighbour
+# (one DPP move per 32 bits of state).  Lane 0 starts from the true carry, so after phase p lanes 0..p hold exact
+# results; a lane that is already exact recomputes the same values, a lane that is not yet exact computes values
+# that are overwritten in a later phase.  After phase 15 all 16*VEC results are exact and lane 15's state is rotated
+# to lane 0 as the carry into the next group.  Per column the wavefront issues one loop body plus 1/VEC state moves,
+# against one loop body plus a 128-bit LDS read and write per VEC columns in the lane = row variant, and rows are
+# spread over four times as many wavefronts.
+# ---------------------------------------------------------------------------------------------------------------------
+
+GROUP_LANES = 16
+SKEW_MAX_BODY = 96
+
+
+def _carried_state(info, p):
+    """Variables declared before the loop and assigned inside it (the loop counter excluded), in DAG order."""
+    range_idx = p.loop_item.node
+    state = []
+    for node in info.nodes:
+        if node.code == lang.ASSIGN_VARIABLE and info.in_loop[node.idx]:
+            target = node.ops[0]
+            if target < range_idx and target != p.counter and target not in state:
+                state.append(target)
+    return sorted(state)
+
+
+def skew_plan(info):
+    """The structural plan when the lane-skewed variant can run this DAG, else None."""
+    p = plan(info)
+    if p is None or p.length % (GROUP_LANES * p.vec) != 0:
+        return None
+    body_nodes = [n for n in info.nodes if info.in_loop[n.idx]]
+    if len(body_nodes) > SKEW_MAX_BODY:
+        return None
+    for idx in _carried_state(info, p):
+        if info.nodes[idx].dtype not in CTYPE:
+            return None
+    return p
+
+
+def generate_skewed(info, kernel_name, depth=None, sets=None):
+    p = skew_plan(info)
+    assert p is not None
+    ctype = CTYPE[p.x.dtype]
+    vec = p.vec
+    group_cols = GROUP_LANES * vec
+    num_groups = p.length // group_cols
+    rows_per_wave = WAVE // GROUP_LANES
+    waves = BLOCK // WAVE
+    rows_per_block = rows_per_wave * waves
+    if depth is None:
+        depth = 4                   # measured on MI355X: 4 groups (1 KiB per row) per request burst is the fastest
+    while num_groups % depth != 0:
+        depth //= 2
+
+    rank = len(info.workgroup_shape)
+    pos_exprs = []
+    stride = 1
+    strides = [1] * rank
+    for k in range(rank - 2, -1, -1):
+        stride *= info.workgroup_shape[k + 1]
+        strides[k] = stride
+    for k in range(rank):
+        expr = 'row'
+        if k > 0:
+            expr = '(row % ' + str(strides[k - 1]) + 'u)'
+        pos_exprs.append(expr + ' / ' + str(strides[k]) + 'u')
+
+    emitter = BodyEmitter(info, pos_exprs,
+                          read_hook=lambda node, tensor, idx: 'OVL_SCAN_IN',
+                          store_hook=lambda node, tensor, idx, value: 'OVL_SCAN_OUT(' + value + ');')
+    tagged = emitter.emit_tagged()
+    range_idx = p.loop_item.node
+    end_idx = max(i for i, _ in tagged)
+    prologue = [t for i, t in tagged if i < range_idx]
+    body = [t.strip() for i, t in tagged if range_idx < i < end_idx]
+    counter_name = 'e' + str(p.counter)
+    counter_type = CTYPE[info.nodes[p.counter].dtype]
+    state = [('e' + str(idx), CTYPE[info.nodes[idx].dtype]) for idx in _carried_state(info, p)]
+
+    vname = 'ovl_scan_vec'
+    src = []
+    src.append('typedef %s %s __attribute__((ext_vector_type(%d)));' % (ctype, vname, vec))
+    src.append('')
+    src.append('extern "C" __global__ void __launch_bounds__(%d)' % BLOCK)
+    src.append('%s(const %s* __restrict__ in%d, %s* __restrict__ out%d) {' % (
+        kernel_name, ctype, p.x.io_index, ctype, p.out.io_index))
+    if info.uses_math_tables():
+        src.append('    OVL_DECLARE_MATH_TABLES();')
+    src.append('    const uint32_t lane = threadIdx.x %% %du;' % WAVE)
+    src.append('    const uint32_t part = lane %% %du;              // which VEC columns of a group this lane holds' % GROUP_LANES)
+    src.append('    const uint32_t row_raw = (blockIdx.x * %du + threadIdx.x / %du) * %du + lane / %du;' % (
+        waves, WAVE, rows_per_wave, GROUP_LANES))
+    src.append('    // A wavefront wholly past the last row leaves; single lanes past it shadow the last row instead (all lanes')
+    src.append('    // must stay active for the lane-to-lane moves): they load, compute and store exactly what its owners do.')
+    src.append('    if ((blockIdx.x * %du + threadIdx.x / %du) * %du >= %du) return;' % (waves, WAVE, rows_per_wave, p.rows))
+    src.append('    const uint32_t row = row_raw < %du ? row_raw : %du;' % (p.rows, p.rows - 1))
+    src.append('    const %s* __restrict__ gin = in%d + (uint64_t)row * %dull + part * %du;' % (
+        ctype, p.x.io_index, p.length, vec))
+    src.append('    %s* __restrict__ gout = out%d + (uint64_t)row * %dull + part * %du;' % (
+        ctype, p.out.io_index, p.length, vec))
+    batch = depth
+    num_batches = num_groups // batch
+    batch_cols = batch * group_cols
+
+    def request(regs, batch_expr):
+        """All loads of one batch, back to back: every row is read in runs of batch * 256 bytes."""
+        src.append('        #pragma unroll')
+        src.append('        for (uint32_t j = 0; j < %du; ++j)' % batch)
+        src.append('            %s[j] = __builtin_nontemporal_load(reinterpret_cast<const %s*>(gin + (%s) * %du + j * %du));' % (
+            regs, vname, batch_expr, batch_cols, group_cols))
+
+    def process(regs, batch_expr, refill_expr):
+        src.append('        {')
+        src.append('        const uint32_t b = %s;' % batch_expr)
+        src.append('        %s ov[%d];' % (vname, batch))
+        src.append('        #pragma unroll')
+        src.append('        for (uint32_t j = 0; j < %du; ++j) {' % batch)
+        src.append('            const %s xv = %s[j];' % (vname, regs))
+        src.append('            const uint32_t col0 = b * %du + j * %du + part * %du;' % (batch_cols, group_cols, vec))
+        src.append('            const bool first_column = (j == 0u) && (b == 0u) && (part == 0u);')
+        src.append('            #pragma unroll')
+        src.append('            for (uint32_t phase = 0; phase < %du; ++phase) {' % GROUP_LANES)
+        for name, _ in state:
+            src.append('                %s = carry_%s;' % (name, name))
+        src.append('                #pragma unroll')
+        src.append('                for (uint32_t u = 0; u < %du; ++u) {' % vec)
+        src.append('                    if (u == 0u && first_column) ov[j][0] = first_out;')
+        src.append('                    else OVL_SCAN_STEP(col0 + u)')
+        src.append('                }')
+        for name, _ in state:
+            src.append('                carry_%s = ovl_dpp_move<OVL_DPP_ROW_SHR1>(carry_%s, %s);' % (name, name, name))
+        src.append('            }')
+        src.append('            // the last lane of the group finished the group: its state is the carry into the next one')
+        for name, _ in state:
+            src.append('            carry_%s = ovl_dpp_move<OVL_DPP_ROW_ROR1>(carry_%s, %s);' % (name, name, name))
+        src.append('        }')
+        src.append('        // The scheduling fences keep the memory traffic of a batch together, after its arithmetic: runs of')
+        src.append('        // batch * 256 bytes per row, and no load is moved ahead of the last use of the registers it fills.')
+        src.append('        __builtin_amdgcn_sched_barrier(0);')
+        src.append('        #pragma unroll')
+        src.append('        for (uint32_t j = 0; j < %du; ++j)' % batch)
+        src.append('            __builtin_nontemporal_store(ov[j], reinterpret_cast<%s*>(gout + b * %du + j * %du));' % (
+            vname, batch_cols, group_cols))
+        if refill_expr is not None:
+            request(regs, refill_expr)
+        src.append('        __builtin_amdgcn_sched_barrier(0);')
+        src.append('        }')
+
+    sets = max(2, min(sets or 2, num_batches)) if num_batches > 1 else 1
+    src.append('    // %d register sets of %d groups each: one is consumed while the others are in flight' % (sets, batch))
+    src.append('    %s %s;' % (vname, ', '.join('q%d[%d]' % (k, batch) for k in range(sets))))
+    src.append('    {')
+    for k in range(sets):
+        request('q%d' % k, '%du' % k)
+    src.append('    }')
+    src.append('    // first column: the statements the worker runs before its loop, in every lane')
+    src.append('    %s first_out;' % ctype)
+    src.append('#define OVL_SCAN_IN (in%d[(uint64_t)row * %dull])' % (p.x.io_index, p.length))
+    src.append('#define OVL_SCAN_OUT(value) first_out = (value)')
+    for stmt in prologue:
+        src.append('    ' + stmt)
+    src.append('#undef OVL_SCAN_IN')
+    src.append('#undef OVL_SCAN_OUT')
+    for name, stype in state:
+        src.append('    %s carry_%s = %s;' % (stype, name, name))
+    src.append('#define OVL_SCAN_IN xv[u]')
+    src.append('#define OVL_SCAN_OUT(value) ov[j][u] = (value)')
+    src.append('#define OVL_SCAN_STEP(column) { %s = (%s)(column); %s }' % (
+        counter_name, counter_type, ' '.join(body)))
+    rounds = num_batches // sets
+    last = num_batches - 1
+    if rounds:
+        src.append('    #pragma unroll 1')
+        src.append('    for (uint32_t b0 = 0; b0 < %du; b0 += %du) {' % (rounds * sets, sets))
+        # past the end a set is refilled with the last batch again, which keeps the loop free of branches
+        for k in range(sets):
+            process('q%d' % k, 'b0 + %du' % k, '(b0 + %du < %du ? b0 + %du : %du)' % (k + sets, num_batches, k + sets, last))
+        src.append('    }')
+    for k in range(num_batches % sets):
+        src.append('    {')
+        process('q%d' % k, '%du' % (rounds * sets + k), None)
+        src.append('    }')
+    src.append('#undef OVL_SCAN_STEP')
+    src.append('#undef OVL_SCAN_IN')
+    src.append('#undef OVL_SCAN_OUT')
+    src.append('}')
+
+    launch = {
+        'template': 'skewscan',
+        'vec': vec,
+        'block': BLOCK,
+        'blocks_needed': (p.rows + rows_per_block - 1) // rows_per_block,
+        'align': {('in', p.x.io_index): 16, ('out', p.out.io_index): 16},
+        'vector_loads': 1,
+        'vector_stores': 1,
+    }
+    return '\n'.join(src) + '\n', launch

@@ -35,6 +35,11 @@ def _io_types(op):
             [TensorType.from_proto(e.tensor_type) for e in outs])
 
 
+# Code generator options applied to every operator that is loaded without explicit options, e.g. {'template': 'map'}
+# to force the general kernel template (see hipgen.generate).
+codegen_options = {}
+
+
 def build_operator(op, options=None):
     """Generate HIP for one operator and make sure its library exists on disk.  Needs hipcc, not a GPU.
 
@@ -99,6 +104,8 @@ class CompiledOperator(object):
 
 
 def load_operator(op, options=None):
+    if options is None and codegen_options:
+        options = dict(codegen_options)
     name = _op_hash(op)
     key = (name, repr(sorted((options or {}).items())))
     with _lock:

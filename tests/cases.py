@@ -568,6 +568,28 @@ def _operators_of(outputs, opt_level):
     return list(dag.operators)
 
 
+# (case, code generator options): the same cases through kernel templates the generator would not pick by itself
+TEMPLATE_VARIANTS = [
+    ('c3_rowscan_shapes', {'template': 'rowscan'}),
+    ('c3_cumsum_f32', {'template': 'rowscan'}),
+    ('c3_cumprod_f64', {'template': 'rowscan'}),
+    ('c3_rowscan_shapes', {'template': 'map'}),
+    ('c3_rowscan_shapes', {'scan_depth': 1, 'scan_sets': 3}),
+    ('c3_cumsum_f32', {'scan_depth': 2, 'scan_sets': 2}),
+    ('c5_variants', {'template': 'map'}),
+    ('c2_chain', {'vec': 2}),
+]
+
+
+def run_variant_on_gpu(name, options):
+    from opveclib_amd import runtime
+    runtime.codegen_options = dict(options)
+    try:
+        run_case_on_gpu(CASE_BY_NAME[name], 3)
+    finally:
+        runtime.codegen_options = {}
+
+
 def prebuild_all(cases=None, workers=8, with_oracle=True):
     """Compile the HIP library (and the oracle library) of every operator used by the cases and the benchmark."""
     from concurrent.futures import ThreadPoolExecutor
@@ -588,10 +610,17 @@ def prebuild_all(cases=None, workers=8, with_oracle=True):
         for op in _operators_of(outs, 3):
             ops[op.SerializeToString()] = op
 
+    variants = []
+    if cases is None:
+        for name, options in TEMPLATE_VARIANTS:
+            for op in _operators_of(CASE_BY_NAME[name].outputs(), 3):
+                variants.append((op, options))
+
     compiler.prebuild_mode = True
     try:
         with ThreadPoolExecutor(max_workers=workers) as pool:
             list(pool.map(runtime.build_operator, ops.values()))
+            list(pool.map(lambda v: runtime.build_operator(*v), variants))
             if with_oracle:
                 list(pool.map(oracle.compile_op, oracle_ops.values()))
     finally:

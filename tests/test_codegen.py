@@ -77,8 +77,10 @@ def test_template_selection():
     assert template(stdops.add(f32, f32))['template'] == 'map'
     # last-axis accumulation with a chunkable row length: the order-preserving row scan
     scan = template(cumsum(np.zeros((48, 1024), np.float32), axis=1))
-    assert scan['template'] == 'rowscan' and scan['blocks_needed'] == 48
-    assert template(cumsum(np.zeros((1024, 16384), np.float64), axis=1))['blocks_needed'] == 256
+    assert scan['template'] == 'skewscan' and scan['blocks_needed'] == 3       # 16 rows per workgroup
+    assert template(cumsum(np.zeros((1024, 16384), np.float64), axis=1))['blocks_needed'] == 64
+    lds = template(cumsum(np.zeros((48, 1024), np.float32), axis=1), {'template': 'rowscan'})
+    assert lds['template'] == 'rowscan' and lds['blocks_needed'] == 48
     assert template(cumsum(np.zeros((48, 1024), np.float32), axis=1), {'template': 'map'})['template'] == 'map'
     # rows that are not a multiple of 64 long, other axes, and loop bodies with branches use the general template
     assert template(cumsum(np.zeros((48, 1000), np.float32), axis=1))['template'] == 'map'

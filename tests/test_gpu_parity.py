@@ -33,6 +33,13 @@ def test_case_matches_oracle(case):
         cases.run_case_on_gpu(case, level)
 
 
+@pytest.mark.parametrize('name,options', cases.TEMPLATE_VARIANTS,
+                         ids=['%s-%s' % (n, '-'.join('%s=%s' % kv for kv in sorted(o.items())))
+                              for n, o in cases.TEMPLATE_VARIANTS])
+def test_forced_template_matches_oracle(name, options):
+    cases.run_variant_on_gpu(name, options)
+
+
 def test_loaded_operators_come_from_the_hip_extension():
     """The results above were produced by hipcc-built operator libraries loaded through libovl_launch.so."""
     from opveclib_amd import launcher
@@ -40,4 +47,4 @@ def test_loaded_operators_come_from_the_hip_extension():
     assert len(runtime._loaded) > 0
     for compiled in runtime._loaded.values():
         assert compiled.so_path.endswith('_generic_hip.so')
-        assert compiled.lib.info['template'] in ('map', 'transpose', 'rowscan')
+        assert compiled.lib.info['template'] in ('map', 'transpose', 'rowscan', 'skewscan')
