@@ -32,9 +32,10 @@ import numpy as np
 
 HBM_PEAK_GBPS = 8000.0
 
-# HBM bytes per launch of the chain8 kernel from rocprofv3 counters (FETCH_SIZE + WRITE_SIZE, scaled by the same
-# counters' reading for a copy kernel of known size); None until measured.  Source: profiles/chain8_*.txt
-CHAIN8_TRAFFIC_BYTES = None
+# HBM bytes per launch of the chain8 kernel from rocprofv3 counters (FETCH_SIZE 262231.6, WRITE_SIZE 262144.0, each
+# scaled by the same counter's reading for the copy kernel of known size: factors 1.99982 and 0.99957).
+# Source: profiles/bench_all_kernels_hbm_traffic_counters.md
+CHAIN8_TRAFFIC_BYTES = 805322727
 
 
 class Spec(object):
@@ -51,6 +52,20 @@ class Spec(object):
 def chain8_outputs(a, b, s):
     from tests.cases import chain8
     return [chain8(a, b, s)[-1][0]]
+
+
+def copy_outputs(x):
+    """out[pos] = x[pos]: the plain copy kernel that calibrates the profiler's byte counters."""
+    import opveclib_amd as ovl
+
+    @ovl.operator()
+    def copy(arg):
+        pos = ovl.position_in(arg.shape)
+        out = ovl.output_like(arg)
+        out[pos] = arg[pos]
+        return out
+
+    return [copy(x)[0]]
 
 
 def c1_outputs(x):
@@ -90,6 +105,7 @@ def all_workload_outputs():
     f32, f64 = np.float32, np.float64
     yield chain8_outputs(Spec((8192, 8192)), Spec((8192, 8192)), Spec((1,)))
     yield chain8_outputs(Spec((2048, 8192)), Spec((2048, 8192)), Spec((1,)))
+    yield copy_outputs(Spec((8192, 8192)))
     yield c1_outputs(Spec((1 << 20,)))
     yield cumsum_outputs(Spec((4096, 16384), f32))
     yield cumprod_outputs(Spec((4096, 16384), f32))
@@ -249,6 +265,8 @@ def main():
     if not args.no_others:
         others = []
         steps = max(5, min(args.steps, 20))
+        others.append(side_workload('copy f32[8192,8192] (counter calibration, plain copy bandwidth)',
+                                    copy_outputs(a), steps, args.warmup))
         g = np.random.default_rng(0)
         others.append(side_workload('c1 shift_cyclic -> expm1 -> log1p, f32[2^20]',
                                     c1_outputs(uniform(g, -0.9, 0.9, 1 << 20)), steps, args.warmup))
