@@ -126,7 +126,7 @@ def uniform(rng, lo, hi, shape, dtype=np.float32):
 class Prepared(object):
     """A fused operator DAG with its device tensors, ready to be launched repeatedly."""
 
-    def __init__(self, outputs):
+    def __init__(self, outputs, options=None):
         import torch
         from opveclib_amd import runtime
         from opveclib_amd.operator import _build_op_dag
@@ -136,7 +136,7 @@ class Prepared(object):
         self.device = torch.device('cuda', 0)
         self.leaves = [x if isinstance(x, torch.Tensor) else torch.from_numpy(np.ascontiguousarray(x)).to(self.device)
                        for x in op_dag.inputs]
-        self.ops = [runtime.load_operator(op) for op in self.dag.operators]
+        self.ops = [runtime.load_operator(op, options) for op in self.dag.operators]
         self.buffers = []
         self.steps = []
         for op_index, compiled in enumerate(self.ops):
@@ -181,8 +181,8 @@ def measure(prepared, steps, warmup):
     return (t1 - t0) * 1e3 / steps, float(np.mean(per_launch)), float(np.min(per_launch))
 
 
-def side_workload(name, outputs, steps, warmup):
-    prepared = Prepared(outputs)
+def side_workload(name, outputs, steps, warmup, options=None):
+    prepared = Prepared(outputs, options)
     wall_ms, event_ms, min_ms = measure(prepared, steps, warmup)
     gbps = prepared.algorithmic_bytes / (event_ms * 1e-3) / 1e9
     return {'workload': name, 'us': round(event_ms * 1e3, 2), 'min_us': round(min_ms * 1e3, 2),
@@ -265,6 +265,21 @@ def main():
     if not args.no_others:
         others = []
         steps = max(5, min(args.steps, 20))
+        # The optional 'fast' math mode (device math library, reciprocal-based division): not bit-compatible with the
+        # reference, so it is reported beside the headline, with its distance from the exact result.
+        fast = Prepared(chain8_outputs(chain.leaves[0], chain.leaves[1], chain.leaves[2]), {'math': 'fast'})
+        _, fast_ms, fast_min = measure(fast, steps, args.warmup)
+        exact_y, fast_y = chain.results()[0], fast.results()[0]
+        err = (fast_y.double() - exact_y.double()).abs()
+        ulps = (fast_y.view(torch.int32).long() - exact_y.view(torch.int32).long()).abs()
+        fast_gbps = nbytes / (fast_ms * 1e-3) / 1e9
+        others.append({'workload': "chain8 in the optional 'fast' math mode (not the parity path)",
+                       'us': round(fast_ms * 1e3, 2), 'min_us': round(fast_min * 1e3, 2),
+                       'GB/s': round(fast_gbps, 1), 'frac': round(fast_gbps / HBM_PEAK_GBPS, 4),
+                       'algorithmic_bytes': nbytes, 'kernels': [k['kernel'] for k in fast.kernels],
+                       'vs_exact': {'max_abs_err': float(err.max()), 'frac_bit_equal': float((ulps == 0).double().mean()),
+                                    'frac_within_2ulp': float((ulps <= 2).double().mean())}})
+        del fast, exact_y, fast_y, err, ulps
         others.append(side_workload('copy f32[8192,8192] (counter calibration, plain copy bandwidth)',
                                     copy_outputs(a), steps, args.warmup))
         g = np.random.default_rng(0)
@@ -288,6 +303,10 @@ def main():
                                     args.warmup))
         others.append(side_workload('c4 lstm cell gradient [4096, 4x1024]',
                                     lstm_grad_outputs(concat, c, dc, dh), steps, args.warmup))
+        others.append(side_workload("c4 lstm cell forward in the optional 'fast' math mode", lstm_outputs(concat, c),
+                                    steps, args.warmup, {'math': 'fast'}))
+        others.append(side_workload("c4 lstm cell gradient in the optional 'fast' math mode",
+                                    lstm_grad_outputs(concat, c, dc, dh), steps, args.warmup, {'math': 'fast'}))
         torch.cuda.empty_cache()
         g5 = torch.Generator(device='cuda')
         g5.manual_seed(5)

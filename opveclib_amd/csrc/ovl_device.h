@@ -59,6 +59,16 @@ __device__ __forceinline__ T ovl_dpp_move(T old, T src) {
 #define ovl_logf(x) ovl_math::logf_((x), ovl_log_tab)
 #define ovl_tanhf(x) ovl_math::tanhf_(x)
 
+// Division for the 'fast' math mode: hardware reciprocal plus one residual correction.  Faithfully rounded (at most one
+// unit in the last place from the exact quotient) when the divisor's magnitude lies in [2^-126, 2^126] and the
+// quotient is a normal number; outside that range use the exact mode.
+__device__ __forceinline__ float ovl_fast_divf(float a, float b) {
+    const float r = __builtin_amdgcn_rcpf(b);
+    const float q = a * r;
+    const float e = __builtin_fmaf(-b, q, a);
+    return __builtin_fmaf(e, r, q);
+}
+
 #define OVL_DECLARE_MATH_TABLES()                                              \
     __shared__ ovl_math::lds_tables ovl_lds_tables;                            \
     ovl_math::load_tables(ovl_lds_tables);                                     \

@@ -312,6 +312,8 @@ class DagInfo(object):
     # -- queries ---------------------------------------------------------------------------------------------------
     def uses_math_tables(self):
         """True when the body calls the table-driven float32 exp or log."""
+        if getattr(self, 'math', 'exact') != 'exact':
+            return False
         return any(n.code in (lang.EXP, lang.LOG) and n.dtype == lang.FLOAT32 for n in self.nodes)
 
     def tensor_accesses(self):

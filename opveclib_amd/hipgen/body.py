@@ -39,6 +39,15 @@ UNARY = {
     lang.ISFINITE: {lang.FLOAT32: 'isfinite', lang.FLOAT64: 'isfinite'},
     lang.ISNAN: {lang.FLOAT32: 'isnan', lang.FLOAT64: 'isnan'},
 }
+# Float32 math per mode: {mode: {expression code: function name}}; DIVIDE maps to a two-argument function.
+# 'exact' (the default) is the table above plus the IEEE '/' operator: the host C library's bits.  'fast' calls the
+# device math library (each result within one unit in the last place of the correctly rounded one over the whole
+# argument range) and divides with a corrected hardware reciprocal.
+MATH_MODES = {
+    'exact': {},
+    'fast': {lang.TANH: 'tanhf', lang.EXP: 'expf', lang.LOG: 'logf', lang.DIVIDE: 'ovl_fast_divf'},
+}
+
 _NEGATABLE = (lang.FLOAT32, lang.FLOAT64, lang.INT8, lang.INT16, lang.INT32, lang.INT64)
 UNARY[lang.NEGATE] = dict((t, '-') for t in _NEGATABLE)
 UNARY[lang.NOT] = dict((t, '!') for t in CTYPE)
@@ -125,6 +134,7 @@ class BodyEmitter(object):
     def emit_tagged(self):
         """[(index of the expression that produced it, statement text)] in program order."""
         info = self.info
+        fast = MATH_MODES[getattr(info, 'math', 'exact')]
         names = {}
         stmts = []
         indent = 0
@@ -193,7 +203,12 @@ class BodyEmitter(object):
                 put('} else {')
                 indent += 1
             elif code in UNARY:
-                put(CTYPE[node.dtype] + ' ' + name + ' = ' + UNARY[code][node.dtype] + '(' + names[ops[0]] + ');')
+                fcn = UNARY[code][node.dtype]
+                if node.dtype == lang.FLOAT32 and code in fast:
+                    fcn = fast[code]
+                put(CTYPE[node.dtype] + ' ' + name + ' = ' + fcn + '(' + names[ops[0]] + ');')
+            elif code == lang.DIVIDE and node.dtype == lang.FLOAT32 and code in fast:
+                put('float ' + name + ' = ' + fast[code] + '(' + names[ops[0]] + ', ' + names[ops[1]] + ');')
             elif code in INFIX or code in (lang.MIN, lang.MAX, lang.POW, lang.ATAN2):
                 put(CTYPE[node.dtype] + ' ' + name + ' = ' +
                     binary_text(code, node.dtype, names[ops[0]], names[ops[1]]) + ';')

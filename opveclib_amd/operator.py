@@ -497,38 +497,69 @@ def _normalise_output_list(output_list):
     return list(output_list)
 
 
-def evaluate(output_list, target_language='hip', opt_level=3):
+MATH_MODES = ('exact', 'fast')
+_default_math_mode = [None]
+
+
+def set_math_mode(mode):
+    """
+    Choose the float32 math library of operators evaluated from now on.
+
+    'exact' (the default) reproduces the host C library's expf/logf/tanhf bit for bit and divides with IEEE rounding,
+    so results equal those of the reference's generated C++ on the same inputs.  'fast' uses the device math library
+    and a reciprocal-based division: every exp/log/tanh and every quotient is within one or two units in the last
+    place of the exact mode's, at roughly half the arithmetic cost.  The environment variable OPVECLIB_MATH sets the
+    initial mode.
+    """
+    if mode not in MATH_MODES:
+        raise ValueError('math mode must be one of ' + str(MATH_MODES))
+    _default_math_mode[0] = mode
+
+
+def get_math_mode():
+    if _default_math_mode[0] is None:
+        import os
+        set_math_mode(os.environ.get('OPVECLIB_MATH', 'exact'))
+    return _default_math_mode[0]
+
+
+def evaluate(output_list, target_language='hip', opt_level=3, math_mode=None):
     """
     Evaluate a collection of OVL operator outputs on the GPU (operator.py:2099-2117).
 
     :param output_list: an operator, an operator output, or a list of either
     :param target_language: must be 'hip'
     :param opt_level: operators are fused when opt_level >= 3
+    :param math_mode: 'exact' or 'fast' for this call (see :func:`set_math_mode`); None uses the current default
     :return: one array for a single requested output, otherwise a list in request order.  Arrays are numpy arrays
         when every DAG input was a numpy array, otherwise torch tensors on the inputs' device.
     """
-    evaluated_outputs = _run(output_list, target_language, 1, opt_level, timed=False)[0]
+    evaluated_outputs = _run(output_list, target_language, 1, opt_level, timed=False, math_mode=math_mode)[0]
     if len(evaluated_outputs) == 1:
         return evaluated_outputs[0]
     return evaluated_outputs
 
 
-def profile(output_list, target_language='hip', profiling_iterations=1, opt_level=3):
+def profile(output_list, target_language='hip', profiling_iterations=1, opt_level=3, math_mode=None):
     """
     Evaluate a collection of OVL operator outputs and time every generated operator (operator.py:2120-2335).
 
     :param profiling_iterations: number of timed launches per operator, a positive int
     :return: (outputs, {operator hash name: float64[profiling_iterations] milliseconds})
     """
-    return _run(output_list, target_language, profiling_iterations, opt_level, timed=True)
+    return _run(output_list, target_language, profiling_iterations, opt_level, timed=True, math_mode=math_mode)
 
 
-def _run(output_list, target_language, profiling_iterations, opt_level, timed):
+def _run(output_list, target_language, profiling_iterations, opt_level, timed, math_mode=None):
     if target_language != 'hip':
         raise ValueError('Unsupported target_language: ' + str(target_language) +
                          '. This package generates HIP kernels for gfx950 only (target_language=\'hip\').')
     if not isinstance(profiling_iterations, int) or profiling_iterations < 1:
         raise ValueError('profiling_iterations must be a positive int')
+    if math_mode is None:
+        math_mode = get_math_mode()
+    if math_mode not in MATH_MODES:
+        raise ValueError('math_mode must be one of ' + str(MATH_MODES))
 
     from .fusion import _merge_op_dag
     from . import runtime
@@ -537,4 +568,5 @@ def _run(output_list, target_language, profiling_iterations, opt_level, timed):
     dag = op_dag.proto_dag
     if opt_level >= 3:
         dag, _ = _merge_op_dag(dag, None)
-    return runtime.run_op_dag(dag, op_dag.inputs, profiling_iterations, timed=timed)
+    options = None if math_mode == 'exact' else {'math': math_mode}
+    return runtime.run_op_dag(dag, op_dag.inputs, profiling_iterations, timed=timed, options=options)

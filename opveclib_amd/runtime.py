@@ -104,8 +104,8 @@ class CompiledOperator(object):
 
 
 def load_operator(op, options=None):
-    if options is None and codegen_options:
-        options = dict(codegen_options)
+    if codegen_options:
+        options = dict(codegen_options, **(options or {}))
     name = _op_hash(op)
     key = (name, repr(sorted((options or {}).items())))
     with _lock:

@@ -10,6 +10,7 @@ import numpy as np
 
 import opveclib_amd as ovl
 from opveclib_amd import stdops
+from opveclib_amd import language as lang
 from opveclib_amd.examples import (shift_cyclic, cumsum, cumprod, accumulate, expm1, log1p, absolute,
                                    gather_transpose)
 from opveclib_amd.lstm import lstm, lstm_grad
@@ -568,6 +569,96 @@ def _operators_of(outputs, opt_level):
     return list(dag.operators)
 
 
+# ----------------------------------------------------------------------------------------------------------------------
+# 'fast' math mode: every transcendental operator on its own, compared with the oracle in units in the last place
+# ----------------------------------------------------------------------------------------------------------------------
+def _log_uniform(rng, lo_exp, hi_exp, n):
+    """Magnitudes spread evenly over binades 2^lo_exp .. 2^hi_exp."""
+    return np.exp2(rng.uniform(lo_exp, hi_exp, n)).astype(np.float32)
+
+
+def fast_stage_inputs(rng, n=1 << 16):
+    """Stage inputs of the 8-op chain drawn like the benchmark's (A, B uniform[-1, 1]) plus wide-range sweeps."""
+    a = uniform(rng, -1, 1, n)
+    b = uniform(rng, -1, 1, n)
+    t2 = (a + b) * np.float32(1.0001)
+    t3 = np.tanh(t2).astype(np.float32)
+    t4 = (1.0 / (1.0 + np.exp(-t3.astype(np.float64)))).astype(np.float32)
+    t5 = np.log1p(t4.astype(np.float64)).astype(np.float32)
+    sign = np.where(rng.random(n) < 0.5, -1.0, 1.0).astype(np.float32)
+    return {
+        'tanh_chain': t2, 'sigmoid_chain': t3, 'log1p_chain': t4, 'expm1_chain': t5,
+        'tanh_wide': sign * _log_uniform(rng, -30, 5, n),
+        'sigmoid_wide': sign * _log_uniform(rng, -30, 6.4, n),
+        'log1p_wide': np.concatenate([_log_uniform(rng, -30, 30, n // 2), -_log_uniform(rng, -30, -0.01, n // 2)]),
+        'expm1_wide': sign * _log_uniform(rng, -30, 6.4, n),
+        'exp_wide': sign * _log_uniform(rng, -20, 6.6, n),
+        'log_wide': _log_uniform(rng, -140, 127, n),
+        'div_wide': (sign * _log_uniform(rng, -60, 60, n), _log_uniform(rng, -60, 60, n)),
+    }
+
+
+def _fast_case(name, key, fcn, max_ulp=2):
+    def build(rng):
+        x = fast_stage_inputs(rng)[key]
+        return [fcn(*x)[0]] if isinstance(x, tuple) else [fcn(x)[0]]
+    return Case('fast_' + name, build, max_ulp=max_ulp, seed=2)
+
+
+def _raw_exp_op():
+    @ovl.operator()
+    def raw_exp(x):
+        pos = ovl.position_in(x.shape)
+        out = ovl.output_like(x)
+        out[pos] = ovl.exp(x[pos])
+        return out
+    return raw_exp
+
+
+def _raw_log_op():
+    @ovl.operator()
+    def raw_log(x):
+        pos = ovl.position_in(x.shape)
+        out = ovl.output_like(x)
+        out[pos] = ovl.log(x[pos])
+        return out
+    return raw_log
+
+
+# Single library calls and the division stay within 2 units in the last place of the oracle.  Operators composed of
+# several of them (sigmoid = 1/(1+exp(-x)), log1p = log(u)*x/(u-1), expm1 = (e-1)*x/log(e)) add the differences up:
+# 4 units is the largest distance observed over these sweeps.
+FAST_CASES = [
+    _fast_case('tanh_chain', 'tanh_chain', stdops.tanh),
+    _fast_case('sigmoid_chain', 'sigmoid_chain', stdops.sigmoid, 4),
+    _fast_case('log1p_chain', 'log1p_chain', log1p, 4),
+    _fast_case('expm1_chain', 'expm1_chain', expm1, 4),
+    _fast_case('tanh_wide', 'tanh_wide', stdops.tanh),
+    _fast_case('sigmoid_wide', 'sigmoid_wide', stdops.sigmoid, 4),
+    _fast_case('log1p_wide', 'log1p_wide', log1p, 4),
+    _fast_case('expm1_wide', 'expm1_wide', expm1, 4),
+    _fast_case('exp_wide', 'exp_wide', _raw_exp_op()),
+    _fast_case('log_wide', 'log_wide', _raw_log_op()),
+    _fast_case('div_wide', 'div_wide', stdops.div),
+]
+
+
+def run_fast_case_on_gpu(case):
+    """The case's operators unfused in 'fast' mode against the oracle (exact by construction); returns the distances."""
+    import oracle
+    outs = case.outputs()
+    ref = oracle.profile(outs, 1, 0)[0]
+    got = ovl.evaluate(outs, target_language='hip', opt_level=0, math_mode='fast')
+    got = got if isinstance(got, list) else [got]
+    dists = []
+    for g, r in zip(got, ref):
+        assert g.dtype == r.dtype and g.shape == r.shape
+        nan = np.isnan(r)
+        assert np.array_equal(np.isnan(g), nan), case.name + ': NaN pattern differs'
+        dists.append(ulp_distance(np.where(nan, 0, g).astype(r.dtype), np.where(nan, 0, r).astype(r.dtype)))
+    return dists
+
+
 # (case, code generator options): the same cases through kernel templates the generator would not pick by itself
 TEMPLATE_VARIANTS = [
     ('c3_rowscan_shapes', {'template': 'rowscan'}),
@@ -579,6 +670,10 @@ TEMPLATE_VARIANTS = [
     ('c5_variants', {'template': 'map'}),
     ('c2_chain', {'vec': 2}),
 ]
+
+
+# fused cases also evaluated end to end in 'fast' mode (tolerance on the absolute error, see the test)
+FAST_FUSED_CASES = ['c2_chain', 'c4_lstm', 'c4_lstm_grad', 'c1_shift_expm1_log1p']
 
 
 def run_variant_on_gpu(name, options):
@@ -615,6 +710,18 @@ def prebuild_all(cases=None, workers=8, with_oracle=True):
         for name, options in TEMPLATE_VARIANTS:
             for op in _operators_of(CASE_BY_NAME[name].outputs(), 3):
                 variants.append((op, options))
+        for case in FAST_CASES:
+            outs = case.outputs()
+            for op in _operators_of(outs, 0):
+                variants.append((op, {'math': 'fast'}))
+                oracle_ops[op.SerializeToString()] = op
+        for name in FAST_FUSED_CASES:
+            for op in _operators_of(CASE_BY_NAME[name].outputs(), 3):
+                variants.append((op, {'math': 'fast'}))
+        for outs in bench.all_workload_outputs():
+            for op in _operators_of(outs, 3):
+                if any(e.code in (lang.EXP, lang.LOG, lang.TANH, lang.DIVIDE) for e in op.expressions):
+                    variants.append((op, {'math': 'fast'}))
 
     compiler.prebuild_mode = True
     try:

@@ -1,0 +1,67 @@
+"""
+The 'fast' float32 math mode on the GPU.
+
+The 'fast' mode is an option next to the default 'exact' mode, which is the one that reproduces the reference's results.
+Stage-wise: every transcendental operator of the benchmark chain (tanh, sigmoid, log1p, expm1), the raw exp and log
+expressions and the division run unfused in 'fast' mode on inputs drawn like the chain's stage inputs and on
+wide-range sweeps.  Single library calls and the division must be within 2 units in the last place (float32) of the
+CPU oracle, operators composed of several of them within 4.  End to end the fused
+chain cannot be compared in units in the last place (its last stages subtract nearly equal numbers, so a one-unit
+difference in a 0.3 .. 0.7 valued intermediate is many units of a small difference): there the absolute error is
+bounded instead and the distribution is reported.
+"""
+import numpy as np
+import pytest
+
+import opveclib_amd as ovl
+import oracle
+from tests import cases
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize('case', cases.FAST_CASES, ids=[c.name for c in cases.FAST_CASES])
+def test_fast_stage_within_tolerance(case):
+    for dist in cases.run_fast_case_on_gpu(case):
+        assert dist.max() <= case.max_ulp, '%s: %d ulp, %.4f of the elements within 2' % (
+            case.name, int(dist.max()), float((dist <= 2).mean()))
+
+
+@pytest.mark.parametrize('name', cases.FAST_FUSED_CASES)
+def test_fast_fused_absolute_error(name):
+    case = cases.CASE_BY_NAME[name]
+    outs = case.outputs()
+    ref = oracle.profile(outs, 1, 0)[0]
+    got = ovl.evaluate(outs, opt_level=3, math_mode='fast')
+    got = got if isinstance(got, list) else [got]
+    for g, r in zip(got, ref):
+        scale = max(1.0, float(np.abs(r).max()))
+        # a few float32 roundings of O(1) intermediates
+        assert float(np.abs(g.astype(np.float64) - r).max()) <= 8 * np.finfo(np.float32).eps * scale
+
+
+def test_exact_ops_stay_exact_in_fast_mode():
+    """Operators without exp/log/tanh/division do not change with the math mode."""
+    rng = np.random.default_rng(9)
+    a = rng.standard_normal((64, 128), dtype=np.float32)
+    b = rng.standard_normal((64, 128), dtype=np.float32)
+    out = cases.absolute(cases.stdops.sub(cases.stdops.mul(cases.stdops.add(a, b), b), a))
+    assert np.array_equal(ovl.evaluate(out, math_mode='fast'), ovl.evaluate(out, math_mode='exact'))
+
+
+def test_math_mode_default_and_errors():
+    assert ovl.get_math_mode() in ('exact', 'fast')
+    with pytest.raises(ValueError):
+        ovl.set_math_mode('sloppy')
+    x = np.linspace(-3, 3, 256).astype(np.float32)
+    with pytest.raises(ValueError):
+        ovl.evaluate(cases.stdops.tanh(x), math_mode='sloppy')
+    previous = ovl.get_math_mode()
+    try:
+        ovl.set_math_mode('fast')
+        fast = ovl.evaluate(cases.stdops.tanh(x))
+    finally:
+        ovl.set_math_mode(previous)
+    exact = ovl.evaluate(cases.stdops.tanh(x), math_mode='exact')
+    assert cases.ulp_distance(fast, exact).max() <= 2
+    assert np.array_equal(exact, oracle.evaluate(cases.stdops.tanh(x)))
