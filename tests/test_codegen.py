@@ -90,7 +90,7 @@ def test_template_selection():
     tr = template(gather_transpose(np.zeros((192, 320), np.float32), np.zeros(192 * 320, np.float32),
                                    alpha=0.5, stride=3))
     assert tr['template'] == 'transpose' and tr['vector_loads'] == 2 and tr['vector_stores'] == 1
-    assert tr['blocks_needed'] == 3 * 5
+    assert tr['blocks_needed'] == 6 * 2                    # tiles of 32 x 256 workers
     wraps = template(gather_transpose(np.zeros((192, 320), np.float32), np.zeros(192 * 320, np.float32),
                                       alpha=0.5, stride=7919))
     assert wraps['template'] == 'transpose' and wraps['vector_loads'] == 1        # the gather index may wrap: scalar
