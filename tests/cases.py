@@ -718,6 +718,11 @@ def prebuild_all(cases=None, workers=8, with_oracle=True):
         for name in FAST_FUSED_CASES:
             for op in _operators_of(CASE_BY_NAME[name].outputs(), 3):
                 variants.append((op, {'math': 'fast'}))
+        from tests import autograd_cases
+        for outs in autograd_cases.graphs_to_build():
+            for level in (0, 3):
+                for op in _operators_of(outs, level):
+                    ops[op.SerializeToString()] = op
         for outs in bench.all_workload_outputs():
             for op in _operators_of(outs, 3):
                 if any(e.code in (lang.EXP, lang.LOG, lang.TANH, lang.DIVIDE) for e in op.expressions):
