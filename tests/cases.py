@@ -443,6 +443,28 @@ def _edge_expm1_log1p(rng):
     return [expm1(a)[0], log1p(b)[0], expm1(a32)[0], log1p(np.abs(a32))[0]]
 
 
+def _conv1d(rng):
+    from opveclib_amd.examples.conv1d import conv_1d
+    outs = []
+    for mode, orientation, taps, dtype in (('same', 'as-is', 5, np.float32), ('valid', 'flipped', 4, np.float32),
+                                           ('full', 'as-is', 3, np.float64), ('same', 'flipped', 1, np.float32)):
+        x = rng.standard_normal((2, 3, 37)).astype(dtype)
+        v = rng.standard_normal((4, 3, taps)).astype(dtype)
+        outs.append(conv_1d(x, v, kernel_orientation=orientation, mode=mode)[0])
+    x = rng.standard_normal((2, 37, 3))
+    v = rng.standard_normal((4, 5, 3))
+    outs.append(conv_1d(x, v, mode='same', data_format='NEC')[0])
+    return outs
+
+
+def _triangles(rng):
+    from opveclib_amd.examples import graph
+    outs = [graph.triangles_op(*graph.adjacency_from_edges(graph.EXAMPLE_EDGES))[0]]
+    for vertices, edges in ((40, 300), (300, 4000)):
+        outs.append(graph.triangles_op(*graph.adjacency_from_edges(rng.integers(0, vertices, size=(edges, 2))))[0])
+    return outs
+
+
 def _odd_sizes(rng):
     # sizes that are not multiples of the vector width, rank 1 and rank 3
     a = rng.standard_normal(1001, dtype=np.float32)
@@ -483,6 +505,8 @@ CASES = [
     _simple('accumulate_max', _accumulate_max),
     _simple('edge_expm1_log1p', _edge_expm1_log1p, max_ulp=2, rel=1e-12),
     _simple('odd_sizes', _odd_sizes),
+    _simple('conv1d', _conv1d),
+    _simple('triangles', _triangles),
 ]
 for _name, _fcn, _np, _kind in UNARY_FLOAT:
     for _dt in (np.float32, np.float64):

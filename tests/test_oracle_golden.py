@@ -260,6 +260,63 @@ def test_chain8_against_numpy():
     assert np.allclose(y, ref, rtol=0, atol=5e-7)
 
 
+def test_triangle_counting_example_graph_and_dense_check():
+    # examples/test_graph.py:121-130: the 7-vertex, 20-edge-record example graph has 3 triangles
+    from opveclib_amd.examples import graph
+    start, frm, to = graph.adjacency_from_edges(graph.EXAMPLE_EDGES)
+    assert len(to) == 10 and start[-1] == 10
+    count = oracle.evaluate(graph.triangles_op(start, frm, to))
+    assert count.dtype == np.uint64 and int(count.sum()) == graph.EXAMPLE_TRIANGLES == 3
+    rng = np.random.default_rng(7)
+    for vertices, edges in ((12, 40), (60, 700)):
+        pairs = rng.integers(0, vertices, size=(edges, 2))
+        got = oracle.evaluate(graph.triangles_op(*graph.adjacency_from_edges(pairs)), num_threads=3)
+        assert int(got.sum()) == graph.count_triangles_dense(pairs)
+    # a triangle-free graph (a path) and a complete graph K6 (20 triangles)
+    path = [(k, k + 1) for k in range(9)]
+    assert int(oracle.evaluate(graph.triangles_op(*graph.adjacency_from_edges(path))).sum()) == 0
+    k6 = [(a, b) for a in range(6) for b in range(a)]
+    assert int(oracle.evaluate(graph.triangles_op(*graph.adjacency_from_edges(k6))).sum()) == 20
+
+
+def test_conv1d_against_numpy_correlate():
+    # examples/conv1D.py:210-283 compares with an explicit loop; here numpy's correlate on zero-padded signals
+    from opveclib_amd.examples.conv1d import conv_1d
+    rng = np.random.default_rng(8)
+
+    def expected(x, v, mode, orientation):
+        taps = v.shape[2]
+        left, right = taps // 2, taps - taps // 2 - 1
+        pad = {'same': (left, right), 'valid': (0, 0), 'full': (taps - 1, taps - 1)}[mode]
+        out = []
+        for b in range(x.shape[0]):
+            out.append([sum(np.correlate(np.pad(x[b, c].astype(np.float64), pad),
+                                         (v[f, c, ::-1] if orientation == 'flipped' else v[f, c]).astype(np.float64),
+                                         'valid') for c in range(x.shape[1])) for f in range(v.shape[0])])
+        return np.array(out)
+
+    for mode in ('same', 'valid', 'full'):
+        for orientation in ('as-is', 'flipped'):
+            for taps in (1, 4, 5):
+                x = rng.standard_normal((2, 3, 23))
+                v = rng.standard_normal((4, 3, taps))
+                got = oracle.evaluate(conv_1d(x, v, kernel_orientation=orientation, mode=mode), num_threads=3)
+                want = expected(x, v, mode, orientation)
+                assert got.shape == want.shape
+                assert np.allclose(got, want, rtol=1e-13, atol=1e-13)
+    x = rng.standard_normal((2, 23, 3)).astype(np.float32)
+    v = rng.standard_normal((4, 5, 3)).astype(np.float32)
+    got = oracle.evaluate(conv_1d(x, v, data_format='NEC'))
+    want = expected(x.transpose(0, 2, 1), v.transpose(0, 2, 1), 'same', 'as-is').transpose(0, 2, 1)
+    assert got.dtype == np.float32 and np.allclose(got, want, rtol=1e-6, atol=1e-6)
+    with pytest.raises(ValueError):
+        conv_1d(x, v, mode='circular', data_format='NEC')
+    with pytest.raises(ValueError):
+        conv_1d(x, v[:, :, :2], data_format='NEC')
+    with pytest.raises(ValueError):
+        conv_1d(x, v, kernel_orientation='sideways', data_format='NEC')
+
+
 def test_driver_reports_argument_errors():
     import ctypes
     a = np.zeros(8, np.float32)
