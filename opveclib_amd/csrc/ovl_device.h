@@ -31,6 +31,12 @@ typedef struct ovl_tensor {
 __device__ __forceinline__ int8_t ovl_abs_8(int8_t x) { return (x < 0) ? -x : x; }
 __device__ __forceinline__ int16_t ovl_abs_16(int16_t x) { return (x < 0) ? -x : x; }
 
+// Vector accesses with and without the non-temporal (streaming) hint; the code generator picks per template.
+#define OVL_LOAD_NT(ptr) __builtin_nontemporal_load(ptr)
+#define OVL_LOAD_PLAIN(ptr) (*(ptr))
+#define OVL_STORE_NT(value, ptr) __builtin_nontemporal_store(value, ptr)
+#define OVL_STORE_PLAIN(value, ptr) (*(ptr) = (value))
+
 // Lane-to-lane moves inside a wavefront (data-parallel-primitive modifiers of the vector ALU).
 //   OVL_DPP_ROW_SHR1: lane i of every 16-lane row receives the value of lane i-1; lane 0 of the row keeps `old`
 //   OVL_DPP_ROW_ROR1: lane i receives lane i-1, lane 0 of the row receives lane 15

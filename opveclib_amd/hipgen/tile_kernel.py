@@ -63,7 +63,9 @@ def applicable(info):
     return vec
 
 
-def generate(info, kernel_name, tile_i=None, tile_j=None):
+def generate(info, kernel_name, tile_i=None, tile_j=None, nt='ls'):
+    load_fn = 'OVL_LOAD_NT' if 'l' in nt else 'OVL_LOAD_PLAIN'
+    store_fn = 'OVL_STORE_NT' if 's' in nt else 'OVL_STORE_PLAIN'
     vec = applicable(info)
     assert vec is not None
     # Measured on MI355X (float32 [16384, 16384], gather + transposed store): 32 x 256 workers per tile, i.e. one
@@ -169,8 +171,8 @@ def generate(info, kernel_name, tile_i=None, tile_j=None):
     for acc in loads.values():
         vname = vec_types[CTYPE[acc.tensor.dtype]]
         wide = acc.aff.hi >= 2 ** 32
-        src.append('                const %s %s = __builtin_nontemporal_load(reinterpret_cast<const %s*>(in%d + (%s)));'
-                   % (vname, acc.reg, vname, acc.tensor.io_index, _index_expr(acc.aff, pos_names, wide)))
+        src.append('                const %s %s = %s(reinterpret_cast<const %s*>(in%d + (%s)));'
+                   % (vname, acc.reg, load_fn, vname, acc.tensor.io_index, _index_expr(acc.aff, pos_names, wide)))
     for acc in unaligned.values():
         vname = vec_types[CTYPE[acc.tensor.dtype]]
         wide = acc.aff.hi >= 2 ** 32
@@ -186,8 +188,8 @@ def generate(info, kernel_name, tile_i=None, tile_j=None):
     for acc in stores.values():
         vname = vec_types[CTYPE[acc.tensor.dtype]]
         wide = acc.aff.hi >= 2 ** 32
-        src.append('                __builtin_nontemporal_store(%s, reinterpret_cast<%s*>(out%d + (%s)));' % (
-            acc.reg, vname, acc.tensor.io_index, _index_expr(acc.aff, pos_names, wide)))
+        src.append('                %s(%s, reinterpret_cast<%s*>(out%d + (%s)));' % (
+            store_fn, acc.reg, vname, acc.tensor.io_index, _index_expr(acc.aff, pos_names, wide)))
     src.append('            }')
     src.append('        }')
     src.append('        __syncthreads();')
@@ -206,8 +208,8 @@ def generate(info, kernel_name, tile_i=None, tile_j=None):
         src.append('                #pragma unroll')
         src.append('                for (uint32_t lane = 0; lane < %du; ++lane) v_%s[lane] = %s[oj][oi + lane];' % (
             vec, acc.reg, acc.reg))
-        src.append('                __builtin_nontemporal_store(v_%s, reinterpret_cast<%s*>(out%d + (%s)));' % (
-            acc.reg, vname, acc.tensor.io_index, _index_expr(acc.aff, pos_names, wide)))
+        src.append('                %s(v_%s, reinterpret_cast<%s*>(out%d + (%s)));' % (
+            store_fn, acc.reg, vname, acc.tensor.io_index, _index_expr(acc.aff, pos_names, wide)))
     src.append('            }')
     src.append('        }')
     src.append('        __syncthreads();')
