@@ -64,6 +64,7 @@ __device__ __forceinline__ T ovl_dpp_move(T old, T src) {
 #define ovl_expf(x) ovl_math::expf_((x), ovl_exp_tab)
 #define ovl_logf(x) ovl_math::logf_((x), ovl_log_tab)
 #define ovl_tanhf(x) ovl_math::tanhf_(x)
+#define ovl_recipf(x) ovl_math::recipf_(x)
 
 // Division for the 'fast' math mode: hardware reciprocal plus one residual correction.  Faithfully rounded (at most one
 // unit in the last place from the exact quotient) when the divisor's magnitude lies in [2^-126, 2^126] and the

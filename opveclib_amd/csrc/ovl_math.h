@@ -270,6 +270,22 @@ OVL_HD float expm1f_(float x) {
 // one is selected, which costs less on a wavefront than branching five ways; every selected value is produced by
 // exactly the operations fdlibm performs for that case, so results are unchanged (checked against the host C
 // library over all 2^32 arguments).
+// The two quotients inside tanh.  On the device the IEEE division (scaling, reciprocal, three refinements, fix-up:
+// about 14 issue slots) is replaced by reciprocal, product and one residual correction (7 slots).  That shortcut is
+// not correctly rounded for arbitrary operands, but for the operands tanh produces it returns the same bits: the
+// results of tanhf_ with it and with IEEE division were compared on MI355X over all 2^32 arguments, zero differences
+// (the generated test library tests/native/exhaustive_math.hip repeats that comparison).
+#if defined(__HIPCC__) && !defined(OVL_TANH_DIV)
+OVL_HD float tanh_div_(float a, float b) {
+    const float r = __builtin_amdgcn_rcpf(b);
+    const float q = a * r;
+    return __builtin_fmaf(__builtin_fmaf(-b, q, a), r, q);
+}
+#define OVL_TANH_DIV(a, b) tanh_div_((a), (b))
+#endif
+#ifndef OVL_TANH_DIV
+#define OVL_TANH_DIV(a, b) ((a) / (b))
+#endif
 OVL_HD float tanhf_(float x) {
     const float one = 1.0f, two = 2.0f, tiny = 1.0e-30f;
     const float ln2_hi = 6.9313812256e-01f, ln2_lo = 9.0580006145e-06f, invln2 = 1.4426950216e+00f;
@@ -305,7 +321,7 @@ OVL_HD float tanhf_(float x) {
     float hxs = xr * hfx;
     float r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
     float t3 = 3.0f - r1 * hfx;
-    float e = hxs * ((r1 - t3) / (6.0f - xr * t3));
+    float e = hxs * OVL_TANH_DIV(r1 - t3, 6.0f - xr * t3);
 
     float res0 = xr - (xr * e - hxs);               // k == 0
     float e2 = xr * (e - c) - c;
@@ -324,10 +340,24 @@ OVL_HD float tanhf_(float x) {
     float resk = tail_a ? y - one : y;
     float em1 = (k == 0) ? res0 : ((k == -1) ? resm1 : resk);
 
-    float q = (big ? two : -em1) / (em1 + two);
+    float q = OVL_TANH_DIV(big ? two : -em1, em1 + two);
     float z = big ? one - q : q;
     return negative ? -z : z;
 }
+
+#if defined(__HIPCC__)
+// 1.0f / b.  Hardware reciprocal plus one Newton refinement is the correctly rounded reciprocal for every divisor
+// with 2^-126 <= |b| < 2^126 (compared with IEEE division on MI355X over all 2^32 divisors: the only differences are
+// subnormal divisors and divisors of 2^126 and above, whose reciprocals are subnormal); those, zeros, infinities and
+// NaN take the IEEE division.
+OVL_HD float recipf_(float b) {
+    float r = __builtin_amdgcn_rcpf(b);
+    r = __builtin_fmaf(__builtin_fmaf(-b, r, 1.0f), r, r);
+    const float ab = __builtin_fabsf(b);
+    if (!(ab >= 0x1p-126f && ab < 0x1p126f)) r = 1.0f / b;
+    return r;
+}
+#endif
 
 }  // namespace ovl_math
 

@@ -127,6 +127,13 @@ class BodyEmitter(object):
             return 'position'
         return 'e' + str(node.idx) + self.suffix
 
+    def _is_constant_one(self, idx):
+        """The expression is the literal 1, directly or through casts (a VARIABLE could be reassigned: excluded)."""
+        node = self.info.nodes[idx]
+        while node.code == lang.CAST:
+            node = self.info.nodes[node.ops[0]]
+        return node.code == lang.CONST_SCALAR and len(node.data) == 1 and float(node.data[0]) == 1.0
+
     def emit(self):
         """All statements of the worker, in order."""
         return [text for _, text in self.emit_tagged()]
@@ -207,6 +214,10 @@ class BodyEmitter(object):
                 if node.dtype == lang.FLOAT32 and code in fast:
                     fcn = fast[code]
                 put(CTYPE[node.dtype] + ' ' + name + ' = ' + fcn + '(' + names[ops[0]] + ');')
+            elif code == lang.DIVIDE and node.dtype == lang.FLOAT32 and code not in fast and \
+                    self._is_constant_one(ops[0]):
+                # 1/x: the verified correctly rounded reciprocal (ovl_math.h) instead of the general division
+                put('float ' + name + ' = ovl_recipf(' + names[ops[1]] + ');')
             elif code == lang.DIVIDE and node.dtype == lang.FLOAT32 and code in fast:
                 put('float ' + name + ' = ' + fast[code] + '(' + names[ops[0]] + ', ' + names[ops[1]] + ');')
             elif code in INFIX or code in (lang.MIN, lang.MAX, lang.POW, lang.ATAN2):

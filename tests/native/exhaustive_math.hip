@@ -1,0 +1,151 @@
+// Test infrastructure: exhaustive checks of the device float32 math over all 2^32 argument bit patterns.
+//
+//   ovl_exh_against_host   device expf / logf / tanhf / reciprocal (opveclib_amd/csrc/ovl_math.h, as generated kernels
+//                          call them) against the host C library's expf / logf / tanhf / (1.0f / x) on this machine
+//                          (function 4 evaluates the device math library's own expf instead: a self-test of the
+//                          checker, which must report differences for it)
+//   ovl_exh_tanh_division  device tanhf with its shortened divisions against the same code with IEEE divisions
+//
+// Built by tests/native/build.py into tests/native/libexhaustive_math.so; called through ctypes by
+// tests/test_gpu_math_exhaustive.py.  Plain C ABI: returns 0 on success, a HIP error code otherwise.
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdint.h>
+#include <string.h>
+#include <thread>
+#include <vector>
+
+#include "ovl_device.h"
+
+// a second copy of tanhf_ with IEEE divisions, for the division check
+namespace ovl_ieee {
+using namespace ovl_math;
+#undef OVL_TANH_DIV
+#define OVL_TANH_DIV(a, b) ((a) / (b))
+#define tanhf_ tanhf_ieee_
+#include "tanh_body.inc"
+#undef tanhf_
+}  // namespace ovl_ieee
+
+namespace {
+
+enum { FN_EXP = 0, FN_LOG = 1, FN_TANH = 2, FN_RECIP = 3, FN_DEVICE_LIBRARY_EXP = 4 };
+
+__global__ void __launch_bounds__(256) eval_kernel(int fn, uint32_t first, uint32_t count, float* __restrict__ out) {
+    OVL_DECLARE_MATH_TABLES();
+    const uint32_t stride = gridDim.x * blockDim.x;
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride) {
+        const float x = __builtin_bit_cast(float, first + i);
+        float y;
+        if (fn == FN_EXP) y = ovl_expf(x);
+        else if (fn == FN_LOG) y = ovl_logf(x);
+        else if (fn == FN_TANH) y = ovl_tanhf(x);
+        else if (fn == FN_RECIP) y = ovl_recipf(x);
+        else y = expf(x);            // the device math library's own expf: differs from the host's in the last place
+        out[i] = y;
+    }
+}
+
+__global__ void __launch_bounds__(256) tanh_division_kernel(unsigned long long* __restrict__ mismatches,
+                                                            uint32_t* __restrict__ first_bad) {
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    unsigned long long bad = 0;
+    for (uint64_t u = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; u < (1ull << 32); u += stride) {
+        const float x = __builtin_bit_cast(float, (uint32_t)u);
+        const float a = ovl_math::tanhf_(x), b = ovl_ieee::tanhf_ieee_(x);
+        const bool same = __builtin_bit_cast(uint32_t, a) == __builtin_bit_cast(uint32_t, b) || (a != a && b != b);
+        if (!same) {
+            ++bad;
+            atomicMin(first_bad, (uint32_t)u);
+        }
+    }
+    if (bad) atomicAdd(mismatches, bad);
+}
+
+float host_value(int fn, float x) {
+    if (fn == FN_EXP || fn == FN_DEVICE_LIBRARY_EXP) return expf(x);
+    if (fn == FN_LOG) return logf(x);
+    if (fn == FN_TANH) return tanhf(x);
+    volatile float one = 1.0f;          // keep the division at run time
+    return one / x;
+}
+
+}  // namespace
+
+extern "C" int ovl_exh_tanh_division(uint64_t* mismatches, uint32_t* first_bad) {
+    unsigned long long* d_count = nullptr;
+    uint32_t* d_first = nullptr;
+    hipError_t err = hipMalloc(&d_count, sizeof(unsigned long long));
+    if (err != hipSuccess) return (int)err;
+    err = hipMalloc(&d_first, sizeof(uint32_t));
+    if (err != hipSuccess) return (int)err;
+    unsigned long long zero = 0;
+    uint32_t all = 0xffffffffu;
+    hipMemcpy(d_count, &zero, sizeof(zero), hipMemcpyHostToDevice);
+    hipMemcpy(d_first, &all, sizeof(all), hipMemcpyHostToDevice);
+    hipLaunchKernelGGL(tanh_division_kernel, dim3(4096), dim3(256), 0, 0, d_count, d_first);
+    err = hipDeviceSynchronize();
+    unsigned long long h = 0;
+    hipMemcpy(&h, d_count, sizeof(h), hipMemcpyDeviceToHost);
+    hipMemcpy(first_bad, d_first, sizeof(uint32_t), hipMemcpyDeviceToHost);
+    *mismatches = h;
+    hipFree(d_count);
+    hipFree(d_first);
+    return (int)err;
+}
+
+// Compare fn over the bit patterns first, first + step, ... (count of them) with the host C library.
+// step = 1 and count = 2^32 is the exhaustive run.  threads = host threads used for the host side.
+extern "C" int ovl_exh_against_host(int fn, uint64_t count, uint32_t step, uint32_t threads, uint64_t* mismatches,
+                                    uint32_t* first_bad) {
+    const uint32_t chunk = 1u << 26;
+    float* d_out = nullptr;
+    float* h_out = nullptr;
+    hipError_t err = hipMalloc(&d_out, (size_t)chunk * sizeof(float));
+    if (err != hipSuccess) return (int)err;
+    err = hipHostMalloc(&h_out, (size_t)chunk * sizeof(float), hipHostMallocDefault);
+    if (err != hipSuccess) { hipFree(d_out); return (int)err; }
+    uint64_t total_bad = 0;
+    uint32_t lowest = 0xffffffffu;
+    if (threads == 0) threads = 1;
+    // with step > 1 the device still evaluates whole chunks; the host then samples every step-th pattern
+    for (uint64_t base = 0; base < (1ull << 32) && base / step < count; base += chunk) {
+        hipLaunchKernelGGL(eval_kernel, dim3(2048), dim3(256), 0, 0, fn, (uint32_t)base, chunk, d_out);
+        err = hipMemcpy(h_out, d_out, (size_t)chunk * sizeof(float), hipMemcpyDeviceToHost);
+        if (err != hipSuccess) break;
+        std::vector<uint64_t> bad(threads, 0);
+        std::vector<uint32_t> low(threads, 0xffffffffu);
+        std::vector<std::thread> pool;
+        for (uint32_t t = 0; t < threads; ++t) {
+            pool.emplace_back([&, t]() {
+                const uint32_t begin = (uint32_t)((uint64_t)chunk * t / threads);
+                const uint32_t end = (uint32_t)((uint64_t)chunk * (t + 1) / threads);
+                uint32_t i = begin + (step - (base + begin) % step) % step;
+                for (; i < end; i += step) {
+                    const uint32_t bits = (uint32_t)base + i;
+                    float x;
+                    memcpy(&x, &bits, 4);
+                    const float want = host_value(fn, x);
+                    const float got = h_out[i];
+                    uint32_t wb, gb;
+                    memcpy(&wb, &want, 4);
+                    memcpy(&gb, &got, 4);
+                    if (wb != gb && !(want != want && got != got)) {
+                        ++bad[t];
+                        if (bits < low[t]) low[t] = bits;
+                    }
+                }
+            });
+        }
+        for (auto& th : pool) th.join();
+        for (uint32_t t = 0; t < threads; ++t) {
+            total_bad += bad[t];
+            if (low[t] < lowest) lowest = low[t];
+        }
+    }
+    hipFree(d_out);
+    hipHostFree(h_out);
+    *mismatches = total_bad;
+    *first_bad = lowest;
+    return (int)err;
+}

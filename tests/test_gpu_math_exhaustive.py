@@ -1,0 +1,61 @@
+"""
+Exhaustive checks of the device float32 math on the GPU, through the native test library of tests/native.
+
+`test_device_math_equals_host_libm_*`: the device expf / logf / tanhf and the reciprocal that generated kernels call are
+evaluated for float bit patterns and compared bit for bit with the host C library's expf / logf / tanhf / (1.0f / x) on
+the machine the test runs on.  By default every 16th bit pattern is compared (2^28 arguments per function, all
+exponents and both signs); OVL_EXHAUSTIVE=1 compares all 2^32 (about 10 s per function with 16 host threads).
+`test_tanh_shortened_divisions_*`: all 2^32 arguments, device against device.
+"""
+import ctypes
+import os
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIBRARY = os.path.join(HERE, 'native', 'libexhaustive_math.so')
+FUNCTIONS = {'expf': 0, 'logf': 1, 'tanhf': 2, 'reciprocal': 3}
+
+
+@pytest.fixture(scope='module')
+def lib():
+    if not os.path.exists(LIBRARY):
+        from tests.native import build
+        build.build()
+    handle = ctypes.CDLL(LIBRARY)
+    handle.ovl_exh_against_host.argtypes = [ctypes.c_int, ctypes.c_uint64, ctypes.c_uint32, ctypes.c_uint32,
+                                            ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint32)]
+    handle.ovl_exh_tanh_division.argtypes = [ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint32)]
+    return handle
+
+
+@pytest.mark.parametrize('name', sorted(FUNCTIONS))
+def test_device_math_equals_host_libm(lib, name):
+    step = 1 if os.environ.get('OVL_EXHAUSTIVE') == '1' else 16
+    count = (1 << 32) // step
+    bad = ctypes.c_uint64(0)
+    first = ctypes.c_uint32(0)
+    threads = min(16, os.cpu_count() or 1)
+    err = lib.ovl_exh_against_host(FUNCTIONS[name], count, step, threads, ctypes.byref(bad), ctypes.byref(first))
+    assert err == 0, 'HIP error %d' % err
+    assert bad.value == 0, '%s: %d of %d arguments differ from the host C library, first at bits 0x%08x' % (
+        name, bad.value, count, first.value)
+
+
+def test_checker_reports_a_library_that_differs_in_the_last_place(lib):
+    """Self-test: the device math library's own expf is a correct expf but not the host's; the checker must see it."""
+    bad = ctypes.c_uint64(0)
+    first = ctypes.c_uint32(0)
+    err = lib.ovl_exh_against_host(4, (1 << 32) // 16, 16, 16, ctypes.byref(bad), ctypes.byref(first))
+    assert err == 0
+    assert bad.value > 1000
+
+
+def test_tanh_shortened_divisions_equal_ieee_divisions_for_all_arguments(lib):
+    bad = ctypes.c_uint64(0)
+    first = ctypes.c_uint32(0)
+    err = lib.ovl_exh_tanh_division(ctypes.byref(bad), ctypes.byref(first))
+    assert err == 0, 'HIP error %d' % err
+    assert bad.value == 0, '%d arguments differ, first at bits 0x%08x' % (bad.value, first.value)
