@@ -24,6 +24,7 @@ from .analysis import ITEMSIZE
 from .body import BodyEmitter, CTYPE
 
 BLOCK = 256
+MAX_GRID = 1 << 24          # largest grid the generated entry points launch
 
 
 class Access(object):
@@ -181,11 +182,23 @@ def generate(info, kernel_name, vec=None, nt=None):
     src.append('')
     src.append('extern "C" __global__ void __launch_bounds__(%d)' % BLOCK)
     src.append(kernel_name + '(' + ', '.join(args) + ') {')
-    if info.uses_math_tables():
-        src.append('    OVL_DECLARE_MATH_TABLES();')
+    blocks_needed = (num_vectors + BLOCK - 1) // BLOCK
+    # Kernels that use the LDS math tables and whose grid covers every vector run one vector per thread without a
+    # loop: the thread requests its operands first and copies the tables (with the barrier that implies) while
+    # they are in flight, instead of waiting for the tables before the first request.
+    single_pass = info.uses_math_tables() and blocks_needed <= MAX_GRID
     src.append('    const uint32_t num_vectors = %du;' % num_vectors)
-    src.append('    const uint32_t stride = gridDim.x * %du;' % BLOCK)
-    src.append('    for (uint32_t v = blockIdx.x * %du + threadIdx.x; v < num_vectors; v += stride) {' % BLOCK)
+    if single_pass:
+        src.append('    const uint32_t v_raw = blockIdx.x * %du + threadIdx.x;' % BLOCK)
+        src.append('    const bool active = v_raw < num_vectors;')
+        src.append('    // idle threads of the last workgroup request vector 0 and store nothing')
+        src.append('    const uint32_t v = active ? v_raw : 0u;')
+        src.append('    {')
+    else:
+        if info.uses_math_tables():
+            src.append('    OVL_DECLARE_MATH_TABLES();')
+        src.append('    const uint32_t stride = gridDim.x * %du;' % BLOCK)
+        src.append('    for (uint32_t v = blockIdx.x * %du + threadIdx.x; v < num_vectors; v += stride) {' % BLOCK)
     src.append('        const uint32_t worker0 = v * %du;' % vec)
     # position of the first of this thread's workers
     block = 1
@@ -209,6 +222,9 @@ def generate(info, kernel_name, vec=None, nt=None):
         wide = acc.aff.hi >= 2 ** 32
         src.append('        const %s %s = *reinterpret_cast<const %s_u*>(in%d + (%s));' % (
             vname, acc.reg, vname, acc.tensor.io_index, _index_expr(acc.aff, pos_names, wide)))
+    if single_pass:
+        src.append('        OVL_DECLARE_MATH_TABLES();')
+        src.append('        if (active) {')
     for acc in stores.values():
         src.append('        %s %s;' % (vec_types[CTYPE[acc.tensor.dtype]], acc.reg))
 
@@ -227,6 +243,8 @@ def generate(info, kernel_name, vec=None, nt=None):
         wide = acc.aff.hi >= 2 ** 32
         src.append('        %s(%s, reinterpret_cast<%s*>(out%d + (%s)));' % (
             store_fn, acc.reg, vname, acc.tensor.io_index, _index_expr(acc.aff, pos_names, wide)))
+    if single_pass:
+        src.append('        }')
     src.append('    }')
     src.append('}')
 
@@ -242,7 +260,7 @@ def generate(info, kernel_name, vec=None, nt=None):
         'template': 'map',
         'vec': vec,
         'block': BLOCK,
-        'blocks_needed': (num_vectors + BLOCK - 1) // BLOCK,
+        'blocks_needed': blocks_needed,
         'align': align,
         'vector_loads': len(loads) + len(unaligned),
         'vector_stores': len(stores),
