@@ -27,9 +27,16 @@
 #if defined(__HIPCC__)
 #define OVL_HD __device__ __forceinline__
 #define OVL_TABLE static __device__ const
+// True when the condition holds in any lane of the wavefront: a wave-uniform value, so `if (OVL_ANY(c))` is a scalar
+// branch around a block that every lane executes or skips together.  The functions below compute their common path
+// unconditionally and repair rare arguments (NaN, infinities, overflow, subnormals) inside such blocks with per-lane
+// selects: no execution-mask juggling on the common path, and identical calls in one kernel can be merged by the
+// compiler because the common path is not nested in a condition.
+#define OVL_ANY(cond) (__builtin_amdgcn_ballot_w64(cond) != 0)
 #else
 #define OVL_HD static inline
 #define OVL_TABLE static const
+#define OVL_ANY(cond) (cond)
 #endif
 
 // Every multiply-add site can be switched between fused (bit set) and separately rounded (bit clear); the default
@@ -77,13 +84,6 @@ OVL_HD float expf_(float x, const uint64_t* tab = exp2f_tab) {
 
     double xd = (double)x;
     uint32_t abstop = top12(x) & 0x7ff;
-    if (abstop >= top12(88.0f)) {
-        // |x| >= 88 or x is nan
-        if (as_u32(x) == as_u32(-__builtin_inff())) return 0.0f;
-        if (abstop >= top12(__builtin_inff())) return x + x;
-        if (x > 0x1.62e42ep6f) return __builtin_inff();     // overflow
-        if (x < -0x1.9fe368p6f) return 0.0f;                // underflow
-    }
     // x*N/Ln2 = k + r with r in [-1/2, 1/2] and int k
     double kd = OVL_MADD(0, InvLn2N, xd, Shift);
     uint64_t ki = as_u64(kd);
@@ -98,7 +98,16 @@ OVL_HD float expf_(float x, const uint64_t* tab = exp2f_tab) {
     double y = OVL_MADD(3, C2, r, 1.0);
     y = OVL_MADD(4, z2, r2, y);
     y = y * s;
-    return (float)y;
+    float result = (float)y;
+    const bool special = abstop >= top12(88.0f);        // |x| >= 88 or x is NaN
+    if (OVL_ANY(special)) {
+        float fixed = result;                                               // 88 <= |x| below the thresholds: as computed
+        if (x < -0x1.9fe368p6f) fixed = 0.0f;                               // underflow, also -inf
+        if (x > 0x1.62e42ep6f) fixed = __builtin_inff();                    // overflow, also +inf
+        if (x != x) fixed = x + x;                                          // NaN
+        result = special ? fixed : result;
+    }
+    return result;
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
@@ -145,22 +154,10 @@ __device__ __forceinline__ void load_tables(lds_tables& t) {
 }
 #endif
 
-OVL_HD float logf_(float x, const logf_entry* tab = logf_tab) {
+OVL_HD float logf_main_(uint32_t ix, const logf_entry* tab) {
     const double Ln2 = 0x1.62e42fefa39efp-1;
     const double A0 = -0x1.00ea348b88334p-2, A1 = 0x1.5575b0be00b6ap-2, A2 = -0x1.ffffef20a4123p-2;
     const uint32_t Off = 0x3f330000;
-
-    uint32_t ix = as_u32(x);
-    if (ix == 0x3f800000) return 0.0f;
-    if (ix - 0x00800000 >= 0x7f800000 - 0x00800000) {
-        // x < 0x1p-126 or inf or nan
-        if (ix * 2 == 0) return -__builtin_inff();
-        if (ix == 0x7f800000) return x;
-        if ((ix & 0x80000000) || ix * 2 >= 0xff000000) return __builtin_nanf("");
-        // x is subnormal, normalize it
-        ix = as_u32(x * 0x1p23f);
-        ix -= 23u << 23;
-    }
     // x = 2^k z; z in [Off, 2*Off) is exact; the range is split into N subintervals, c is near the centre of z's
     uint32_t tmp = ix - Off;
     int i = (tmp >> (23 - OVL_LOGF_TABLE_BITS)) % OVL_LOGF_N;
@@ -177,6 +174,24 @@ OVL_HD float logf_(float x, const logf_entry* tab = logf_tab) {
     y = OVL_MADD(11, A0, r2, y);
     y = OVL_MADD(12, y, r2, y0 + r);
     return (float)y;
+}
+
+OVL_HD float logf_(float x, const logf_entry* tab = logf_tab) {
+    uint32_t ix = as_u32(x);
+    // log(1) needs no special case in round-to-nearest: the table entry around 1 has invc = 1 and logc = 0, so the
+    // common path returns +0 (the exhaustive comparison with the host library covers it)
+    float result = logf_main_(ix, tab);
+    const bool special = ix - 0x00800000 >= 0x7f800000 - 0x00800000;    // x < 0x1p-126 or inf or nan
+    if (OVL_ANY(special)) {
+        // subnormal arguments are normalised and evaluated again
+        uint32_t scaled = as_u32(x * 0x1p23f) - (23u << 23);
+        float fixed = logf_main_(scaled, tab);
+        if ((ix & 0x80000000) || ix * 2 >= 0xff000000) fixed = __builtin_nanf("");
+        if (ix == 0x7f800000) fixed = x;
+        if (ix * 2 == 0) fixed = -__builtin_inff();
+        result = special ? fixed : result;
+    }
+    return result;
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
@@ -296,12 +311,6 @@ OVL_HD float tanhf_(float x) {
     uint32_t ix = jx & 0x7fffffffu;
     bool negative = (jx & 0x80000000u) != 0;
 
-    if (ix >= 0x41b00000u || ix < 0x24000000u) {    // |x| >= 22 (or inf, NaN), |x| < 2**-55 (or zero)
-        if (ix >= 0x7f800000u) return negative ? one / x - one : one / x + one;
-        if (ix >= 0x41b00000u) return negative ? -(one - tiny) : (one - tiny);
-        if (ix == 0) return x;
-        return x * (one + x);
-    }
 
     float ax = as_f32(ix);
     bool big = ix >= 0x3f800000u;                   // |x| >= 1
@@ -342,7 +351,16 @@ OVL_HD float tanhf_(float x) {
 
     float q = OVL_TANH_DIV(big ? two : -em1, em1 + two);
     float z = big ? one - q : q;
-    return negative ? -z : z;
+    float result = negative ? -z : z;
+    const bool special = ix >= 0x41b00000u || ix < 0x24000000u;     // |x| >= 22 (or inf, NaN), |x| < 2**-55 (or zero)
+    if (OVL_ANY(special)) {
+        float fixed = x * (one + x);                                                // tiny
+        if (ix == 0) fixed = x;
+        if (ix >= 0x41b00000u) fixed = negative ? -(one - tiny) : (one - tiny);
+        if (ix >= 0x7f800000u) fixed = negative ? one / x - one : one / x + one;    // +-1 for infinities, NaN for NaN
+        result = special ? fixed : result;
+    }
+    return result;
 }
 
 #if defined(__HIPCC__)
@@ -354,7 +372,8 @@ OVL_HD float recipf_(float b) {
     float r = __builtin_amdgcn_rcpf(b);
     r = __builtin_fmaf(__builtin_fmaf(-b, r, 1.0f), r, r);
     const float ab = __builtin_fabsf(b);
-    if (!(ab >= 0x1p-126f && ab < 0x1p126f)) r = 1.0f / b;
+    const bool special = !(ab >= 0x1p-126f && ab < 0x1p126f);
+    if (OVL_ANY(special)) r = special ? 1.0f / b : r;
     return r;
 }
 #endif
