@@ -111,12 +111,14 @@ class BodyEmitter(object):
         plain global store ``out<k>[index] = value;``
     """
 
-    def __init__(self, info, position_exprs, read_hook=None, store_hook=None, suffix=''):
+    def __init__(self, info, position_exprs, read_hook=None, store_hook=None, suffix='', register_stores=True):
         self.info = info
         self.position_exprs = position_exprs
         self.read_hook = read_hook
         self.store_hook = store_hook
         self.suffix = suffix
+        # True when every statement the store hook returns assigns a register (so it may be turned into a select)
+        self.register_stores = register_stores
 
     def tensor_name(self, node):
         if node.code == lang.INPUT:
@@ -134,6 +136,88 @@ class BodyEmitter(object):
             node = self.info.nodes[node.ops[0]]
         return node.code == lang.CONST_SCALAR and len(node.data) == 1 and float(node.data[0]) == 1.0
 
+    # ------------------------------------------------------------------------------------------------------------
+    # If-conversion.  A conditional chain whose branches only compute values and assign variables (or registers that
+    # buffer a vector store) is emitted as straight-line code: every branch is evaluated and each assignment becomes a
+    # select on "this branch is the one taken".  Lanes of a wavefront that disagree execute all branches anyway; what
+    # the conversion removes is the execution-mask bookkeeping around every branch, and it lets the compiler schedule
+    # across the chain.  Speculating a branch is safe when it cannot fault or trap: no memory access of its own, no
+    # integer division.  At most one branch may be expensive (the others would otherwise be pure overhead when the
+    # whole wavefront takes the same branch).
+    # ------------------------------------------------------------------------------------------------------------
+    _CHEAP_BRANCH = 6
+
+    def _plan_if_conversion(self):
+        info = self.info
+        self._predicate = {}        # statement node index -> name of the bool "its branch is taken"
+        self._converted = {}        # IF node index -> [(predicate name, condition node index or None)]
+        if not getattr(info, 'if_conversion', True):
+            return
+        expensive_codes = (lang.DIVIDE, lang.MODULO, lang.POW, lang.ATAN2, lang.EXP, lang.LOG, lang.LOG10, lang.TANH,
+                           lang.SIN, lang.COS, lang.TAN, lang.SINH, lang.COSH, lang.ASIN, lang.ACOS, lang.ATAN,
+                           lang.SQRT)
+
+        def branch_cost(items):
+            """Number of operations of a branch, or None when it cannot be speculated."""
+            cost = 0
+            for item in items:
+                if item.kind != 'stmt':
+                    return None
+                node = info.nodes[item.node]
+                code = node.code
+                if code in (lang.CONST_SCALAR, lang.MIN_VALUE, lang.MAX_VALUE, lang.EPSILON):
+                    continue
+                if code in (lang.CAST, lang.VARIABLE):
+                    cost += 1 if node.dtype in (lang.FLOAT32, lang.FLOAT64) else 0
+                elif code == lang.ASSIGN_VARIABLE:
+                    cost += 1
+                elif code == lang.READ_TENSOR and info.nodes[node.ops[0]].code == lang.POSITION:
+                    continue                # a component of the worker's position: a register
+                elif code == lang.READ_TENSOR:
+                    tensor = info.nodes[node.ops[0]]
+                    if tensor.code != lang.INPUT or self.read_hook is None or \
+                            self.read_hook(node, tensor, 'index') is None:
+                        return None         # a memory access of its own
+                    cost += 1
+                elif code == lang.ASSIGN_TENSOR:
+                    tensor = info.nodes[node.ops[0]]
+                    if tensor.code != lang.OUTPUT or self.store_hook is None or not self.register_stores:
+                        return None
+                    text = self.store_hook(node, tensor, 'index', 'value')
+                    if not text or not text.endswith('= value;'):
+                        return None         # a real store, not a register that buffers one
+                    cost += 1
+                elif code in UNARY or code in INFIX or code in (lang.MIN, lang.MAX, lang.POW, lang.ATAN2):
+                    if code in (lang.DIVIDE, lang.MODULO) and node.dtype not in (lang.FLOAT32, lang.FLOAT64):
+                        return None         # integer division by zero must stay guarded
+                    if node.dtype in (lang.FLOAT32, lang.FLOAT64):
+                        cost += 20 if code in expensive_codes else 1
+                    # integer arithmetic in a branch is almost always index arithmetic that folds away: not counted
+                else:
+                    return None
+            return cost
+
+        def walk(items):
+            for item in items:
+                if item.kind == 'loop':
+                    walk(item.body)
+                elif item.kind == 'if':
+                    costs = [branch_cost(body) for _, body in item.branches]
+                    if all(c is not None for c in costs) and \
+                            sum(1 for c in costs if c > self._CHEAP_BRANCH) <= 1:
+                        names = []
+                        for k, (cond, body) in enumerate(item.branches):
+                            pred = 't%d_%d%s' % (item.node, k, self.suffix)
+                            names.append((pred, cond))
+                            for stmt in body:
+                                self._predicate[stmt.node] = pred
+                        self._converted[item.node] = names
+                    else:
+                        for _, body in item.branches:
+                            walk(body)
+
+        walk(info.tree)
+
     def emit(self):
         """All statements of the worker, in order."""
         return [text for _, text in self.emit_tagged()]
@@ -142,10 +226,19 @@ class BodyEmitter(object):
         """[(index of the expression that produced it, statement text)] in program order."""
         info = self.info
         fast = MATH_MODES[getattr(info, 'math', 'exact')]
+        self._plan_if_conversion()
         names = {}
         stmts = []
         indent = 0
         current = [0]
+        open_chains = []        # True for a converted chain, False for one emitted as branches
+
+        def assign(node, target, value):
+            """target = value, as a select when the statement sits in a converted branch."""
+            pred = self._predicate.get(node.idx)
+            if pred is None:
+                return target + ' = ' + value + ';'
+            return target + ' = ' + pred + ' ? (' + value + ') : ' + target + ';'
 
         def put(text):
             stmts.append((current[0], '    ' * indent + text))
@@ -172,12 +265,15 @@ class BodyEmitter(object):
             elif code == lang.TENSOR:
                 put(CTYPE[node.dtype] + ' ' + name + '[' + str(node.size) + '] = ' + names[ops[0]] + ';')
             elif code == lang.ASSIGN_VARIABLE:
-                put(names[ops[0]] + ' = ' + names[ops[1]] + ';')
+                put(assign(node, names[ops[0]], names[ops[1]]))
             elif code == lang.ASSIGN_TENSOR:
                 tensor = info.nodes[ops[0]]
                 text = None
                 if tensor.code == lang.OUTPUT and self.store_hook is not None:
                     text = self.store_hook(node, tensor, names[ops[1]], names[ops[2]])
+                    if text and node.idx in self._predicate:
+                        target = text[:text.index(' = ')]
+                        text = assign(node, target, names[ops[2]])
                 if text is None:
                     text = names[ops[0]] + '[' + names[ops[1]] + '] = ' + names[ops[2]] + ';'
                 if text:
@@ -195,20 +291,37 @@ class BodyEmitter(object):
                 put('for(' + i + ' = ' + start + '; ((' + i + ' < ' + stop + ')&&(' + step + '>0)) || ((' +
                     i + ' > ' + stop + ')&&(' + step + '<0)); ' + i + '+=' + step + '){')
                 indent += 1
-            elif code in (lang.ENDRANGE, lang.ENDIF):
+            elif code == lang.ENDRANGE:
                 indent -= 1
                 put('}')
+            elif code == lang.ENDIF:
+                if not open_chains.pop():
+                    indent -= 1
+                    put('}')
             elif code == lang.IF:
-                put('if(' + names[ops[0]] + '){')
-                indent += 1
+                if node.idx in self._converted:
+                    open_chains.append(True)
+                    earlier = []
+                    for pred, cond in self._converted[node.idx]:
+                        terms = ['!' + e for e in earlier]
+                        if cond is not None:
+                            terms.append('(' + names[cond] + ' != 0)')
+                        put('const bool ' + pred + ' = ' + (' && '.join(terms) if terms else 'true') + ';')
+                        earlier.append(pred)
+                else:
+                    open_chains.append(False)
+                    put('if(' + names[ops[0]] + '){')
+                    indent += 1
             elif code == lang.ELSEIF:
-                indent -= 1
-                put('} else if(' + names[ops[0]] + '){')
-                indent += 1
+                if not open_chains[-1]:
+                    indent -= 1
+                    put('} else if(' + names[ops[0]] + '){')
+                    indent += 1
             elif code == lang.ELSE:
-                indent -= 1
-                put('} else {')
-                indent += 1
+                if not open_chains[-1]:
+                    indent -= 1
+                    put('} else {')
+                    indent += 1
             elif code in UNARY:
                 fcn = UNARY[code][node.dtype]
                 if node.dtype == lang.FLOAT32 and code in fast:

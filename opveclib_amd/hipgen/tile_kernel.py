@@ -125,7 +125,7 @@ def generate(info, kernel_name, tile_i=None, tile_j=None, nt='ls'):
                 return tstores[key].reg + '[tj + lane][ti] = ' + value_name + ';'
         return None
 
-    body = BodyEmitter(info, ['p0', 'p1 + lane'], read_hook, store_hook).emit()
+    body = BodyEmitter(info, ['p0', 'p1 + lane'], read_hook, store_hook, register_stores=False).emit()
 
     threads_per_row = tile_j // vec             # phase 1: a tile row is tile_j workers along j
     rows_per_pass = BLOCK // threads_per_row

@@ -155,3 +155,48 @@ def test_entry_point_validates_before_touching_the_gpu(launcher_library):
     with pytest.raises(launcher.LauncherError) as err:
         lib.launch(bad_len, 2, out, 1, None)
     assert err.value.code == launcher.OVL_EARGS
+
+
+def test_if_conversion_of_pure_conditional_chains():
+    """Chains that only compute and assign become selects; chains with memory accesses of their own stay branches."""
+    from opveclib_amd.examples import expm1
+    x = np.zeros((8, 64), np.float32)
+    converted = hipgen.generate(expm1(x).expression_dag, 'f' + '5' * 56).source
+    assert 'if(' not in converted and converted.count('const bool t') == 4      # four branches, four predicates
+    assert converted.count(' ? (') == 4
+    kept = hipgen.generate(expm1(x).expression_dag, 'f' + '5' * 56, {'if_conversion': False}).source
+    assert kept.count('if(') == 3 and 'const bool t' not in kept
+    # clip stores a constant or the input under three conditions: also convertible (register-buffered vector store)
+    clipped = hipgen.generate(cases.clip(np.zeros(256), threshold1=0.1, threshold2=0.9).expression_dag,
+                              'f' + '5' * 56).source
+    assert 'if(' not in clipped
+    # a branch that reads a tensor at a computed index must not be speculated
+    @ovl.operator()
+    def guarded_gather(x, idx):
+        pos = ovl.position_in(x.shape)
+        out = ovl.output_like(x)
+        i = idx[pos]
+        with ovl.if_(i < x.shape[0]):
+            out[pos] = x[i]
+        with ovl.else_():
+            out[pos] = 0
+        return out
+    guarded = hipgen.generate(guarded_gather(np.zeros(64, np.float32), np.zeros(64, np.uint32)).expression_dag,
+                              'f' + '5' * 56).source
+    assert 'if(' in guarded
+    # integer division stays guarded
+    @ovl.operator()
+    def guarded_divide(a, b):
+        pos = ovl.position_in(a.shape)
+        out = ovl.output_like(a)
+        with ovl.if_(b[pos] != 0):
+            out[pos] = a[pos] / b[pos]
+        with ovl.else_():
+            out[pos] = 0
+        return out
+    ints = hipgen.generate(guarded_divide(np.zeros(64, np.int32), np.zeros(64, np.int32)).expression_dag,
+                           'f' + '5' * 56).source
+    assert 'if(' in ints
+    floats = hipgen.generate(guarded_divide(np.zeros(64, np.float32), np.zeros(64, np.float32)).expression_dag,
+                             'f' + '5' * 56).source
+    assert 'if(' not in floats
