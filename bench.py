@@ -9,6 +9,13 @@ one launch of the fused kernel on inputs that are already resident in HBM.  The 
 in GB/s counted on algorithmic bytes (each input element read once, each output element written once:
 3 * 2^26 * 4 + 4 bytes per launch).
 
+Defaults: 100 untimed warm-up launches, then 100 timed ones.  The warm-up is that long on purpose: under this kernel's
+vector ALU load the GPU's power management lets the first ten launches slow down by a third and needs about sixty
+launches (25 ms) to settle (measured series: 310, 310, 310, 347, 377 ... 428 ... 340 ... 307, 307, 307 us), so a short
+warm-up times the transient rather than the kernel.  For the same reason the headline kernel is first launched until
+its time is stable (at least 40 ms of launches, reported as config.clock_settling_launches_before_warmup), whatever
+--warmup says; so is every workload under `others`.
+
 The JSON line also carries
   roofline      algorithmic bytes / average kernel duration (HIP events recorded around every launch on the launch
                 stream) against the 8 TB/s HBM peak,
@@ -160,6 +167,33 @@ class Prepared(object):
         return [self.buffers[ref.op_index][ref.op_output_index] for ref in self.dag.dag_outputs]
 
 
+def settle(prepared, busy_ms=40.0, limit_ms=250.0, window=8, tolerance=0.02):
+    """
+    Launch until the GPU's clocks have settled under this kernel: for at least ``busy_ms`` of kernel time and until
+    the last ``window`` launch times lie within ``tolerance`` of each other, at most ``limit_ms``.  Untimed
+    conditioning before the warm-up; returns the number of launches it took.
+    """
+    import torch
+    stream_obj = torch.cuda.current_stream()
+    stream = stream_obj.cuda_stream
+    recent = []
+    total = 0.0
+    launches = 0
+    while total < limit_ms:
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record(stream_obj)
+        prepared.launch(stream)
+        stop.record(stream_obj)
+        stop.synchronize()
+        elapsed = start.elapsed_time(stop)
+        total += elapsed
+        launches += 1
+        recent = (recent + [elapsed])[-window:]
+        if total >= busy_ms and len(recent) == window and max(recent) <= (1.0 + tolerance) * min(recent):
+            break
+    return launches
+
+
 def measure(prepared, steps, warmup):
     """Returns (ms per step from the host clock around the timed region, mean ms per launch from HIP events)."""
     import torch
@@ -183,6 +217,7 @@ def measure(prepared, steps, warmup):
 
 def side_workload(name, outputs, steps, warmup, options=None):
     prepared = Prepared(outputs, options)
+    settle(prepared)
     wall_ms, event_ms, min_ms = measure(prepared, steps, warmup)
     gbps = prepared.algorithmic_bytes / (event_ms * 1e-3) / 1e9
     return {'workload': name, 'us': round(event_ms * 1e3, 2), 'min_us': round(min_ms * 1e3, 2),
@@ -210,8 +245,8 @@ def cpu_baseline(seed_arrays, rows, iters=3):
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument('--gpus', type=int, default=1)
-    parser.add_argument('--steps', type=int, default=50)
-    parser.add_argument('--warmup', type=int, default=5)
+    parser.add_argument('--steps', type=int, default=100)
+    parser.add_argument('--warmup', type=int, default=100)
     parser.add_argument('--no-others', action='store_true', help='skip the secondary configurations')
     parser.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline')
     args = parser.parse_args()
@@ -231,6 +266,7 @@ def main():
 
     chain = Prepared(chain8_outputs(a, b, s))
     assert len(chain.ops) == 1, 'the 8-op chain must fuse into one kernel'
+    settled_after = settle(chain)
     wall_ms, event_ms, min_ms = measure(chain, args.steps, args.warmup)
     nbytes = chain.algorithmic_bytes
     value = nbytes / (wall_ms * 1e-3) / 1e9
@@ -244,7 +280,8 @@ def main():
         'config': {'workload': 'chain8: add, mul 1.0001, tanh, sigmoid, log1p, expm1, sub, abs fused into one kernel; '
                                'A, B float32 [8192, 8192] uniform[-1, 1], numpy default_rng(2)',
                    'algorithmic_bytes': nbytes, 'kernel': chain.kernels[0]['kernel'],
-                   'pct_of_hbm_peak': round(100.0 * value / HBM_PEAK_GBPS, 2)},
+                   'pct_of_hbm_peak': round(100.0 * value / HBM_PEAK_GBPS, 2),
+                   'clock_settling_launches_before_warmup': settled_after},
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
                      'frac': round(achieved / HBM_PEAK_GBPS, 4), 'traffic': CHAIN8_TRAFFIC_BYTES,
                      'kernel_us': round(event_ms * 1e3, 2), 'kernel_min_us': round(min_ms * 1e3, 2)},
@@ -268,6 +305,7 @@ def main():
         # The optional 'fast' math mode (device math library, reciprocal-based division): not bit-compatible with the
         # reference, so it is reported beside the headline, with its distance from the exact result.
         fast = Prepared(chain8_outputs(chain.leaves[0], chain.leaves[1], chain.leaves[2]), {'math': 'fast'})
+        settle(fast)
         _, fast_ms, fast_min = measure(fast, steps, args.warmup)
         exact_y, fast_y = chain.results()[0], fast.results()[0]
         err = (fast_y.double() - exact_y.double()).abs()
