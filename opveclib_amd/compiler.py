@@ -26,7 +26,7 @@ HIPCC_FLAGS = ('--offload-arch=' + local.gpu_arch, '-O3', '-std=c++17', '-fPIC',
 #: while True, operators are compiled into the package's prebuilt directory
 prebuild_mode = False
 
-_header_paths = [os.path.join(local.csrc_directory, name) for name in ('ovl_device.h', 'ovl_math.h')]
+_header_paths = [os.path.join(local.csrc_directory, name) for name in ('ovl_device.h', 'ovl_math.h', 'ovl_fast_math.h')]
 _lock = threading.Lock()
 _header_cache = []
 

@@ -11,6 +11,7 @@
 #include <float.h>
 
 #include "ovl_math.h"
+#include "ovl_fast_math.h"
 
 // Same layout as ovl_tensor in include/ovl_launch.h.
 typedef struct ovl_tensor {
@@ -66,15 +67,11 @@ __device__ __forceinline__ T ovl_dpp_move(T old, T src) {
 #define ovl_tanhf(x) ovl_math::tanhf_(x)
 #define ovl_recipf(x) ovl_math::recipf_(x)
 
-// Division for the 'fast' math mode: hardware reciprocal plus one residual correction.  Faithfully rounded (at most one
-// unit in the last place from the exact quotient) when the divisor's magnitude lies in [2^-126, 2^126] and the
-// quotient is a normal number; outside that range use the exact mode.
-__device__ __forceinline__ float ovl_fast_divf(float a, float b) {
-    const float r = __builtin_amdgcn_rcpf(b);
-    const float q = a * r;
-    const float e = __builtin_fmaf(-b, q, a);
-    return __builtin_fmaf(e, r, q);
-}
+// Entry points of the optional 'fast' math mode (ovl_fast_math.h).
+#define ovl_fast_expf(x) ovl_fast::expf_(x)
+#define ovl_fast_logf(x) ovl_fast::logf_(x)
+#define ovl_fast_tanhf(x) ovl_fast::tanhf_(x)
+#define ovl_fast_divf(a, b) ovl_fast::divf_((a), (b))
 
 #define OVL_DECLARE_MATH_TABLES()                                              \
     __shared__ ovl_math::lds_tables ovl_lds_tables;                            \

@@ -33,10 +33,16 @@
 // selects: no execution-mask juggling on the common path, and identical calls in one kernel can be merged by the
 // compiler because the common path is not nested in a condition.
 #define OVL_ANY(cond) (__builtin_amdgcn_ballot_w64(cond) != 0)
+// OVL_RARE() as first statement of such a block keeps the compiler from turning the block into unconditional code
+// with selects, which it does when it judges the block cheap.  That is welcome for the few selects of the routines in
+// this file (measured: faster without the marker) and unwelcome for blocks that call a library routine
+// (ovl_fast_math.h).
+#define OVL_RARE() asm volatile("; rare arguments")
 #else
 #define OVL_HD static inline
 #define OVL_TABLE static const
 #define OVL_ANY(cond) (cond)
+#define OVL_RARE() ((void)0)
 #endif
 
 // Every multiply-add site can be switched between fused (bit set) and separately rounded (bit clear); the default

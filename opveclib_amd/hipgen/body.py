@@ -41,11 +41,12 @@ UNARY = {
 }
 # Float32 math per mode: {mode: {expression code: function name}}; DIVIDE maps to a two-argument function.
 # 'exact' (the default) is the table above plus the IEEE '/' operator: the host C library's bits.  'fast' calls the
-# device math library (each result within one unit in the last place of the correctly rounded one over the whole
-# argument range) and divides with a corrected hardware reciprocal.
+# routines of csrc/ovl_fast_math.h (hardware exp2 / log2 / reciprocal with extended-precision range handling, each
+# within two units in the last place of the host library's result).
 MATH_MODES = {
     'exact': {},
-    'fast': {lang.TANH: 'tanhf', lang.EXP: 'expf', lang.LOG: 'logf', lang.DIVIDE: 'ovl_fast_divf'},
+    'fast': {lang.TANH: 'ovl_fast_tanhf', lang.EXP: 'ovl_fast_expf', lang.LOG: 'ovl_fast_logf',
+             lang.DIVIDE: 'ovl_fast_divf'},
 }
 
 _NEGATABLE = (lang.FLOAT32, lang.FLOAT64, lang.INT8, lang.INT16, lang.INT32, lang.INT64)

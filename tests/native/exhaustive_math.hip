@@ -29,7 +29,8 @@ using namespace ovl_math;
 
 namespace {
 
-enum { FN_EXP = 0, FN_LOG = 1, FN_TANH = 2, FN_RECIP = 3, FN_DEVICE_LIBRARY_EXP = 4 };
+enum { FN_EXP = 0, FN_LOG = 1, FN_TANH = 2, FN_RECIP = 3, FN_DEVICE_LIBRARY_EXP = 4,
+       FN_FAST_EXP = 5, FN_FAST_LOG = 6, FN_FAST_TANH = 7, FN_FAST_RECIP = 8 };
 
 __global__ void __launch_bounds__(256) eval_kernel(int fn, uint32_t first, uint32_t count, float* __restrict__ out) {
     OVL_DECLARE_MATH_TABLES();
@@ -41,6 +42,10 @@ __global__ void __launch_bounds__(256) eval_kernel(int fn, uint32_t first, uint3
         else if (fn == FN_LOG) y = ovl_logf(x);
         else if (fn == FN_TANH) y = ovl_tanhf(x);
         else if (fn == FN_RECIP) y = ovl_recipf(x);
+        else if (fn == FN_FAST_EXP) y = ovl_fast_expf(x);
+        else if (fn == FN_FAST_LOG) y = ovl_fast_logf(x);
+        else if (fn == FN_FAST_TANH) y = ovl_fast_tanhf(x);
+        else if (fn == FN_FAST_RECIP) y = ovl_fast_divf(1.0f, x);
         else y = expf(x);            // the device math library's own expf: differs from the host's in the last place
         out[i] = y;
     }
@@ -63,9 +68,9 @@ __global__ void __launch_bounds__(256) tanh_division_kernel(unsigned long long* 
 }
 
 float host_value(int fn, float x) {
-    if (fn == FN_EXP || fn == FN_DEVICE_LIBRARY_EXP) return expf(x);
-    if (fn == FN_LOG) return logf(x);
-    if (fn == FN_TANH) return tanhf(x);
+    if (fn == FN_EXP || fn == FN_DEVICE_LIBRARY_EXP || fn == FN_FAST_EXP) return expf(x);
+    if (fn == FN_LOG || fn == FN_FAST_LOG) return logf(x);
+    if (fn == FN_TANH || fn == FN_FAST_TANH) return tanhf(x);
     volatile float one = 1.0f;          // keep the division at run time
     return one / x;
 }
@@ -96,8 +101,31 @@ extern "C" int ovl_exh_tanh_division(uint64_t* mismatches, uint32_t* first_bad) 
 
 // Compare fn over the bit patterns first, first + step, ... (count of them) with the host C library.
 // step = 1 and count = 2^32 is the exhaustive run.  threads = host threads used for the host side.
+static int against_host(int fn, uint64_t count, uint32_t step, uint32_t threads, uint64_t* mismatches,
+                        uint32_t* first_bad, uint64_t* beyond_two_ulp, uint32_t* max_ulp, uint32_t* worst_bits);
+
 extern "C" int ovl_exh_against_host(int fn, uint64_t count, uint32_t step, uint32_t threads, uint64_t* mismatches,
                                     uint32_t* first_bad) {
+    uint64_t beyond = 0;
+    uint32_t max_ulp = 0, worst = 0;
+    return against_host(fn, count, step, threads, mismatches, first_bad, &beyond, &max_ulp, &worst);
+}
+
+// The same comparison reporting distances in units in the last place: the number of arguments whose results lie more
+// than two units apart, the largest distance and an argument where it occurs.
+extern "C" int ovl_exh_ulp_against_host(int fn, uint64_t count, uint32_t step, uint32_t threads,
+                                        uint64_t* mismatches, uint64_t* beyond_two_ulp, uint32_t* max_ulp,
+                                        uint32_t* worst_bits) {
+    uint32_t first = 0;
+    return against_host(fn, count, step, threads, mismatches, &first, beyond_two_ulp, max_ulp, worst_bits);
+}
+
+static int64_t ordered(uint32_t bits) {       // float bit pattern -> integer that grows with the value
+    return (bits & 0x80000000u) ? -(int64_t)(bits & 0x7fffffffu) : (int64_t)bits;
+}
+
+static int against_host(int fn, uint64_t count, uint32_t step, uint32_t threads, uint64_t* mismatches,
+                        uint32_t* first_bad, uint64_t* beyond_two_ulp, uint32_t* max_ulp, uint32_t* worst_bits) {
     const uint32_t chunk = 1u << 26;
     float* d_out = nullptr;
     float* h_out = nullptr;
@@ -105,16 +133,16 @@ extern "C" int ovl_exh_against_host(int fn, uint64_t count, uint32_t step, uint3
     if (err != hipSuccess) return (int)err;
     err = hipHostMalloc(&h_out, (size_t)chunk * sizeof(float), hipHostMallocDefault);
     if (err != hipSuccess) { hipFree(d_out); return (int)err; }
-    uint64_t total_bad = 0;
-    uint32_t lowest = 0xffffffffu;
+    uint64_t total_bad = 0, total_far = 0;
+    uint32_t lowest = 0xffffffffu, largest = 0, largest_at = 0;
     if (threads == 0) threads = 1;
     // with step > 1 the device still evaluates whole chunks; the host then samples every step-th pattern
     for (uint64_t base = 0; base < (1ull << 32) && base / step < count; base += chunk) {
         hipLaunchKernelGGL(eval_kernel, dim3(2048), dim3(256), 0, 0, fn, (uint32_t)base, chunk, d_out);
         err = hipMemcpy(h_out, d_out, (size_t)chunk * sizeof(float), hipMemcpyDeviceToHost);
         if (err != hipSuccess) break;
-        std::vector<uint64_t> bad(threads, 0);
-        std::vector<uint32_t> low(threads, 0xffffffffu);
+        std::vector<uint64_t> bad(threads, 0), far(threads, 0);
+        std::vector<uint32_t> low(threads, 0xffffffffu), worst(threads, 0), worst_at(threads, 0);
         std::vector<std::thread> pool;
         for (uint32_t t = 0; t < threads; ++t) {
             pool.emplace_back([&, t]() {
@@ -133,6 +161,11 @@ extern "C" int ovl_exh_against_host(int fn, uint64_t count, uint32_t step, uint3
                     if (wb != gb && !(want != want && got != got)) {
                         ++bad[t];
                         if (bits < low[t]) low[t] = bits;
+                        int64_t d = ordered(wb) - ordered(gb);
+                        if (d < 0) d = -d;
+                        if (want != want || got != got || d > 0x7fffffff) d = 0x7fffffff;   // NaN against a number
+                        if (d > 2) ++far[t];
+                        if ((uint32_t)d > worst[t]) { worst[t] = (uint32_t)d; worst_at[t] = bits; }
                     }
                 }
             });
@@ -140,12 +173,17 @@ extern "C" int ovl_exh_against_host(int fn, uint64_t count, uint32_t step, uint3
         for (auto& th : pool) th.join();
         for (uint32_t t = 0; t < threads; ++t) {
             total_bad += bad[t];
+            total_far += far[t];
             if (low[t] < lowest) lowest = low[t];
+            if (worst[t] > largest) { largest = worst[t]; largest_at = worst_at[t]; }
         }
     }
     hipFree(d_out);
     hipHostFree(h_out);
     *mismatches = total_bad;
     *first_bad = lowest;
+    *beyond_two_ulp = total_far;
+    *max_ulp = largest;
+    *worst_bits = largest_at;
     return (int)err;
 }

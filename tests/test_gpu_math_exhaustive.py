@@ -6,6 +6,8 @@ evaluated for float bit patterns and compared bit for bit with the host C librar
 the machine the test runs on.  By default every 16th bit pattern is compared (2^28 arguments per function, all
 exponents and both signs); OVL_EXHAUSTIVE=1 compares all 2^32 (about 10 s per function with 16 host threads).
 `test_tanh_shortened_divisions_*`: all 2^32 arguments, device against device.
+`test_fast_mode_routines_*`: the optional fast routines against the host C library, largest distance in units in the
+last place (measured over all 2^32 arguments: expf 1, logf 2, tanhf 2, reciprocal 0).
 """
 import ctypes
 import os
@@ -42,6 +44,27 @@ def test_device_math_equals_host_libm(lib, name):
     assert err == 0, 'HIP error %d' % err
     assert bad.value == 0, '%s: %d of %d arguments differ from the host C library, first at bits 0x%08x' % (
         name, bad.value, count, first.value)
+
+
+FAST_FUNCTIONS = {'expf': (5, 1), 'logf': (6, 2), 'tanhf': (7, 2), 'reciprocal': (8, 0)}
+
+
+@pytest.mark.parametrize('name', sorted(FAST_FUNCTIONS))
+def test_fast_mode_routines_within_two_ulp_of_host_libm(lib, name):
+    """The routines of the optional 'fast' math mode: distance from the host C library in units in the last place."""
+    lib.ovl_exh_ulp_against_host.argtypes = [ctypes.c_int, ctypes.c_uint64, ctypes.c_uint32, ctypes.c_uint32,
+                                             ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint64),
+                                             ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_uint32)]
+    fn, bound = FAST_FUNCTIONS[name]
+    step = 1 if os.environ.get('OVL_EXHAUSTIVE') == '1' else 16
+    differing, beyond = ctypes.c_uint64(0), ctypes.c_uint64(0)
+    largest, where = ctypes.c_uint32(0), ctypes.c_uint32(0)
+    err = lib.ovl_exh_ulp_against_host(fn, (1 << 32) // step, step, min(16, os.cpu_count() or 1),
+                                       ctypes.byref(differing), ctypes.byref(beyond), ctypes.byref(largest),
+                                       ctypes.byref(where))
+    assert err == 0, 'HIP error %d' % err
+    assert beyond.value == 0 and largest.value <= bound, '%s: %d ulp at bits 0x%08x, %d arguments beyond 2 ulp' % (
+        name, largest.value, where.value, beyond.value)
 
 
 def test_checker_reports_a_library_that_differs_in_the_last_place(lib):
