@@ -75,7 +75,8 @@ __device__ __forceinline__ float divf_(float a, float b) {
     float result = __builtin_fmaf(__builtin_fmaf(-b, q, a), r, q);
     // divisors outside [2^-126, 2^126), quotients in or near the subnormal range, infinities and NaN
     const float ab = __builtin_fabsf(b), aq = __builtin_fabsf(q);
-    const bool special = !(ab >= 0x1p-126f && ab < 0x1p126f && aq >= 0x1p-100f && aq < __builtin_inff());
+    // (a zero dividend needs nothing special: the quotient is a correctly signed zero)
+    const bool special = !(ab >= 0x1p-126f && ab < 0x1p126f && ((aq >= 0x1p-100f && aq < __builtin_inff()) || a == 0.0f));
     if (OVL_ANY(special)) {
         OVL_RARE();
         result = special ? a / b : result;
