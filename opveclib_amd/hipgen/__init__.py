@@ -67,6 +67,9 @@ def generate(expression_dag, function_name, options=None):
     """
     options = options or {}
     info = DagInfo(expression_dag)
+    if info.num_workers >= 2 ** 32:
+        # positions are 32-bit, as in the reference (worker_index is uint32, expression.py:582-608)
+        raise ValueError('workgroup of %d workers: at most 2^32 - 1 are supported' % info.num_workers)
     info.math = options.get('math', 'exact')
     info.if_conversion = options.get('if_conversion', True)
     kernel_name = 'ovl_' + _kernel_label(info.name) + '_' + function_name[1:9]

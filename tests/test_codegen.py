@@ -200,3 +200,14 @@ def test_if_conversion_of_pure_conditional_chains():
     floats = hipgen.generate(guarded_divide(np.zeros(64, np.float32), np.zeros(64, np.float32)).expression_dag,
                              'f' + '5' * 56).source
     assert 'if(' not in floats
+
+
+def test_workgroups_beyond_32_bit_positions_are_refused():
+    @ovl.operator()
+    def fill(shape_like):
+        pos = ovl.position_in([1 << 16, 1 << 16])
+        out = ovl.output([4], ovl.float32)
+        out[pos[0] % 4] = 1
+        return out
+    with pytest.raises(ValueError):
+        hipgen.generate(fill(np.zeros(4, np.float32)).expression_dag, 'f' + '6' * 56)
