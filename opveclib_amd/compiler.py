@@ -25,6 +25,8 @@ HIPCC_FLAGS = ('--offload-arch=' + local.gpu_arch, '-O3', '-std=c++17', '-fPIC',
 
 #: while True, operators are compiled into the package's prebuilt directory
 prebuild_mode = False
+#: while True, operators are compiled even when a built library exists (the "does it build" check)
+force_rebuild = False
 
 _header_paths = [os.path.join(local.csrc_directory, name) for name in ('ovl_device.h', 'ovl_math.h', 'ovl_fast_math.h')]
 _lock = threading.Lock()
@@ -62,7 +64,7 @@ def find_library(source):
 def build_library(source):
     """Return the path of the operator library for ``source``, compiling it when no cached copy exists."""
     found = find_library(source)
-    if found is not None:
+    if found is not None and not force_rebuild:
         return found
 
     directory = local.prebuilt_directory if prebuild_mode else local.ensure_cache_directory()

@@ -709,7 +709,7 @@ def run_variant_on_gpu(name, options):
         runtime.codegen_options = {}
 
 
-def prebuild_all(cases=None, workers=8, with_oracle=True):
+def prebuild_all(cases=None, workers=8, with_oracle=True, force_benchmark=False):
     """Compile the HIP library (and the oracle library) of every operator used by the cases and the benchmark."""
     from concurrent.futures import ThreadPoolExecutor
     from opveclib_amd import compiler, runtime
@@ -754,6 +754,19 @@ def prebuild_all(cases=None, workers=8, with_oracle=True):
 
     compiler.prebuild_mode = True
     try:
+        if force_benchmark:
+            # the benchmark's and the smoke check's kernels are compiled again even when built libraries exist
+            forced = {}
+            for outs in list(bench.all_workload_outputs()) + [CASE_BY_NAME[n].outputs() for n in SMOKE_CASES]:
+                for op in _operators_of(outs, 3):
+                    forced[op.SerializeToString()] = op
+            compiler.force_rebuild = True
+            try:
+                with ThreadPoolExecutor(max_workers=workers) as pool:
+                    list(pool.map(runtime.build_operator, forced.values()))
+            finally:
+                compiler.force_rebuild = False
+            runtime._generated.clear()
         with ThreadPoolExecutor(max_workers=workers) as pool:
             list(pool.map(runtime.build_operator, ops.values()))
             list(pool.map(lambda v: runtime.build_operator(*v), variants))
@@ -775,6 +788,9 @@ def run_case_on_gpu(case, opt_level):
         assert_matches(case, g, r, 'output %d opt_level %d' % (n, opt_level))
 
 
+SMOKE_CASES = ('c2_chain', 'c4_lstm', 'c1_shift')
+
+
 def smoke_check():
-    for name in ('c2_chain', 'c4_lstm', 'c1_shift'):
+    for name in SMOKE_CASES:
         run_case_on_gpu(CASE_BY_NAME[name], 3)
