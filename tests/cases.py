@@ -465,6 +465,39 @@ def _triangles(rng):
     return outs
 
 
+@ovl.operator()
+def scatter_affine(x, a=None, c=None):
+    """out[(a * p + c) mod n] = x[p]"""
+    n = x.shape[0]
+    pos = ovl.position_in(x.shape)
+    out = ovl.output_like(x)
+    out[(pos[0] * a + c) % n] = x[pos]
+    return out
+
+
+@ovl.operator()
+def transpose_scaled(x):
+    pos = ovl.position_in(x.shape)
+    out = ovl.output([x.shape[1], x.shape[0]], x.dtype)
+    out[pos[1], pos[0]] = 2 * x[pos]
+    return out
+
+
+def _adopted_position(rng):
+    """Element-wise consumers fused into producers whose store permutes the workgroup."""
+    x = uniform(rng, -0.9, 0.9, 1000)
+    y = rng.standard_normal(4096, dtype=np.float32)
+    w = rng.standard_normal(4096, dtype=np.float32)
+    m = rng.standard_normal((96, 160), dtype=np.float32)
+    v = rng.standard_normal((160, 96), dtype=np.float32)
+    shifted = shift_cyclic(x)
+    return [log1p(expm1(shifted))[0], shifted[0],
+            stdops.mul(scatter_affine(y, a=3, c=1), w)[0],
+            stdops.sub(scatter_affine(y, a=4095, c=7), w)[0],
+            stdops.tanh(stdops.neg(transpose_scaled(m)))[0],
+            stdops.tanh(stdops.add(transpose_scaled(m), v))[0]]
+
+
 def _odd_sizes(rng):
     # sizes that are not multiples of the vector width, rank 1 and rank 3
     a = rng.standard_normal(1001, dtype=np.float32)
@@ -505,6 +538,7 @@ CASES = [
     _simple('accumulate_max', _accumulate_max),
     _simple('edge_expm1_log1p', _edge_expm1_log1p, max_ulp=2, rel=1e-12),
     _simple('odd_sizes', _odd_sizes),
+    _simple('adopted_position', _adopted_position),
     _simple('conv1d', _conv1d),
     _simple('triangles', _triangles),
 ]

@@ -417,10 +417,75 @@ def test_no_merge_cases():
     # broadcast across the edge: shapes differ
     s = stdops.mul(stdops.add(np.ones((1,)), np.ones((1,))), np.ones((4,)))
     assert _get_merge_refs_for_op_dag(_build_op_dag(s).proto_dag) == []
-    # the shift writes at (p+1) mod n, the consumer reads at p
-    from opveclib_amd.examples import shift_cyclic
-    sh = expm1(shift_cyclic(np.zeros(8, np.float32)))
-    assert _get_merge_refs_for_op_dag(_build_op_dag(sh).proto_dag) == []
+
+
+@ovl.operator()
+def t_scatter(x, a=None, c=None):
+    """out[(a * p + c) mod n] = x[p]: a permutation of the workgroup exactly when gcd(a, n) = 1."""
+    n = x.shape[0]
+    pos = ovl.position_in(x.shape)
+    out = ovl.output_like(x)
+    out[(pos[0] * a + c) % n] = x[pos]
+    return out
+
+
+@ovl.operator()
+def t_transpose(x):
+    pos = ovl.position_in(x.shape)
+    out = ovl.output([x.shape[1], x.shape[0]], x.dtype)
+    out[pos[1], pos[0]] = 2 * x[pos]
+    return out
+
+
+def test_consumer_adopts_the_store_index_of_a_permuting_producer():
+    """A producer whose store permutes its workgroup fuses with an element-wise consumer (the reference keeps such
+    chains apart: its shift -> expm1 -> log1p runs as two operators)."""
+    from opveclib_amd.examples import shift_cyclic, log1p
+    from opveclib_amd.fusion import _merge_op_dag
+    rng = np.random.default_rng(5)
+
+    def fused_ops(outputs):
+        dag, _ = _merge_op_dag(_build_op_dag(*outputs).proto_dag, None)
+        return [op.name for op in dag.operators]
+
+    x = rng.uniform(-0.9, 0.9, 64).astype(np.float32)
+    chain = [log1p(expm1(shift_cyclic(x)))[0]]
+    assert len(_get_merge_refs_for_op_dag(_build_op_dag(*chain).proto_dag)) == 2
+    assert fused_ops(chain) == ['shift_cyclic_expm1_log1p']
+    assert np.array_equal(oracle.evaluate(chain, opt_level=3), oracle.evaluate(chain, opt_level=0))
+    # the shifted tensor itself is also requested: it stays an output of the merged operator
+    shifted = shift_cyclic(x)
+    both = [shifted[0], expm1(shifted)[0]]
+    assert fused_ops(both) == ['shift_cyclic_expm1']
+    for fused, plain in zip(oracle.evaluate(both, opt_level=3), oracle.evaluate(both, opt_level=0)):
+        assert np.array_equal(fused, plain)
+
+    # (3p + 1) mod 64 is a permutation, (2p + 1) mod 64 is not; a second input of the consumer is gathered
+    y = rng.standard_normal(64)
+    w = rng.standard_normal(64)
+    ok = [stdops.mul(t_scatter(y, a=3, c=1), w)[0]]
+    assert fused_ops(ok) == ['t_scatter_mul']
+    assert np.array_equal(oracle.evaluate(ok, opt_level=3), oracle.evaluate(ok, opt_level=0))
+    assert np.array_equal(oracle.evaluate(ok, opt_level=3)[(3 * np.arange(64) + 1) % 64], y * w[(3 * np.arange(64) + 1) % 64])
+    not_ok = [stdops.mul(t_scatter(y, a=2, c=1), w)[0]]
+    assert fused_ops(not_ok) == ['t_scatter', 'mul']
+
+    # a transposed store followed by element-wise operators over the transposed shape
+    m = rng.standard_normal((6, 10))
+    v = rng.standard_normal((10, 6))
+    tr = [stdops.tanh(stdops.neg(t_transpose(m)))[0]]
+    assert fused_ops(tr) == ['t_transpose_neg_tanh']
+    got = oracle.evaluate(tr, opt_level=3)
+    assert np.array_equal(got, oracle.evaluate(tr, opt_level=0))
+    assert np.allclose(got, np.tanh(-2 * m.T), rtol=1e-15, atol=1e-15)
+    # ... but not by a consumer that reads a second tensor, which it would then have to read transposed
+    tr2 = [stdops.tanh(stdops.add(t_transpose(m), v))[0]]
+    assert fused_ops(tr2) == ['t_transpose', 'add_tanh']
+    assert np.array_equal(oracle.evaluate(tr2, opt_level=3), oracle.evaluate(tr2, opt_level=0))
+
+    # a consumer that takes two tensors from the permuting producer, or is not element-wise, keeps its own launch
+    sq = rng.standard_normal((5, 5))
+    assert len(fused_ops([t_cum_sum_cols(t_transpose(sq))[0]])) == 2
 
 
 def fused_equals_unfused(outputs, expected_ops=None):
