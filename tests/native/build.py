@@ -6,6 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(os.path.dirname(os.path.dirname(HERE)), 'opveclib_amd', 'csrc')
 LIBRARY = os.path.join(HERE, 'libexhaustive_math.so')
+HAND_WRITTEN = os.path.join(HERE, 'libhand_written_add.so')
 
 
 def _tanh_body():
@@ -29,6 +30,8 @@ def build():
     cmd = [local.hipcc] + list(HIPCC_FLAGS) + ['-I', CSRC, '-I', include, '-pthread',
                                                 os.path.join(HERE, 'exhaustive_math.hip'), '-o', LIBRARY]
     subprocess.check_call(cmd)
+    subprocess.check_call([local.hipcc] + list(HIPCC_FLAGS) + ['-I', CSRC, os.path.join(HERE, 'hand_written_add.hip'),
+                                                            '-o', HAND_WRITTEN])
     return LIBRARY
 
 

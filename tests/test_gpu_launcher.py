@@ -113,3 +113,38 @@ def test_launch_is_asynchronous_on_the_callers_stream():
         out = ovl.evaluate(stdops.mul(stdops.add(a, a), a))
     side.synchronize()
     assert torch.all(out == 8.0)
+
+
+def test_hand_written_library_through_the_c_abi():
+    """A library written by hand against include/ovl_launch.h (the reference's addgpu.cu test, restated): open it,
+    resolve its entry point and launch it with the launcher; wrong argument lists come back as error code 1."""
+    import os
+    import torch
+    from opveclib_amd import launcher
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'native', 'libhand_written_add.so')
+    if not os.path.exists(path):
+        from tests.native import build
+        build.build()
+    op = launcher.OperatorLibrary(path, 'hand_written_add_generic_hip')
+    stream = torch.cuda.current_stream().cuda_stream
+    for dtype, code in ((torch.float32, 2), (torch.float64, 3)):
+        a = torch.randn(100003, device='cuda', dtype=dtype)
+        b = torch.randn(100003, device='cuda', dtype=dtype)
+        total, diff = torch.empty_like(a), torch.empty_like(a)
+        ins = launcher.tensor_array([(a.data_ptr(), code, a.numel()), (b.data_ptr(), code, b.numel())])
+        outs = launcher.tensor_array([(total.data_ptr(), code, a.numel()), (diff.data_ptr(), code, a.numel())])
+        op.launch(ins, 2, outs, 2, stream)
+        torch.cuda.synchronize()
+        assert torch.equal(total, a + b) and torch.equal(diff, a - b)
+        op.launch(ins, 2, outs, 1, stream)                      # the second output is optional
+        times = op.time(ins, 2, outs, 1, stream, 3)
+        assert len(times) == 3 and all(t > 0 for t in times)
+    with pytest.raises(launcher.LauncherError) as err:
+        op.launch(ins, 1, outs, 1, stream)                      # one input only
+    assert err.value.code == 1
+    mixed = launcher.tensor_array([(a.data_ptr(), 3, a.numel()), (b.data_ptr(), 2, b.numel())])
+    with pytest.raises(launcher.LauncherError):
+        op.launch(mixed, 2, outs, 1, stream)                    # dtypes disagree
+    with pytest.raises(launcher.LauncherError) as err:
+        launcher.OperatorLibrary(path, 'no_such_entry_point')
+    assert err.value.code == 3
