@@ -39,7 +39,7 @@ from .expression import arange
 from .expression import if_, elif_, else_
 
 # @ Operator functions
-from .operator import operator, gradient, evaluate, profile, set_math_mode, get_math_mode
+from .operator import operator, gradient, evaluate, profile, set_math_mode, get_math_mode, set_trace_cache
 from .autograd import as_torch
 
 # @ Local runtime environment functions

@@ -40,6 +40,7 @@ from collections import namedtuple
 
 from . import language as lang
 from .local import version, logger
+from .operator import _op_hash, _freeze_op
 
 
 class _MergeRef(namedtuple('_MergeRef', ['to_op_index', 'to_in_expr_index', 'to_in_arg_index', 'from_op_index',
@@ -696,6 +697,21 @@ def _merge_pair(proto_op_dag, to_op_index, from_op_index):
 _merged_dag_registry = {}
 
 
+def _dag_key(proto_op_dag):
+    """Content hash of an operator DAG from its operators' content names (computed once per traced operator) and
+    the serialised wiring."""
+    wiring = lang.OperatorDAG()
+    wiring.dag_input_types.extend(proto_op_dag.dag_input_types)
+    wiring.references.extend(proto_op_dag.references)
+    wiring.dag_outputs.extend(proto_op_dag.dag_outputs)
+    digest = hashlib.sha224()
+    for op in proto_op_dag.operators:
+        digest.update(_op_hash(op).encode('utf-8'))
+    digest.update(wiring.SerializeToString())
+    digest.update(version.encode('utf-8'))
+    return digest.hexdigest()
+
+
 def _merge_op_dag(proto_op_dag, grad_dags):
     """
     Merge operators until no candidate is left (operator.py:1672-2034); memoised by the hash of the input DAG.
@@ -705,7 +721,7 @@ def _merge_op_dag(proto_op_dag, grad_dags):
         of the result is None whenever a merge happened.
     :return: (merged operator DAG, gradient DAGs or None)
     """
-    key = hashlib.sha224(proto_op_dag.SerializeToString() + version.encode('utf-8')).hexdigest()
+    key = _dag_key(proto_op_dag)
     if key in _merged_dag_registry:
         return _merged_dag_registry[key]
 
@@ -717,6 +733,9 @@ def _merge_op_dag(proto_op_dag, grad_dags):
         merged = _merge_pair(merged, to_op_index, from_op_index)
         pairs = _group_merge_refs(merged, _get_merge_refs_for_op_dag(merged))
 
+    if merged is not proto_op_dag:
+        for op in merged.operators:
+            _freeze_op(op)
     result = (merged, grad_dags if merged is proto_op_dag else None)
     _merged_dag_registry[key] = result
     return result

@@ -177,12 +177,21 @@ class _Repeated(list):
 
 
 class Message(object):
-    """Base class of the schema messages: field table driven storage, equality and wire codec."""
-    _fields = ()
+    """
+    Base class of the schema messages: field table driven storage, equality and wire codec.
 
-    def __init__(self):
-        for f in self._fields:
-            object.__setattr__(self, f.name, self._default(f))
+    Storage is sparse: a field lives in the instance dictionary only once it has been read or written, so creating,
+    copying and encoding a message cost in proportion to the fields in use (an Expression has ten fields and
+    typically uses two or three).
+    """
+    _fields = ()
+    _by_name = {}
+    _by_number = {}
+
+    def __init_subclass__(cls, **kwargs):
+        super(Message, cls).__init_subclass__(**kwargs)
+        cls._by_name = dict((f.name, f) for f in cls._fields)
+        cls._by_number = dict((f.number, f) for f in cls._fields)
 
     @staticmethod
     def _default(f):
@@ -194,21 +203,31 @@ class Message(object):
             return ''
         return _SCALAR_KINDS[f.kind][3]
 
+    def __getattr__(self, key):
+        # reached only for names that are not in the instance dictionary yet: materialise the field's default
+        f = type(self)._by_name.get(key)
+        if f is None:
+            raise AttributeError('%s has no field "%s"' % (type(self).__name__, key))
+        value = self._default(f)
+        self.__dict__[key] = value
+        return value
+
     def __setattr__(self, key, value):
-        for f in self._fields:
-            if f.name == key:
-                if f.repeated or f.kind == 'message':
-                    raise AttributeError('Assignment not allowed to composite field "%s"; use CopyFrom/extend.' % key)
-                object.__setattr__(self, key, value)
-                return
-        raise AttributeError('%s has no field "%s"' % (type(self).__name__, key))
+        f = self._by_name.get(key)
+        if f is None:
+            raise AttributeError('%s has no field "%s"' % (type(self).__name__, key))
+        if f.repeated or f.kind == 'message':
+            raise AttributeError('Assignment not allowed to composite field "%s"; use CopyFrom/extend.' % key)
+        self.__dict__[key] = value
 
     def __eq__(self, other):
         if type(other) is not type(self):
             return False
+        mine, theirs = self.__dict__, other.__dict__
         for f in self._fields:
-            if getattr(self, f.name) != getattr(other, f.name):
-                return False
+            if f.name in mine or f.name in theirs:
+                if getattr(self, f.name) != getattr(other, f.name):
+                    return False
         return True
 
     def __ne__(self, other):
@@ -221,10 +240,21 @@ class Message(object):
             raise TypeError('CopyFrom expects a %s' % type(self).__name__)
         if other is self:
             return
-        for f in self._fields:
-            src = getattr(other, f.name)
+        mine, theirs = self.__dict__, other.__dict__
+        # containers and sub-messages handed out earlier keep their identity: they are emptied, not replaced
+        for name in list(mine):
+            if name not in theirs:
+                f = self._by_name[name]
+                if f.repeated:
+                    del mine[name][:]
+                elif f.kind == 'message':
+                    mine[name].Clear()
+                else:
+                    del mine[name]
+        for name, src in theirs.items():
+            f = self._by_name[name]
             if f.repeated:
-                dst = getattr(self, f.name)
+                dst = getattr(self, name)
                 del dst[:]
                 if f.kind == 'message':
                     for item in src:
@@ -232,17 +262,26 @@ class Message(object):
                 else:
                     dst.extend(src)
             elif f.kind == 'message':
-                getattr(self, f.name).CopyFrom(src)
+                getattr(self, name).CopyFrom(src)
             else:
-                object.__setattr__(self, f.name, src)
+                mine[name] = src
 
     def Clear(self):
         self.CopyFrom(type(self)())
 
+    def __getstate__(self):
+        return self.__dict__
+
+    def __setstate__(self, state):
+        self.__dict__.update(state)
+
     # -- encoding ------------------------------------------------------------------------------------------------
     def _encode(self, buf):
+        stored = self.__dict__
         for f in self._fields:
-            value = getattr(self, f.name)
+            value = stored.get(f.name)
+            if value is None:
+                continue
             if f.kind == 'message':
                 items = value if f.repeated else [value]
                 for item in items:
@@ -280,7 +319,7 @@ class Message(object):
 
     # -- decoding ------------------------------------------------------------------------------------------------
     def _decode(self, data, pos, end):
-        by_number = dict((f.number, f) for f in self._fields)
+        by_number = self._by_number
         while pos < end:
             key, pos = _get_varint(data, pos)
             number, wire = key >> 3, key & 7

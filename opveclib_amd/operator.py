@@ -165,8 +165,23 @@ def _resolve_output(x):
     return x
 
 
+_frozen_hashes = {}      # id(expression DAG message) -> (the message, its content name)
+
+
+def _freeze_op(op):
+    """Declare that ``op`` (an ExpressionDAG message) will not be modified any more; its name is computed once."""
+    entry = _frozen_hashes.get(id(op))
+    if entry is None or entry[0] is not op:
+        entry = (op, 'f' + hashlib.sha224(op.SerializeToString() + version.encode('utf-8')).hexdigest())
+        _frozen_hashes[id(op)] = entry
+    return entry[1]
+
+
 def _op_hash(op):
     """Content name of an operator: 'f' + sha224(serialised DAG + library version) (operator.py:357-358)."""
+    entry = _frozen_hashes.get(id(op))
+    if entry is not None and entry[0] is op:
+        return entry[1]
     return 'f' + hashlib.sha224(op.SerializeToString() + version.encode('utf-8')).hexdigest()
 
 
@@ -197,8 +212,11 @@ def _with_full_inputs(found_dag, full_inputs):
             raise ValueError('Gradient DAG depends on a tensor that is not one of its declared inputs.')
 
     reordered = lang.OperatorDAG()
-    reordered.CopyFrom(found_dag.proto_dag)
-    del reordered.dag_input_types[:]
+    reordered.operators.extend(found_dag.proto_dag.operators)       # traced expression DAGs are shared, not copied
+    for ref in found_dag.proto_dag.references:
+        reordered.references.add().CopyFrom(ref)
+    for ref in found_dag.proto_dag.dag_outputs:
+        reordered.dag_outputs.add().CopyFrom(ref)
     for placeholder in full_inputs:
         reordered.dag_input_types.add().CopyFrom(placeholder.tensor_type.as_proto())
     for ref in reordered.references:
@@ -206,6 +224,49 @@ def _with_full_inputs(found_dag, full_inputs):
             if input_ref.is_leaf:
                 input_ref.dag_input_index = remap[input_ref.dag_input_index]
     return reordered
+
+
+class _Uncacheable(Exception):
+    pass
+
+
+def _freeze(value):
+    """A hashable stand-in that distinguishes any two constants an operator function could tell apart."""
+    if value is None or isinstance(value, (bool, str, bytes)):
+        return (type(value).__name__, value)
+    if isinstance(value, int):
+        return ('int', value)
+    if isinstance(value, float):
+        return ('float', value.hex())
+    if isinstance(value, (tuple, list)):
+        return (type(value).__name__,) + tuple(_freeze(v) for v in value)
+    if isinstance(value, np.generic):
+        return ('numpy', value.dtype.str, value.tobytes())
+    if isinstance(value, np.ndarray) and value.size <= 4096:
+        return ('ndarray', value.dtype.str, value.shape, value.tobytes())
+    if isinstance(value, np.dtype):
+        return ('numpy dtype', value.str)
+    from .expression import DType as _DType
+    if isinstance(value, _DType):
+        return ('ovl dtype', value.proto_dtype)
+    if isinstance(value, type):
+        return ('type', value)
+    if type(value).__module__ == 'torch' and type(value).__name__ == 'dtype':
+        return ('torch dtype', str(value))
+    raise _Uncacheable()
+
+
+#: re-use the trace of an operator function applied again to the same input types and constants
+trace_cache_enabled = [True]
+
+
+def set_trace_cache(enabled):
+    """
+    Operator functions are pure functions of their input types and constants, so a repeated application re-uses the
+    expression DAG (and gradient DAG) traced the first time.  Switch this off for operator functions that read
+    mutable state from outside their arguments.
+    """
+    trace_cache_enabled[0] = bool(enabled)
 
 
 class _OpGenerator(object):
@@ -216,6 +277,8 @@ class _OpGenerator(object):
         self.forbid_none_valued_constants = forbid_none_valued_constants
         self.name = op_function.__name__ if name is None else name
         self.grad_function = None
+        self._spec = inspect.getfullargspec(op_function)
+        self._traces = {}
 
     def __str__(self):
         return self.op_function.__name__
@@ -229,7 +292,7 @@ class _OpGenerator(object):
             elif isinstance(inp, OperatorOutput) and inp.parent.from_gradient:
                 from_gradient = True
 
-        spec = inspect.getfullargspec(self.op_function)
+        spec = self._spec
         if spec.defaults is None:
             input_names = spec.args
             constants = dict(defined_constants)
@@ -269,6 +332,18 @@ class _OpGenerator(object):
                 remaining_names = input_names[num_inputs - len(input_names):]
                 err_msg += 'Should ' + str(remaining_names) + ' be passed to constructor as constant?'
             raise TypeError(err_msg)
+
+        trace_key = None
+        if trace_cache_enabled[0]:
+            try:
+                trace_key = (tuple((tuple(t.shape), t.dtype.proto_dtype) for t in input_types),
+                             tuple(sorted((k, _freeze(v)) for k, v in constants.items())), from_gradient)
+            except _Uncacheable:
+                trace_key = None
+            else:
+                cached = self._traces.get(trace_key)
+                if cached is not None and cached[0] is self.grad_function:
+                    return _Operator(cached[1], list(cached[2]), inputs, cached[3], from_gradient, self.name)
 
         ExpressionDAG.clear()
         input_exprs = [input(cur_type) for cur_type in input_types]
@@ -322,6 +397,9 @@ class _OpGenerator(object):
                                         str(grad_output_index) + ', with TensorType: ' + str(cur_input_type))
                 grad_dag = _with_full_inputs(_build_op_dag(*grad_outputs), grad_inputs)
 
+        if trace_key is not None:
+            _freeze_op(expression_dag)
+            self._traces[trace_key] = (self.grad_function, expression_dag, tuple(output_types), grad_dag)
         return _Operator(expression_dag, output_types, inputs, grad_dag, from_gradient, self.name)
 
     def add_grad(self, grad_function):
@@ -464,7 +542,8 @@ def _build_op_dag(*outputs):
 
     op_dag = lang.OperatorDAG()
     for op in sorted_ops:
-        op_dag.operators.add().CopyFrom(op.expression_dag)
+        # expression DAGs are never modified once traced: the operator DAG shares them instead of copying
+        op_dag.operators.append(op.expression_dag)
     for dag_input in dag_inputs:
         op_dag.dag_input_types.add().CopyFrom(TensorType.like(dag_input).as_proto())
     for slot in order:

@@ -551,3 +551,89 @@ def test_merge_is_memoised():
     dag = _build_op_dag(t_add(t_add(a, a), a)).proto_dag
     first = _merge_op_dag(dag, None)
     assert _merge_op_dag(dag, None) is first
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# trace re-use
+# ----------------------------------------------------------------------------------------------------------------------
+def _traced_scale():
+    calls = []
+
+    @ovl.operator()
+    def scale(x, factor=None, offsets=None):
+        calls.append(1)
+        pos = ovl.position_in(x.shape)
+        out = ovl.output_like(x)
+        value = x[pos] * factor
+        for offset in offsets:
+            value = value + offset
+        out[pos] = value
+        return out
+
+    return scale, calls
+
+
+def test_repeated_applications_share_one_trace():
+    scale, calls = _traced_scale()
+    a = np.zeros(8, dtype=np.float32)
+    b = np.ones(8, dtype=np.float32)
+    first = scale(a, factor=2.0, offsets=(1, 2))
+    second = scale(b, factor=2.0, offsets=(1, 2))
+    assert len(calls) == 1
+    assert second.expression_dag is first.expression_dag
+    assert second.inputs[0] is b and first.inputs[0] is a           # the handles stay separate
+    assert _op_hash(first.expression_dag) == 'f' + __import__('hashlib').sha224(
+        first.expression_dag.SerializeToString() + ovl.local.version.encode('utf-8')).hexdigest()
+
+
+def test_a_trace_is_keyed_by_types_and_constants():
+    scale, calls = _traced_scale()
+    a = np.zeros(8, dtype=np.float32)
+    base = scale(a, factor=2.0, offsets=(1, 2))
+    variants = [scale(a, factor=3.0, offsets=(1, 2)),
+                scale(a, factor=2, offsets=(1, 2)),                 # an int is not the float of the same value
+                scale(a, factor=2.0, offsets=(1, 3)),
+                scale(a, factor=2.0, offsets=[1, 2]),
+                scale(a, factor=-0.0, offsets=()),
+                scale(a, factor=0.0, offsets=()),
+                scale(np.zeros(9, dtype=np.float32), factor=2.0, offsets=(1, 2)),
+                scale(np.zeros(8, dtype=np.float64), factor=2.0, offsets=(1, 2)),
+                scale(np.zeros((2, 4), dtype=np.float32), factor=2.0, offsets=(1, 2))]
+    assert len(calls) == 1 + len(variants)
+    for v in variants:
+        assert v.expression_dag is not base.expression_dag
+
+
+def test_trace_reuse_can_be_switched_off_and_skips_unhashable_constants():
+    scale, calls = _traced_scale()
+    a = np.zeros(8, dtype=np.float32)
+    ovl.set_trace_cache(False)
+    try:
+        scale(a, factor=2.0, offsets=(1,))
+        scale(a, factor=2.0, offsets=(1,))
+    finally:
+        ovl.set_trace_cache(True)
+    assert len(calls) == 2
+    # a constant that cannot be keyed (a generator here) is traced every time
+    scale(a, factor=2.0, offsets=iter((1,)))
+    scale(a, factor=2.0, offsets=iter((1,)))
+    assert len(calls) == 4
+
+
+def test_a_gradient_registered_later_invalidates_the_trace():
+    scale, calls = _traced_scale()
+    a = np.zeros(8, dtype=np.float32)
+    before = scale(a, factor=2.0, offsets=())
+    assert before.grad_dag is None
+
+    @ovl.gradient(scale)
+    @ovl.operator()
+    def scale_grad(x, dy, factor=None, offsets=None):
+        pos = ovl.position_in(x.shape)
+        dx = ovl.output_like(x)
+        dx[pos] = dy[pos] * factor
+        return dx
+
+    after = scale(a, factor=2.0, offsets=())
+    assert after.grad_dag is not None
+    assert len(calls) == 2

@@ -150,3 +150,44 @@ def test_real_dag_round_trip():
     dag = op[0].parent.expression_dag
     data = dag.SerializeToString()
     assert lang.ExpressionDAG.FromString(data) == dag
+
+
+def test_sparse_storage_keeps_message_semantics():
+    # fields exist only once touched, yet unset and default-valued fields are indistinguishable from outside
+    a, b = lang.Expression(), lang.Expression()
+    assert a == b
+    assert a.io_index == 0 and list(a.float_data) == [] and a.tensor_type == lang.TensorType()
+    assert a == b                                  # reading a field does not change equality
+    b.io_index = 0
+    assert a == b and a.SerializeToString() == b.SerializeToString() == b''
+    b.io_index = 3
+    assert a != b
+
+    # CopyFrom empties what the source leaves unset, keeping containers handed out earlier alive
+    target = lang.Expression()
+    kept_list = target.sint64_data
+    kept_list.extend([1, 2])
+    kept_type = target.tensor_type
+    kept_type.shape.extend([4])
+    target.dtype = lang.INT64
+    source = lang.Expression()
+    source.code = lang.CONST_SCALAR
+    source.double_data.append(2.5)
+    target.CopyFrom(source)
+    assert target == source
+    assert target.sint64_data is kept_list and kept_list == []
+    assert target.tensor_type is kept_type and list(kept_type.shape) == []
+    assert target.dtype == 0
+
+    with pytest.raises(AttributeError):
+        target.no_such_field
+    with pytest.raises(AttributeError):
+        target.no_such_field = 1
+    with pytest.raises(AttributeError):
+        target.tensor_type = lang.TensorType()
+
+    import copy
+    import pickle
+    dag = sample_dag()
+    assert copy.deepcopy(dag) == dag
+    assert pickle.loads(pickle.dumps(dag)) == dag
