@@ -62,16 +62,26 @@ __device__ __forceinline__ T ovl_dpp_move(T old, T src) {
 // float32 transcendental entry points used by generated code: bit-compatible with the host C library's
 // expf/logf/tanhf (see ovl_math.h).  ovl_exp_tab / ovl_log_tab name the lookup tables in scope: kernels that call
 // exp or log declare them with OVL_DECLARE_MATH_TABLES at their top, pointing at copies in LDS.
-#define ovl_expf(x) ovl_math::expf_((x), ovl_exp_tab)
+#define ovl_expf(x) ovl_math::expf_<true>((x), ovl_exp_tab)
 #define ovl_logf(x) ovl_math::logf_((x), ovl_log_tab)
 #define ovl_tanhf(x) ovl_math::tanhf_(x)
-#define ovl_recipf(x) ovl_math::recipf_(x)
+#define ovl_recipf(x) ovl_math::recipf_<true>(x)
+// Variants for arguments that the code generator has proved to lie where the routine's common path is valid
+// (hipgen/ranges.py): no rare-argument block.
+#define ovl_expf_inrange(x) ovl_math::expf_<false>((x), ovl_exp_tab)
+#define ovl_logf_inrange(x) ovl_math::logf_inrange_<false>((x), ovl_log_tab)
+#define ovl_logf_inrange_nan(x) ovl_math::logf_inrange_<true>((x), ovl_log_tab)
+#define ovl_recipf_inrange(x) ovl_math::recipf_<false>(x)
+#define ovl_divf_inrange(a, b) ovl_math::divf_inrange_((a), (b))
 
 // Entry points of the optional 'fast' math mode (ovl_fast_math.h).
-#define ovl_fast_expf(x) ovl_fast::expf_(x)
-#define ovl_fast_logf(x) ovl_fast::logf_(x)
+#define ovl_fast_expf(x) ovl_fast::expf_<true>(x)
+#define ovl_fast_logf(x) ovl_fast::logf_<true>(x)
 #define ovl_fast_tanhf(x) ovl_fast::tanhf_(x)
-#define ovl_fast_divf(a, b) ovl_fast::divf_((a), (b))
+#define ovl_fast_divf(a, b) ovl_fast::divf_<true>((a), (b))
+#define ovl_fast_expf_inrange(x) ovl_fast::expf_<false>(x)
+#define ovl_fast_logf_inrange(x) ovl_fast::logf_<false>(x)
+#define ovl_fast_divf_inrange(a, b) ovl_fast::divf_<false>((a), (b))
 
 #define OVL_DECLARE_MATH_TABLES()                                              \
     __shared__ ovl_math::lds_tables ovl_lds_tables;                            \

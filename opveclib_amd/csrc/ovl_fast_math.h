@@ -14,6 +14,9 @@ namespace ovl_fast {
 
 // exp(x) = 2^(x * log2 e).  The product is formed to about 48 bits (p + e1); 2^p comes from the hardware and the
 // factor 2^e1 ~ 1 + e1 ln 2 is applied with one fused multiply-add.
+// (CHECKED = false in this file: the caller knows that no argument needs the rare-argument block; NaN propagates
+// through the common path of every routine.)
+template <bool CHECKED = true>
 __device__ __forceinline__ float expf_(float x) {
     const float log2e = 0x1.715476p+0f, log2e_lo = 0x1.4ae0cp-26f, ln2 = 0x1.62e43p-1f;
     const float p = x * log2e;
@@ -23,7 +26,7 @@ __device__ __forceinline__ float expf_(float x) {
     float result = __builtin_fmaf(r, e1 * ln2, r);
     // |x| >= 87: the result may be subnormal, zero or infinite (or x is NaN)
     const bool special = !(__builtin_fabsf(x) < 87.0f);
-    if (OVL_ANY(special)) {
+    if (CHECKED && OVL_ANY(special)) {
         OVL_RARE();
         result = special ? expf(x) : result;
     }
@@ -31,6 +34,7 @@ __device__ __forceinline__ float expf_(float x) {
 }
 
 // log(x) = log2(x) * ln 2 with the product carried to about 48 bits.
+template <bool CHECKED = true>
 __device__ __forceinline__ float logf_(float x) {
     const float ln2 = 0x1.62e430p-1f, ln2_lo = -0x1.05c610p-29f;
     const float l = __builtin_amdgcn_logf(x);
@@ -38,7 +42,7 @@ __device__ __forceinline__ float logf_(float x) {
     float result = r + __builtin_fmaf(l, ln2_lo, __builtin_fmaf(l, ln2, -r));
     // subnormal, zero, negative, infinite or NaN arguments
     const bool special = !(x >= 0x1p-126f && x < __builtin_inff());
-    if (OVL_ANY(special)) {
+    if (CHECKED && OVL_ANY(special)) {
         OVL_RARE();
         result = special ? logf(x) : result;
     }
@@ -69,6 +73,7 @@ __device__ __forceinline__ float tanhf_(float x) {
 }
 
 // a / b: hardware reciprocal, product and one residual correction.
+template <bool CHECKED = true>
 __device__ __forceinline__ float divf_(float a, float b) {
     const float r = __builtin_amdgcn_rcpf(b);
     const float q = a * r;
@@ -77,7 +82,7 @@ __device__ __forceinline__ float divf_(float a, float b) {
     const float ab = __builtin_fabsf(b), aq = __builtin_fabsf(q);
     // (a zero dividend needs nothing special: the quotient is a correctly signed zero)
     const bool special = !(ab >= 0x1p-126f && ab < 0x1p126f && ((aq >= 0x1p-100f && aq < __builtin_inff()) || a == 0.0f));
-    if (OVL_ANY(special)) {
+    if (CHECKED && OVL_ANY(special)) {
         OVL_RARE();
         result = special ? a / b : result;
     }

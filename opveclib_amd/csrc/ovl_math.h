@@ -81,6 +81,9 @@ OVL_TABLE uint64_t exp2f_tab[OVL_EXP2F_N] = OVL_EXP2F_TABLE;
 
 OVL_HD uint32_t top12(float x) { return as_u32(x) >> 20; }
 
+// CHECKED = false leaves out the repair of |x| >= 88 and NaN: for callers that know -88 < x < 88 (NaN still gives
+// NaN, through the polynomial in r).
+template <bool CHECKED = true>
 OVL_HD float expf_(float x, const uint64_t* tab = exp2f_tab) {
     const double InvLn2N = 0x1.71547652b82fep+0 * OVL_EXP2F_N;
     const double Shift = 0x1.8p+52;
@@ -106,7 +109,7 @@ OVL_HD float expf_(float x, const uint64_t* tab = exp2f_tab) {
     y = y * s;
     float result = (float)y;
     const bool special = abstop >= top12(88.0f);        // |x| >= 88 or x is NaN
-    if (OVL_ANY(special)) {
+    if (CHECKED && OVL_ANY(special)) {
         float fixed = result;                                               // 88 <= |x| below the thresholds: as computed
         if (x < -0x1.9fe368p6f) fixed = 0.0f;                               // underflow, also -inf
         if (x > 0x1.62e42ep6f) fixed = __builtin_inff();                    // overflow, also +inf
@@ -180,6 +183,15 @@ OVL_HD float logf_main_(uint32_t ix, const logf_entry* tab) {
     y = OVL_MADD(11, A0, r2, y);
     y = OVL_MADD(12, y, r2, y0 + r);
     return (float)y;
+}
+
+// logf_inrange_: for callers that know x is a positive normal number or, with MAYBE_NAN, possibly NaN.  The common
+// path works on the bits of x and would turn NaN into a number; adding x * 0 (+0 for every number) puts the NaN back.
+template <bool MAYBE_NAN>
+OVL_HD float logf_inrange_(float x, const logf_entry* tab = logf_tab) {
+    float result = logf_main_(as_u32(x), tab);
+    if (MAYBE_NAN) result = __builtin_fmaf(x, 0.0f, result);
+    return result;
 }
 
 OVL_HD float logf_(float x, const logf_entry* tab = logf_tab) {
@@ -374,13 +386,28 @@ OVL_HD float tanhf_(float x) {
 // with 2^-126 <= |b| < 2^126 (compared with IEEE division on MI355X over all 2^32 divisors: the only differences are
 // subnormal divisors and divisors of 2^126 and above, whose reciprocals are subnormal); those, zeros, infinities and
 // NaN take the IEEE division.
+// CHECKED = false: for callers that know 2^-126 <= |b| < 2^126 (or NaN, which propagates).
+template <bool CHECKED = true>
 OVL_HD float recipf_(float b) {
     float r = __builtin_amdgcn_rcpf(b);
     r = __builtin_fmaf(__builtin_fmaf(-b, r, 1.0f), r, r);
     const float ab = __builtin_fabsf(b);
     const bool special = !(ab >= 0x1p-126f && ab < 0x1p126f);
-    if (OVL_ANY(special)) r = special ? 1.0f / b : r;
+    if (CHECKED && OVL_ANY(special)) r = special ? 1.0f / b : r;
     return r;
+}
+
+// a / b for operands whose quotient needs none of the IEEE division's operand scaling and no fix-up: both normal and
+// nonzero, |b| <= 2^120, 2^-120 <= |a / b| <= 2^90 (NaN propagates).  These are the operations the device's division
+// sequence performs between its scaling and fix-up instructions (reciprocal, two refinements of it, quotient, three
+// residual corrections), which leave operands in that range untouched; the result is the correctly rounded quotient
+// (tests/native/exhaustive_math.hip compares it with the '/' operator on 2^32 operand pairs).
+OVL_HD float divf_inrange_(float a, float b) {
+    float r = __builtin_amdgcn_rcpf(b);
+    r = __builtin_fmaf(__builtin_fmaf(-b, r, 1.0f), r, r);
+    float q = a * r;
+    q = __builtin_fmaf(__builtin_fmaf(-b, q, a), r, q);
+    return __builtin_fmaf(__builtin_fmaf(-b, q, a), r, q);
 }
 #endif
 

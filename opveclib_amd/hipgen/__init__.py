@@ -26,7 +26,7 @@ from . import tile_kernel
 from . import rowscan_kernel
 
 #: bump when generated code changes for an unchanged DAG, so cached binaries are not reused
-CODEGEN_VERSION = 19
+CODEGEN_VERSION = 20
 
 
 
@@ -72,6 +72,7 @@ def generate(expression_dag, function_name, options=None):
         raise ValueError('workgroup of %d workers: at most 2^32 - 1 are supported' % info.num_workers)
     info.math = options.get('math', 'exact')
     info.if_conversion = options.get('if_conversion', True)
+    info.value_ranges = options.get('value_ranges', True)
     kernel_name = 'ovl_' + _kernel_label(info.name) + '_' + function_name[1:9]
     if info.math != 'exact':
         kernel_name += '_' + info.math         # so that profiles tell the math modes of one operator apart

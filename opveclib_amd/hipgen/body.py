@@ -10,6 +10,7 @@ tiles, plain global accesses).
 """
 
 from .. import language as lang
+from . import ranges as value_ranges
 
 CTYPE = {
     lang.FLOAT32: 'float', lang.FLOAT64: 'double',
@@ -47,6 +48,15 @@ MATH_MODES = {
     'exact': {},
     'fast': {lang.TANH: 'ovl_fast_tanhf', lang.EXP: 'ovl_fast_expf', lang.LOG: 'ovl_fast_logf',
              lang.DIVIDE: 'ovl_fast_divf'},
+}
+# Variants without the rare-argument block, chosen when the value-range analysis (ranges.py) proves that no argument
+# can need it: {mode: {expression code: function name}}.  The exact mode's logarithm works on the bits of its
+# argument and has a second variant that also passes NaN on.
+IN_RANGE = {
+    'exact': {lang.EXP: 'ovl_expf_inrange', lang.LOG: 'ovl_logf_inrange', 'log nan': 'ovl_logf_inrange_nan',
+              'reciprocal': 'ovl_recipf_inrange', lang.DIVIDE: 'ovl_divf_inrange'},
+    'fast': {lang.EXP: 'ovl_fast_expf_inrange', lang.LOG: 'ovl_fast_logf_inrange', 'log nan': 'ovl_fast_logf_inrange',
+             lang.DIVIDE: 'ovl_fast_divf_inrange'},
 }
 
 _NEGATABLE = (lang.FLOAT32, lang.FLOAT64, lang.INT8, lang.INT16, lang.INT32, lang.INT64)
@@ -226,7 +236,10 @@ class BodyEmitter(object):
     def emit_tagged(self):
         """[(index of the expression that produced it, statement text)] in program order."""
         info = self.info
-        fast = MATH_MODES[getattr(info, 'math', 'exact')]
+        math_mode = getattr(info, 'math', 'exact')
+        fast = MATH_MODES[math_mode]
+        in_range = IN_RANGE[math_mode]
+        known = value_ranges.analyse(info) if getattr(info, 'value_ranges', True) else None
         self._plan_if_conversion()
         names = {}
         stmts = []
@@ -323,15 +336,30 @@ class BodyEmitter(object):
                     indent -= 1
                     put('} else {')
                     indent += 1
+            elif known is not None and known.constant(node.idx) is not None:
+                # the operands' value ranges decide this comparison / logical operation / predicate
+                put(CTYPE[node.dtype] + ' ' + name + ' = ' + str(known.constant(node.idx)) + ';')
             elif code in UNARY:
                 fcn = UNARY[code][node.dtype]
                 if node.dtype == lang.FLOAT32 and code in fast:
                     fcn = fast[code]
+                if node.dtype == lang.FLOAT32 and known is not None:
+                    x = known.operand(node.idx, 0)
+                    if code == lang.EXP and value_ranges.exp_in_range(x, math_mode):
+                        fcn = in_range[code]
+                    elif code == lang.LOG and value_ranges.log_in_range(x):
+                        fcn = in_range['log nan' if x.nan else code]
                 put(CTYPE[node.dtype] + ' ' + name + ' = ' + fcn + '(' + names[ops[0]] + ');')
             elif code == lang.DIVIDE and node.dtype == lang.FLOAT32 and code not in fast and \
                     self._is_constant_one(ops[0]):
                 # 1/x: the verified correctly rounded reciprocal (ovl_math.h) instead of the general division
-                put('float ' + name + ' = ovl_recipf(' + names[ops[1]] + ');')
+                fcn = 'ovl_recipf'
+                if known is not None and value_ranges.recip_in_range(known.operand(node.idx, 1)):
+                    fcn = in_range['reciprocal']
+                put('float ' + name + ' = ' + fcn + '(' + names[ops[1]] + ');')
+            elif code == lang.DIVIDE and node.dtype == lang.FLOAT32 and known is not None and \
+                    value_ranges.div_in_range(known.operand(node.idx, 0), known.operand(node.idx, 1)):
+                put('float ' + name + ' = ' + in_range[code] + '(' + names[ops[0]] + ', ' + names[ops[1]] + ');')
             elif code == lang.DIVIDE and node.dtype == lang.FLOAT32 and code in fast:
                 put('float ' + name + ' = ' + fast[code] + '(' + names[ops[0]] + ', ' + names[ops[1]] + ');')
             elif code in INFIX or code in (lang.MIN, lang.MAX, lang.POW, lang.ATAN2):

@@ -5,6 +5,8 @@
 //                          (function 4 evaluates the device math library's own expf instead: a self-test of the
 //                          checker, which must report differences for it)
 //   ovl_exh_tanh_division  device tanhf with its shortened divisions against the same code with IEEE divisions
+//   ovl_exh_in_range       the variants without a rare-argument block (expf, logf, reciprocal, division) against the
+//                          full routines / the '/' operator, on every argument the code generator may hand them
 //
 // Built by tests/native/build.py into tests/native/libexhaustive_math.so; called through ctypes by
 // tests/test_gpu_math_exhaustive.py.  Plain C ABI: returns 0 on success, a HIP error code otherwise.
@@ -67,6 +69,69 @@ __global__ void __launch_bounds__(256) tanh_division_kernel(unsigned long long* 
     if (bad) atomicAdd(mismatches, bad);
 }
 
+enum { IN_RANGE_EXP = 0, IN_RANGE_LOG = 1, IN_RANGE_RECIP = 2, IN_RANGE_DIV = 3 };
+
+__device__ __forceinline__ uint64_t mix64(uint64_t z) {        // splitmix64 finaliser
+    z += 0x9e3779b97f4a7c15ull;
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+    return z ^ (z >> 31);
+}
+
+__device__ __forceinline__ bool same_bits(float a, float b) {
+    return __builtin_bit_cast(uint32_t, a) == __builtin_bit_cast(uint32_t, b) || (a != a && b != b);
+}
+
+// which = exp / log / reciprocal: all 2^32 bit patterns, those outside the variant's domain skipped (NaN stays in).
+// which = division: 2^32 operand pairs drawn from the variant's domain (|a| in [2^-100, 2^120], |b| in
+// [2^-120, 2^120], |a / b| in [2^-120, 2^90]; every 16th pair has an all-ones or all-zeros significand).
+__global__ void __launch_bounds__(256) in_range_kernel(int which, unsigned long long* __restrict__ mismatches,
+                                                       unsigned long long* __restrict__ compared,
+                                                       uint32_t* __restrict__ first_bad) {
+    OVL_DECLARE_MATH_TABLES();
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    unsigned long long bad = 0, done = 0;
+    for (uint64_t u = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; u < (1ull << 32); u += stride) {
+        const uint32_t bits = (uint32_t)u;
+        const float x = __builtin_bit_cast(float, bits);
+        const float ax = __builtin_fabsf(x);
+        bool same = true, use = false;
+        if (which == IN_RANGE_EXP) {
+            use = ax < 88.0f || x != x;
+            if (use) same = same_bits(ovl_expf_inrange(x), ovl_expf(x));
+        } else if (which == IN_RANGE_LOG) {
+            const bool normal = x >= 0x1p-126f && x < __builtin_inff();
+            use = normal || x != x;
+            if (use) same = same_bits(ovl_logf_inrange_nan(x), ovl_logf(x));
+            if (normal) same = same && same_bits(ovl_logf_inrange(x), ovl_logf(x));
+        } else if (which == IN_RANGE_RECIP) {
+            use = (ax >= 0x1p-125f && ax <= 0x1p125f) || x != x;
+            if (use) same = same_bits(ovl_recipf_inrange(x), 1.0f / x);
+        } else {
+            const uint64_t h = mix64(u);
+            const int ea = -100 + (int)((h >> 48) % 220u);                      // 2^ea <= |a| < 2^(ea+1)
+            const int eb = -120 + (int)((h >> 56) % 240u + ((h >> 40) & 0xffu) % 240u) % 240;
+            uint32_t ma = (uint32_t)h & 0x7fffffu, mb = (uint32_t)(h >> 23) & 0x7fffffu;
+            if ((u & 15u) == 0) {
+                ma = (h & (1ull << 46)) ? 0x7fffffu : 0u;
+                mb = (h & (1ull << 47)) ? 0x7fffffu : 0u;
+            }
+            const uint32_t sa = (uint32_t)(h >> 62) & 1u, sb = (uint32_t)(h >> 63) & 1u;
+            const float a = __builtin_bit_cast(float, (sa << 31) | ((uint32_t)(ea + 127) << 23) | ma);
+            const float b = __builtin_bit_cast(float, (sb << 31) | ((uint32_t)(eb + 127) << 23) | mb);
+            use = (ea - eb) <= 88 && (ea - eb) >= -119 && (ea < 120 || ma == 0u) && (eb < 120 || mb == 0u);
+            if (use) same = same_bits(ovl_divf_inrange(a, b), a / b);
+        }
+        if (use) ++done;
+        if (!same) {
+            ++bad;
+            atomicMin(first_bad, bits);
+        }
+    }
+    if (bad) atomicAdd(mismatches, bad);
+    atomicAdd(compared, done);
+}
+
 float host_value(int fn, float x) {
     if (fn == FN_EXP || fn == FN_DEVICE_LIBRARY_EXP || fn == FN_FAST_EXP) return expf(x);
     if (fn == FN_LOG || fn == FN_FAST_LOG) return logf(x);
@@ -95,6 +160,29 @@ extern "C" int ovl_exh_tanh_division(uint64_t* mismatches, uint32_t* first_bad) 
     hipMemcpy(first_bad, d_first, sizeof(uint32_t), hipMemcpyDeviceToHost);
     *mismatches = h;
     hipFree(d_count);
+    hipFree(d_first);
+    return (int)err;
+}
+
+extern "C" int ovl_exh_in_range(int which, uint64_t* mismatches, uint64_t* compared, uint32_t* first_bad) {
+    unsigned long long* d_counts = nullptr;
+    uint32_t* d_first = nullptr;
+    hipError_t err = hipMalloc(&d_counts, 2 * sizeof(unsigned long long));
+    if (err != hipSuccess) return (int)err;
+    err = hipMalloc(&d_first, sizeof(uint32_t));
+    if (err != hipSuccess) { hipFree(d_counts); return (int)err; }
+    unsigned long long zero[2] = {0, 0};
+    uint32_t all = 0xffffffffu;
+    hipMemcpy(d_counts, zero, sizeof(zero), hipMemcpyHostToDevice);
+    hipMemcpy(d_first, &all, sizeof(all), hipMemcpyHostToDevice);
+    hipLaunchKernelGGL(in_range_kernel, dim3(4096), dim3(256), 0, 0, which, d_counts, d_counts + 1, d_first);
+    err = hipDeviceSynchronize();
+    unsigned long long h[2] = {0, 0};
+    hipMemcpy(h, d_counts, sizeof(h), hipMemcpyDeviceToHost);
+    hipMemcpy(first_bad, d_first, sizeof(uint32_t), hipMemcpyDeviceToHost);
+    *mismatches = h[0];
+    *compared = h[1];
+    hipFree(d_counts);
     hipFree(d_first);
     return (int)err;
 }

@@ -6,6 +6,8 @@ evaluated for float bit patterns and compared bit for bit with the host C librar
 the machine the test runs on.  By default every 16th bit pattern is compared (2^28 arguments per function, all
 exponents and both signs); OVL_EXHAUSTIVE=1 compares all 2^32 (about 10 s per function with 16 host threads).
 `test_tanh_shortened_divisions_*`: all 2^32 arguments, device against device.
+`test_in_range_variants_*`: the variants of expf / logf / reciprocal / division without a rare-argument block, on every
+argument the code generator may hand them (division: 2^32 operand pairs), device against device.
 `test_fast_mode_routines_*`: the optional fast routines against the host C library, largest distance in units in the
 last place (measured over all 2^32 arguments: expf 1, logf 2, tanhf 2, reciprocal 0).
 """
@@ -82,3 +84,22 @@ def test_tanh_shortened_divisions_equal_ieee_divisions_for_all_arguments(lib):
     err = lib.ovl_exh_tanh_division(ctypes.byref(bad), ctypes.byref(first))
     assert err == 0, 'HIP error %d' % err
     assert bad.value == 0, '%d arguments differ, first at bits 0x%08x' % (bad.value, first.value)
+
+
+IN_RANGE = {'expf': (0, 1 << 31), 'logf': (1, 1 << 30), 'reciprocal': (2, 1 << 31), 'division': (3, 1 << 31)}
+
+
+@pytest.mark.parametrize('name', sorted(IN_RANGE))
+def test_in_range_variants_equal_the_full_routines(lib, name):
+    """What the code generator emits for arguments it has proved harmless returns the same bits as the full routine
+    (for division: as the IEEE '/' operator) on all of those arguments."""
+    lib.ovl_exh_in_range.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint64),
+                                     ctypes.POINTER(ctypes.c_uint32)]
+    which, at_least = IN_RANGE[name]
+    bad, compared = ctypes.c_uint64(0), ctypes.c_uint64(0)
+    first = ctypes.c_uint32(0)
+    err = lib.ovl_exh_in_range(which, ctypes.byref(bad), ctypes.byref(compared), ctypes.byref(first))
+    assert err == 0, 'HIP error %d' % err
+    assert compared.value >= at_least, 'only %d arguments were compared' % compared.value
+    assert bad.value == 0, '%s: %d of %d arguments differ, first at 0x%08x' % (name, bad.value, compared.value,
+                                                                               first.value)

@@ -1,0 +1,230 @@
+"""Value-range analysis of the code generator: soundness of the interval arithmetic and what it decides."""
+import math
+
+import numpy as np
+import pytest
+
+import opveclib_amd as ovl
+from opveclib_amd import hipgen, language as lang, stdops
+from opveclib_amd.examples import expm1, log1p, cumsum
+from opveclib_amd.fusion import _merge_op_dag
+from opveclib_amd.hipgen import ranges
+from opveclib_amd.hipgen.analysis import DagInfo
+from opveclib_amd.hipgen.ranges import Range
+from opveclib_amd.operator import _build_op_dag, _normalise_output_list
+
+F32 = np.float32
+
+
+def _engine():
+    engine = ranges.RangeInfo.__new__(ranges.RangeInfo)
+    engine.inexact_division = False
+    return engine
+
+
+def _samples(r, rng, n=200):
+    """Values of a finite range: both ends, values next to them and random interior points, as float32."""
+    lo, hi = F32(r.lo), F32(r.hi)
+    pts = [lo, hi, np.nextafter(lo, hi), np.nextafter(hi, lo), F32(0.5) * (lo + hi)]
+    pts += list((lo + (hi - lo) * rng.random(n, dtype=np.float32)).astype(F32))
+    if lo <= 0 <= hi:
+        pts += [F32(0.0), F32(-0.0)]
+    return np.array([p for p in pts if lo <= p <= hi], dtype=F32)
+
+
+def _random_range(rng):
+    scale = 10.0 ** rng.integers(-6, 7)
+    a, b = sorted(F32(x) for x in rng.normal(0, scale, 2))
+    if rng.random() < 0.2:
+        b = a
+    return Range(a, b, False)
+
+
+def _contains(r, values):
+    values = values[~np.isnan(values)]
+    return bool(np.all(values >= r.lo) and np.all(values <= r.hi))
+
+
+def test_interval_arithmetic_contains_every_sampled_result():
+    rng = np.random.default_rng(7)
+    engine = _engine()
+    ops = {lang.ADD: np.add, lang.SUBTRACT: np.subtract, lang.MULTIPLY: np.multiply, lang.DIVIDE: np.divide}
+    with np.errstate(all='ignore'):
+        for _ in range(300):
+            a, b = _random_range(rng), _random_range(rng)
+            xs, ys = _samples(a, rng, 40), _samples(b, rng, 40)
+            for code, fn in ops.items():
+                out = engine._float_op(code, lang.FLOAT32, [a, b])
+                got = fn(xs[:, None], ys[None, :]).astype(F32).ravel()
+                assert _contains(out, got), (code, a, b, out)
+                if np.isnan(got).any():
+                    assert out.nan
+
+
+def test_math_routine_images_contain_every_sampled_result():
+    rng = np.random.default_rng(8)
+    engine = _engine()
+    routines = {lang.TANH: np.tanh, lang.EXP: np.exp, lang.LOG: np.log, lang.SQRT: np.sqrt, lang.ABS: np.abs,
+                lang.NEGATE: np.negative, lang.SIN: np.sin, lang.COS: np.cos, lang.FLOOR: np.floor, lang.CEIL: np.ceil}
+    with np.errstate(all='ignore'):
+        for _ in range(300):
+            a = _random_range(rng)
+            xs = _samples(a, rng)
+            for code, fn in routines.items():
+                out = engine._float_op(code, lang.FLOAT32, [a])
+                got = fn(xs).astype(F32)
+                assert _contains(out, got), (code, a, out)
+                if np.isnan(got).any():
+                    assert out.nan
+    # unbounded arguments
+    everything = ranges.top()
+    assert engine._float_op(lang.TANH, lang.FLOAT32, [everything]) == Range(-1.0, 1.0, True)
+    assert engine._float_op(lang.EXP, lang.FLOAT32, [everything]) == Range(0.0, math.inf, True)
+    assert engine._float_op(lang.LOG, lang.FLOAT32, [Range(-1.0, 2.0, False)]) == ranges.top()
+    assert engine._float_op(lang.ADD, lang.FLOAT32, [Range(0, math.inf, False), Range(-math.inf, 0, False)]).nan
+    assert engine._float_op(lang.DIVIDE, lang.FLOAT32, [Range(1, 2, False), Range(-1, 1, False)]) == ranges.top()
+
+
+def test_comparisons_respect_nan():
+    num, maybe_nan = Range(2.0, 3.0, False), Range(2.0, 3.0, True)
+    five = Range(5.0, 5.0, False)
+    assert ranges._compare(lang.LESS, num, five) is True
+    assert ranges._compare(lang.LESS, maybe_nan, five) is None           # NaN < 5 is false
+    assert ranges._compare(lang.GREATER, maybe_nan, five) is False       # false for numbers and for NaN
+    assert ranges._compare(lang.GREATER_EQ, five, maybe_nan) is None
+    assert ranges._compare(lang.EQUAL, maybe_nan, five) is False
+    assert ranges._compare(lang.NOTEQUAL, maybe_nan, five) is True       # NaN != 5 is true as well
+    assert ranges._compare(lang.EQUAL, five, five) is True
+    assert ranges._compare(lang.EQUAL, Range(5.0, 5.0, True), five) is None
+    assert ranges._compare(lang.LESS_EQ, Range(1.0, 5.0, False), five) is True
+    assert ranges._compare(lang.LESS, Range(1.0, 5.0, False), five) is None
+    # truth of a condition: NaN is nonzero
+    assert ranges._truth(Range(1.0, 2.0, True)) is True
+    assert ranges._truth(Range(0.0, 0.0, True)) is None
+    assert ranges._truth(Range(0.0, 0.0, False)) is False
+    assert ranges._truth(Range(-1.0, 1.0, False)) is None
+    engine = _engine()
+    assert engine._predicate(lang.ISINF, maybe_nan) == ranges.BOOL_FALSE
+    assert engine._predicate(lang.ISNAN, maybe_nan) == ranges.BOOL_UNKNOWN
+    assert engine._predicate(lang.ISFINITE, maybe_nan) == ranges.BOOL_UNKNOWN
+    assert engine._predicate(lang.ISFINITE, num) == ranges.BOOL_TRUE
+    assert engine._predicate(lang.ISINF, ranges.top()) == ranges.BOOL_UNKNOWN
+
+
+def _merged_single(outputs):
+    dag, _ = _merge_op_dag(_build_op_dag(*_normalise_output_list(outputs)).proto_dag, None)
+    assert len(dag.operators) == 1
+    return dag.operators[0]
+
+
+def _source(op, **options):
+    return hipgen.generate(op, 'f' + '0' * 56, options or None).source
+
+
+def test_bounded_activations_prune_the_guards_of_log1p_and_expm1():
+    x = np.zeros((4, 64), dtype=np.float32)
+    op = _merged_single(expm1(log1p(stdops.sigmoid(stdops.tanh(x)))))
+    info = DagInfo(op)
+    known = ranges.analyse(info)
+    decided = [known.constant(n.idx) for n in info.nodes if known.constant(n.idx) is not None]
+    # isinf x2, logical_and x2, (u - 1 == 0), (e == 1), (e - 1 == -1): all false
+    assert decided == [0] * 7
+    tanh = [n for n in info.nodes if n.code == lang.TANH][0]
+    assert known.ranges[tanh.idx] == Range(-1.0, 1.0, True)
+
+    exact = _source(op)
+    for name in ('ovl_expf_inrange(', 'ovl_recipf_inrange(', 'ovl_logf_inrange_nan(', 'ovl_divf_inrange('):
+        assert name in exact
+    for name in ('ovl_expf(', 'ovl_logf(', 'ovl_recipf(', 'isinf('):
+        assert name not in exact
+    fast = _source(op, math='fast')
+    for name in ('ovl_fast_expf_inrange(', 'ovl_fast_logf_inrange(', 'ovl_fast_divf_inrange('):
+        assert name in fast
+    for name in ('ovl_fast_expf(', 'ovl_fast_logf(', 'ovl_fast_divf('):
+        assert name not in fast
+    unpruned = _source(op, value_ranges=False)
+    assert 'inrange' not in unpruned and 'isinf(' in unpruned and 'ovl_expf(' in unpruned
+
+
+def test_unknown_arguments_keep_every_guard():
+    x = np.zeros((4, 64), dtype=np.float32)
+    for op in (expm1(x), log1p(x), stdops.sigmoid(x)):
+        source = _source(op.expression_dag)
+        assert 'inrange' not in source
+        assert ranges.analyse(DagInfo(op.expression_dag)).constant(0) is None
+    info = DagInfo(expm1(x).expression_dag)
+    known = ranges.analyse(info)
+    assert all(known.constant(n.idx) is None for n in info.nodes)
+
+
+@ovl.operator()
+def _branchy(x, with_else=None):
+    pos = ovl.position_in(x.shape)
+    out = ovl.output_like(x)
+    v = ovl.variable(0.5, x.dtype)
+    with ovl.if_(x[pos] > 0.0):
+        v <<= 5.0
+    if with_else:
+        with ovl.else_():
+            v <<= 7.0
+    out[pos] = ovl.exp(v) / (v + 1.0)
+    return out
+
+
+def test_variables_take_the_union_of_the_branches_that_can_run():
+    x = np.zeros(64, dtype=np.float32)
+    for with_else, expected in ((True, Range(5.0, 7.0, False)), (False, Range(0.5, 5.0, False))):
+        info = DagInfo(_branchy(x, with_else=with_else).expression_dag)
+        known = ranges.analyse(info)
+        exp_node = [n for n in info.nodes if n.code == lang.EXP][0]
+        assert known.operand(exp_node.idx, 0) == expected
+        source = _source(_branchy(x, with_else=with_else).expression_dag)
+        assert 'ovl_expf_inrange(' in source and 'ovl_divf_inrange(' in source
+
+
+@ovl.operator()
+def _dead_branch(x):
+    pos = ovl.position_in(x.shape)
+    out = ovl.output_like(x)
+    t = ovl.tanh(x[pos])
+    v = ovl.variable(1.0, x.dtype)
+    with ovl.if_(t > 2.0):              # never: tanh is at most 1 (and NaN > 2 is false)
+        v <<= 1000.0
+    with ovl.elif_(t != 3.0):           # always, also for NaN: later branches cannot run
+        v <<= 2.0
+    with ovl.else_():
+        v <<= -1000.0
+    out[pos] = ovl.exp(v)
+    return out
+
+
+def test_branches_that_cannot_run_do_not_widen_ranges():
+    info = DagInfo(_dead_branch(np.zeros(64, dtype=np.float32)).expression_dag)
+    known = ranges.analyse(info)
+    exp_node = [n for n in info.nodes if n.code == lang.EXP][0]
+    assert known.operand(exp_node.idx, 0) == Range(2.0, 2.0, False)
+
+
+def test_variables_assigned_in_a_loop_are_unknown():
+    x = np.zeros((4, 32), dtype=np.float32)
+    info = DagInfo(cumsum(x, axis=1).expression_dag)
+    known = ranges.analyse(info)
+    for n in info.nodes:
+        if n.code == lang.ADD and n.dtype == lang.FLOAT32:
+            assert known.ranges[n.idx] == ranges.top()
+
+
+def test_in_range_conditions():
+    assert ranges.exp_in_range(Range(-87.0, 87.0, True), 'exact')
+    assert not ranges.exp_in_range(Range(-87.0, 88.0, False), 'exact')
+    assert not ranges.exp_in_range(Range(-87.0, 87.0, False), 'fast')
+    assert not ranges.exp_in_range(None, 'exact')
+    assert ranges.log_in_range(Range(2.0 ** -126, 1e38, True))
+    assert not ranges.log_in_range(Range(0.0, 1.0, False))
+    assert not ranges.log_in_range(Range(1.0, math.inf, False))
+    assert ranges.recip_in_range(Range(-4.0, -0.5, False))
+    assert not ranges.recip_in_range(Range(-1.0, 1.0, False))
+    assert ranges.div_in_range(Range(0.1, 10.0, False), Range(-3.0, -0.01, True))
+    assert not ranges.div_in_range(Range(0.0, 10.0, False), Range(1.0, 2.0, False))         # a zero dividend
+    assert not ranges.div_in_range(Range(1.0, 2.0 ** 100, False), Range(2.0 ** -100, 1.0, False))   # quotient too large
+    assert not ranges.div_in_range(Range(1.0, 2.0, False), Range(-1.0, 1.0, False))
