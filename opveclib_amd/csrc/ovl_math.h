@@ -337,7 +337,13 @@ OVL_HD float tanhf_(float x) {
 
     // argument reduction a = k*ln2 + xr (+ correction c); k = 0 leaves a untouched
     int32_t kg = (int32_t)(invln2 * a + (big ? 0.5f : -0.5f));
+#if defined(OVL_TANH_FDLIBM_K)
     int32_t k = (ha > 0x3eb17218u) ? ((ha < 0x3F851592u) ? -1 : kg) : 0;
+#else
+    // fdlibm sets k = 0 for |a| <= 0.5 ln2 and k = -+1 for |a| < 1.5 ln2 without computing it; the rounded quotient
+    // gives the same k for every argument tanh passes on (checked over all 2^32 arguments against the host library)
+    int32_t k = kg;
+#endif
     float t = (float)k;
     float hi = a - t * ln2_hi;
     float lo = t * ln2_lo;
@@ -350,10 +356,11 @@ OVL_HD float tanhf_(float x) {
     float t3 = 3.0f - r1 * hfx;
     float e = hxs * OVL_TANH_DIV(r1 - t3, 6.0f - xr * t3);
 
-    float res0 = xr - (xr * e - hxs);               // k == 0
     float e2 = xr * (e - c) - c;
     e2 -= hxs;
     float d = e2 - xr;
+    // k == 0: fdlibm returns xr - (xr*e - hxs); c is zero then, so e2 is that same xr*e - hxs and the result is -d
+    float res0 = -d;
     float resm1 = 0.5f * (-d) - 0.5f;               // k == -1: 0.5*(xr-e2) - 0.5
     // k <= -2 or k > 56: (1 - d) * 2^k - 1;  3 <= k < 23: ((1 - 2^-k) - d) * 2^k;  23 <= k <= 56: ((xr-(e2+2^-k))+1) * 2^k
     bool tail_a = (k <= -2) || (k > 56);
@@ -369,7 +376,7 @@ OVL_HD float tanhf_(float x) {
 
     float q = OVL_TANH_DIV(big ? two : -em1, em1 + two);
     float z = big ? one - q : q;
-    float result = negative ? -z : z;
+    float result = as_f32(as_u32(z) | (jx & 0x80000000u));      // z >= +0: give it the sign of x
     const bool special = ix >= 0x41b00000u || ix < 0x24000000u;     // |x| >= 22 (or inf, NaN), |x| < 2**-55 (or zero)
     if (OVL_ANY(special)) {
         float fixed = x * (one + x);                                                // tiny
