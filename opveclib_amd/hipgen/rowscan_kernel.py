@@ -334,18 +334,29 @@ def skew_plan(info):
     return p
 
 
-def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s'):
+def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None):
     p = skew_plan(info)
     assert p is not None
     ctype = CTYPE[p.x.dtype]
     vec = p.vec
-    group_cols = GROUP_LANES * vec
+    # width = 128-bit vectors per lane and phase: a lane owns vec * width consecutive columns of a group, so the
+    # hand-over to the neighbouring lane (a move and its wait states on the critical path of the recurrence) comes
+    # once per vec * width columns
+    # (measured on MI355X: float64 [1024, 16384] 104 us with one vector per phase, 76 us with two, 126 us with four,
+    # whose 64-byte stride between lanes wastes the memory pipeline; float32 [4096, 16384], which runs at the speed of
+    # memory, 85 us with one and 111 us with two)
+    if width is None:
+        width = 2 if vec == 2 else 1
+    while width > 1 and p.length % (GROUP_LANES * vec * width) != 0:
+        width //= 2
+    group_cols = GROUP_LANES * vec * width
     num_groups = p.length // group_cols
     rows_per_wave = WAVE // GROUP_LANES
     waves = BLOCK // WAVE
     rows_per_block = rows_per_wave * waves
     if depth is None:
-        depth = 4                   # measured on MI355X: 4 groups (1 KiB per row) per request burst is the fastest
+        # measured on MI355X: request bursts of 1 KiB per row are the fastest
+        depth = max(1, 4 // width)
     while num_groups % depth != 0:
         depth //= 2
 
@@ -392,9 +403,9 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s'):
     src.append('    if ((blockIdx.x * %du + threadIdx.x / %du) * %du >= %du) return;' % (waves, WAVE, rows_per_wave, p.rows))
     src.append('    const uint32_t row = row_raw < %du ? row_raw : %du;' % (p.rows, p.rows - 1))
     src.append('    const %s* __restrict__ gin = in%d + (uint64_t)row * %dull + part * %du;' % (
-        ctype, p.x.io_index, p.length, vec))
+        ctype, p.x.io_index, p.length, vec * width))
     src.append('    %s* __restrict__ gout = out%d + (uint64_t)row * %dull + part * %du;' % (
-        ctype, p.out.io_index, p.length, vec))
+        ctype, p.out.io_index, p.length, vec * width))
     # measured on MI355X (float32 [4096, 16384]): non-temporal stores with plain loads 85 us, hint on both 100 us,
     # on the loads only 90 us, on neither 102 us
     batch = depth
@@ -405,30 +416,35 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s'):
         """All loads of one batch, back to back: every row is read in runs of batch * 256 bytes."""
         src.append('        #pragma unroll')
         src.append('        for (uint32_t j = 0; j < %du; ++j)' % batch)
+        src.append('            #pragma unroll')
+        src.append('            for (uint32_t w = 0; w < %du; ++w)' % width)
         if 'l' in nt:
-            src.append('            %s[j] = __builtin_nontemporal_load(reinterpret_cast<const %s*>(gin + (%s) * %du + j * %du));' % (
-                regs, vname, batch_expr, batch_cols, group_cols))
+            src.append('                %s[j][w] = __builtin_nontemporal_load(reinterpret_cast<const %s*>(gin + (%s) * %du + j * %du + w * %du));' % (
+                regs, vname, batch_expr, batch_cols, group_cols, vec))
         else:
-            src.append('            %s[j] = *(reinterpret_cast<const %s*>(gin + (%s) * %du + j * %du));' % (
-                regs, vname, batch_expr, batch_cols, group_cols))
+            src.append('                %s[j][w] = *(reinterpret_cast<const %s*>(gin + (%s) * %du + j * %du + w * %du));' % (
+                regs, vname, batch_expr, batch_cols, group_cols, vec))
 
     def process(regs, batch_expr, refill_expr):
         src.append('        {')
         src.append('        const uint32_t b = %s;' % batch_expr)
-        src.append('        %s ov[%d];' % (vname, batch))
+        src.append('        %s ov[%d][%d];' % (vname, batch, width))
         src.append('        #pragma unroll')
         src.append('        for (uint32_t j = 0; j < %du; ++j) {' % batch)
-        src.append('            const %s xv = %s[j];' % (vname, regs))
-        src.append('            const uint32_t col0 = b * %du + j * %du + part * %du;' % (batch_cols, group_cols, vec))
+        src.append('            const uint32_t col0 = b * %du + j * %du + part * %du;' % (batch_cols, group_cols, vec * width))
         src.append('            const bool first_column = (j == 0u) && (b == 0u) && (part == 0u);')
         src.append('            #pragma unroll')
         src.append('            for (uint32_t phase = 0; phase < %du; ++phase) {' % GROUP_LANES)
         for name, _ in state:
             src.append('                %s = carry_%s;' % (name, name))
         src.append('                #pragma unroll')
-        src.append('                for (uint32_t u = 0; u < %du; ++u) {' % vec)
-        src.append('                    if (u == 0u && first_column) ov[j][0] = first_out;')
-        src.append('                    else OVL_SCAN_STEP(col0 + u)')
+        src.append('                for (uint32_t w = 0; w < %du; ++w) {' % width)
+        src.append('                    const %s xv = %s[j][w];' % (vname, regs))
+        src.append('                    #pragma unroll')
+        src.append('                    for (uint32_t u = 0; u < %du; ++u) {' % vec)
+        src.append('                        if (w == 0u && u == 0u && first_column) ov[j][0][0] = first_out;')
+        src.append('                        else OVL_SCAN_STEP(col0 + w * %du + u)' % vec)
+        src.append('                    }')
         src.append('                }')
         for name, _ in state:
             src.append('                carry_%s = ovl_dpp_move<OVL_DPP_ROW_SHR1>(carry_%s, %s);' % (name, name, name))
@@ -442,12 +458,14 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s'):
         src.append('        __builtin_amdgcn_sched_barrier(0);')
         src.append('        #pragma unroll')
         src.append('        for (uint32_t j = 0; j < %du; ++j)' % batch)
+        src.append('            #pragma unroll')
+        src.append('            for (uint32_t w = 0; w < %du; ++w)' % width)
         if 's' in nt:
-            src.append('            __builtin_nontemporal_store(ov[j], reinterpret_cast<%s*>(gout + b * %du + j * %du));' % (
-                vname, batch_cols, group_cols))
+            src.append('                __builtin_nontemporal_store(ov[j][w], reinterpret_cast<%s*>(gout + b * %du + j * %du + w * %du));' % (
+                vname, batch_cols, group_cols, vec))
         else:
-            src.append('            *(reinterpret_cast<%s*>(gout + b * %du + j * %du)) = ov[j];' % (
-                vname, batch_cols, group_cols))
+            src.append('                *(reinterpret_cast<%s*>(gout + b * %du + j * %du + w * %du)) = ov[j][w];' % (
+                vname, batch_cols, group_cols, vec))
         if refill_expr is not None:
             request(regs, refill_expr)
         src.append('        __builtin_amdgcn_sched_barrier(0);')
@@ -455,7 +473,7 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s'):
 
     sets = max(2, min(sets or 2, num_batches)) if num_batches > 1 else 1
     src.append('    // %d register sets of %d groups each: one is consumed while the others are in flight' % (sets, batch))
-    src.append('    %s %s;' % (vname, ', '.join('q%d[%d]' % (k, batch) for k in range(sets))))
+    src.append('    %s %s;' % (vname, ', '.join('q%d[%d][%d]' % (k, batch, width) for k in range(sets))))
     src.append('    {')
     for k in range(sets):
         request('q%d' % k, '%du' % k)
@@ -471,7 +489,7 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s'):
     for name, stype in state:
         src.append('    %s carry_%s = %s;' % (stype, name, name))
     src.append('#define OVL_SCAN_IN xv[u]')
-    src.append('#define OVL_SCAN_OUT(value) ov[j][u] = (value)')
+    src.append('#define OVL_SCAN_OUT(value) ov[j][w][u] = (value)')
     src.append('#define OVL_SCAN_STEP(column) { %s = (%s)(column); %s }' % (
         counter_name, counter_type, ' '.join(body)))
     rounds = num_batches // sets
