@@ -26,7 +26,7 @@ from . import tile_kernel
 from . import rowscan_kernel
 
 #: bump when generated code changes for an unchanged DAG, so cached binaries are not reused
-CODEGEN_VERSION = 21
+CODEGEN_VERSION = 22
 
 
 

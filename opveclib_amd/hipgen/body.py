@@ -54,7 +54,7 @@ MATH_MODES = {
 # argument and has a second variant that also passes NaN on.
 IN_RANGE = {
     'exact': {lang.EXP: 'ovl_expf_inrange', lang.LOG: 'ovl_logf_inrange', 'log nan': 'ovl_logf_inrange_nan',
-              'reciprocal': 'ovl_recipf_inrange', lang.DIVIDE: 'ovl_divf_inrange'},
+              lang.DIVIDE: 'ovl_divf_inrange'},
     'fast': {lang.EXP: 'ovl_fast_expf_inrange', lang.LOG: 'ovl_fast_logf_inrange', 'log nan': 'ovl_fast_logf_inrange',
              lang.DIVIDE: 'ovl_fast_divf_inrange'},
 }
@@ -350,12 +350,12 @@ class BodyEmitter(object):
                     elif code == lang.LOG and value_ranges.log_in_range(x):
                         fcn = in_range['log nan' if x.nan else code]
                 put(CTYPE[node.dtype] + ' ' + name + ' = ' + fcn + '(' + names[ops[0]] + ');')
-            elif code == lang.DIVIDE and node.dtype == lang.FLOAT32 and code not in fast and \
-                    self._is_constant_one(ops[0]):
-                # 1/x: the verified correctly rounded reciprocal (ovl_math.h) instead of the general division
+            elif code == lang.DIVIDE and node.dtype == lang.FLOAT32 and self._is_constant_one(ops[0]):
+                # 1/x: the verified correctly rounded reciprocal (ovl_math.h) instead of the general division, in
+                # every math mode (it is also the cheapest form: hardware reciprocal and one refinement)
                 fcn = 'ovl_recipf'
                 if known is not None and value_ranges.recip_in_range(known.operand(node.idx, 1)):
-                    fcn = in_range['reciprocal']
+                    fcn = 'ovl_recipf_inrange'
                 put('float ' + name + ' = ' + fcn + '(' + names[ops[1]] + ');')
             elif code == lang.DIVIDE and node.dtype == lang.FLOAT32 and known is not None and \
                     value_ranges.div_in_range(known.operand(node.idx, 0), known.operand(node.idx, 1)):
