@@ -1,6 +1,7 @@
 """
 Build step for the package's native code: ``python -m opveclib_amd.build`` compiles the C-ABI launcher
-(csrc/ovl_launch.cpp -> csrc/libovl_launch.so) with hipcc.  Generated operators are compiled on demand and cached;
+(csrc/ovl_launch.cpp -> csrc/libovl_launch.so) and the hand-written LSTM cell kernels (csrc/ovl_lstm.hip ->
+csrc/libovl_lstm.so) with hipcc.  Generated operators are compiled on demand and cached;
 ``python -m opveclib_amd.build --check`` additionally compiles one small operator to verify the toolchain.
 """
 
@@ -8,8 +9,9 @@ import sys
 
 
 def build_all(force=True, check=False):
-    from . import launcher
+    from . import launcher, lstm_cell
     path = launcher.build(force=force)
+    lstm_cell.build(force=force)
     if check:
         import numpy as np
         from . import runtime

@@ -74,3 +74,63 @@ def test_missing_launcher_is_a_loud_error(monkeypatch):
     monkeypatch.setattr(launcher, 'library_path', '/nonexistent/libovl_launch.so')
     with pytest.raises(RuntimeError):
         launcher.library()
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# the hand-written LSTM cell library (include/ovl_lstm.h)
+# ----------------------------------------------------------------------------------------------------------------------
+LSTM_HEADER = os.path.join(ROOT, 'include', 'ovl_lstm.h')
+
+
+def lstm_declared_functions():
+    text = open(LSTM_HEADER).read()
+    text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
+    return sorted(set(re.findall(r'\b(ovl_[a-z_0-9]+)\s*\(', text)))
+
+
+@pytest.fixture(scope='module')
+def lstm_library():
+    from opveclib_amd import lstm_cell
+    if not os.path.exists(lstm_cell.library_path):
+        lstm_cell.build()
+    return lstm_cell.library()
+
+
+def test_lstm_header_and_binding_agree(lstm_library):
+    from opveclib_amd import lstm_cell
+    assert lstm_declared_functions() == sorted(lstm_cell.EXPORTED_SYMBOLS)
+    raw = ctypes.CDLL(lstm_cell.library_path)
+    for name in lstm_declared_functions():
+        assert hasattr(raw, name), name
+
+
+def test_lstm_argument_errors_are_reported_before_any_gpu_work(lstm_library):
+    L = lstm_library
+    p = ctypes.c_void_p(64)             # never dereferenced: every call below is refused first
+    assert L.ovl_lstm_forward(None, p, 1.0, 4, 8, 0, p, p, None) == launcher.OVL_EINVAL
+    assert b'null' in L.ovl_lstm_last_error()
+    assert L.ovl_lstm_forward(p, p, 1.0, 0, 8, 0, p, p, None) == launcher.OVL_EINVAL
+    assert L.ovl_lstm_forward(p, p, 1.0, 4, 0, 0, p, p, None) == launcher.OVL_EINVAL
+    assert L.ovl_lstm_forward(p, p, 1.0, 1 << 16, 1 << 16, 0, p, p, None) == launcher.OVL_EINVAL
+    assert b'2^32' in L.ovl_lstm_last_error()
+    assert L.ovl_lstm_backward(p, p, p, None, 1.0, 4, 8, 0, p, p, None) == launcher.OVL_EINVAL
+    assert L.ovl_lstm_backward(p, p, p, p, 1.0, 0, 8, 0, p, p, None) == launcher.OVL_EINVAL
+
+
+def test_lstm_python_wrapper_validates_its_arguments():
+    import numpy as np
+    import torch
+    from opveclib_amd import lstm_cell
+    concat = torch.zeros(4, 32)
+    c = torch.zeros(4, 8)
+    with pytest.raises(RuntimeError):
+        lstm_cell.lstm_cell(concat, c, 1.0)                         # host tensors
+    with pytest.raises((TypeError, AttributeError)):
+        lstm_cell.lstm_cell(np.zeros((4, 32), np.float32), c, 1.0)
+    with pytest.raises(ValueError):
+        lstm_cell._fast('sloppy')
+    with pytest.raises(TypeError):
+        lstm_cell._shapes(torch.zeros(4, 30), [], [])
+    with pytest.raises(TypeError):
+        lstm_cell._shapes(concat, [torch.zeros(4, 9)], ['c'])
+    assert lstm_cell._shapes(concat, [c], ['c']) == (4, 8)
