@@ -11,6 +11,7 @@ current PyTorch HIP stream.  There is no CPU execution path in this package.
 import dis
 import hashlib
 import inspect
+import types
 from collections import namedtuple
 
 import numpy as np
@@ -251,20 +252,81 @@ def _freeze(value):
         return ('ovl dtype', value.proto_dtype)
     if isinstance(value, type):
         return ('type', value)
+    if isinstance(value, types.FunctionType):
+        # a function passed as a constant (accumulate's inner function): the same code with the same defaults and
+        # surroundings is the same function, even when a lambda expression creates a new object on every call
+        return ('function', value.__code__, tuple(_freeze(d) for d in (value.__defaults__ or ())),
+                _environment_key(value))
     if type(value).__module__ == 'torch' and type(value).__name__ == 'dtype':
         return ('torch dtype', str(value))
     raise _Uncacheable()
 
 
+class _ById(object):
+    """Key component for an object compared by identity; holds the object, so its id cannot be re-used by another
+    object while a cache entry refers to it."""
+    __slots__ = ('obj',)
+
+    def __init__(self, obj):
+        self.obj = obj
+
+    def __hash__(self):
+        return id(self.obj)
+
+    def __eq__(self, other):
+        return isinstance(other, _ById) and other.obj is self.obj
+
+    def __ne__(self, other):
+        return not self == other
+
+
+def _freeze_environment_value(value):
+    try:
+        return _freeze(value)
+    except _Uncacheable:
+        return _ById(value)                 # modules, classes, large arrays, other objects: by identity
+
+
+def _code_names(code):
+    """Global names a code object refers to, nested functions and lambdas included."""
+    names = list(code.co_names)
+    for const in code.co_consts:
+        if hasattr(const, 'co_names'):
+            names.extend(_code_names(const))
+    return names
+
+
+def _environment_key(function):
+    """
+    What an operator function can see besides its arguments: the contents of its closure cells and the globals its
+    code names.  Part of the trace key, so rebinding such a name to another value (``scale = 3``) traces again;
+    objects that cannot be frozen count by identity (changing one in place is not noticed).
+    """
+    code = function.__code__
+    items = []
+    for name, cell in zip(code.co_freevars, function.__closure__ or ()):
+        try:
+            items.append((name, _freeze_environment_value(cell.cell_contents)))
+        except ValueError:                  # an empty cell
+            items.append((name, ('empty',)))
+    module_globals = function.__globals__
+    for name in _code_names(code):
+        if name in module_globals:
+            items.append((name, _freeze_environment_value(module_globals[name])))
+    return tuple(items)
+
+
 #: re-use the trace of an operator function applied again to the same input types and constants
 trace_cache_enabled = [True]
+_MAX_TRACES_PER_OPERATOR = 256
 
 
 def set_trace_cache(enabled):
     """
-    Operator functions are pure functions of their input types and constants, so a repeated application re-uses the
-    expression DAG (and gradient DAG) traced the first time.  Switch this off for operator functions that read
-    mutable state from outside their arguments.
+    Operator functions are pure functions of their input types, their constants and the closure variables and
+    globals they name, so a repeated application with all of those unchanged re-uses the expression DAG (and gradient
+    DAG) traced the first time.  Switch this off for operator functions that depend on anything else (an object
+    modified in place, a file, a random number).
     """
     trace_cache_enabled[0] = bool(enabled)
 
@@ -337,7 +399,8 @@ class _OpGenerator(object):
         if trace_cache_enabled[0]:
             try:
                 trace_key = (tuple((tuple(t.shape), t.dtype.proto_dtype) for t in input_types),
-                             tuple(sorted((k, _freeze(v)) for k, v in constants.items())), from_gradient)
+                             tuple(sorted((k, _freeze(v)) for k, v in constants.items())), from_gradient,
+                             _environment_key(self.op_function))
             except _Uncacheable:
                 trace_key = None
             else:
@@ -398,6 +461,8 @@ class _OpGenerator(object):
                 grad_dag = _with_full_inputs(_build_op_dag(*grad_outputs), grad_inputs)
 
         if trace_key is not None:
+            if len(self._traces) >= _MAX_TRACES_PER_OPERATOR:
+                self._traces.clear()
             _freeze_op(expression_dag)
             self._traces[trace_key] = (self.grad_function, expression_dag, tuple(output_types), grad_dag)
         return _Operator(expression_dag, output_types, inputs, grad_dag, from_gradient, self.name)

@@ -556,8 +556,21 @@ def test_merge_is_memoised():
 # ----------------------------------------------------------------------------------------------------------------------
 # trace re-use
 # ----------------------------------------------------------------------------------------------------------------------
+class _Counter(object):
+    """Counts traces; an object of its own so that the trace key sees it by identity, not by value."""
+
+    def __init__(self):
+        self.count = 0
+
+    def append(self, _):
+        self.count += 1
+
+    def __len__(self):
+        return self.count
+
+
 def _traced_scale():
-    calls = []
+    calls = _Counter()
 
     @ovl.operator()
     def scale(x, factor=None, offsets=None):
@@ -637,3 +650,67 @@ def test_a_gradient_registered_later_invalidates_the_trace():
     after = scale(a, factor=2.0, offsets=())
     assert after.grad_dag is not None
     assert len(calls) == 2
+
+
+_TRACE_SCALE = 2.0
+
+
+def test_rebinding_a_global_or_closure_variable_traces_again():
+    global _TRACE_SCALE
+    offset = [1.0]
+    bias = 0.5
+    calls = _Counter()
+
+    @ovl.operator()
+    def affine(x):
+        calls.append(1)
+        pos = ovl.position_in(x.shape)
+        out = ovl.output_like(x)
+        out[pos] = x[pos] * _TRACE_SCALE + bias + (lambda: offset[0])()
+        return out
+
+    a = np.zeros(8, dtype=np.float32)
+    first = affine(a)
+    assert affine(a).expression_dag is first.expression_dag and len(calls) == 1
+    _TRACE_SCALE = 3.0
+    try:
+        second = affine(a)
+        assert len(calls) == 2 and second.expression_dag is not first.expression_dag
+        assert affine(a).expression_dag is second.expression_dag
+    finally:
+        _TRACE_SCALE = 2.0
+    assert affine(a).expression_dag is first.expression_dag         # the earlier trace is still there
+    bias = 0.75                                                     # a rebound closure variable
+    assert affine(a).expression_dag is not first.expression_dag
+    assert len(calls) == 3
+    offset[0] = 9.0                                                 # a list changed in place: frozen by value
+    affine(a)
+    assert len(calls) == 4
+
+
+def test_function_valued_constants_are_keyed_by_code_and_surroundings():
+    from opveclib_amd.examples import accumulate, cumprod
+    x = np.zeros((4, 32), dtype=np.float32)
+    # each call of cumsum creates a new lambda object from the same code
+    assert cumsum(x, axis=1).expression_dag is cumsum(x, axis=1).expression_dag
+    assert cumsum(x, axis=1).expression_dag is not cumprod(x, axis=1).expression_dag
+
+    def scaled_sum(factor):
+        return accumulate(x, inner_fcn=lambda acc, elem: acc + elem * factor, axis=1)
+
+    assert scaled_sum(2.0).expression_dag is scaled_sum(2.0).expression_dag
+    assert scaled_sum(2.0).expression_dag is not scaled_sum(3.0).expression_dag
+    # default arguments are part of the function
+    first = accumulate(x, inner_fcn=lambda acc, elem, w=2.0: acc + elem * w, axis=1)
+    second = accumulate(x, inner_fcn=lambda acc, elem, w=4.0: acc + elem * w, axis=1)
+    assert first.expression_dag is not second.expression_dag
+
+
+def test_objects_keyed_by_identity_are_kept_alive():
+    from opveclib_amd.operator import _ById, _freeze_environment_value
+    big = np.zeros(100000)
+    key = _freeze_environment_value(big)
+    assert isinstance(key, _ById) and key.obj is big
+    assert key == _freeze_environment_value(big) and hash(key) == hash(_freeze_environment_value(big))
+    assert key != _freeze_environment_value(np.zeros(100000))
+    assert _freeze_environment_value(np.arange(4)) == _freeze_environment_value(np.arange(4))   # small: by value
