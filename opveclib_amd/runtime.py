@@ -117,6 +117,32 @@ def load_operator(op, options=None):
     return compiled
 
 
+#: compiler processes run side by side when several operators of one DAG have no library yet
+max_parallel_builds = 8
+
+
+def _build_missing(operators, options):
+    """
+    Cold start: generate and compile, in parallel, every operator of the DAG that is neither loaded nor built.  One
+    hipcc run takes 10-20 s, so an unfused eight operator DAG starts in the time of one compilation instead of eight
+    (the reference compiles its operators one after the other, opveclib/operator.py:2262-2300).
+    """
+    if codegen_options:
+        options = dict(codegen_options, **(options or {}))
+    option_key = repr(sorted((options or {}).items()))
+    missing = {}
+    for op in operators:
+        name = _op_hash(op)
+        with _lock:
+            known = (name, option_key) in _loaded or (name, option_key) in _generated
+        if not known:
+            missing[name] = op
+    if len(missing) > 1:
+        from concurrent.futures import ThreadPoolExecutor
+        with ThreadPoolExecutor(max_workers=min(max_parallel_builds, len(missing))) as pool:
+            list(pool.map(lambda op: build_operator(op, options), missing.values()))
+
+
 def _require_gpu():
     import torch
     if not torch.cuda.is_available():
@@ -165,6 +191,7 @@ def run_op_dag(dag, leaf_inputs, profiling_iterations=1, timed=True, options=Non
         all_host = all_host and from_host
         leaves.append(t)
 
+    _build_missing(dag.operators, options)
     with torch.cuda.device(device):
         stream = torch.cuda.current_stream(device).cuda_stream
         buffers = []

@@ -211,3 +211,38 @@ def test_workgroups_beyond_32_bit_positions_are_refused():
         return out
     with pytest.raises(ValueError):
         hipgen.generate(fill(np.zeros(4, np.float32)).expression_dag, 'f' + '6' * 56)
+
+
+def test_missing_operators_of_a_dag_are_built_side_by_side(tmp_path, monkeypatch):
+    """Cold start: every operator of a DAG without a library is generated and compiled before the first launch."""
+    import os
+    import threading
+    import numpy as np
+    from opveclib_amd import compiler, local, runtime, stdops
+    from opveclib_amd.operator import _build_op_dag, _normalise_output_list, _op_hash
+
+    monkeypatch.setattr(local, 'cache_directory', str(tmp_path))
+    monkeypatch.setattr(local, 'prebuilt_directory', str(tmp_path / 'none'))
+    monkeypatch.setattr(compiler, 'prebuild_mode', False)
+    seen_threads = set()
+    real_build = compiler.build_library
+
+    def recording_build(source):
+        seen_threads.add(threading.get_ident())
+        return real_build(source)
+
+    monkeypatch.setattr(compiler, 'build_library', recording_build)
+    x = np.zeros((3, 20), dtype=np.float32)                # a shape no other test uses
+    out = stdops.sub(stdops.mul(stdops.add(x, x), x), x)
+    dag = _build_op_dag(*_normalise_output_list(out)).proto_dag
+    assert len(dag.operators) == 3
+    runtime._build_missing(dag.operators, None)
+    for op in dag.operators:
+        key = (_op_hash(op), repr([]))
+        assert key in runtime._generated
+        assert os.path.exists(runtime._generated[key][1])
+    assert len(seen_threads) == 3 and threading.get_ident() not in seen_threads
+    # nothing left to do the second time
+    seen_threads.clear()
+    runtime._build_missing(dag.operators, None)
+    assert not seen_threads
