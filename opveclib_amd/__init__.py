@@ -41,6 +41,7 @@ from .expression import if_, elif_, else_
 # @ Operator functions
 from .operator import operator, gradient, evaluate, profile, set_math_mode, get_math_mode, set_trace_cache
 from .autograd import as_torch
+from .graph import CapturedDag
 
 # @ Local runtime environment functions
 from .local import version, logger, cache_directory, clear_op_cache

@@ -138,6 +138,17 @@ def bounded_mix(rng, shape=(32, 256)):
     return all_outputs(_bounded_mix(special_values(rng, shape)))
 
 
+def graph_capture_dag(x, y):
+    """Several kernels even at opt_level 3: a scan between element-wise stages, two requested outputs."""
+    stage = stdops.tanh(stdops.add(x, y))
+    scanned = cumsum(stage, axis=1)
+    return [log1p(expm1(stdops.mul(scanned, y)))[0], stdops.sub(scanned, x)[0]]
+
+
+def graph_capture_single(x):
+    return [log1p(expm1(shift_cyclic(x)))[0]]
+
+
 def c3_cumsum_f32(rng, shape=(48, 1024)):
     return [cumsum(rng.standard_normal(shape, dtype=np.float32), axis=1)[0]]
 
@@ -834,6 +845,12 @@ def prebuild_all(cases=None, workers=8, with_oracle=True, force_benchmark=False)
         for name in FAST_FUSED_CASES:
             for op in _operators_of(CASE_BY_NAME[name].outputs(), 3):
                 variants.append((op, {'math': 'fast'}))
+        zeros = np.zeros((48, 256), np.float32)
+        for level in (0, 3):
+            for op in _operators_of(graph_capture_dag(zeros, zeros), level):
+                ops[op.SerializeToString()] = op
+        for op in _operators_of(graph_capture_single(np.zeros(4096, np.float32)), 3):
+            variants.append((op, {'math': 'fast'}))
         from tests import autograd_cases
         for outs in autograd_cases.graphs_to_build():
             for level in (0, 3):
