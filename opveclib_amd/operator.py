@@ -287,12 +287,19 @@ def _freeze_environment_value(value):
         return _ById(value)                 # modules, classes, large arrays, other objects: by identity
 
 
+_code_names_cache = {}
+
+
 def _code_names(code):
-    """Global names a code object refers to, nested functions and lambdas included."""
-    names = list(code.co_names)
-    for const in code.co_consts:
-        if hasattr(const, 'co_names'):
-            names.extend(_code_names(const))
+    """Global names a code object refers to, nested functions and lambdas included (code objects are immutable)."""
+    names = _code_names_cache.get(code)
+    if names is None:
+        names = list(code.co_names)
+        for const in code.co_consts:
+            if hasattr(const, 'co_names'):
+                names.extend(_code_names(const))
+        names = tuple(dict.fromkeys(names))
+        _code_names_cache[code] = names
     return names
 
 
