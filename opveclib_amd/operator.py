@@ -281,10 +281,14 @@ class _ById(object):
 
 
 def _freeze_environment_value(value):
+    # functions, modules and classes that an operator function names count by identity (looking into them would
+    # never end for functions that name each other); so does anything else that cannot be frozen by value
+    if isinstance(value, (types.FunctionType, types.ModuleType, type, types.BuiltinFunctionType)):
+        return _ById(value)
     try:
         return _freeze(value)
     except _Uncacheable:
-        return _ById(value)                 # modules, classes, large arrays, other objects: by identity
+        return _ById(value)
 
 
 _code_names_cache = {}

@@ -714,3 +714,23 @@ def test_objects_keyed_by_identity_are_kept_alive():
     assert key == _freeze_environment_value(big) and hash(key) == hash(_freeze_environment_value(big))
     assert key != _freeze_environment_value(np.zeros(100000))
     assert _freeze_environment_value(np.arange(4)) == _freeze_environment_value(np.arange(4))   # small: by value
+
+
+def _ping(n):
+    return n if n <= 0 else _pong(n - 1)
+
+
+def _pong(n):
+    return n if n <= 0 else _ping(n - 1)
+
+
+def test_operator_functions_may_name_functions_that_name_each_other():
+    @ovl.operator()
+    def uses_helpers(x):
+        pos = ovl.position_in(x.shape)
+        out = ovl.output_like(x)
+        out[pos] = x[pos] + float(_ping(3))
+        return out
+
+    a = np.zeros(8, dtype=np.float32)
+    assert uses_helpers(a).expression_dag is uses_helpers(a).expression_dag
