@@ -125,9 +125,15 @@ class DType(object):
             raise KeyError(self.proto_dtype)
         return cstr
 
+    _torch_dtypes = {}
+
     def as_torch(self):
-        import torch
-        return getattr(torch, np.dtype(self.as_numpy()).name)
+        found = DType._torch_dtypes.get(self.proto_dtype)
+        if found is None:
+            import torch
+            found = getattr(torch, np.dtype(self.as_numpy()).name)
+            DType._torch_dtypes[self.proto_dtype] = found
+        return found
 
     def as_proto(self):
         return self.proto_dtype
