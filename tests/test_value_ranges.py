@@ -228,3 +228,163 @@ def test_in_range_conditions():
     assert not ranges.div_in_range(Range(0.0, 10.0, False), Range(1.0, 2.0, False))         # a zero dividend
     assert not ranges.div_in_range(Range(1.0, 2.0 ** 100, False), Range(2.0 ** -100, 1.0, False))   # quotient too large
     assert not ranges.div_in_range(Range(1.0, 2.0, False), Range(-1.0, 1.0, False))
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# Soundness on whole operators: a concrete interpreter of the expression DAG runs one worker on sample inputs; every
+# value it computes must lie in the range the analysis assigned (NaN only where NaN is declared possible), operands
+# must lie in the operand ranges recorded at their point of use, and every decided comparison must have the decided
+# outcome.
+# ----------------------------------------------------------------------------------------------------------------------
+_NP_TYPE = {lang.FLOAT32: np.float32, lang.FLOAT64: np.float64, lang.INT8: np.int8, lang.INT16: np.int16,
+            lang.INT32: np.int32, lang.INT64: np.int64, lang.UINT8: np.uint8, lang.UINT16: np.uint16,
+            lang.UINT32: np.uint32, lang.UINT64: np.uint64}
+_UNARY_FN = {lang.TANH: np.tanh, lang.EXP: np.exp, lang.LOG: np.log, lang.SQRT: np.sqrt, lang.ABS: np.abs,
+             lang.NEGATE: np.negative, lang.SIN: np.sin, lang.COS: np.cos, lang.FLOOR: np.floor, lang.CEIL: np.ceil,
+             lang.TAN: np.tan, lang.SINH: np.sinh, lang.COSH: np.cosh, lang.LOG10: np.log10, lang.ASIN: np.arcsin,
+             lang.ACOS: np.arccos, lang.ATAN: np.arctan}
+_BINARY_FN = {lang.ADD: np.add, lang.SUBTRACT: np.subtract, lang.MULTIPLY: np.multiply, lang.DIVIDE: np.divide}
+_COMPARE_FN = {lang.EQUAL: np.equal, lang.NOTEQUAL: np.not_equal, lang.LESS: np.less, lang.LESS_EQ: np.less_equal,
+               lang.GREATER: np.greater, lang.GREATER_EQ: np.greater_equal}
+
+
+class _Interpreter(object):
+    """One worker (position 0) of a loop-free operator on inputs that read ``feed[input index]`` everywhere."""
+
+    def __init__(self, info, known, feed):
+        self.info, self.known, self.feed = info, known, feed
+        self.values = {}
+        self.checked = 0
+
+    def value(self, idx):
+        return self.values.get(idx)
+
+    def check(self, r, v, what):
+        if r is None or v is None or not isinstance(v, (np.floating, np.integer, float, int)):
+            return
+        v = float(v)
+        if v != v:
+            assert r.nan, '%s: NaN but the range %r excludes it' % (what, r)
+        else:
+            assert r.lo <= v <= r.hi, '%s: %r outside %r' % (what, v, r)
+        self.checked += 1
+
+    def run(self, items):
+        nodes = self.info.nodes
+        for item in items:
+            if item.kind == 'stmt':
+                self.step(nodes[item.node])
+            elif item.kind == 'if':
+                for cond, body in item.branches:
+                    if cond is None or self.value(cond) != 0:      # NaN is true, as in C
+                        self.run(body)
+                        break
+            else:
+                raise NotImplementedError('loops')
+
+    def step(self, node):
+        code, ops = node.code, node.ops
+        args = [self.value(o) for o in ops]
+        for k, a in enumerate(args):
+            self.check(self.known.operand(node.idx, k), a, 'operand %d of node %d' % (k, node.idx))
+        cast = _NP_TYPE.get(node.dtype)
+        result = None
+        with np.errstate(all='ignore'):
+            if code == lang.CONST_SCALAR:
+                result = cast(node.data[0])
+            elif code in (lang.MIN_VALUE, lang.MAX_VALUE, lang.EPSILON):
+                fi = np.finfo(cast)
+                result = {lang.MIN_VALUE: fi.tiny, lang.MAX_VALUE: fi.max, lang.EPSILON: fi.eps}[code]
+            elif code in (lang.CAST, lang.VARIABLE):
+                result = None if args[0] is None else cast(args[0])
+            elif code == lang.ASSIGN_VARIABLE:
+                target = self.info.nodes[ops[0]]
+                self.values[ops[0]] = None if args[1] is None else _NP_TYPE[target.dtype](args[1])
+                return
+            elif code == lang.READ_TENSOR:
+                tensor = self.info.nodes[ops[0]]
+                if tensor.code == lang.INPUT:
+                    result = cast(self.feed[tensor.io_index])
+                elif tensor.code == lang.POSITION:
+                    result = cast(0)
+            elif code in _COMPARE_FN:
+                if args[0] is not None and args[1] is not None:
+                    result = cast(bool(_COMPARE_FN[code](args[0], args[1])))
+            elif code == lang.AND:
+                if args[0] is not None and args[1] is not None:
+                    result = cast(bool(args[0] != 0) and bool(args[1] != 0))
+            elif code == lang.OR:
+                if args[0] is not None and args[1] is not None:
+                    result = cast(bool(args[0] != 0) or bool(args[1] != 0))
+            elif code == lang.NOT:
+                if args[0] is not None:
+                    result = cast(not bool(args[0] != 0))
+            elif code == lang.ISINF:
+                result = cast(bool(np.isinf(args[0])))
+            elif code == lang.ISNAN:
+                result = cast(bool(np.isnan(args[0])))
+            elif code == lang.ISFINITE:
+                result = cast(bool(np.isfinite(args[0])))
+            elif code in (lang.MIN, lang.MAX) and args[0] is not None and args[1] is not None:
+                first = args[0] < args[1] if code == lang.MIN else args[0] > args[1]
+                result = args[0] if first else args[1]
+            elif node.dtype in (lang.FLOAT32, lang.FLOAT64) and all(a is not None for a in args):
+                if code in _UNARY_FN:
+                    result = cast(_UNARY_FN[code](args[0]))
+                elif code in _BINARY_FN:
+                    result = cast(_BINARY_FN[code](args[0], args[1]))
+        if result is None:
+            return
+        self.values[node.idx] = result
+        self.check(self.known.ranges.get(node.idx), result, 'node %d (code %d)' % (node.idx, node.code))
+        decided = self.known.constant(node.idx)
+        if decided is not None:
+            assert float(result) == decided, 'node %d decided %d but is %r' % (node.idx, decided, result)
+
+
+def _sample_values():
+    rng = np.random.default_rng(11)
+    special = [np.nan, np.inf, -np.inf, 0.0, -0.0, 3.4028235e38, -3.4028235e38, 1.1754944e-38, 1e-45, -1e-45, 88.0,
+               -88.0, 87.3, -87.4, 103.9, -104.0, 22.0, -22.0, 50.0, -50.0, 49.99, 1.0, -1.0, 0.5, 1e-8, -1e-8, 1e20,
+               -1e20, 2.0 ** 126, 2.0 ** -126, 0.6, -0.6, 10.0, -10.0]
+    return special + list(rng.standard_normal(60)) + list(rng.uniform(-100, 100, 40)) + list(10.0 ** rng.uniform(-40, 38, 30))
+
+
+def _operators_to_interpret():
+    from opveclib_amd.lstm import lstm, lstm_grad
+    from tests import cases
+    x = np.zeros((2, 64), dtype=np.float32)
+    v = np.zeros(64, dtype=np.float32)
+    concat, c = np.zeros((2, 256), np.float32), np.zeros((2, 64), np.float32)
+    yield 'chain8', _merged_single(cases.chain8(x, x, np.ones(1, np.float32))[-1][0])
+    yield 'activation chain', _merged_single(expm1(log1p(stdops.sigmoid(stdops.tanh(x)))))
+    yield 'bounded_mix', cases._bounded_mix(x).expression_dag
+    yield 'branchy', _branchy(v, with_else=True).expression_dag
+    yield 'branchy without else', _branchy(v, with_else=False).expression_dag
+    yield 'dead branch', _dead_branch(v).expression_dag
+    yield 'expm1', expm1(x).expression_dag
+    yield 'log1p', log1p(x).expression_dag
+    yield 'lstm', lstm(concat, c, forget_bias=1.0).expression_dag
+    yield 'lstm_grad', lstm_grad(concat, c, c, c, forget_bias=1.0)[0].parent.expression_dag
+    yield 'division', stdops.div(x, x).expression_dag
+
+
+@pytest.mark.parametrize('math_mode', ['exact', 'fast'])
+def test_ranges_hold_for_every_value_a_worker_computes(math_mode):
+    samples = [np.float32(s) for s in _sample_values()]
+    rng = np.random.default_rng(12)
+    total = 0
+    for name, op in _operators_to_interpret():
+        info = DagInfo(op)
+        info.math = math_mode
+        known = ranges.analyse(info)
+        for s in samples:
+            # every input tensor reads the sample, or (second round) independent samples
+            for feed in ([s] * len(info.inputs), [samples[k] for k in rng.integers(0, len(samples), len(info.inputs))]):
+                machine = _Interpreter(info, known, feed)
+                try:
+                    machine.run(info.tree)
+                except AssertionError as error:
+                    raise AssertionError('%s, inputs %r: %s' % (name, feed, error))
+                total += machine.checked
+    assert total > 100000
