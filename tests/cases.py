@@ -845,6 +845,10 @@ def prebuild_all(cases=None, workers=8, with_oracle=True, force_benchmark=False)
         for name in FAST_FUSED_CASES:
             for op in _operators_of(CASE_BY_NAME[name].outputs(), 3):
                 variants.append((op, {'math': 'fast'}))
+        from tests import golden
+        for _name, out, _expected, _sum, _atol in golden.known_answers():
+            for op in _operators_of(all_outputs(out), 0):
+                ops[op.SerializeToString()] = op
         zeros = np.zeros((48, 256), np.float32)
         for level in (0, 3):
             for op in _operators_of(graph_capture_dag(zeros, zeros), level):

@@ -48,3 +48,17 @@ def test_loaded_operators_come_from_the_hip_extension():
     for compiled in runtime._loaded.values():
         assert compiled.so_path.endswith('_generic_hip.so')
         assert compiled.lib.info['template'] in ('map', 'transpose', 'rowscan', 'skewscan')
+
+
+def test_known_answer_fixtures_on_the_gpu():
+    """tests/golden/known_answers.json: the answers the reference's README and tests state, through the HIP path."""
+    from tests import golden
+    for name, out, expected, expected_sum, atol in golden.known_answers():
+        for opt_level in (0, 3):
+            got = ovl.evaluate(out, opt_level=opt_level)
+            if expected_sum is not None:
+                assert int(got.sum()) == expected_sum, name
+            elif atol:
+                assert got.dtype == expected.dtype and np.allclose(got, expected, rtol=0, atol=atol), name
+            else:
+                assert got.dtype == expected.dtype and np.array_equal(got, expected), name

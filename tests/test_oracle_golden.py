@@ -335,3 +335,19 @@ def test_driver_reports_argument_errors():
     assert lib.ovl_cpu_run(so_path.encode(), entry.encode(), good_in, 2, good_out, 1, 2, None, 1) == 1
     assert lib.ovl_cpu_run(so_path.encode(), b'no_such_symbol', good_in, 1, good_out, 1, 2, None, 1) == 3
     assert lib.ovl_cpu_run(b'/nonexistent/lib.so', entry.encode(), good_in, 1, good_out, 1, 2, None, 1) == 2
+
+
+def test_known_answer_fixtures():
+    """tests/golden/known_answers.json: the answers the reference's README and tests state, through the oracle."""
+    from tests import golden
+    names = []
+    for name, out, expected, expected_sum, atol in golden.known_answers():
+        got = oracle.evaluate(out)
+        if expected_sum is not None:
+            assert int(got.sum()) == expected_sum, name
+        elif atol:
+            assert got.dtype == expected.dtype and np.allclose(got, expected, rtol=0, atol=atol), name
+        else:
+            assert got.dtype == expected.dtype and np.array_equal(got, expected), name
+        names.append(name)
+    assert len(names) == 8
