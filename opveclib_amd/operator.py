@@ -11,6 +11,7 @@ current PyTorch HIP stream.  There is no CPU execution path in this package.
 import dis
 import hashlib
 import inspect
+import threading
 import types
 from collections import namedtuple
 
@@ -327,6 +328,8 @@ def _environment_key(function):
     return tuple(items)
 
 
+_trace_lock = threading.RLock()
+
 #: re-use the trace of an operator function applied again to the same input types and constants
 trace_cache_enabled = [True]
 _MAX_TRACES_PER_OPERATOR = 256
@@ -419,37 +422,7 @@ class _OpGenerator(object):
                 if cached is not None and cached[0] is self.grad_function:
                     return _Operator(cached[1], list(cached[2]), inputs, cached[3], from_gradient, self.name)
 
-        ExpressionDAG.clear()
-        input_exprs = [input(cur_type) for cur_type in input_types]
-
-        # interpret function to build up ExpressionDAG
-        output_exprs = self.op_function(*input_exprs, **constants)
-        if output_exprs is None:
-            raise ValueError('No outputs returned from op function')
-        output_exprs = _as_list(output_exprs)
-
-        if len(output_exprs) != ExpressionDAG.num_outputs:
-            raise ValueError('Defined ' + str(ExpressionDAG.num_outputs) + ' outputs, but returned ' +
-                             str(len(output_exprs)) +
-                             '. Number of defined outputs must equal number of returned outputs.')
-
-        # outputs are numbered by return position, not by declaration order, and their declarations are permuted
-        # so that they appear in the DAG in that order too
-        output_types = []
-        slots = []
-        for index, expr in enumerate(output_exprs):
-            if type(expr) is not OutputTensor:
-                raise TypeError('User functions must only return outputs. Instead got:\n' + str(expr))
-            slots.append(ExpressionDAG.expr_index(expr))
-            output_types.append(TensorType.like(expr))
-        for index, expr in enumerate(output_exprs):
-            expr.proto_expr.io_index = index
-        for slot, expr in zip(sorted(slots), output_exprs):
-            ExpressionDAG.replace(slot, expr)
-
-        expression_dag = ExpressionDAG.as_proto()
-        ExpressionDAG.clear()
-        expression_dag.name = self.name
+        expression_dag, output_types = self._trace(input_types, constants)
 
         grad_dag = None
         if self.grad_function is not None and not from_gradient:
@@ -477,6 +450,43 @@ class _OpGenerator(object):
             _freeze_op(expression_dag)
             self._traces[trace_key] = (self.grad_function, expression_dag, tuple(output_types), grad_dag)
         return _Operator(expression_dag, output_types, inputs, grad_dag, from_gradient, self.name)
+
+    def _trace(self, input_types, constants):
+        """Run the operator function on input expressions; returns (expression DAG, output types).  The recorder of
+        expressions is one global list (as in the reference, expression.py:250-352), so traces take turns."""
+        with _trace_lock:
+            ExpressionDAG.clear()
+            input_exprs = [input(cur_type) for cur_type in input_types]
+
+            # interpret function to build up ExpressionDAG
+            output_exprs = self.op_function(*input_exprs, **constants)
+            if output_exprs is None:
+                raise ValueError('No outputs returned from op function')
+            output_exprs = _as_list(output_exprs)
+
+            if len(output_exprs) != ExpressionDAG.num_outputs:
+                raise ValueError('Defined ' + str(ExpressionDAG.num_outputs) + ' outputs, but returned ' +
+                                 str(len(output_exprs)) +
+                                 '. Number of defined outputs must equal number of returned outputs.')
+
+            # outputs are numbered by return position, not by declaration order, and their declarations are permuted
+            # so that they appear in the DAG in that order too
+            output_types = []
+            slots = []
+            for index, expr in enumerate(output_exprs):
+                if type(expr) is not OutputTensor:
+                    raise TypeError('User functions must only return outputs. Instead got:\n' + str(expr))
+                slots.append(ExpressionDAG.expr_index(expr))
+                output_types.append(TensorType.like(expr))
+            for index, expr in enumerate(output_exprs):
+                expr.proto_expr.io_index = index
+            for slot, expr in zip(sorted(slots), output_exprs):
+                ExpressionDAG.replace(slot, expr)
+
+            expression_dag = ExpressionDAG.as_proto()
+            ExpressionDAG.clear()
+            expression_dag.name = self.name
+            return expression_dag, output_types
 
     def add_grad(self, grad_function):
         if self.grad_function is not None:

@@ -734,3 +734,28 @@ def test_operator_functions_may_name_functions_that_name_each_other():
 
     a = np.zeros(8, dtype=np.float32)
     assert uses_helpers(a).expression_dag is uses_helpers(a).expression_dag
+
+
+def test_concurrent_traces_do_not_mix():
+    """The expression recorder is global; applications from several threads take turns."""
+    import threading
+    a = np.zeros((4, 32), dtype=np.float32)
+    serial = {'expm1': expm1(a).expression_dag.SerializeToString(),
+              'log1p': log1p(a).expression_dag.SerializeToString(),
+              'tanh': stdops.tanh(a).expression_dag.SerializeToString()}
+    builders = {'expm1': lambda: expm1(a), 'log1p': lambda: log1p(a), 'tanh': lambda: stdops.tanh(a)}
+    failures = []
+    ovl.set_trace_cache(False)
+    try:
+        def worker(name):
+            for _ in range(40):
+                if builders[name]().expression_dag.SerializeToString() != serial[name]:
+                    failures.append(name)
+        threads = [threading.Thread(target=worker, args=(name,)) for name in builders for _ in range(2)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+    finally:
+        ovl.set_trace_cache(True)
+    assert not failures
