@@ -248,8 +248,27 @@ class HandWrittenLstm(object):
             raise RuntimeError(self.lib.ovl_lstm_last_error().decode())
 
 
+class HandWrittenScan(object):
+    """The hand-written row scan kernels (include/ovl_scan.h) behind the interface settle() and measure() use."""
+
+    def __init__(self, x, entry):
+        import torch
+        from opveclib_amd import row_scan
+        self.lib = row_scan.library()
+        self.entry = getattr(self.lib, entry)
+        self.x = torch.from_numpy(np.ascontiguousarray(x)).cuda()
+        self.out = torch.empty_like(self.x)
+        self.rows, self.cols = self.x.shape
+        self.algorithmic_bytes = 2 * self.x.numel() * self.x.element_size()
+        self.kernels = [{'kernel': 'skewed_scan_kernel'}]
+
+    def launch(self, stream):
+        if self.entry(self.x.data_ptr(), self.rows, self.cols, self.out.data_ptr(), stream) != 0:
+            raise RuntimeError(self.lib.ovl_scan_last_error().decode())
+
+
 def side_workload(name, outputs, steps, warmup, options=None):
-    prepared = outputs if isinstance(outputs, HandWrittenLstm) else Prepared(outputs, options)
+    prepared = outputs if isinstance(outputs, (HandWrittenLstm, HandWrittenScan)) else Prepared(outputs, options)
     return _side_workload(name, prepared, steps, warmup)
 
 
@@ -372,6 +391,10 @@ def main():
         others.append(side_workload('c3 cumprod f32[4096,16384] last axis', cumprod_outputs(xp), steps, args.warmup))
         xd = g.standard_normal((1024, 16384))
         others.append(side_workload('c3 cumsum f64[1024,16384] last axis', cumsum_outputs(xd), steps, args.warmup))
+        others.append(side_workload('c3 cumsum f32[4096,16384], hand-written kernel (run-time shape, same bits)',
+                                    HandWrittenScan(xs, 'ovl_cumsum_f32'), steps, args.warmup))
+        others.append(side_workload('c3 cumsum f64[1024,16384], hand-written kernel (run-time shape, same bits)',
+                                    HandWrittenScan(xd, 'ovl_cumsum_f64'), steps, args.warmup))
         g = np.random.default_rng(4)
         concat = g.standard_normal((4096, 4096), dtype=np.float32)
         c = g.standard_normal((4096, 1024), dtype=np.float32)

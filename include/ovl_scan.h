@@ -1,0 +1,50 @@
+/*
+ * C ABI of the hand-written row scan kernels for AMD GPUs (libovl_scan.so).
+ *
+ * The reference's `accumulate` operator (opveclib/examples/test_accumulate.py:22-78; `cumsum` 81-113, `cumprod`
+ * 116-147) is generated for one fixed shape per trace: one worker per row runs
+ * `acc = x[row, 0]; out[row, 0] = acc; for i in 1 .. n-1: acc = f(acc, x[row, i]); out[row, i] = acc`
+ * strictly left to right in the tensor's type.  These entry points compute the running sum and the running product
+ * along the last axis of a dense C-ordered [rows, cols] tensor with exactly that order of operations - so results
+ * equal the generated operator's and `numpy.cumsum` / `numpy.cumprod` bit for bit - but take the shape at run time
+ * and need no code generation or compiler on the machine that calls them:
+ *
+ *   reference interface                                   replaced by
+ *   ----------------------------------------------------  ------------------------------------------
+ *   cumsum(x, axis=-1)    test_accumulate.py:81-113        ovl_cumsum_f32 / ovl_cumsum_f64
+ *   cumprod(x, axis=-1)   test_accumulate.py:116-147       ovl_cumprod_f32 / ovl_cumprod_f64
+ *
+ * Kernel: the lane-skewed order-preserving scan.  Sixteen neighbouring lanes share a row; a lane owns a run of
+ * consecutive columns of the current group (one 128-bit access for float32, two for float64), runs the recurrence
+ * over its run from the carried state it holds and hands its state to its right neighbour with a lane-to-lane move;
+ * after sixteen such phases the group is exact and the last lane's state is the carry into the next group.  Column
+ * counts that are not a multiple of the group (64 columns for float32, 64 for float64) or unaligned tensors take a
+ * plain kernel with one lane per row.
+ *
+ * Conventions: tensor memory belongs to the caller and must be device accessible; `out` may not overlap `x`; the
+ * functions enqueue one kernel on `hip_stream` (a hipStream_t; NULL is the default stream), return without
+ * synchronising and allocate nothing.  They return an ovl_status (ovl_launch.h): OVL_EINVAL for null pointers, zero
+ * sizes or rows * cols of 2^32 or more, OVL_EHIP for a HIP error (text from ovl_scan_last_error).
+ */
+#ifndef OVL_SCAN_H_
+#define OVL_SCAN_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+int ovl_cumsum_f32(const float* x, uint32_t rows, uint32_t cols, float* out, void* hip_stream);
+int ovl_cumprod_f32(const float* x, uint32_t rows, uint32_t cols, float* out, void* hip_stream);
+int ovl_cumsum_f64(const double* x, uint32_t rows, uint32_t cols, double* out, void* hip_stream);
+int ovl_cumprod_f64(const double* x, uint32_t rows, uint32_t cols, double* out, void* hip_stream);
+
+/* Text of the last error on the calling thread ("" if none). */
+const char* ovl_scan_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif  /* OVL_SCAN_H_ */

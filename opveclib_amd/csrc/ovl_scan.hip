@@ -1,0 +1,208 @@
+// Hand-written order-preserving row scans (running sum and product along the last axis) for gfx950 behind the C ABI
+// of include/ovl_scan.h.
+//
+// The recurrence of the reference's accumulate operator (opveclib/examples/test_accumulate.py:63-76) is kept exactly:
+// out[r, 0] = x[r, 0], out[r, i] = f(out[r, i-1], x[r, i]) in the tensor's own type, left to right.  Floating point
+// addition and multiplication are not associative, so a tree-shaped wavefront scan would give other bits; what is
+// parallel here is the rows (four per wavefront) and the movement of data.
+//
+// Lane-skewed scan: sixteen neighbouring lanes share one row.  Lane p of the group owns RUN = VEC * WIDTH consecutive
+// columns of the current group of 16 * RUN columns, loaded and stored as WIDTH 128-bit accesses.  In phase 0..15 every
+// lane runs the recurrence over its own run starting from the carried state it holds, then hands its final state to
+// its right neighbour (a DPP row_shr:1 move; lane 0 keeps the true carry).  After phase p lanes 0..p hold exact
+// results: a lane that is already exact recomputes the same values, a lane that is not yet exact computes values that
+// a later phase overwrites.  After phase 15 the group is exact and lane 15's state is rotated to lane 0 (row_ror:1)
+// as the carry into the next group.  Global accesses are issued in bursts of DEPTH groups into two register sets, so
+// one burst is in flight while the other is consumed.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <string>
+#include <type_traits>
+
+#include "ovl_device.h"
+#include "ovl_scan.h"
+
+// ovl_device.h carries the status codes generated operators return; this one (ovl_status in ovl_launch.h) is the
+// launcher's own
+#define OVL_EINVAL 6
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const std::string& detail) {
+    g_last_error = detail;
+    return code;
+}
+
+constexpr uint32_t BLOCK = 256, WAVE = 64, GROUP = 16;
+constexpr uint32_t ROWS_PER_WAVE = WAVE / GROUP, ROWS_PER_BLOCK = ROWS_PER_WAVE * (BLOCK / WAVE);
+
+// `start` is the value s with f(s, x) == x bit for bit for every x, signed zeros and infinities included (-0 for the
+// sum: +0 would turn a leading -0 into +0).  Starting the recurrence from it makes column 0 an ordinary step, with no
+// special case on the critical path: out[r, 0] = f(start, x[r, 0]) = x[r, 0].
+struct op_sum {
+    template <typename T> static __device__ __forceinline__ T apply(T a, T b) { return a + b; }
+    template <typename T> static __device__ __forceinline__ T start() { return (T)-0.0; }
+};
+struct op_product {
+    template <typename T> static __device__ __forceinline__ T apply(T a, T b) { return a * b; }
+    template <typename T> static __device__ __forceinline__ T start() { return (T)1.0; }
+};
+
+template <typename T, int VEC> struct vec_of { typedef T type __attribute__((ext_vector_type(VEC))); };
+
+// cols must be a multiple of 16 * VEC * WIDTH * DEPTH; x and out 16-byte aligned.
+template <typename T, typename OP, int VEC, int WIDTH, int DEPTH>
+__global__ void __launch_bounds__(BLOCK)
+skewed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, uint32_t cols) {
+    typedef typename vec_of<T, VEC>::type vec;
+    constexpr uint32_t RUN = VEC * WIDTH, GROUP_COLS = GROUP * RUN, BATCH_COLS = GROUP_COLS * DEPTH;
+    const uint32_t lane = threadIdx.x % WAVE;
+    const uint32_t part = lane % GROUP;
+    const uint32_t first_row = (blockIdx.x * (BLOCK / WAVE) + threadIdx.x / WAVE) * ROWS_PER_WAVE;
+    // A wavefront wholly past the last row leaves; single lanes past it shadow the last row instead (all lanes must
+    // stay active for the lane-to-lane moves): they load, compute and store exactly what its owners do.
+    if (first_row >= rows) return;
+    const uint32_t row_raw = first_row + lane / GROUP;
+    const uint32_t row = row_raw < rows ? row_raw : rows - 1u;
+    const T* __restrict__ gin = x + (uint64_t)row * cols + part * RUN;
+    T* __restrict__ gout = out + (uint64_t)row * cols + part * RUN;
+    const uint32_t num_batches = cols / BATCH_COLS;
+    const uint32_t last_batch = num_batches - 1u;
+
+    vec q[2][DEPTH][WIDTH];
+#pragma unroll
+    for (uint32_t s = 0; s < 2u; ++s) {
+        const uint32_t b = s < num_batches ? s : last_batch;
+#pragma unroll
+        for (uint32_t j = 0; j < (uint32_t)DEPTH; ++j)
+#pragma unroll
+            for (uint32_t w = 0; w < (uint32_t)WIDTH; ++w)
+                q[s][j][w] = *reinterpret_cast<const vec*>(gin + (uint64_t)b * BATCH_COLS + j * GROUP_COLS + w * VEC);
+    }
+    T carry = OP::template start<T>();
+
+    // One batch: scan the DEPTH groups held in register set s, store them, refill the set with batch b + 2.
+    auto process = [&](auto set, uint32_t b) {
+        constexpr uint32_t s = decltype(set)::value;
+        vec ov[DEPTH][WIDTH];
+#pragma unroll
+        for (uint32_t j = 0; j < (uint32_t)DEPTH; ++j) {
+            T acc = carry;
+#pragma unroll
+            for (uint32_t phase = 0; phase < GROUP; ++phase) {
+                acc = carry;
+#pragma unroll
+                for (uint32_t w = 0; w < (uint32_t)WIDTH; ++w) {
+#pragma unroll
+                    for (uint32_t u = 0; u < (uint32_t)VEC; ++u) {
+                        acc = OP::apply(acc, q[s][j][w][u]);
+                        ov[j][w][u] = acc;
+                    }
+                }
+                carry = ovl_dpp_move<OVL_DPP_ROW_SHR1>(carry, acc);
+            }
+            carry = ovl_dpp_move<OVL_DPP_ROW_ROR1>(carry, acc);
+        }
+        // The scheduling fences keep the memory traffic of a batch together, after its arithmetic, and no load is
+        // moved ahead of the last use of the registers it fills.
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (uint32_t j = 0; j < (uint32_t)DEPTH; ++j)
+#pragma unroll
+            for (uint32_t w = 0; w < (uint32_t)WIDTH; ++w)
+                __builtin_nontemporal_store(ov[j][w], reinterpret_cast<vec*>(
+                    gout + (uint64_t)b * BATCH_COLS + j * GROUP_COLS + w * VEC));
+        // past the end a set is refilled with the last batch again, which keeps the loop free of branches
+        const uint32_t next = b + 2u < num_batches ? b + 2u : last_batch;
+#pragma unroll
+        for (uint32_t j = 0; j < (uint32_t)DEPTH; ++j)
+#pragma unroll
+            for (uint32_t w = 0; w < (uint32_t)WIDTH; ++w)
+                q[s][j][w] = *reinterpret_cast<const vec*>(gin + (uint64_t)next * BATCH_COLS + j * GROUP_COLS + w * VEC);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    typedef std::integral_constant<uint32_t, 0> set0;
+    typedef std::integral_constant<uint32_t, 1> set1;
+
+    // straight-line pairs of batches (the wait counters of the loads in flight stay exact), then the odd one
+    uint32_t b0 = 0;
+#pragma unroll 1
+    for (; b0 + 1u < num_batches; b0 += 2u) {
+        process(set0(), b0);
+        process(set1(), b0 + 1u);
+    }
+    if (b0 < num_batches) process(set0(), b0);
+}
+
+// Any shape, any alignment: one lane per row.
+template <typename T, typename OP>
+__global__ void __launch_bounds__(BLOCK)
+row_per_lane_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, uint32_t cols) {
+    const uint32_t row = blockIdx.x * BLOCK + threadIdx.x;
+    if (row >= rows) return;
+    const T* in_row = x + (uint64_t)row * cols;
+    T* out_row = out + (uint64_t)row * cols;
+    T acc = in_row[0];
+    out_row[0] = acc;
+    for (uint32_t i = 1; i < cols; ++i) {
+        acc = OP::apply(acc, in_row[i]);
+        out_row[i] = acc;
+    }
+}
+
+template <typename T, typename OP>
+int scan(const char* who, const T* x, uint32_t rows, uint32_t cols, T* out, void* hip_stream) {
+    if (x == nullptr || out == nullptr) return fail(OVL_EINVAL, std::string(who) + ": null tensor");
+    if (rows == 0 || cols == 0) return fail(OVL_EINVAL, std::string(who) + ": rows and cols must be positive");
+    if ((uint64_t)rows * cols >= (1ull << 32)) return fail(OVL_EINVAL, std::string(who) + ": rows * cols must be below 2^32");
+    hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    // measured on MI355X: one 128-bit vector per lane and phase for 4-byte elements (the scan runs at the speed of
+    // memory), two for 8-byte elements (it runs at the latency of the recurrence, and the hand-over is paid half as
+    // often); request bursts of 1 KiB per row
+    constexpr int VEC = 16 / sizeof(T), WIDTH = sizeof(T) == 8 ? 2 : 1, DEPTH = 4 / WIDTH;
+    constexpr uint32_t GROUP_COLS = GROUP * VEC * WIDTH;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+    const dim3 block(BLOCK);
+    if (aligned && cols % GROUP_COLS == 0) {
+        const dim3 grid((rows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK);
+        if (cols % (GROUP_COLS * DEPTH) == 0)
+            hipLaunchKernelGGL((skewed_scan_kernel<T, OP, VEC, WIDTH, DEPTH>), grid, block, 0, stream, x, out, rows, cols);
+        else
+            hipLaunchKernelGGL((skewed_scan_kernel<T, OP, VEC, WIDTH, 1>), grid, block, 0, stream, x, out, rows, cols);
+    } else {
+        const dim3 grid((rows + BLOCK - 1) / BLOCK);
+        hipLaunchKernelGGL((row_per_lane_scan_kernel<T, OP>), grid, block, 0, stream, x, out, rows, cols);
+    }
+    const hipError_t err = hipPeekAtLastError();
+    if (err != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(OVL_EHIP, std::string(who) + ": " + hipGetErrorString(err));
+    }
+    return OVL_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* ovl_scan_last_error(void) { return g_last_error.c_str(); }
+
+int ovl_cumsum_f32(const float* x, uint32_t rows, uint32_t cols, float* out, void* hip_stream) {
+    return scan<float, op_sum>("ovl_cumsum_f32", x, rows, cols, out, hip_stream);
+}
+
+int ovl_cumprod_f32(const float* x, uint32_t rows, uint32_t cols, float* out, void* hip_stream) {
+    return scan<float, op_product>("ovl_cumprod_f32", x, rows, cols, out, hip_stream);
+}
+
+int ovl_cumsum_f64(const double* x, uint32_t rows, uint32_t cols, double* out, void* hip_stream) {
+    return scan<double, op_sum>("ovl_cumsum_f64", x, rows, cols, out, hip_stream);
+}
+
+int ovl_cumprod_f64(const double* x, uint32_t rows, uint32_t cols, double* out, void* hip_stream) {
+    return scan<double, op_product>("ovl_cumprod_f64", x, rows, cols, out, hip_stream);
+}
+
+}  // extern "C"

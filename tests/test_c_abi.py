@@ -134,3 +134,45 @@ def test_lstm_python_wrapper_validates_its_arguments():
     with pytest.raises(TypeError):
         lstm_cell._shapes(concat, [torch.zeros(4, 9)], ['c'])
     assert lstm_cell._shapes(concat, [c], ['c']) == (4, 8)
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# the hand-written row scan library (include/ovl_scan.h)
+# ----------------------------------------------------------------------------------------------------------------------
+SCAN_HEADER = os.path.join(ROOT, 'include', 'ovl_scan.h')
+
+
+def scan_declared_functions():
+    text = open(SCAN_HEADER).read()
+    text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
+    return sorted(set(re.findall(r'\b(ovl_[a-z_0-9]+)\s*\(', text)))
+
+
+def test_scan_header_binding_and_argument_errors():
+    from opveclib_amd import row_scan
+    if not os.path.exists(row_scan.library_path):
+        row_scan.build()
+    L = row_scan.library()
+    assert scan_declared_functions() == sorted(row_scan.EXPORTED_SYMBOLS)
+    raw = ctypes.CDLL(row_scan.library_path)
+    for name in scan_declared_functions():
+        assert hasattr(raw, name), name
+    p = ctypes.c_void_p(64)             # never dereferenced: every call below is refused first
+    for entry in (L.ovl_cumsum_f32, L.ovl_cumprod_f32, L.ovl_cumsum_f64, L.ovl_cumprod_f64):
+        assert entry(None, 4, 8, p, None) == launcher.OVL_EINVAL
+        assert b'null' in L.ovl_scan_last_error()
+        assert entry(p, 4, 8, None, None) == launcher.OVL_EINVAL
+        assert entry(p, 0, 8, p, None) == launcher.OVL_EINVAL
+        assert entry(p, 4, 0, p, None) == launcher.OVL_EINVAL
+        assert entry(p, 1 << 16, 1 << 16, p, None) == launcher.OVL_EINVAL
+        assert b'2^32' in L.ovl_scan_last_error()
+
+
+def test_scan_python_wrapper_validates_its_arguments():
+    import numpy as np
+    import torch
+    from opveclib_amd import row_scan
+    with pytest.raises(TypeError):
+        row_scan.cumsum(np.zeros((4, 8), np.float32))
+    with pytest.raises(RuntimeError):
+        row_scan.cumsum(torch.zeros(4, 8))                          # a host tensor

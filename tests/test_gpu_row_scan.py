@@ -1,0 +1,72 @@
+"""
+The hand-written row scans (include/ovl_scan.h) on the GPU: the same bits as numpy's strictly sequential
+cumsum / cumprod (which is what the reference's accumulate operator computes, examples/test_accumulate.py:63-76), as
+the CPU oracle and as the generated operator, on shapes that take the lane-skewed kernel with deep and shallow request
+bursts, the one-lane-per-row kernel (ragged column counts, unaligned views) and the benchmark's full sizes.
+"""
+import numpy as np
+import pytest
+import torch
+
+import opveclib_amd as ovl
+import oracle
+from opveclib_amd import row_scan
+from opveclib_amd.examples import cumsum, cumprod
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(48, 1024), (7, 256), (5, 64), (3, 192), (515, 64), (259, 128), (4, 70, 128), (5, 70), (7, 3), (1, 1),
+          (2, 4096), (4096,)]
+
+
+def _data(rng, shape, dtype, kind):
+    if kind == 'sum':
+        return rng.standard_normal(shape).astype(dtype)
+    return (0.9 + 0.2 * rng.random(shape)).astype(dtype)
+
+
+@pytest.mark.parametrize('dtype', [np.float32, np.float64])
+@pytest.mark.parametrize('shape', SHAPES, ids=[str(s) for s in SHAPES])
+def test_equal_to_sequential_accumulation(shape, dtype):
+    rng = np.random.default_rng(len(shape) * 100 + shape[-1])
+    for kind, fn, ref_fn in (('sum', row_scan.cumsum, np.cumsum), ('product', row_scan.cumprod, np.cumprod)):
+        x = _data(rng, shape, dtype, kind)
+        got = fn(torch.from_numpy(x).cuda()).cpu().numpy()
+        ref = ref_fn(x, axis=-1, dtype=dtype)           # numpy accumulates strictly left to right
+        assert got.dtype == ref.dtype and got.shape == ref.shape
+        assert np.array_equal(got, ref), '%s %s %s: %d elements differ' % (kind, shape, np.dtype(dtype).name,
+                                                                           int((got != ref).sum()))
+
+
+def test_equal_to_the_oracle_with_special_values():
+    x = np.random.default_rng(5).standard_normal((6, 128)).astype(np.float32)
+    x[1, 5] = np.inf
+    x[2, 9] = np.nan
+    x[3, 0] = -0.0
+    x[4, 17] = 3.0e38
+    x[4, 18] = 3.0e38
+    for op, fn in ((cumsum, row_scan.cumsum), (cumprod, row_scan.cumprod)):
+        ref = oracle.evaluate(op(x, axis=1))
+        got = fn(torch.from_numpy(x).cuda()).cpu().numpy()
+        assert np.array_equal(got, ref, equal_nan=True)
+        assert np.array_equal(np.signbit(got[~np.isnan(ref)]), np.signbit(ref[~np.isnan(ref)]))
+
+
+def test_unaligned_views_take_the_row_per_lane_kernel():
+    x = np.random.default_rng(6).standard_normal((9, 64)).astype(np.float32)
+    backing = torch.zeros(x.size + 1, device='cuda')
+    view = backing[1:].view(x.shape)
+    view.copy_(torch.from_numpy(x))
+    assert view.data_ptr() % 16 != 0
+    assert np.array_equal(row_scan.cumsum(view).cpu().numpy(), np.cumsum(x, axis=1, dtype=np.float32))
+
+
+def test_full_sizes_equal_the_generated_operators():
+    g = torch.Generator(device='cuda')
+    g.manual_seed(3)
+    xs = torch.randn((4096, 16384), device='cuda', generator=g)
+    assert torch.equal(row_scan.cumsum(xs), ovl.evaluate(cumsum(xs, axis=1)))
+    xp = 0.99 + 0.02 * torch.rand((4096, 16384), device='cuda', generator=g)
+    assert torch.equal(row_scan.cumprod(xp), ovl.evaluate(cumprod(xp, axis=1)))
+    xd = torch.randn((1024, 16384), device='cuda', generator=g, dtype=torch.float64)
+    assert torch.equal(row_scan.cumsum(xd), ovl.evaluate(cumsum(xd, axis=1)))
