@@ -845,6 +845,13 @@ def prebuild_all(cases=None, workers=8, with_oracle=True, force_benchmark=False)
         for name in FAST_FUSED_CASES:
             for op in _operators_of(CASE_BY_NAME[name].outputs(), 3):
                 variants.append((op, {'math': 'fast'}))
+        from tests import random_programs
+        for seed in random_programs.GPU_SEEDS:
+            program = random_programs.application(seed).expression_dag
+            ops[program.SerializeToString()] = program
+            oracle_ops[program.SerializeToString()] = program
+            variants.append((program, {'value_ranges': False}))
+            variants.append((program, {'math': 'fast'}))
         from tests import golden
         for _name, out, _expected, _sum, _atol in golden.known_answers():
             for op in _operators_of(all_outputs(out), 0):

@@ -1,0 +1,29 @@
+"""Random element-wise programs (tests/random_programs.py) through the HIP path, with and without the value-range
+pruning, against the CPU oracle: bit-exact apart from the sign and payload of NaN."""
+import numpy as np
+import pytest
+
+import opveclib_amd as ovl
+import oracle
+from opveclib_amd import runtime
+from tests import random_programs
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize('seed', random_programs.GPU_SEEDS)
+def test_random_program_equals_the_oracle(seed):
+    op = random_programs.application(seed)
+    outs = [op[0], op[1]]
+    ref = oracle.evaluate(outs)
+    for options in ({}, {'value_ranges': False}):
+        runtime.codegen_options = dict(options)
+        try:
+            got = ovl.evaluate(outs, opt_level=0)
+        finally:
+            runtime.codegen_options = {}
+        for k, (g, r) in enumerate(zip(got, ref)):
+            equal = ((g == r) & (np.signbit(g) == np.signbit(r))) | (np.isnan(g) & np.isnan(r))
+            assert equal.all(), 'seed %d %r output %d: %d elements differ' % (seed, options, k, int((~equal).sum()))
+    # the fast math mode evaluates the same program without error
+    ovl.evaluate(outs, opt_level=0, math_mode='fast')

@@ -388,3 +388,26 @@ def test_ranges_hold_for_every_value_a_worker_computes(math_mode):
                     raise AssertionError('%s, inputs %r: %s' % (name, feed, error))
                 total += machine.checked
     assert total > 100000
+
+
+def test_ranges_hold_on_random_programs():
+    """The same check on random programs (tests/random_programs.py): nested conditionals, comparisons against
+    constants, min / max, floor / ceil, square roots."""
+    from tests import random_programs
+    samples = [np.float32(s) for s in _sample_values()]
+    rng = np.random.default_rng(13)
+    total = decided = 0
+    for seed in range(60):
+        op = random_programs.application(seed).expression_dag
+        info = DagInfo(op)
+        known = ranges.analyse(info)
+        decided += sum(1 for n in info.nodes if known.constant(n.idx) is not None)
+        for s in samples[::2]:
+            feed = [s, samples[int(rng.integers(0, len(samples)))]]
+            machine = _Interpreter(info, known, feed)
+            try:
+                machine.run(info.tree)
+            except AssertionError as error:
+                raise AssertionError('seed %d, inputs %r: %s' % (seed, feed, error))
+            total += machine.checked
+    assert total > 50000 and decided > 50
