@@ -852,6 +852,13 @@ def prebuild_all(cases=None, workers=8, with_oracle=True, force_benchmark=False)
             oracle_ops[program.SerializeToString()] = program
             variants.append((program, {'value_ranges': False}))
             variants.append((program, {'math': 'fast'}))
+        for seed in random_programs.DAG_SEEDS:
+            outs = random_programs.random_dag(seed)
+            for level in (0, 3):
+                for op in _operators_of(outs, level):
+                    ops[op.SerializeToString()] = op
+            for op in _operators_of(outs, 0):
+                oracle_ops[op.SerializeToString()] = op
         from tests import golden
         for _name, out, _expected, _sum, _atol in golden.known_answers():
             for op in _operators_of(all_outputs(out), 0):

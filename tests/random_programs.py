@@ -82,3 +82,38 @@ def application(seed):
 
 
 GPU_SEEDS = list(range(16))
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# random DAGs of library operators (fusion)
+# ----------------------------------------------------------------------------------------------------------------------
+def random_dag(seed):
+    """Outputs of a random DAG of 3 to 9 element-wise library operators (cyclic shifts included) over three vectors."""
+    from opveclib_amd import stdops
+    from opveclib_amd.examples import expm1, log1p, shift_cyclic, absolute
+    from tests import cases
+    unary = [stdops.tanh, stdops.sigmoid, stdops.neg, lambda t: log1p(t)[0], lambda t: expm1(t)[0],
+             lambda t: absolute(t)[0], lambda t: shift_cyclic(t)[0]]
+    binary = [stdops.add, stdops.sub, stdops.mul, stdops.div]
+    rng = random.Random(seed)
+    nrng = np.random.default_rng(seed)
+    n = rng.choice([256, 1024, 4096])
+    leaves = [cases.special_values(nrng, (n,)) if rng.random() < 0.3 else nrng.uniform(-2, 2, n).astype(np.float32)
+              for _ in range(3)]
+    scalar = np.array([rng.choice([1.0001, 0.5, -2.0])], np.float32)
+    nodes = list(leaves)
+    for _ in range(rng.randint(3, 9)):
+        r = rng.random()
+        if r < 0.45:
+            nodes.append(rng.choice(unary)(rng.choice(nodes)))
+        elif r < 0.9:
+            nodes.append(rng.choice(binary)(rng.choice(nodes), rng.choice(nodes)))
+        else:
+            nodes.append(stdops.mul(rng.choice(nodes), scalar))
+    produced = nodes[3:]
+    count = rng.randint(1, min(3, len(produced)))
+    outs = [produced[-1]] + (rng.sample(produced[:-1], count - 1) if len(produced) > 1 else [])
+    return [o if not hasattr(o, 'output_types') else o[0] for o in outs]
+
+
+DAG_SEEDS = list(range(100, 112))

@@ -27,3 +27,17 @@ def test_random_program_equals_the_oracle(seed):
             assert equal.all(), 'seed %d %r output %d: %d elements differ' % (seed, options, k, int((~equal).sum()))
     # the fast math mode evaluates the same program without error
     ovl.evaluate(outs, opt_level=0, math_mode='fast')
+
+
+@pytest.mark.parametrize('seed', random_programs.DAG_SEEDS)
+def test_random_dag_fused_and_unfused_equal_the_oracle(seed):
+    outs = random_programs.random_dag(seed)
+    ref = oracle.evaluate(outs)
+    ref = ref if isinstance(ref, list) else [ref]
+    for opt_level in (0, 3):
+        got = ovl.evaluate(outs, opt_level=opt_level)
+        got = got if isinstance(got, list) else [got]
+        for k, (g, r) in enumerate(zip(got, ref)):
+            equal = ((g == r) & (np.signbit(g) == np.signbit(r))) | (np.isnan(g) & np.isnan(r))
+            assert equal.all(), 'seed %d opt_level %d output %d: %d elements differ' % (
+                seed, opt_level, k, int((~equal).sum()))
