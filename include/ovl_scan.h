@@ -24,7 +24,7 @@
  * Conventions: tensor memory belongs to the caller and must be device accessible; `out` may not overlap `x`; the
  * functions enqueue one kernel on `hip_stream` (a hipStream_t; NULL is the default stream), return without
  * synchronising and allocate nothing.  They return an ovl_status (ovl_launch.h): OVL_EINVAL for null pointers, zero
- * sizes or rows * cols of 2^32 or more, OVL_EHIP for a HIP error (text from ovl_scan_last_error).
+ * sizes, rows * cols of 2^32 or more, or more than 2^32 - 257 rows, OVL_EHIP for a HIP error (text from ovl_scan_last_error).
  */
 #ifndef OVL_SCAN_H_
 #define OVL_SCAN_H_

@@ -16,6 +16,7 @@
 #include <string>
 
 #include "ovl_device.h"
+#include "ovl_index_div.h"
 #include "ovl_lstm.h"
 
 // ovl_device.h carries the status codes generated operators return; this one (ovl_status in ovl_launch.h) is the
@@ -63,27 +64,6 @@ __device__ __forceinline__ float sig_grad_(float x, float e) {
     return (x > -50.0f && x < 50.0f) ? q : 0.0f;
 }
 
-// Division of a 32-bit index by a divisor fixed per launch (multiply-high and shifts; Granlund & Montgomery).
-struct index_divisor {
-    uint32_t divisor, magic, shift1, shift2;
-};
-
-__device__ __forceinline__ uint32_t divide(uint32_t n, const index_divisor& d) {
-    const uint32_t t = __umulhi(d.magic, n);
-    return (t + ((n - t) >> d.shift1)) >> d.shift2;
-}
-
-index_divisor make_divisor(uint32_t divisor) {
-    uint32_t log2_ceil = 0;
-    while ((1ull << log2_ceil) < divisor) ++log2_ceil;
-    index_divisor d;
-    d.divisor = divisor;
-    d.magic = (uint32_t)(((1ull << 32) * ((1ull << log2_ceil) - divisor)) / divisor + 1);
-    d.shift1 = log2_ceil < 1 ? log2_ceil : 1;
-    d.shift2 = log2_ceil > 1 ? log2_ceil - 1 : 0;
-    return d;
-}
-
 template <typename V>
 __device__ __forceinline__ V load_nt(const float* p) {
     return __builtin_nontemporal_load(reinterpret_cast<const V*>(p));
@@ -96,8 +76,10 @@ lstm_forward_kernel(const float* __restrict__ concat, const float* __restrict__ 
                     float* __restrict__ new_c, float* __restrict__ new_h) {
     typedef typename vec_of<VEC>::type vec;
     OVL_DECLARE_MATH_TABLES();
+    // v + stride may pass 2^32 (scalar variant on more than 2^32 - 2^28 elements): step only while it stays in range
     const uint32_t stride = gridDim.x * BLOCK;
-    for (uint32_t v = blockIdx.x * BLOCK + threadIdx.x; v < num_vectors; v += stride) {
+    for (uint32_t v = blockIdx.x * BLOCK + threadIdx.x; v < num_vectors;
+         v = (num_vectors - v > stride) ? v + stride : num_vectors) {
         const uint32_t row = divide(v, vectors_per_row);
         const uint32_t elem = (v - row * vectors_per_row.divisor) * VEC;
         const float* gates = concat + (uint64_t)row * 4u * units + elem;
@@ -133,8 +115,10 @@ lstm_backward_kernel(const float* __restrict__ concat, const float* __restrict__
                      float* __restrict__ d_concat, float* __restrict__ d_c) {
     typedef typename vec_of<VEC>::type vec;
     OVL_DECLARE_MATH_TABLES();
+    // v + stride may pass 2^32 (scalar variant on more than 2^32 - 2^28 elements): step only while it stays in range
     const uint32_t stride = gridDim.x * BLOCK;
-    for (uint32_t v = blockIdx.x * BLOCK + threadIdx.x; v < num_vectors; v += stride) {
+    for (uint32_t v = blockIdx.x * BLOCK + threadIdx.x; v < num_vectors;
+         v = (num_vectors - v > stride) ? v + stride : num_vectors) {
         const uint32_t row = divide(v, vectors_per_row);
         const uint32_t elem = (v - row * vectors_per_row.divisor) * VEC;
         const uint64_t gate_at = (uint64_t)row * 4u * units + elem;
@@ -211,8 +195,8 @@ int ovl_lstm_forward(const float* concat, const float* c, float forget_bias, uin
     const uint32_t vec = wide ? 4u : 1u;
     const index_divisor per_row = make_divisor(units / vec);
     const uint32_t total = batch * per_row.divisor;
-    const uint32_t blocks = (total + BLOCK - 1) / BLOCK;
-    const dim3 grid(blocks < MAX_GRID ? blocks : MAX_GRID), block(BLOCK);
+    const uint64_t blocks = ((uint64_t)total + BLOCK - 1) / BLOCK;
+    const dim3 grid(blocks < MAX_GRID ? (uint32_t)blocks : MAX_GRID), block(BLOCK);
 #define OVL_LSTM_LAUNCH(FAST, VEC)                                                                           \
     hipLaunchKernelGGL((lstm_forward_kernel<FAST, VEC>), grid, block, 0, stream, concat, c, forget_bias,    \
                        units, per_row, total, new_c, new_h)
@@ -236,8 +220,8 @@ int ovl_lstm_backward(const float* concat, const float* c, const float* d_new_c,
     const uint32_t vec = wide ? 4u : 1u;
     const index_divisor per_row = make_divisor(units / vec);
     const uint32_t total = batch * per_row.divisor;
-    const uint32_t blocks = (total + BLOCK - 1) / BLOCK;
-    const dim3 grid(blocks < MAX_GRID ? blocks : MAX_GRID), block(BLOCK);
+    const uint64_t blocks = ((uint64_t)total + BLOCK - 1) / BLOCK;
+    const dim3 grid(blocks < MAX_GRID ? (uint32_t)blocks : MAX_GRID), block(BLOCK);
 #define OVL_LSTM_LAUNCH(FAST, VEC)                                                                           \
     hipLaunchKernelGGL((lstm_backward_kernel<FAST, VEC>), grid, block, 0, stream, concat, c, d_new_c,       \
                        d_new_h, forget_bias, units, per_row, total, d_concat, d_c)

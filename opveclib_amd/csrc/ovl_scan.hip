@@ -140,7 +140,7 @@ skewed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, 
 template <typename T, typename OP>
 __global__ void __launch_bounds__(BLOCK)
 row_per_lane_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, uint32_t cols) {
-    const uint32_t row = blockIdx.x * BLOCK + threadIdx.x;
+    const uint32_t row = blockIdx.x * BLOCK + threadIdx.x;     // the grid has at most 2^24 - 1 workgroups
     if (row >= rows) return;
     const T* in_row = x + (uint64_t)row * cols;
     T* out_row = out + (uint64_t)row * cols;
@@ -172,6 +172,9 @@ int scan(const char* who, const T* x, uint32_t rows, uint32_t cols, T* out, void
         else
             hipLaunchKernelGGL((skewed_scan_kernel<T, OP, VEC, WIDTH, 1>), grid, block, 0, stream, x, out, rows, cols);
     } else {
+        // (a launch has fewer than 2^32 threads)
+        if (rows > 0xffffffffu - BLOCK)
+            return fail(OVL_EINVAL, std::string(who) + ": more than 2^32 - 257 rows");
         const dim3 grid((rows + BLOCK - 1) / BLOCK);
         hipLaunchKernelGGL((row_per_lane_scan_kernel<T, OP>), grid, block, 0, stream, x, out, rows, cols);
     }

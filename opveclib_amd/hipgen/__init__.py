@@ -26,7 +26,7 @@ from . import tile_kernel
 from . import rowscan_kernel
 
 #: bump when generated code changes for an unchanged DAG, so cached binaries are not reused
-CODEGEN_VERSION = 22
+CODEGEN_VERSION = 23
 
 
 
@@ -63,7 +63,8 @@ def generate(expression_dag, function_name, options=None):
         map template with that vector width; ``scan_depth`` / ``scan_sets`` / ``scan_width`` set the request burst (groups), the
         number of register sets and the 128-bit vectors per lane and phase of the lane-skewed scan; ``math``: 'exact'
         or 'fast'; ``if_conversion`` / ``value_ranges``: False switches that transformation off; ``scan_rows`` / ``scan_chunk`` the LDS tile of the row scan; ``nt`` /
-        ``scan_nt`` which vector accesses carry the non-temporal hint ('l' loads, 's' stores, 'ls', '')
+        ``scan_nt`` which vector accesses carry the non-temporal hint ('l' loads, 's' stores, 'ls', ''); ``grid_cap``
+        the largest grid of the map and transpose templates (their kernels then stride over the rest)
     :return: a :class:`GeneratedOperator`
     """
     options = options or {}
@@ -89,7 +90,8 @@ def generate(expression_dag, function_name, options=None):
         kernel_src, launch = tile_kernel.generate(info, kernel_name, options.get('tile_i'), options.get('tile_j'),
                                                   options.get('nt', 'ls'))
     else:
-        kernel_src, launch = map_kernel.generate(info, kernel_name, options.get('vec'), options.get('nt'))
+        kernel_src, launch = map_kernel.generate(info, kernel_name, options.get('vec'), options.get('nt'),
+                                                 options.get('grid_cap'))
 
     num_inputs = len(info.inputs)
     num_outputs = len(info.outputs)
@@ -114,8 +116,13 @@ def generate(expression_dag, function_name, options=None):
                     kind, i, need - 1))
             const = 'const ' if kind == 'in' else ''
             call_args.append('static_cast<%s%s*>(%s[%d].data)' % (const, CTYPE[node.dtype], kind, i))
-    grid_cap = options.get('grid_cap') or MAX_GRID
-    src.append('    uint32_t grid = %du;' % min(launch['blocks_needed'], grid_cap))
+    grid = launch['blocks_needed']
+    if launch['template'] in ('map', 'transpose'):
+        # these kernels stride over what the grid does not cover
+        grid = min(grid, options.get('grid_cap') or MAX_GRID, MAX_GRID)
+    elif grid > MAX_GRID:
+        raise ValueError('%d workgroups: the %s template launches at most %d' % (grid, launch['template'], MAX_GRID))
+    src.append('    uint32_t grid = %du;' % grid)
     src.append('    hipLaunchKernelGGL(%s, dim3(grid), dim3(%du), 0, static_cast<hipStream_t>(stream),' % (
         kernel_name, launch['block']))
     src.append('                       ' + ', '.join(call_args) + ');')

@@ -24,7 +24,9 @@ from .analysis import ITEMSIZE
 from .body import BodyEmitter, CTYPE
 
 BLOCK = 256
-MAX_GRID = 1 << 24          # largest grid the generated entry points launch
+# largest grid the generated entry points launch: 2^24 - 1 workgroups of 256 threads keep the number of threads of a
+# launch, and with it gridDim.x * 256 inside the kernels, below 2^32
+MAX_GRID = (1 << 24) - 1
 
 
 class Access(object):
@@ -99,7 +101,7 @@ def contiguous_unaligned(info, node, tensor, aff, vec):
     return not _is_vector_access(info, node, tensor, aff, vec)
 
 
-def generate(info, kernel_name, vec=None, nt=None):
+def generate(info, kernel_name, vec=None, nt=None, grid_cap=None):
     """
     :return: (kernel source text, launch description dict) for the map template.
     """
@@ -183,10 +185,12 @@ def generate(info, kernel_name, vec=None, nt=None):
     src.append('extern "C" __global__ void __launch_bounds__(%d)' % BLOCK)
     src.append(kernel_name + '(' + ', '.join(args) + ') {')
     blocks_needed = (num_vectors + BLOCK - 1) // BLOCK
-    # Kernels that use the LDS math tables and whose grid covers every vector run one vector per thread without a
-    # loop: the thread requests its operands first and copies the tables (with the barrier that implies) while
-    # they are in flight, instead of waiting for the tables before the first request.
-    single_pass = info.uses_math_tables() and blocks_needed <= MAX_GRID
+    # When the grid covers every vector (always, unless the workgroup has more than 2^32 - 256 workers at VEC = 1 or
+    # the caller caps the grid) a thread runs one vector without a loop.  Kernels that use the LDS math tables then
+    # request their operands first and copy the tables (with the barrier that implies) while they are in flight,
+    # instead of waiting for the tables before the first request.
+    covers = blocks_needed <= min(grid_cap or MAX_GRID, MAX_GRID)
+    single_pass = info.uses_math_tables() and covers
     src.append('    const uint32_t num_vectors = %du;' % num_vectors)
     if single_pass:
         src.append('    const uint32_t v_raw = blockIdx.x * %du + threadIdx.x;' % BLOCK)
@@ -194,11 +198,16 @@ def generate(info, kernel_name, vec=None, nt=None):
         src.append('    // idle threads of the last workgroup request vector 0 and store nothing')
         src.append('    const uint32_t v = active ? v_raw : 0u;')
         src.append('    {')
+    elif covers:
+        src.append('    const uint32_t v = blockIdx.x * %du + threadIdx.x;' % BLOCK)
+        src.append('    if (v < num_vectors) {')
     else:
         if info.uses_math_tables():
             src.append('    OVL_DECLARE_MATH_TABLES();')
+        src.append('    // v + stride may pass 2^32: the step is taken only while it stays below num_vectors')
         src.append('    const uint32_t stride = gridDim.x * %du;' % BLOCK)
-        src.append('    for (uint32_t v = blockIdx.x * %du + threadIdx.x; v < num_vectors; v += stride) {' % BLOCK)
+        src.append('    for (uint32_t v = blockIdx.x * %du + threadIdx.x; v < num_vectors;' % BLOCK)
+        src.append('         v = (num_vectors - v > stride) ? v + stride : num_vectors) {')
     src.append('        const uint32_t worker0 = v * %du;' % vec)
     # position of the first of this thread's workers
     block = 1

@@ -23,7 +23,7 @@ EXPORTED_SYMBOLS = ('ovl_lstm_forward', 'ovl_lstm_backward', 'ovl_lstm_last_erro
 def build(force=False):
     """Compile the library with hipcc next to its source (same flags as generated operators); returns its path."""
     from .compiler import HIPCC_FLAGS
-    headers = [os.path.join(local.csrc_directory, n) for n in ('ovl_device.h', 'ovl_math.h', 'ovl_fast_math.h')]
+    headers = [os.path.join(local.csrc_directory, n) for n in ('ovl_device.h', 'ovl_math.h', 'ovl_fast_math.h', 'ovl_index_div.h')]
     newest = max(os.path.getmtime(p) for p in [source_path] + headers)
     if not force and os.path.exists(library_path) and os.path.getmtime(library_path) >= newest:
         return library_path

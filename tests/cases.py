@@ -796,6 +796,12 @@ TEMPLATE_VARIANTS = [
     ('c2_chain', {'value_ranges': False}),
     ('c2_chain_special', {'value_ranges': False}),
     ('bounded_mix', {'value_ranges': False}),
+    # grids smaller than the work: the map and transpose kernels stride over the rest
+    ('c2_chain', {'grid_cap': 3}),
+    ('odd_sizes', {'grid_cap': 1}),
+    ('pad_crop', {'grid_cap': 2}),
+    ('c5_variants', {'grid_cap': 2}),
+    ('c5_variants', {'template': 'map', 'grid_cap': 5}),
 ]
 
 
@@ -869,6 +875,9 @@ def prebuild_all(cases=None, workers=8, with_oracle=True, force_benchmark=False)
                 ops[op.SerializeToString()] = op
         for op in _operators_of(graph_capture_single(np.zeros(4096, np.float32)), 3):
             variants.append((op, {'math': 'fast'}))
+        from tests import large_cases
+        for op in large_cases.operators_to_build():
+            ops[op.SerializeToString()] = op
         from tests import autograd_cases
         for outs in autograd_cases.graphs_to_build():
             for level in (0, 3):

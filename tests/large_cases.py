@@ -1,0 +1,71 @@
+"""
+Operators at the largest sizes the path supports: workgroups just below 2^32 workers (positions are 32-bit, as in the
+reference: opveclib/expression.py:582-608), tensors beyond 2^31 and 2^32 elements (flat indices are 64-bit:
+expression.py:859-973).  Data-movement and integer operators only, so that PyTorch on the GPU is an independent,
+bit-exact reference at sizes the CPU oracle would need minutes for.
+
+`cases(make)` yields (name, operator output, reference function); `make(shape, dtype)` supplies the tensors: shape-only
+placeholders when the kernels are compiled ahead of time, device tensors in the GPU test.
+"""
+import numpy as np
+
+import opveclib_amd as ovl
+from opveclib_amd import stdops
+from opveclib_amd.examples import shift_cyclic, cumsum, gather_transpose
+
+
+@ovl.operator()
+def reverse(x):
+    """out[n - 1 - p] = x[p]: nothing to vectorise on 1-byte elements, one worker per thread."""
+    pos = ovl.position_in(x.shape)
+    out = ovl.output_like(x)
+    out[(x.shape[0] - 1) - pos[0]] = x[pos]
+    return out
+
+
+def placeholder(shape, dtype):
+    """An array of the given shape that owns one element (every stride is zero): enough to trace an operator."""
+    shape = shape if isinstance(shape, tuple) else (shape,)
+    return np.lib.stride_tricks.as_strided(np.zeros(1, dtype), shape=shape, strides=(0,) * len(shape))
+
+
+def cases(make):
+    import torch
+
+    n = 2 ** 32 - 3       # 2^24 workgroups of 256 one-worker threads would be 2^32 threads: the kernel strides
+    x = make(n, np.uint8)
+    yield 'reverse uint8 [2^32 - 3]', reverse(x), lambda: torch.flip(x, [0])
+
+    n = 2 ** 32 - 256     # sixteen workers per thread
+    a, b = make(n, np.uint8), make(n, np.uint8)
+    yield 'add uint8 [2^32 - 256]', stdops.add(a, b), lambda: a + b
+
+    n = 2 ** 31 + 2 ** 20     # byte offsets beyond 2^33
+    a, b = make(n, np.float32), make(n, np.float32)
+    yield 'add float32 [2^31 + 2^20]', stdops.add(a, b), lambda: a + b
+
+    n = 2 ** 31 + 4
+    a = make(n, np.float32)
+    yield 'shift_cyclic float32 [2^31 + 4]', shift_cyclic(a), lambda: torch.roll(a, 1)
+
+    a = make((131088, 32832), np.int32)     # 2^32 + 2^23.3 elements, 131088 workers
+    yield 'cumsum int32 [131088, 32832]', cumsum(a, axis=1), lambda: torch.cumsum(a, 1, dtype=torch.int32)
+
+    rows, cols = 65536, 32768 + 256         # 2^31 + 2^24 workers, transposed store
+    a, flat = make((rows, cols), np.float32), make(rows * cols, np.float32)
+
+    def gathered_and_transposed():
+        out = torch.empty((cols, rows), dtype=torch.float32, device=a.device)
+        j = torch.arange(cols, device=a.device, dtype=torch.int64)[None, :]
+        for r0 in range(0, rows, 4096):
+            i = torch.arange(r0, r0 + 4096, device=a.device, dtype=torch.int64)[:, None]
+            index = ((i * 7919 + j) & 0xffffffff) % (rows * cols)
+            out[:, r0:r0 + 4096] = (0.5 * a[r0:r0 + 4096] + flat[index]).T
+        return out
+    yield 'gather_transpose float32 [65536, 33024]', gather_transpose(a, flat, alpha=0.5, stride=7919), \
+        gathered_and_transposed
+
+
+def operators_to_build():
+    for _name, out, _ref in cases(placeholder):
+        yield (out if hasattr(out, 'parent') else out[0]).parent.expression_dag

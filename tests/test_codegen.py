@@ -213,6 +213,28 @@ def test_workgroups_beyond_32_bit_positions_are_refused():
         hipgen.generate(fill(np.zeros(4, np.float32)).expression_dag, 'f' + '6' * 56)
 
 
+def test_largest_workgroups_launch_fewer_than_2_to_32_threads_and_step_without_wrapping():
+    """A scalar map over 2^32 - 3 workers: 2^24 workgroups of 256 threads would make gridDim.x * 256 wrap to zero (a
+    stride of zero never ends), and `v += stride` would wrap for the threads that take a second step."""
+    @ovl.operator()
+    def fill(shape_like):
+        pos = ovl.position_in([(1 << 32) - 3])
+        out = ovl.output([7], ovl.float32)
+        out[pos[0] % 7] = 1
+        return out
+    generated = hipgen.generate(fill(np.zeros(4, np.float32)).expression_dag, 'f' + '7' * 56)
+    assert generated.launch['vec'] == 1 and generated.launch['blocks_needed'] == 1 << 24
+    assert 'uint32_t grid = %du;' % ((1 << 24) - 1) in generated.source
+    assert 'v = (num_vectors - v > stride) ? v + stride : num_vectors' in generated.source
+    assert 'v += stride' not in generated.source
+
+    # a grid that covers the work needs no loop at all; a capped grid strides
+    small = stdops.add(np.zeros(4096, np.float32), np.zeros(4096, np.float32)).expression_dag
+    assert 'stride' not in hipgen.generate(small, 'f' + '8' * 56).source
+    capped = hipgen.generate(small, 'f' + '8' * 56, {'grid_cap': 1})
+    assert 'uint32_t grid = 1u;' in capped.source and 'stride' in capped.source
+
+
 def test_missing_operators_of_a_dag_are_built_side_by_side(tmp_path, monkeypatch):
     """Cold start: every operator of a DAG without a library is generated and compiled before the first launch."""
     import os
