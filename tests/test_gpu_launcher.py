@@ -148,3 +148,40 @@ def test_hand_written_library_through_the_c_abi():
     with pytest.raises(launcher.LauncherError) as err:
         launcher.OperatorLibrary(path, 'no_such_entry_point')
     assert err.value.code == 3
+
+
+def test_concurrent_evaluation_from_several_threads_and_streams():
+    """Four Python threads trace, load and launch different operator DAGs at the same time, each on a HIP stream of
+    its own (default priority), ten rounds each: every result equals the oracle's (computed beforehand on the CPU)."""
+    import threading
+    import torch
+    import oracle
+    from tests import cases
+    names = ['c2_chain', 'c4_lstm_grad', 'c5_variants', 'c1_shift_expm1_log1p']
+    expected = {}
+    for name in names:
+        expected[name] = oracle.profile(cases.CASE_BY_NAME[name].outputs(), 1, 0)[0]
+    failures = []
+    start = threading.Barrier(len(names))
+
+    def worker(name):
+        try:
+            case = cases.CASE_BY_NAME[name]
+            stream = torch.cuda.Stream()
+            start.wait(timeout=60)
+            for _ in range(10):
+                with torch.cuda.stream(stream):
+                    got = ovl.evaluate(case.outputs(), opt_level=3)
+                got = got if isinstance(got, list) else [got]
+                for n, (g, r) in enumerate(zip(got, expected[name])):
+                    cases.assert_matches(case, g, r, '%s output %d' % (name, n))
+        except Exception as exception:      # reported by the main thread
+            failures.append((name, repr(exception)))
+
+    threads = [threading.Thread(target=worker, args=(name,)) for name in names]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=120)
+    assert not any(t.is_alive() for t in threads)
+    assert failures == []
