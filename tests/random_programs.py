@@ -117,3 +117,143 @@ def random_dag(seed):
 
 
 DAG_SEEDS = list(range(100, 112))
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# Random index programs: gathers through computed indices, guarded neighbour reads, stores through one-to-one index maps.
+# They exercise what the code generator decides from index expressions: which accesses become vector accesses, which
+# loads may move ahead of the conditions that guard them, which modulo operations cannot wrap, which template runs.
+# ----------------------------------------------------------------------------------------------------------------------
+INDEX_DTYPES = [np.float32, np.float32, np.float64, np.int32, np.uint8, np.int16]
+LAST_DIMS = [4, 8, 12, 16, 20, 32, 64, 100, 7, 33, 128, 256]
+OUTER_DIMS = [1, 2, 3, 5, 8, 16, 17]
+MULTIPLIERS = [1, 2, 3, 4, 5, 7, 16, 31, 7919, 65537, 2 ** 31 + 1, 2 ** 32 - 1]
+
+
+def _coprime(rng, n):
+    import math
+    while True:
+        a = rng.choice([1, 3, 5, 7, 11, 13, 7919, n - 1 if n > 1 else 1, n + 1])
+        if math.gcd(a, n) == 1:
+            return a
+
+
+def index_program_shapes(seed):
+    """(workgroup shape, dtype, shapes of the gathered operands) of the program of ``seed``."""
+    rng = random.Random(seed * 7919 + 1)
+    rank = rng.choice([1, 2, 2, 3])
+    shape = [rng.choice(OUTER_DIMS) for _ in range(rank - 1)] + [rng.choice(LAST_DIMS)]
+    dtype = rng.choice(INDEX_DTYPES)
+    gathered = []
+    for _ in range(2):
+        g_rank = rng.choice([1, 1, 2, 3])
+        gathered.append([rng.choice([1, 2, 3, 5, 8, 16, 17, 64, 100, 257]) for _ in range(g_rank)])
+    return shape, dtype, gathered
+
+
+def make_index_operator(seed):
+    shape, _, _ = index_program_shapes(seed)
+    rank = len(shape)
+
+    @ovl.operator()
+    def index_program(x, g0, g1):
+        rng = random.Random(seed)
+        pos = ovl.position_in(x.shape)
+        p = [pos[k] for k in range(rank)]
+
+        def component(n):
+            """An index expression with values in [0, n)."""
+            form = rng.randrange(9)
+            k = rng.randrange(rank)
+            if form == 0:
+                return p[k] % n
+            if form == 1:
+                return (p[k] + rng.choice([1, 2, 3, n - 1, n, 1000])) % n
+            if form == 2:
+                return (p[k] * rng.choice(MULTIPLIERS) + rng.choice([0, 1, 5, 2 ** 31])) % n
+            if form == 3:
+                j = rng.randrange(rank)
+                return (p[k] * rng.choice(MULTIPLIERS) + p[j] * rng.choice([1, 2, 3])) % n
+            if form == 4:
+                return (n - 1) - (p[k] % n)
+            if form == 5:
+                return (p[k] / rng.choice([1, 2, 3, 4, 7])) % n
+            if form == 6:
+                return rng.randrange(n)
+            if form == 7:
+                return ovl.minimum(p[k], n - 1)
+            return (p[k] % rng.choice([2, 3, 4, 8])) % n
+
+        def gather(g):
+            return g[[component(n) for n in g.shape]]
+
+        value = x[pos] + gather(g0)
+        if rng.random() < 0.7:
+            value = value + gather(g1)
+
+        # neighbour reads along one dimension, guarded against the ends of the tensor
+        for _ in range(rng.randint(0, 2)):
+            k = rng.randrange(rank)
+            n = x.shape[k]
+            delta = rng.choice([1, 1, 2, 4])
+            neighbour = ovl.variable(0, x.dtype)
+            forward = rng.random() < 0.5
+            where = list(p)
+            if forward:
+                where[k] = p[k] + delta
+                with ovl.if_(p[k] + delta < n):
+                    neighbour <<= x[where]
+                if rng.random() < 0.5:
+                    with ovl.else_():
+                        neighbour <<= x[pos]
+            else:
+                where[k] = p[k] - delta
+                with ovl.if_(p[k] >= delta):
+                    neighbour <<= x[where]
+            value = value + neighbour
+
+        # stores: one output at the worker's position, one through a one-to-one map of every dimension
+        out0 = ovl.output_like(x)
+        out0[pos] = value
+        permuted = list(range(rank))
+        if rank >= 2 and rng.random() < 0.5:
+            a, b = rng.sample(range(rank), 2)
+            permuted[a], permuted[b] = permuted[b], permuted[a]
+        transposition = rank == 2 and rng.random() < 0.3
+        if transposition:
+            permuted = [1, 0]
+        target = []
+        for k in permuted:
+            n = x.shape[k]
+            form = 0 if transposition else rng.randrange(4)
+            if form == 0:
+                target.append(p[k])
+            elif form == 1:
+                target.append((p[k] + rng.choice([1, 2, n - 1, 5])) % n)
+            elif form == 2:
+                target.append((n - 1) - p[k])
+            else:
+                target.append((p[k] * _coprime(rng, n) + rng.choice([0, 1, 3])) % n)
+        out1 = ovl.output([x.shape[k] for k in permuted], x.dtype)
+        out1[target] = value + x[pos]
+        return out0, out1
+    return index_program
+
+
+def index_inputs(seed):
+    shape, dtype, gathered = index_program_shapes(seed)
+    rng = np.random.default_rng(seed)
+
+    def data(s):
+        if np.dtype(dtype).kind == 'f':
+            return rng.standard_normal(s).astype(dtype)
+        return rng.integers(0, 50, s).astype(dtype)
+    return [data(shape)] + [data(g) for g in gathered]
+
+
+def index_application(seed):
+    """The index program of ``seed`` applied to its inputs (an operator with two outputs)."""
+    return make_index_operator(seed)(*index_inputs(seed))
+
+
+INDEX_SEEDS = range(200, 224)

@@ -41,3 +41,19 @@ def test_random_dag_fused_and_unfused_equal_the_oracle(seed):
             equal = ((g == r) & (np.signbit(g) == np.signbit(r))) | (np.isnan(g) & np.isnan(r))
             assert equal.all(), 'seed %d opt_level %d output %d: %d elements differ' % (
                 seed, opt_level, k, int((~equal).sum()))
+
+
+@pytest.mark.parametrize('seed', random_programs.INDEX_SEEDS)
+def test_random_index_program_equals_the_oracle(seed):
+    """Gathers through computed indices, guarded neighbour reads and stores through one-to-one index maps: bit-exact
+    (unwritten elements would show as the 0xFE fill)."""
+    op = random_programs.index_application(seed)
+    outs = [op[0], op[1]]
+    ref = oracle.evaluate(outs)
+    runtime.poison_outputs = True
+    try:
+        got = ovl.evaluate(outs, opt_level=3)
+    finally:
+        runtime.poison_outputs = False
+    for k, (g, r) in enumerate(zip(got, ref)):
+        assert g.dtype == r.dtype and g.shape == r.shape and np.array_equal(g, r), 'seed %d output %d' % (seed, k)

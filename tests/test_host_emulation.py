@@ -1,0 +1,111 @@
+"""
+The generated HIP sources on the CPU: every operator source the code generator emits for the parity cases (all four
+kernel templates, fused and unfused, plus the forced template variants and the random programs) is compiled as plain
+C++ against tests/native/host_emulation/ovl_device.h, run with one host thread per GPU thread under AddressSanitizer
+on buffers of exactly the tensors' sizes, and compared bit for bit with the oracle.  This checks, without a GPU, the
+text the GPU compiles: index arithmetic, vector accesses, loads moved ahead of conditions, LDS tiles and barriers,
+lane-to-lane moves, and that no access leaves its tensor.  (What only the device can show - its math instructions,
+memory model, the lockstep of the 64 lanes of a wavefront, timing - stays with the `gpu` tests.)  The 'fast' math mode is built on device instructions and is
+not emulated.
+"""
+import os
+from concurrent.futures import ThreadPoolExecutor
+
+import numpy as np
+import pytest
+
+import oracle
+from tests import cases, host_emulation, random_programs
+
+pytestmark = pytest.mark.skipif(not os.path.exists(host_emulation.CLANG), reason='needs the ROCm clang++ as host compiler')
+
+WORKERS = min(8, os.cpu_count() or 1)
+
+
+def _same(got, ref):
+    return len(got) == len(ref) and all(
+        g.dtype == r.dtype and g.shape == r.shape and np.array_equal(g, r, equal_nan=(r.dtype.kind == 'f'))
+        for g, r in zip(got, ref))
+
+
+def _check(job):
+    """job = (label, outputs, opt level, code generator options); returns the label when something is wrong."""
+    label, outs, level, options = job
+    try:
+        ref = oracle.profile(outs, 1, 0)[0]
+        got = host_emulation.evaluate(outs, level, options)
+        return None if _same(got, ref) else label + ': differs from the oracle'
+    except Exception as exception:
+        return label + ': ' + str(exception)[-1500:]
+
+
+def _run_all(jobs):
+    with ThreadPoolExecutor(WORKERS) as pool:
+        return [problem for problem in pool.map(_check, jobs) if problem]
+
+
+def test_an_access_outside_a_tensor_ends_the_run():
+    """Control: an operator that reads one element past its input is reported, not silently accepted."""
+    source = r'''
+#include "ovl_device.h"
+extern "C" __global__ void __launch_bounds__(256) k(const float* __restrict__ in0, float* __restrict__ out0, uint32_t n, uint32_t off) {
+    const uint32_t v = blockIdx.x * 256u + threadIdx.x;
+    if (v < n) out0[v] = in0[v + off];
+}
+extern "C" int beyond(const ovl_tensor* in, uint32_t n_in, ovl_tensor* out, uint32_t n_out, void* stream) {
+    hipLaunchKernelGGL(k, dim3(2u), dim3(256u), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const float*>(in[0].data), static_cast<float*>(out[0].data), 300u, 1u);
+    return OVL_OK;
+}
+extern "C" int within(const ovl_tensor* in, uint32_t n_in, ovl_tensor* out, uint32_t n_out, void* stream) {
+    hipLaunchKernelGGL(k, dim3(2u), dim3(256u), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const float*>(in[0].data), static_cast<float*>(out[0].data), 300u, 0u);
+    return OVL_OK;
+}
+'''
+    x = np.arange(300, dtype=np.float32)
+    types = [(1, np.float32, [300])]
+    good = host_emulation.run_program(host_emulation.build_source(source, 'within'), [x], types, types)
+    assert np.array_equal(good[0], x)
+    with pytest.raises(host_emulation.EmulationError) as failure:
+        host_emulation.run_program(host_emulation.build_source(source, 'beyond'), [x], types, types)
+    assert 'AddressSanitizer' in str(failure.value) and 'heap-buffer-overflow' in str(failure.value)
+
+
+def test_every_parity_case_emulated_on_the_host_equals_the_oracle():
+    jobs = []
+    for case in cases.CASES:
+        outs = case.outputs()
+        for level in (0, 3):
+            jobs.append(('%s opt_level %d' % (case.name, level), outs, level, None))
+    assert _run_all(jobs) == []
+
+
+def test_forced_templates_emulated_on_the_host_equal_the_oracle():
+    jobs = []
+    for name, options in cases.TEMPLATE_VARIANTS:
+        if options.get('template') == 'rowscan':
+            # The LDS row scan lets the surplus lanes of its scanning wavefront shadow the last row of the tile: they
+            # read, compute and write the same LDS words as the row's owner, instruction by instruction.  That is
+            # harmless only because the 64 lanes of a wavefront run in lockstep (all reads of an instruction precede
+            # the writes of the next), which independent host threads do not model.
+            continue
+        jobs.append(('%s %r' % (name, options), cases.CASE_BY_NAME[name].outputs(), 3, options))
+    assert _run_all(jobs) == []
+
+
+def test_random_programs_emulated_on_the_host_equal_the_oracle():
+    jobs = []
+    for seed in random_programs.INDEX_SEEDS:
+        op = random_programs.index_application(seed)
+        jobs.append(('index program %d' % seed, [op[0], op[1]], 3, None))
+    for seed in random_programs.GPU_SEEDS:
+        op = random_programs.application(seed)
+        jobs.append(('element-wise program %d' % seed, [op[0], op[1]], 3, None))
+        jobs.append(('element-wise program %d without value ranges' % seed, [op[0], op[1]], 3,
+                     {'value_ranges': False}))
+    for seed in random_programs.DAG_SEEDS:
+        outs = random_programs.random_dag(seed)
+        for level in (0, 3):
+            jobs.append(('operator DAG %d opt_level %d' % (seed, level), outs, level, None))
+    assert _run_all(jobs) == []
