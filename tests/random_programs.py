@@ -257,3 +257,90 @@ def index_application(seed):
 
 
 INDEX_SEEDS = range(200, 224)
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# Random scan programs: one worker per row walks the last axis with loop-carried state.  The scan templates find the
+# carried state in the DAG, so the body can be any straight-line update: one or two state variables, sums, products,
+# running extrema, decayed sums, integer and floating point types; row lengths that do and do not fit the lane-skewed
+# template (a multiple of 16 vectors).
+# ----------------------------------------------------------------------------------------------------------------------
+SCAN_DTYPES = [np.float32, np.float32, np.float64, np.int32, np.int64, np.int16]
+SCAN_LENGTHS = [64, 128, 192, 256, 320, 512, 1024, 32, 96, 100, 7, 2, 130]
+SCAN_ROWS = [[1], [3], [4], [5], [16], [17], [67], [2, 3], [4, 9], [2, 2, 5]]
+
+
+def scan_program_shape(seed):
+    rng = random.Random(seed * 104729 + 7)
+    return rng.choice(SCAN_ROWS) + [rng.choice(SCAN_LENGTHS)], rng.choice(SCAN_DTYPES)
+
+
+def make_scan_operator(seed):
+    shape, dtype = scan_program_shape(seed)
+    floating = np.dtype(dtype).kind == 'f'
+
+    @ovl.operator()
+    def scan_program(x):
+        rng = random.Random(seed)
+        length = x.shape[-1]
+        pos = ovl.position_in(x.shape[:-1])
+        out = ovl.output_like(x)
+
+        def at(i):
+            return [pos[k] for k in range(x.rank - 1)] + [i]
+
+        def update(state, other, element):
+            form = rng.randrange(8)
+            if form == 0:
+                return state + element
+            if form == 1:
+                return state * element if floating else state + element * 3
+            if form == 2:
+                return ovl.maximum(state, element)
+            if form == 3:
+                return ovl.minimum(state, element)
+            if form == 4:
+                return state + element * element
+            if form == 5:
+                return state * 0.5 + element if floating else state - element
+            if form == 6 and other is not None:
+                return ovl.maximum(state, other)
+            if form == 7 and other is not None:
+                return state + other
+            return element - state
+
+        two_states = rng.random() < 0.4
+        first = x[at(0)]
+        s0 = ovl.variable(first, x.dtype)
+        s1 = ovl.variable(first if rng.random() < 0.5 else 0, x.dtype) if two_states else None
+        emit_second = two_states and rng.random() < 0.5
+        out[at(0)] = s1 if emit_second else s0
+        for i in ovl.arange(1, length):
+            element = x[at(i)]
+            s0 <<= update(s0, None, element)
+            if two_states:
+                s1 <<= update(s1, s0, element)
+            if emit_second:
+                out[at(i)] = s1
+            elif rng.random() < 0.3:
+                out[at(i)] = s0 + element
+            else:
+                out[at(i)] = s0
+        return out
+    return scan_program
+
+
+def scan_input(seed):
+    shape, dtype = scan_program_shape(seed)
+    rng = np.random.default_rng(seed)
+    if np.dtype(dtype).kind == 'f':
+        # magnitudes around one keep running products finite and interesting
+        return (rng.uniform(0.7, 1.3, shape) * rng.choice([-1.0, 1.0], shape, p=[0.2, 0.8])).astype(dtype)
+    return rng.integers(-3, 4, shape).astype(dtype)
+
+
+def scan_application(seed):
+    return make_scan_operator(seed)(scan_input(seed))
+
+
+SCAN_SEEDS = range(300, 324)

@@ -57,3 +57,19 @@ def test_random_index_program_equals_the_oracle(seed):
         runtime.poison_outputs = False
     for k, (g, r) in enumerate(zip(got, ref)):
         assert g.dtype == r.dtype and g.shape == r.shape and np.array_equal(g, r), 'seed %d output %d' % (seed, k)
+
+
+@pytest.mark.parametrize('seed', random_programs.SCAN_SEEDS)
+def test_random_scan_program_equals_the_oracle(seed):
+    """Row scans with one or two loop-carried variables and assorted update rules, through whichever template the
+    generator picks (lane-skewed scan when the row length fits, else the map kernel): bit-exact."""
+    out = random_programs.scan_application(seed)[0]
+    ref = oracle.evaluate([out])
+    ref = ref[0] if isinstance(ref, list) else ref
+    runtime.poison_outputs = True
+    try:
+        got = ovl.evaluate(out, opt_level=3)
+    finally:
+        runtime.poison_outputs = False
+    assert got.dtype == ref.dtype and got.shape == ref.shape
+    assert np.array_equal(got, ref, equal_nan=(ref.dtype.kind == 'f')), 'seed %d' % seed
