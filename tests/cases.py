@@ -862,6 +862,10 @@ def prebuild_all(cases=None, workers=8, with_oracle=True, force_benchmark=False)
             program = random_programs.index_application(seed).expression_dag
             ops[program.SerializeToString()] = program
             oracle_ops[program.SerializeToString()] = program
+        for seed in random_programs.TYPED_SEEDS:
+            program = random_programs.typed_application(seed).expression_dag
+            ops[program.SerializeToString()] = program
+            oracle_ops[program.SerializeToString()] = program
         for seed in random_programs.SCAN_SEEDS:
             program = random_programs.scan_application(seed).expression_dag
             ops[program.SerializeToString()] = program

@@ -344,3 +344,113 @@ def scan_application(seed):
 
 
 SCAN_SEEDS = range(300, 324)
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# Random typed programs: element-wise expressions over all ten element types with casts between them, integer
+# division and remainder (C truncation), comparisons that yield 0/1 in the operand type, small counted loops and
+# worker-local tensors.  Inputs are small integers, so that no signed arithmetic overflows (undefined in C, for the
+# reference's generated code as much as for this one) and every float is exactly representable.
+# ----------------------------------------------------------------------------------------------------------------------
+TYPED_DTYPES = [np.float32, np.float64, np.int8, np.int16, np.int32, np.int64, np.uint8, np.uint16, np.uint32,
+                np.uint64]
+
+
+def typed_program_types(seed):
+    rng = random.Random(seed * 31337 + 3)
+    return rng.choice(TYPED_DTYPES), rng.choice(TYPED_DTYPES), rng.choice([[64], [5, 12], [3, 7], [2, 3, 16], [100]])
+
+
+def make_typed_operator(seed):
+    @ovl.operator()
+    def typed_program(x, y):
+        rng = random.Random(seed)
+        pos = ovl.position_in(x.shape)
+        out0 = ovl.output_like(x)
+        out1 = ovl.output_like(y)
+        dtypes = [ovl.float32, ovl.float64, ovl.int8, ovl.int16, ovl.int32, ovl.int64, ovl.uint8, ovl.uint16,
+                  ovl.uint32, ovl.uint64]
+
+        def leaf(dtype):
+            source = rng.choice([x, y])
+            value = source[pos]
+            if source.dtype == dtype:
+                return value
+            floats = (ovl.float32, ovl.float64)
+            if source.dtype in floats and dtype not in floats and dtype != ovl.int32:
+                value = ovl.cast(value, ovl.int32)
+            return ovl.cast(value, dtype)
+
+        def expr(dtype, depth):
+            """An expression of type ``dtype`` whose magnitude stays below a few thousand."""
+            if depth <= 0:
+                return leaf(dtype)
+            form = rng.randrange(10)
+            if form == 0:
+                return expr(dtype, depth - 1) + expr(dtype, depth - 1)
+            if form == 1:
+                return expr(dtype, depth - 1) - leaf(dtype)
+            if form == 2:
+                return leaf(dtype) * leaf(dtype)
+            if form == 3:
+                # the divisor is made odd, hence never zero
+                if dtype in (ovl.float32, ovl.float64):
+                    return expr(dtype, depth - 1) / (leaf(dtype) * 2 + 1)
+                return expr(dtype, depth - 1) / (leaf(dtype) * 2 + 1)
+            if form == 4 and dtype not in (ovl.float32, ovl.float64):
+                return expr(dtype, depth - 1) % (leaf(dtype) * 2 + 1)
+            if form == 5:
+                return ovl.minimum(expr(dtype, depth - 1), leaf(dtype))
+            if form == 6:
+                return ovl.maximum(expr(dtype, depth - 1), leaf(dtype))
+            if form == 7:
+                other = rng.choice(dtypes)
+                value = expr(other, depth - 1)
+                floats = (ovl.float32, ovl.float64)
+                if other in floats and dtype not in floats and dtype != ovl.int32:
+                    # a float outside the target's range (a negative one for an unsigned target) converts with
+                    # undefined behaviour in C: go through int32, which holds every value that occurs here
+                    value = ovl.cast(value, ovl.int32)
+                return ovl.cast(value, dtype)
+            if form == 8:
+                a, b = expr(dtype, depth - 1), leaf(dtype)
+                return rng.choice([lambda: a < b, lambda: a <= b, lambda: a == b, lambda: a != b, lambda: a >= b])()
+            return leaf(dtype) + rng.choice([0, 1, 2, 3])
+
+        first = expr(x.dtype, 3)
+        # a small counted loop over a worker-local tensor
+        if rng.random() < 0.5:
+            taps = rng.randint(2, 5)
+            window = ovl.zeros(taps, x.dtype)
+            for k in ovl.arange(taps):
+                window[k] = leaf(x.dtype) + ovl.cast(k, x.dtype)
+            total = ovl.variable(0, x.dtype)
+            for k in ovl.arange(taps - 1, -1, -1):
+                total <<= total + window[k]
+            first = first + total
+        out0[pos] = first
+        chosen = ovl.variable(0, y.dtype)
+        with ovl.if_(expr(x.dtype, 1) < leaf(x.dtype)):
+            chosen <<= expr(y.dtype, 2)
+        with ovl.else_():
+            chosen <<= expr(y.dtype, 3)
+        out1[pos] = chosen
+        return out0, out1
+    return typed_program
+
+
+def typed_inputs(seed):
+    dx, dy, shape = typed_program_types(seed)
+    rng = np.random.default_rng(seed)
+
+    def data(dtype):
+        lo = 0 if np.dtype(dtype).kind == 'u' else -6
+        return rng.integers(lo, 7, shape).astype(dtype)
+    return data(dx), data(dy)
+
+
+def typed_application(seed):
+    return make_typed_operator(seed)(*typed_inputs(seed))
+
+
+TYPED_SEEDS = range(400, 424)

@@ -73,3 +73,15 @@ def test_random_scan_program_equals_the_oracle(seed):
         runtime.poison_outputs = False
     assert got.dtype == ref.dtype and got.shape == ref.shape
     assert np.array_equal(got, ref, equal_nan=(ref.dtype.kind == 'f')), 'seed %d' % seed
+
+
+@pytest.mark.parametrize('seed', random_programs.TYPED_SEEDS)
+def test_random_typed_program_equals_the_oracle(seed):
+    """Expressions over all ten element types with casts, integer division and remainder, comparisons in the operand
+    type, counted loops over worker-local tensors: bit-exact."""
+    op = random_programs.typed_application(seed)
+    outs = [op[0], op[1]]
+    ref = oracle.evaluate(outs)
+    got = ovl.evaluate(outs, opt_level=3)
+    for k, (g, r) in enumerate(zip(got, ref)):
+        assert g.dtype == r.dtype and g.shape == r.shape and np.array_equal(g, r), 'seed %d output %d' % (seed, k)
