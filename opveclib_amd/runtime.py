@@ -16,6 +16,7 @@ from . import language as lang
 from . import compiler
 from . import hipgen
 from . import launcher
+from . import transfer
 from .expression import TensorType
 from .operator import _op_hash
 
@@ -153,7 +154,7 @@ def _require_gpu():
 def _to_device(x, torch, device):
     """Contiguous, 16-byte aligned device tensor for a DAG input; returns (tensor, came_from_host_array)."""
     if isinstance(x, np.ndarray):
-        return torch.from_numpy(np.ascontiguousarray(x)).to(device), True
+        return transfer.to_device(x, torch, device), True
     if isinstance(x, torch.Tensor):
         t = x.detach()
         if t.device.type != 'cuda':
@@ -162,7 +163,7 @@ def _to_device(x, torch, device):
         if t.data_ptr() % 16 != 0:
             t = t.clone()       # a view into the middle of an allocation: vector loads need an aligned base
         return t, False
-    return torch.from_numpy(np.ascontiguousarray(np.asarray(x))).to(device), True
+    return transfer.to_device(np.asarray(x), torch, device), True
 
 
 def run_op_dag(dag, leaf_inputs, profiling_iterations=1, timed=True, options=None):
@@ -215,5 +216,5 @@ def run_op_dag(dag, leaf_inputs, profiling_iterations=1, timed=True, options=Non
 
         results = [buffers[ref.op_index][ref.op_output_index] for ref in dag.dag_outputs]
         if all_host:
-            results = [r.cpu().numpy() for r in results]
+            results = [transfer.to_host(r, torch) for r in results]
     return results, times

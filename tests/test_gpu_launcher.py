@@ -185,3 +185,32 @@ def test_concurrent_evaluation_from_several_threads_and_streams():
         t.join(timeout=120)
     assert not any(t.is_alive() for t in threads)
     assert failures == []
+
+
+def test_staged_host_transfers_round_trip():
+    """Arrays below, at and above the staging threshold and the staging buffer size, five element types, two
+    transfers back to back: what comes back equals what went in, and the device tensor equals PyTorch's own copy."""
+    import torch
+    from opveclib_amd import transfer
+    device = torch.device('cuda', torch.cuda.current_device())
+    rng = np.random.default_rng(1)
+    chunk, least = transfer.CHUNK_BYTES, transfer.MIN_STAGED_BYTES
+    for dtype in (np.float32, np.uint8, np.float64, np.uint16, np.int64):
+        for nbytes in (1, least - 8, least, least + 8, chunk + 24, 2 * chunk, 3 * chunk + 8):
+            n = max(1, nbytes // np.dtype(dtype).itemsize)
+            x = rng.integers(0, 250, n).astype(dtype)
+            t = transfer.to_device(x, torch, device)
+            assert tuple(t.shape) == x.shape and torch.equal(t.cpu(), torch.from_numpy(x))
+            back = transfer.to_host(t, torch)
+            assert back.dtype == x.dtype and back.shape == x.shape and np.array_equal(back, x)
+            y = x[:(n // 3) * 3].reshape(-1, 3) if n >= 3 else x.reshape(1, -1)
+            assert np.array_equal(transfer.to_host(transfer.to_device(y, torch, device), torch), y)
+
+
+def test_evaluate_on_large_host_arrays_uses_the_staged_path_and_matches_torch():
+    import torch
+    rng = np.random.default_rng(2)
+    a = rng.standard_normal((4096, 4096)).astype(np.float32)      # 64 MiB each
+    b = rng.standard_normal((4096, 4096)).astype(np.float32)
+    got = ovl.evaluate(stdops.mul(stdops.add(a, b), a))
+    assert isinstance(got, np.ndarray) and np.array_equal(got, (a + b) * a)
