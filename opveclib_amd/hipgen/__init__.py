@@ -26,7 +26,7 @@ from . import tile_kernel
 from . import rowscan_kernel
 
 #: bump when generated code changes for an unchanged DAG, so cached binaries are not reused
-CODEGEN_VERSION = 23
+CODEGEN_VERSION = 24
 
 
 
@@ -60,8 +60,8 @@ def generate(expression_dag, function_name, options=None):
     :param function_name: unique name of the operator (its content hash)
     :param options: optional dict.  ``template``: 'auto' (default), 'map', 'transpose', 'rowscan' or 'skewscan' restricts
         the choice of kernel template (a template that does not fit the DAG falls back to 'map'); ``vec`` forces the
-        map template with that vector width; ``scan_depth`` / ``scan_sets`` / ``scan_width`` set the request burst (groups), the
-        number of register sets and the 128-bit vectors per lane and phase of the lane-skewed scan; ``math``: 'exact'
+        map template with that vector width; ``scan_depth`` / ``scan_sets`` / ``scan_width`` / ``scan_interleave`` set the request burst (groups), the
+        number of register sets, the 128-bit vectors per lane and phase and the rows per lane group of the lane-skewed scan; ``math``: 'exact'
         or 'fast'; ``if_conversion`` / ``value_ranges``: False switches that transformation off; ``scan_rows`` / ``scan_chunk`` the LDS tile of the row scan; ``nt`` /
         ``scan_nt`` which vector accesses carry the non-temporal hint ('l' loads, 's' stores, 'ls', ''); ``grid_cap``
         the largest grid of the map and transpose templates (their kernels then stride over the rest)
@@ -82,7 +82,7 @@ def generate(expression_dag, function_name, options=None):
     template = options.get('template', 'auto')
     if options.get('vec') is None and template in ('auto', 'skewscan') and rowscan_kernel.skew_plan(info) is not None:
         kernel_src, launch = rowscan_kernel.generate_skewed(info, kernel_name, options.get('scan_depth'), options.get('scan_sets'), options.get('scan_nt', 's'),
-                                                             options.get('scan_width'))
+                                                             options.get('scan_width'), options.get('scan_interleave'))
     elif options.get('vec') is None and template in ('auto', 'rowscan') and rowscan_kernel.plan(info) is not None:
         kernel_src, launch = rowscan_kernel.generate(info, kernel_name, options.get('scan_rows'),
                                                      options.get('scan_chunk'))

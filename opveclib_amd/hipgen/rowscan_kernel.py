@@ -19,6 +19,8 @@ recurrence, so results equal the generic template's (and numpy's accumulate) bit
 coalesced and every element is read and written once.
 """
 
+import re
+
 from .. import language as lang
 from .analysis import ITEMSIZE
 from .body import BodyEmitter, CTYPE
@@ -334,7 +336,24 @@ def skew_plan(info):
     return p
 
 
-def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None):
+def _default_interleave(rows, vec):
+    """Rows per lane group of the lane-skewed scan when the caller does not say."""
+    return 1
+
+
+def _for_slot(text, slot):
+    """The per-row names of a source fragment renamed for the row with number ``slot`` of a lane group (slot 0 keeps
+    the plain names): expression variables e<N> and their carries, position, row, the row's pointers, register sets,
+    output vectors and the step macro."""
+    if slot == 0:
+        return text
+    suffix = '_r%d' % slot
+    text = re.sub(r'\b(carry_e\d+|e\d+|position|row_raw|row|gin|gout|q\d+|ov|xv|first_out|OVL_SCAN_STEP)\b',
+                  lambda m: m.group(1) + suffix, text)
+    return text
+
+
+def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None, interleave=None):
     p = skew_plan(info)
     assert p is not None
     ctype = CTYPE[p.x.dtype]
@@ -351,7 +370,14 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
         width //= 2
     group_cols = GROUP_LANES * vec * width
     num_groups = p.length // group_cols
-    rows_per_wave = WAVE // GROUP_LANES
+    # interleave = rows per group of sixteen lanes.  With few rows there are fewer wavefronts than SIMDs and each runs
+    # at the latency of its one recurrence; a lane group that carries two rows has two independent recurrences whose
+    # additions and hand-overs fill each other's wait states.
+    if interleave is None:
+        interleave = _default_interleave(p.rows, vec)
+    interleave = max(1, min(int(interleave), 4))
+    slots = list(range(interleave))
+    rows_per_wave = (WAVE // GROUP_LANES) * interleave
     waves = BLOCK // WAVE
     rows_per_block = rows_per_wave * waves
     if depth is None:
@@ -387,6 +413,13 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
 
     vname = 'ovl_scan_vec'
     src = []
+
+    def emit(lines, per_row=True):
+        """Append source lines: once, or once per row of the lane group with that row's names."""
+        for slot in (slots if per_row else [0]):
+            for line in lines:
+                src.append(_for_slot(line, slot))
+
     src.append('typedef %s %s __attribute__((ext_vector_type(%d)));' % (ctype, vname, vec))
     src.append('')
     src.append('extern "C" __global__ void __launch_bounds__(%d)' % BLOCK)
@@ -396,16 +429,21 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
         src.append('    OVL_DECLARE_MATH_TABLES();')
     src.append('    const uint32_t lane = threadIdx.x %% %du;' % WAVE)
     src.append('    const uint32_t part = lane %% %du;              // which VEC columns of a group this lane holds' % GROUP_LANES)
-    src.append('    const uint32_t row_raw = (blockIdx.x * %du + threadIdx.x / %du) * %du + lane / %du;' % (
-        waves, WAVE, rows_per_wave, GROUP_LANES))
     src.append('    // A wavefront wholly past the last row leaves; single lanes past it shadow the last row instead (all lanes')
     src.append('    // must stay active for the lane-to-lane moves): they load, compute and store exactly what its owners do.')
     src.append('    if ((blockIdx.x * %du + threadIdx.x / %du) * %du >= %du) return;' % (waves, WAVE, rows_per_wave, p.rows))
-    src.append('    const uint32_t row = row_raw < %du ? row_raw : %du;' % (p.rows, p.rows - 1))
-    src.append('    const %s* __restrict__ gin = in%d + (uint64_t)row * %dull + part * %du;' % (
-        ctype, p.x.io_index, p.length, vec * width))
-    src.append('    %s* __restrict__ gout = out%d + (uint64_t)row * %dull + part * %du;' % (
-        ctype, p.out.io_index, p.length, vec * width))
+    for slot in slots:
+        if interleave == 1:
+            raw = '(blockIdx.x * %du + threadIdx.x / %du) * %du + lane / %du' % (waves, WAVE, rows_per_wave, GROUP_LANES)
+        else:
+            raw = '(blockIdx.x * %du + threadIdx.x / %du) * %du + (lane / %du) * %du + %du' % (
+                waves, WAVE, rows_per_wave, GROUP_LANES, interleave, slot)
+        src.append(_for_slot('    const uint32_t row_raw = %s;' % raw, slot))
+    emit(['    const uint32_t row = row_raw < %du ? row_raw : %du;' % (p.rows, p.rows - 1),
+          '    const %s* __restrict__ gin = in%d + (uint64_t)row * %dull + part * %du;' % (
+              ctype, p.x.io_index, p.length, vec * width),
+          '    %s* __restrict__ gout = out%d + (uint64_t)row * %dull + part * %du;' % (
+              ctype, p.out.io_index, p.length, vec * width)])
     # measured on MI355X (float32 [4096, 16384]): non-temporal stores with plain loads 85 us, hint on both 100 us,
     # on the loads only 90 us, on neither 102 us
     batch = depth
@@ -414,58 +452,61 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
 
     def request(regs, batch_expr):
         """All loads of one batch, back to back: every row is read in runs of batch * 256 bytes."""
-        src.append('        #pragma unroll')
-        src.append('        for (uint32_t j = 0; j < %du; ++j)' % batch)
-        src.append('            #pragma unroll')
-        src.append('            for (uint32_t w = 0; w < %du; ++w)' % width)
+        lines = ['        #pragma unroll',
+                 '        for (uint32_t j = 0; j < %du; ++j)' % batch,
+                 '            #pragma unroll',
+                 '            for (uint32_t w = 0; w < %du; ++w)' % width]
         if 'l' in nt:
-            src.append('                %s[j][w] = __builtin_nontemporal_load(reinterpret_cast<const %s*>(gin + (%s) * %du + j * %du + w * %du));' % (
+            lines.append('                %s[j][w] = __builtin_nontemporal_load(reinterpret_cast<const %s*>(gin + (%s) * %du + j * %du + w * %du));' % (
                 regs, vname, batch_expr, batch_cols, group_cols, vec))
         else:
-            src.append('                %s[j][w] = *(reinterpret_cast<const %s*>(gin + (%s) * %du + j * %du + w * %du));' % (
+            lines.append('                %s[j][w] = *(reinterpret_cast<const %s*>(gin + (%s) * %du + j * %du + w * %du));' % (
                 regs, vname, batch_expr, batch_cols, group_cols, vec))
+        emit(lines)
 
     def process(regs, batch_expr, refill_expr):
         src.append('        {')
         src.append('        const uint32_t b = %s;' % batch_expr)
-        src.append('        %s ov[%d][%d];' % (vname, batch, width))
+        emit(['        %s ov[%d][%d];' % (vname, batch, width)])
         src.append('        #pragma unroll')
         src.append('        for (uint32_t j = 0; j < %du; ++j) {' % batch)
         src.append('            const uint32_t col0 = b * %du + j * %du + part * %du;' % (batch_cols, group_cols, vec * width))
         src.append('            const bool first_column = (j == 0u) && (b == 0u) && (part == 0u);')
         src.append('            #pragma unroll')
         src.append('            for (uint32_t phase = 0; phase < %du; ++phase) {' % GROUP_LANES)
-        for name, _ in state:
-            src.append('                %s = carry_%s;' % (name, name))
+        # the rows of a lane group advance column by column, side by side: their recurrences are independent, and in
+        # this order the additions and hand-overs of one row fill the wait states of the other
+        emit(['                %s = carry_%s;' % (name, name) for name, _ in state])
         src.append('                #pragma unroll')
         src.append('                for (uint32_t w = 0; w < %du; ++w) {' % width)
-        src.append('                    const %s xv = %s[j][w];' % (vname, regs))
+        emit(['                    const %s xv = %s[j][w];' % (vname, regs)])
         src.append('                    #pragma unroll')
         src.append('                    for (uint32_t u = 0; u < %du; ++u) {' % vec)
-        src.append('                        if (w == 0u && u == 0u && first_column) ov[j][0][0] = first_out;')
-        src.append('                        else OVL_SCAN_STEP(col0 + w * %du + u)' % vec)
+        emit(['                        if (w == 0u && u == 0u && first_column) ov[j][0][0] = first_out;',
+              '                        else OVL_SCAN_STEP(col0 + w * %du + u)' % vec])
         src.append('                    }')
         src.append('                }')
-        for name, _ in state:
-            src.append('                carry_%s = ovl_dpp_move<OVL_DPP_ROW_SHR1>(carry_%s, %s);' % (name, name, name))
+        emit(['                carry_%s = ovl_dpp_move<OVL_DPP_ROW_SHR1>(carry_%s, %s);' % (name, name, name)
+              for name, _ in state])
         src.append('            }')
         src.append('            // the last lane of the group finished the group: its state is the carry into the next one')
-        for name, _ in state:
-            src.append('            carry_%s = ovl_dpp_move<OVL_DPP_ROW_ROR1>(carry_%s, %s);' % (name, name, name))
+        emit(['            carry_%s = ovl_dpp_move<OVL_DPP_ROW_ROR1>(carry_%s, %s);' % (name, name, name)
+              for name, _ in state])
         src.append('        }')
         src.append('        // The scheduling fences keep the memory traffic of a batch together, after its arithmetic: runs of')
         src.append('        // batch * 256 bytes per row, and no load is moved ahead of the last use of the registers it fills.')
         src.append('        __builtin_amdgcn_sched_barrier(0);')
-        src.append('        #pragma unroll')
-        src.append('        for (uint32_t j = 0; j < %du; ++j)' % batch)
-        src.append('            #pragma unroll')
-        src.append('            for (uint32_t w = 0; w < %du; ++w)' % width)
+        lines = ['        #pragma unroll',
+                 '        for (uint32_t j = 0; j < %du; ++j)' % batch,
+                 '            #pragma unroll',
+                 '            for (uint32_t w = 0; w < %du; ++w)' % width]
         if 's' in nt:
-            src.append('                __builtin_nontemporal_store(ov[j][w], reinterpret_cast<%s*>(gout + b * %du + j * %du + w * %du));' % (
+            lines.append('                __builtin_nontemporal_store(ov[j][w], reinterpret_cast<%s*>(gout + b * %du + j * %du + w * %du));' % (
                 vname, batch_cols, group_cols, vec))
         else:
-            src.append('                *(reinterpret_cast<%s*>(gout + b * %du + j * %du + w * %du)) = ov[j][w];' % (
+            lines.append('                *(reinterpret_cast<%s*>(gout + b * %du + j * %du + w * %du)) = ov[j][w];' % (
                 vname, batch_cols, group_cols, vec))
+        emit(lines)
         if refill_expr is not None:
             request(regs, refill_expr)
         src.append('        __builtin_amdgcn_sched_barrier(0);')
@@ -473,25 +514,28 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
 
     sets = max(2, min(sets or 2, num_batches)) if num_batches > 1 else 1
     src.append('    // %d register sets of %d groups each: one is consumed while the others are in flight' % (sets, batch))
-    src.append('    %s %s;' % (vname, ', '.join('q%d[%d][%d]' % (k, batch, width) for k in range(sets))))
+    emit(['    %s %s;' % (vname, ', '.join('q%d[%d][%d]' % (k, batch, width) for k in range(sets)))])
     src.append('    {')
     for k in range(sets):
         request('q%d' % k, '%du' % k)
     src.append('    }')
     src.append('    // first column: the statements the worker runs before its loop, in every lane')
-    src.append('    %s first_out;' % ctype)
-    src.append('#define OVL_SCAN_IN (in%d[(uint64_t)row * %dull])' % (p.x.io_index, p.length))
-    src.append('#define OVL_SCAN_OUT(value) first_out = (value)')
-    for stmt in prologue:
-        src.append('    ' + stmt)
-    src.append('#undef OVL_SCAN_IN')
-    src.append('#undef OVL_SCAN_OUT')
-    for name, stype in state:
-        src.append('    %s carry_%s = %s;' % (stype, name, name))
-    src.append('#define OVL_SCAN_IN xv[u]')
-    src.append('#define OVL_SCAN_OUT(value) ov[j][w][u] = (value)')
-    src.append('#define OVL_SCAN_STEP(column) { %s = (%s)(column); %s }' % (
-        counter_name, counter_type, ' '.join(body)))
+    for slot in slots:
+        emit_one = lambda lines: src.extend(_for_slot(line, slot) for line in lines)
+        emit_one(['    %s first_out;' % ctype])
+        src.append('#define OVL_SCAN_IN (in%d[(uint64_t)%s * %dull])' % (p.x.io_index, _for_slot('row', slot), p.length))
+        src.append('#define OVL_SCAN_OUT(value) %s = (value)' % _for_slot('first_out', slot))
+        emit_one(['    ' + stmt for stmt in prologue])
+        src.append('#undef OVL_SCAN_IN')
+        src.append('#undef OVL_SCAN_OUT')
+        emit_one(['    %s carry_%s = %s;' % (stype, name, name) for name, stype in state])
+    for slot in slots:
+        # (the output vector is named in the step macro itself, so that every row writes its own)
+        src.append(_for_slot('#define OVL_SCAN_STEP(column) { %s = (%s)(column); %s }' % (
+            counter_name, counter_type, ' '.join(body)), slot).replace(
+                'OVL_SCAN_OUT(', 'OVL_SCAN_OUT_R%d(' % slot).replace('OVL_SCAN_IN', 'OVL_SCAN_IN_R%d' % slot))
+        src.append('#define OVL_SCAN_IN_R%d %s[u]' % (slot, _for_slot('xv', slot)))
+        src.append('#define OVL_SCAN_OUT_R%d(value) %s[j][w][u] = (value)' % (slot, _for_slot('ov', slot)))
     rounds = num_batches // sets
     last = num_batches - 1
     if rounds:
@@ -505,9 +549,10 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
         src.append('    {')
         process('q%d' % k, '%du' % (rounds * sets + k), None)
         src.append('    }')
-    src.append('#undef OVL_SCAN_STEP')
-    src.append('#undef OVL_SCAN_IN')
-    src.append('#undef OVL_SCAN_OUT')
+    for slot in slots:
+        src.append('#undef %s' % _for_slot('OVL_SCAN_STEP', slot))
+        src.append('#undef OVL_SCAN_OUT_R%d' % slot)
+        src.append('#undef OVL_SCAN_IN_R%d' % slot)
     src.append('}')
 
     launch = {

@@ -791,6 +791,9 @@ TEMPLATE_VARIANTS = [
     ('c3_cumsum_f32', {'scan_width': 2}),
     ('c3_cumprod_f64', {'scan_width': 1}),
     ('c3_rowscan_shapes', {'scan_width': 4, 'scan_depth': 1}),
+    ('c3_rowscan_shapes', {'scan_interleave': 2}),
+    ('c3_cumprod_f64', {'scan_interleave': 3, 'scan_sets': 3}),
+    ('accumulate_max', {'scan_interleave': 4}),
     ('c5_variants', {'template': 'map'}),
     ('c2_chain', {'vec': 2}),
     ('c2_chain', {'value_ranges': False}),
