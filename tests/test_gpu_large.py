@@ -22,8 +22,16 @@ def _device_tensor(shape, dtype):
     return torch.randn(shape, dtype=torch_dtype, device='cuda:0')
 
 
+def _need_free_device_memory(gib):
+    import torch
+    free, _total = torch.cuda.mem_get_info()
+    if free < gib * 2 ** 30:
+        pytest.skip('needs %d GiB of free device memory, %.0f GiB are free' % (gib, free / 2 ** 30))
+
+
 def test_generated_operators_at_the_largest_sizes():
     import torch
+    _need_free_device_memory(48)
     torch.manual_seed(11)
     names = []
     for name, out, reference in large_cases.cases(_device_tensor):
@@ -42,6 +50,7 @@ def test_hand_written_lstm_cell_on_2_to_32_minus_1_elements():
     the result must equal the same function on blocks of rows (which stay far below that)."""
     import torch
     from opveclib_amd.lstm_cell import lstm_cell, lstm_cell_grad
+    _need_free_device_memory(128)
     torch.manual_seed(12)
     batch, units, block = 1431655765, 3, 1 << 27
     assert batch * units == 2 ** 32 - 1
