@@ -44,29 +44,47 @@ def _io_types(op):
     return ([TensorType.from_proto(e.tensor_type) for e in ins], [TensorType.from_proto(e.tensor_type) for e in outs])
 
 
-def build_source(source, entry):
-    """Compile one operator source text (with entry point ``entry``) for the host; returns the program's path."""
+def build_source(source, entry, extra_flags=()):
+    """Compile operator source text (one text, or a list of texts that become one translation unit each) with entry
+    point ``entry`` for the host; returns the program's path."""
+    sources = [source] if isinstance(source, str) else list(source)
     with open(os.path.join(SHIM, 'ovl_device.h'), 'rb') as f:
         shim = f.read()
     with open(os.path.join(SHIM, 'main.cpp'), 'rb') as f:
         shim += f.read()
-    digest = hashlib.sha224(source.encode('utf-8') + entry.encode('utf-8') + shim).hexdigest()[:32]
+    digest = hashlib.sha224('\0'.join(sources).encode('utf-8') + entry.encode('utf-8') + shim).hexdigest()[:32]
     os.makedirs(BUILD, exist_ok=True)
     program = os.path.join(BUILD, 'emu_' + digest)
     if not os.path.exists(program):
-        path = program + '.cpp'
-        with open(path, 'w') as f:
-            f.write(source)
+        paths = []
+        for k, text in enumerate(sources):
+            paths.append(program + ('.cpp' if k == 0 else '.%d.cpp' % k))
+            with open(paths[-1], 'w') as f:
+                f.write(text)
         tmp = program + '.tmp.%d.%d' % (os.getpid(), threading.get_ident())
-        cmd = [CLANG] + FLAGS + ['-I' + SHIM, '-I' + local.csrc_directory, '-DOVL_ENTRY=' + entry,
-                                 '-Wl,-rpath,' + _sanitizer_runtime_directory(),
-                                 os.path.join(SHIM, 'main.cpp'), path, '-o', tmp]
+        cmd = [CLANG] + FLAGS + list(extra_flags) + ['-I' + SHIM, '-I' + local.csrc_directory, '-DOVL_ENTRY=' + entry,
+                                                     '-Wl,-rpath,' + _sanitizer_runtime_directory(),
+                                                     os.path.join(SHIM, 'main.cpp')] + paths + ['-o', tmp]
         try:
             subprocess.check_output(cmd, stderr=subprocess.STDOUT, universal_newlines=True)
         except subprocess.CalledProcessError as exception:
             raise EmulationError('host build of the generated source failed:\n' + exception.output)
         os.replace(tmp, program)
     return program
+
+
+def build_hand_written(entry):
+    """The hand-written kernel libraries (csrc/ovl_lstm.hip, csrc/ovl_scan.hip) compiled for the host together with
+    the adapters of hand_written_adapters.cpp; ``entry`` names the adapter to run.  The sources are compiled from
+    copies in the build directory, so that their ``#include "ovl_device.h"`` finds the stand-in."""
+    parts = []
+    for name in ('ovl_lstm.hip', 'ovl_scan.hip'):
+        with open(os.path.join(local.csrc_directory, name)) as f:
+            parts.append(f.read())
+    with open(os.path.join(SHIM, 'hand_written_adapters.cpp')) as f:
+        parts.append(f.read())
+    include = os.path.normpath(os.path.join(local.csrc_directory, '..', '..', 'include'))
+    return build_source(parts, entry, ['-I' + include])
 
 
 def build(op, options=None):

@@ -56,8 +56,11 @@ struct dim3 {
 static thread_local dim3 blockIdx, threadIdx;
 static dim3 gridDim, blockDim;
 typedef void* hipStream_t;
+typedef int hipError_t;
 enum { hipSuccess = 0 };
-static inline int hipPeekAtLastError() { return hipSuccess; }
+static inline hipError_t hipPeekAtLastError() { return hipSuccess; }
+static inline hipError_t hipGetLastError() { return hipSuccess; }
+static inline const char* hipGetErrorString(hipError_t) { return "no error"; }
 
 static pthread_barrier_t ovl_emulated_block_barrier;
 static pthread_barrier_t ovl_emulated_wave_barrier[16];
@@ -134,6 +137,12 @@ static inline T ovl_dpp_move(T old, T src) {
 #define ovl_logf_inrange_nan(x) ovl_math::logf_inrange_<true>((x), ovl_log_tab)
 #define ovl_recipf_inrange(x) (1.0f / (x))
 #define ovl_divf_inrange(a, b) ((a) / (b))
+
+// The 'fast' math mode is built on device instructions; sources that also instantiate it (the hand-written LSTM
+// cell) compile against the exact routines here, and the emulation tests never select it.
+#define ovl_fast_expf(x) ovl_expf(x)
+#define ovl_fast_tanhf(x) ovl_tanhf(x)
+#define ovl_fast_divf(a, b) ((a) / (b))
 
 #define OVL_DECLARE_MATH_TABLES()                                   \
     const uint64_t* const ovl_exp_tab = ovl_math::exp2f_tab;        \

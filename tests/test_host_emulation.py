@@ -114,3 +114,73 @@ def test_random_programs_emulated_on_the_host_equal_the_oracle():
         for level in (0, 3):
             jobs.append(('operator DAG %d opt_level %d' % (seed, level), outs, level, None))
     assert _run_all(jobs) == []
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# The hand-written kernels with run-time shapes (csrc/ovl_lstm.hip, csrc/ovl_scan.hip) on the host
+# ----------------------------------------------------------------------------------------------------------------------
+F32, F64, U32 = 1, 2, 10        # dtype codes of the launcher ABI (include/ovl_launch.h)
+
+
+def _skewed(array, skew):
+    """The array as the adapters expect it: behind ``skew`` leading elements (which the kernels must not touch)."""
+    flat = np.ascontiguousarray(array).reshape(-1)
+    return np.concatenate([np.full(skew, 77, flat.dtype), flat]) if skew else flat
+
+
+def _lstm_shapes():
+    rng = np.random.default_rng(21)
+    shapes = [(1, 1), (1, 4), (3, 5), (2, 8), (7, 12), (5, 64), (64, 36), (9, 257), (33, 100), (2, 1024), (130, 20)]
+    return [(b, u, int(rng.integers(0, 2))) for b, u in shapes]
+
+
+@pytest.mark.parametrize('batch,units,skew', _lstm_shapes())
+def test_hand_written_lstm_cell_emulated_on_the_host_equals_the_oracle(batch, units, skew):
+    from opveclib_amd.lstm import lstm, lstm_grad
+    rng = np.random.default_rng(batch * 1000 + units)
+    concat = rng.standard_normal((batch, 4 * units)).astype(np.float32) * 3
+    c = rng.standard_normal((batch, units)).astype(np.float32)
+    d_c = rng.standard_normal((batch, units)).astype(np.float32)
+    d_h = rng.standard_normal((batch, units)).astype(np.float32)
+    concat[0, 0] = 60.0          # beyond the range of the sigmoid derivative
+    bias = np.array([1.0], np.float32)
+    dims = np.array([batch, units, skew], np.uint32)
+    n, m = batch * units + skew, 4 * batch * units + skew
+
+    ref_c, ref_h = oracle.evaluate(lstm(concat, c, forget_bias=1.0))
+    got = host_emulation.run_program(
+        host_emulation.build_hand_written('emu_lstm_forward'),
+        [_skewed(concat, skew), _skewed(c, skew), bias, dims],
+        [(F32, np.float32, [m]), (F32, np.float32, [n]), (F32, np.float32, [1]), (U32, np.uint32, [3])],
+        [(F32, np.float32, [n]), (F32, np.float32, [n])])
+    assert np.array_equal(got[0][skew:].reshape(batch, units), ref_c)
+    assert np.array_equal(got[1][skew:].reshape(batch, units), ref_h)
+    # the elements in front of a skewed tensor keep the fill the driver gave them
+    assert all(np.all(g[:skew].view(np.uint32) == 0xFEFEFEFE) for g in got)
+
+    ref_dconcat, ref_dc = oracle.evaluate(lstm_grad(concat, c, d_c, d_h, forget_bias=1.0))
+    got = host_emulation.run_program(
+        host_emulation.build_hand_written('emu_lstm_backward'),
+        [_skewed(concat, skew), _skewed(c, skew), _skewed(d_c, skew), _skewed(d_h, skew), bias, dims],
+        [(F32, np.float32, [m]), (F32, np.float32, [n]), (F32, np.float32, [n]), (F32, np.float32, [n]),
+         (F32, np.float32, [1]), (U32, np.uint32, [3])],
+        [(F32, np.float32, [m]), (F32, np.float32, [n])])
+    assert np.array_equal(got[0][skew:].reshape(batch, 4 * units), ref_dconcat)
+    assert np.array_equal(got[1][skew:].reshape(batch, units), ref_dc)
+
+
+@pytest.mark.parametrize('rows,cols,skew', [(1, 1, 0), (1, 64, 0), (3, 128, 0), (5, 192, 0), (4, 256, 0), (17, 320, 0),
+                                            (9, 64, 1), (6, 100, 0), (2, 7, 1), (70, 33, 0), (67, 512, 0), (1, 1024, 0)])
+def test_hand_written_row_scans_emulated_on_the_host_equal_numpy(rows, cols, skew):
+    rng = np.random.default_rng(rows * 1000 + cols)
+    dims = np.array([rows, cols, skew], np.uint32)
+    n = rows * cols + skew
+    for name, code, dtype in (('cumsum_f32', F32, np.float32), ('cumprod_f32', F32, np.float32),
+                              ('cumsum_f64', F64, np.float64), ('cumprod_f64', F64, np.float64)):
+        x = (rng.uniform(0.7, 1.3, (rows, cols)) * rng.choice([-1.0, 1.0], (rows, cols))).astype(dtype)
+        x[0, 0] = -0.0
+        got = host_emulation.run_program(host_emulation.build_hand_written('emu_' + name), [_skewed(x, skew), dims],
+                                         [(code, dtype, [n]), (U32, np.uint32, [3])], [(code, dtype, [n])])[0]
+        ref = (np.cumsum if 'cumsum' in name else np.cumprod)(x, axis=1, dtype=dtype)
+        out = got[skew:].reshape(rows, cols)
+        assert np.array_equal(out, ref) and np.array_equal(np.signbit(out), np.signbit(ref)), name
