@@ -294,8 +294,13 @@ def cpu_baseline(seed_arrays, rows, iters=3):
     _, times = oracle.profile(outs, profiling_iterations=iters, opt_level=3, num_threads=threads)
     ms = min(min(t) for t in times.values()) if len(times) == 1 else sum(min(t) for t in times.values())
     nbytes = 3 * rows * a.shape[1] * 4 + 4
+    # the same generated C++ built with -O2, as a courtesy next to the reference's own flags (never `value`)
+    _, times_o2 = oracle.profile(outs, profiling_iterations=iters, opt_level=3, num_threads=threads,
+                                 extra_flags=('-O2',))
+    ms_o2 = sum(min(t) for t in times_o2.values())
     return {'value': round(nbytes / (ms * 1e-3) / 1e9, 3), 'unit': 'GB/s', 'cores': threads, 'kind': 'port',
             'ms': round(ms, 2),
+            'with_O2': {'value': round(nbytes / (ms_o2 * 1e-3) / 1e9, 3), 'unit': 'GB/s', 'ms': round(ms_o2, 2)},
             'sample': 'first %d of %d rows of the chain8 inputs; reference-shaped fused C++ (g++, no -O flag as in '
                       'the reference), std::thread block split, thread create/join inside the timed region, '
                       'best of %d' % (rows, a.shape[0], iters)}, outs
