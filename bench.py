@@ -285,6 +285,35 @@ def _side_workload(name, prepared, steps, warmup):
             'kernels': [k['kernel'] for k in prepared.kernels]}
 
 
+def clocks_under_load(prepared, seconds=2.0, per_launch_ms=0.26):
+    """Shader and memory clock (MHz) as rocm-smi reports them while a queue of launches of the workload runs: the
+    median of three readings taken after the first second (the power management needs that long to settle under
+    this kernel); None where the tool is missing or says nothing.  Outside every timed region."""
+    import subprocess
+    import torch
+    stream = torch.cuda.current_stream(prepared.device).cuda_stream
+    for _ in range(int(seconds * 1e3 / per_launch_ms)):
+        prepared.launch(stream)
+    readings = {'sclk_mhz': [], 'mclk_mhz': []}
+    try:
+        time.sleep(1.0)
+        for _ in range(3):
+            text = subprocess.run(['rocm-smi', '--showclocks', '--json'], stdout=subprocess.PIPE,
+                                  stderr=subprocess.DEVNULL, universal_newlines=True, timeout=30).stdout
+            card = next(iter(json.loads(text[text.index('{'):]).values()))
+            for key, value in card.items():
+                digits = ''.join(ch for ch in str(value) if ch.isdigit() or ch == '.')
+                if digits and key.startswith('sclk clock speed'):
+                    readings['sclk_mhz'].append(float(digits))
+                elif digits and key.startswith('mclk clock speed'):
+                    readings['mclk_mhz'].append(float(digits))
+    except Exception:           # the figures are informational: a missing or talkative tool must not end the benchmark
+        pass
+    torch.cuda.synchronize(prepared.device)
+    found = dict((k, sorted(v)[len(v) // 2]) for k, v in readings.items() if v)
+    return found or None
+
+
 def cpu_baseline(seed_arrays, rows, iters=3):
     """The CPU oracle on the first ``rows`` rows of the chain8 inputs, all host threads, best of ``iters``."""
     import oracle
@@ -345,7 +374,8 @@ def main():
                                'A, B float32 [8192, 8192] uniform[-1, 1], numpy default_rng(2)',
                    'algorithmic_bytes': nbytes, 'kernel': chain.kernels[0]['kernel'],
                    'pct_of_hbm_peak': round(100.0 * value / HBM_PEAK_GBPS, 2),
-                   'clock_settling_launches_before_warmup': settled_after},
+                   'clock_settling_launches_before_warmup': settled_after,
+                   'clocks_under_load': clocks_under_load(chain)},
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
                      'frac': round(achieved / HBM_PEAK_GBPS, 4), 'traffic': CHAIN8_TRAFFIC_BYTES,
                      'kernel_us': round(event_ms * 1e3, 2), 'kernel_min_us': round(min_ms * 1e3, 2)},
