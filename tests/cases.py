@@ -890,6 +890,13 @@ def prebuild_all(cases=None, workers=8, with_oracle=True, force_benchmark=False)
                 ops[op.SerializeToString()] = op
         for op in _operators_of(graph_capture_single(np.zeros(4096, np.float32)), 3):
             variants.append((op, {'math': 'fast'}))
+        for k in range(4):      # tests/test_gpu_launcher.py: concurrent evaluation on large host arrays
+            staged = np.zeros((3 << 20) + k, np.float32)
+            for op in _operators_of([stdops.add(staged, staged)[0]], 0):
+                ops[op.SerializeToString()] = op
+        staged = np.zeros((4096, 4096), np.float32)
+        for op in _operators_of([stdops.mul(stdops.add(staged, staged), staged)[0]], 3):
+            ops[op.SerializeToString()] = op
         from tests import large_cases
         for op in large_cases.operators_to_build():
             ops[op.SerializeToString()] = op

@@ -161,6 +161,8 @@ def test_concurrent_evaluation_from_several_threads_and_streams():
     expected = {}
     for name in names:
         expected[name] = oracle.profile(cases.CASE_BY_NAME[name].outputs(), 1, 0)[0]
+    large = dict((name, np.random.default_rng(k).standard_normal((3 << 20) + k).astype(np.float32))
+                 for k, name in enumerate(names))
     failures = []
     start = threading.Barrier(len(names))
 
@@ -175,6 +177,10 @@ def test_concurrent_evaluation_from_several_threads_and_streams():
                 got = got if isinstance(got, list) else [got]
                 for n, (g, r) in enumerate(zip(got, expected[name])):
                     cases.assert_matches(case, g, r, '%s output %d' % (name, n))
+                # host arrays large enough for the page-locked staging buffers, which the threads share
+                with torch.cuda.stream(stream):
+                    big = ovl.evaluate(stdops.add(large[name], large[name]))
+                assert np.array_equal(big, large[name] + large[name]), name + ': staged transfer'
         except Exception as exception:      # reported by the main thread
             failures.append((name, repr(exception)))
 
