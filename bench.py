@@ -121,6 +121,13 @@ def all_workload_outputs():
     yield lstm_outputs(Spec((4096, 4096)), Spec((4096, 1024)))
     yield lstm_grad_outputs(Spec((4096, 4096)), Spec((4096, 1024)), Spec((4096, 1024)), Spec((4096, 1024)))
     yield gather_outputs(Spec((16384, 16384)), Spec((16384 * 16384,)))
+    # the bounded samples that are also run through the CPU oracle
+    yield cumsum_outputs(Spec((512, 16384), f32))
+    yield cumprod_outputs(Spec((512, 16384), f32))
+    yield cumsum_outputs(Spec((256, 16384), f64))
+    yield lstm_outputs(Spec((512, 4096)), Spec((512, 1024)))
+    yield lstm_grad_outputs(Spec((512, 4096)), Spec((512, 1024)), Spec((512, 1024)), Spec((512, 1024)))
+    yield gather_outputs(Spec((2048, 2048)), Spec((2048 * 2048,)))
 
 
 def uniform(rng, lo, hi, shape, dtype=np.float32):
@@ -335,6 +342,24 @@ def cpu_baseline(seed_arrays, rows, iters=3):
                       'best of %d' % (rows, a.shape[0], iters)}, outs
 
 
+def cpu_reference(outputs, sample, iters=3):
+    """
+    The CPU oracle on a bounded sample of a configuration (operators as written, one generated C++ function per
+    operator, the reference's compiler flags, all host threads, best of ``iters``), and whether the HIP path returns
+    the same bits for the same inputs.
+    """
+    import oracle
+    import opveclib_amd as ovl
+    threads = oracle.hardware_threads()
+    ref, times = oracle.profile(outputs, profiling_iterations=iters, opt_level=0, num_threads=threads)
+    ms = sum(float(min(t)) for t in times.values())
+    got = ovl.evaluate(outputs, opt_level=3)
+    got = got if isinstance(got, list) else [got]
+    same = all(g.dtype == r.dtype and g.shape == r.shape and
+               np.array_equal(g, r, equal_nan=(r.dtype.kind == 'f')) for g, r in zip(got, ref))
+    return {'ms': round(ms, 3), 'cores': threads, 'sample': sample, 'bit_exact': bool(same)}
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument('--gpus', type=int, default=1)
@@ -415,17 +440,29 @@ def main():
         others.append(side_workload('copy f32[8192,8192] (counter calibration, plain copy bandwidth)',
                                     copy_outputs(a), steps, args.warmup))
         g = np.random.default_rng(0)
-        others.append(side_workload('c1 shift_cyclic -> expm1 -> log1p, f32[2^20]',
-                                    c1_outputs(uniform(g, -0.9, 0.9, 1 << 20)), steps, args.warmup))
+        x1 = uniform(g, -0.9, 0.9, 1 << 20)
+        others.append(side_workload('c1 shift_cyclic -> expm1 -> log1p, f32[2^20]', c1_outputs(x1), steps,
+                                    args.warmup))
+        if not args.no_cpu:
+            others[-1]['cpu_reference'] = cpu_reference(c1_outputs(x1), 'the full 2^20 elements')
         del chain
         torch.cuda.empty_cache()
         g = np.random.default_rng(3)
         xs = g.standard_normal((4096, 16384), dtype=np.float32)
         others.append(side_workload('c3 cumsum f32[4096,16384] last axis', cumsum_outputs(xs), steps, args.warmup))
+        if not args.no_cpu:
+            others[-1]['cpu_reference'] = cpu_reference(cumsum_outputs(np.ascontiguousarray(xs[:512])),
+                                                        'the first 512 rows')
         xp = uniform(g, 0.99, 1.01, (4096, 16384))
         others.append(side_workload('c3 cumprod f32[4096,16384] last axis', cumprod_outputs(xp), steps, args.warmup))
+        if not args.no_cpu:
+            others[-1]['cpu_reference'] = cpu_reference(cumprod_outputs(np.ascontiguousarray(xp[:512])),
+                                                        'the first 512 rows')
         xd = g.standard_normal((1024, 16384))
         others.append(side_workload('c3 cumsum f64[1024,16384] last axis', cumsum_outputs(xd), steps, args.warmup))
+        if not args.no_cpu:
+            others[-1]['cpu_reference'] = cpu_reference(cumsum_outputs(np.ascontiguousarray(xd[:256])),
+                                                        'the first 256 rows')
         others.append(side_workload('c3 cumsum f32[4096,16384], hand-written kernel (run-time shape, same bits)',
                                     HandWrittenScan(xs, 'ovl_cumsum_f32'), steps, args.warmup))
         others.append(side_workload('c3 cumsum f64[1024,16384], hand-written kernel (run-time shape, same bits)',
@@ -437,8 +474,13 @@ def main():
         dc = g.standard_normal((4096, 1024), dtype=np.float32)
         others.append(side_workload('c4 lstm cell forward [4096, 4x1024]', lstm_outputs(concat, c), steps,
                                     args.warmup))
+        if not args.no_cpu:
+            others[-1]['cpu_reference'] = cpu_reference(lstm_outputs(concat[:512], c[:512]), 'the first 512 rows')
         others.append(side_workload('c4 lstm cell gradient [4096, 4x1024]',
                                     lstm_grad_outputs(concat, c, dc, dh), steps, args.warmup))
+        if not args.no_cpu:
+            others[-1]['cpu_reference'] = cpu_reference(lstm_grad_outputs(concat[:512], c[:512], dc[:512], dh[:512]),
+                                                        'the first 512 rows')
         others.append(side_workload('c4 lstm cell forward, hand-written kernel (run-time shape, same bits)',
                                     HandWrittenLstm(concat, c), steps, args.warmup))
         others.append(side_workload('c4 lstm cell gradient, hand-written kernel (run-time shape, same bits)',
@@ -454,6 +496,12 @@ def main():
         b5 = torch.randn((16384 * 16384,), device='cuda', generator=g5)
         others.append(side_workload('c5 gather + transposed scatter f32[16384,16384]', gather_outputs(a5, b5),
                                     max(3, steps // 4), 2))
+        if not args.no_cpu:
+            g = np.random.default_rng(5)
+            a_small = g.standard_normal((2048, 2048), dtype=np.float32)
+            b_small = g.standard_normal(2048 * 2048, dtype=np.float32)
+            others[-1]['cpu_reference'] = cpu_reference(gather_outputs(a_small, b_small),
+                                                        'the same operator on A, B float32 [2048, 2048]')
         result['others'] = others
 
     print(json.dumps(result))
