@@ -267,7 +267,8 @@ class HandWrittenScan(object):
         self.out = torch.empty_like(self.x)
         self.rows, self.cols = self.x.shape
         self.algorithmic_bytes = 2 * self.x.numel() * self.x.element_size()
-        self.kernels = [{'kernel': 'skewed_scan_kernel'}]
+        self.kernels = [{'kernel': 'reassociated_scan_kernel' if entry.endswith('_reassociated')
+                         else 'skewed_scan_kernel'}]
 
     def launch(self, stream):
         if self.entry(self.x.data_ptr(), self.rows, self.cols, self.out.data_ptr(), stream) != 0:
@@ -467,6 +468,21 @@ def main():
                                     HandWrittenScan(xs, 'ovl_cumsum_f32'), steps, args.warmup))
         others.append(side_workload('c3 cumsum f64[1024,16384], hand-written kernel (run-time shape, same bits)',
                                     HandWrittenScan(xd, 'ovl_cumsum_f64'), steps, args.warmup))
+        # the tree-shaped wavefront scan: another association of the operands, so not the parity path; reported with
+        # its distance from the sequential result
+        for label, data, entry in (('f32[4096,16384]', xs, 'ovl_cumsum_f32'), ('f64[1024,16384]', xd, 'ovl_cumsum_f64')):
+            tree = HandWrittenScan(data, entry + '_reassociated')
+            others.append(side_workload('c3 cumsum %s, reassociating wavefront scan (not the parity path)' % label,
+                                        tree, steps, args.warmup))
+            sequential = HandWrittenScan(data, entry)
+            sequential.launch(torch.cuda.current_stream().cuda_stream)
+            torch.cuda.synchronize()
+            distance = (tree.out.double() - sequential.out.double()).abs()
+            others[-1]['vs_sequential'] = {
+                'max_abs_diff': float(distance.max()),
+                'max_abs_diff_over_max_abs_value': float(distance.max() / sequential.out.double().abs().max()),
+                'frac_bit_equal': float((tree.out == sequential.out).double().mean())}
+            del tree, sequential, distance
         g = np.random.default_rng(4)
         concat = g.standard_normal((4096, 4096), dtype=np.float32)
         c = g.standard_normal((4096, 1024), dtype=np.float32)

@@ -40,6 +40,20 @@ int ovl_cumprod_f32(const float* x, uint32_t rows, uint32_t cols, float* out, vo
 int ovl_cumsum_f64(const double* x, uint32_t rows, uint32_t cols, double* out, void* hip_stream);
 int ovl_cumprod_f64(const double* x, uint32_t rows, uint32_t cols, double* out, void* hip_stream);
 
+/*
+ * The same functions with the operands associated as a tree instead of left to right: one workgroup per row, every
+ * thread scans one 128-bit vector, the threads' totals are combined with wavefront shuffles and through LDS, the total
+ * of the steps before travels in a register.  The reference's accumulate (examples/test_accumulate.py:63-76) is the
+ * sequential recurrence, so these results are NOT its bits: they differ by rounding (for float32 sums of 16384 values
+ * of order one typically in the last one or two digits; relative to a running sum that passes near zero the distance is
+ * unbounded, as for any reordering).  In exchange the kernel runs at the speed of memory for every element type.  Rows
+ * that are not whole 16-byte aligned vectors, and 2^24 rows or more, take the order-preserving kernels above.
+ */
+int ovl_cumsum_f32_reassociated(const float* x, uint32_t rows, uint32_t cols, float* out, void* hip_stream);
+int ovl_cumprod_f32_reassociated(const float* x, uint32_t rows, uint32_t cols, float* out, void* hip_stream);
+int ovl_cumsum_f64_reassociated(const double* x, uint32_t rows, uint32_t cols, double* out, void* hip_stream);
+int ovl_cumprod_f64_reassociated(const double* x, uint32_t rows, uint32_t cols, double* out, void* hip_stream);
+
 /* Text of the last error on the calling thread ("" if none). */
 const char* ovl_scan_last_error(void);
 

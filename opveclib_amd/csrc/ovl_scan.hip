@@ -26,6 +26,11 @@
 // launcher's own
 #define OVL_EINVAL 6
 
+// steps of loads the reassociating scan keeps in flight per thread
+#ifndef OVL_SCAN_AHEAD
+#define OVL_SCAN_AHEAD 8
+#endif
+
 namespace {
 
 thread_local std::string g_last_error;
@@ -186,11 +191,146 @@ int scan(const char* who, const T* x, uint32_t rows, uint32_t cols, T* out, void
     return OVL_OK;
 }
 
+// ---------------------------------------------------------------------------------------------------------------------
+// The reassociating scan (ovl_*_reassociated): one workgroup per row, the row taken in steps of 256 vectors.  Every
+// thread scans its own 128-bit vector, the threads' totals are scanned across the wavefront with six lane-to-lane
+// steps (a tree, hence another association of the operands than the sequential recurrence), the four wavefront totals go through LDS, and the running total of the steps before is
+// carried in a register.  Data moves exactly once in coalesced 128-bit accesses, several steps of loads in flight, so
+// the kernel runs at the speed of memory whatever the latency of one addition; the price is the bits: results differ
+// from the sequential recurrence by rounding (the distance is reported by the tests and the benchmark).
+// Lane-to-lane move with a row mask: rows of 16 lanes whose bit is clear in ROW_MASK, and lanes the pattern gives no
+// source, receive `old`.
+template <int CTRL, int ROW_MASK, typename T>
+__device__ __forceinline__ T masked_lane_move(T old, T src) {
+    if constexpr (sizeof(T) == 8) {
+        const uint64_t o = __builtin_bit_cast(uint64_t, old), v = __builtin_bit_cast(uint64_t, src);
+        const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp((int)(uint32_t)o, (int)(uint32_t)v, CTRL, ROW_MASK, 0xf, false);
+        const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp((int)(uint32_t)(o >> 32), (int)(uint32_t)(v >> 32), CTRL,
+                                                                  ROW_MASK, 0xf, false);
+        return __builtin_bit_cast(T, ((uint64_t)hi << 32) | lo);
+    } else {
+        return __builtin_bit_cast(T, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, src),
+                                                                 CTRL, ROW_MASK, 0xf, false));
+    }
+}
+
+// Inclusive scan over the 64 lanes of a wavefront in six steps: lanes 1, 2, 4 and 8 below within each row of sixteen
+// (row_shr), then the last lane of row 0 into row 1 and of row 2 into row 3 (row_bcast:15), then lane 31 into rows 2
+// and 3 (row_bcast:31).  A lane without a partner combines with the value that leaves it unchanged.
+template <typename T, typename OP>
+__device__ __forceinline__ T wave_inclusive_scan(T v) {
+    const T unit = OP::template start<T>();
+    v = OP::apply(masked_lane_move<0x111, 0xf>(unit, v), v);
+    v = OP::apply(masked_lane_move<0x112, 0xf>(unit, v), v);
+    v = OP::apply(masked_lane_move<0x114, 0xf>(unit, v), v);
+    v = OP::apply(masked_lane_move<0x118, 0xf>(unit, v), v);
+    v = OP::apply(masked_lane_move<0x142, 0xa>(unit, v), v);
+    v = OP::apply(masked_lane_move<0x143, 0xc>(unit, v), v);
+    return v;
+}
+
+template <typename T, typename OP, int VEC, int AHEAD>
+__global__ void __launch_bounds__(BLOCK)
+reassociated_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t cols) {
+    typedef typename vec_of<T, VEC>::type vec;
+    __shared__ T wave_totals[2][BLOCK / WAVE];
+    const uint32_t lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+    const T* __restrict__ in_row = x + (uint64_t)blockIdx.x * cols;
+    T* __restrict__ out_row = out + (uint64_t)blockIdx.x * cols;
+    const uint32_t step_cols = BLOCK * VEC;
+    const uint32_t steps = (cols + step_cols - 1u) / step_cols;
+    T carry = OP::template start<T>();
+    uint32_t buffer = 0;
+    // a vector past the end of the row holds the value that leaves its neighbours unchanged and is not stored
+    auto fetch = [&](uint32_t step) -> vec {
+        const uint32_t col = step * step_cols + threadIdx.x * VEC;
+        vec r;
+        if (step < steps && col < cols) r = *reinterpret_cast<const vec*>(in_row + col);
+        else
+#pragma unroll
+            for (uint32_t u = 0; u < (uint32_t)VEC; ++u) r[u] = OP::template start<T>();
+        return r;
+    };
+    // AHEAD steps of loads are always in flight: a register is refilled as soon as its vector has been taken
+    vec v[AHEAD];
+#pragma unroll
+    for (uint32_t a = 0; a < (uint32_t)AHEAD; ++a) v[a] = fetch(a);
+    for (uint32_t s0 = 0; s0 < steps; s0 += AHEAD) {
+#pragma unroll
+        for (uint32_t a = 0; a < (uint32_t)AHEAD; ++a) {
+            if (s0 + a >= steps) break;         // uniform over the workgroup
+            const uint32_t col = (s0 + a) * step_cols + threadIdx.x * VEC;
+            vec mine = v[a];
+            v[a] = fetch(s0 + a + AHEAD);
+#pragma unroll
+            for (uint32_t u = 1; u < (uint32_t)VEC; ++u) mine[u] = OP::apply(mine[u - 1], mine[u]);
+            // inclusive scan of the threads' totals over the wavefront
+            const T inclusive = wave_inclusive_scan<T, OP>(mine[VEC - 1]);
+            // total of the lanes below this one (wave_shr:1; lane 0 receives the unit)
+            const T before_me = masked_lane_move<0x138, 0xf>(OP::template start<T>(), inclusive);
+            if (lane == WAVE - 1u) wave_totals[buffer][wave] = inclusive;
+            __syncthreads();
+            T base = carry, all = carry;
+#pragma unroll
+            for (uint32_t w = 0; w < BLOCK / WAVE; ++w) {
+                const T t = wave_totals[buffer][w];
+                if (w < wave) base = OP::apply(base, t);
+                all = OP::apply(all, t);
+            }
+            base = OP::apply(base, before_me);
+#pragma unroll
+            for (uint32_t u = 0; u < (uint32_t)VEC; ++u) mine[u] = OP::apply(base, mine[u]);
+            if (col < cols) __builtin_nontemporal_store(mine, reinterpret_cast<vec*>(out_row + col));
+            carry = all;
+            // the next step writes the other buffer: a thread can only get there after every thread has passed this
+            // step's barrier, and can only write this buffer again after the next barrier, behind all reads of it
+            buffer ^= 1u;
+        }
+    }
+}
+
+template <typename T, typename OP>
+int reassociated_scan(const char* who, const T* x, uint32_t rows, uint32_t cols, T* out, void* hip_stream) {
+    if (x == nullptr || out == nullptr) return fail(OVL_EINVAL, std::string(who) + ": null tensor");
+    if (rows == 0 || cols == 0) return fail(OVL_EINVAL, std::string(who) + ": rows and cols must be positive");
+    if ((uint64_t)rows * cols >= (1ull << 32)) return fail(OVL_EINVAL, std::string(who) + ": rows * cols must be below 2^32");
+    constexpr int VEC = 16 / sizeof(T), AHEAD = OVL_SCAN_AHEAD;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+    // rows of whole, aligned vectors only; anything else takes the order-preserving kernels
+    // (column indices of the last, partial step must not wrap: rows that long also go the other way)
+    if (!aligned || cols % VEC != 0 || rows >= (1u << 24) || cols > 0xffffffffu - 16u * BLOCK)
+        return scan<T, OP>(who, x, rows, cols, out, hip_stream);
+    hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    hipLaunchKernelGGL((reassociated_scan_kernel<T, OP, VEC, AHEAD>), dim3(rows), dim3(BLOCK), 0, stream, x, out, cols);
+    const hipError_t err = hipPeekAtLastError();
+    if (err != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(OVL_EHIP, std::string(who) + ": " + hipGetErrorString(err));
+    }
+    return OVL_OK;
+}
+
 }  // namespace
 
 extern "C" {
 
 const char* ovl_scan_last_error(void) { return g_last_error.c_str(); }
+
+int ovl_cumsum_f32_reassociated(const float* x, uint32_t rows, uint32_t cols, float* out, void* hip_stream) {
+    return reassociated_scan<float, op_sum>("ovl_cumsum_f32_reassociated", x, rows, cols, out, hip_stream);
+}
+
+int ovl_cumprod_f32_reassociated(const float* x, uint32_t rows, uint32_t cols, float* out, void* hip_stream) {
+    return reassociated_scan<float, op_product>("ovl_cumprod_f32_reassociated", x, rows, cols, out, hip_stream);
+}
+
+int ovl_cumsum_f64_reassociated(const double* x, uint32_t rows, uint32_t cols, double* out, void* hip_stream) {
+    return reassociated_scan<double, op_sum>("ovl_cumsum_f64_reassociated", x, rows, cols, out, hip_stream);
+}
+
+int ovl_cumprod_f64_reassociated(const double* x, uint32_t rows, uint32_t cols, double* out, void* hip_stream) {
+    return reassociated_scan<double, op_product>("ovl_cumprod_f64_reassociated", x, rows, cols, out, hip_stream);
+}
 
 int ovl_cumsum_f32(const float* x, uint32_t rows, uint32_t cols, float* out, void* hip_stream) {
     return scan<float, op_sum>("ovl_cumsum_f32", x, rows, cols, out, hip_stream);

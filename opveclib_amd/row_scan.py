@@ -5,7 +5,7 @@ Running sum and running product along the last axis with the strict left-to-righ
 ``accumulate`` operator (opveclib/examples/test_accumulate.py:22-147) - the same bits as the generated operator and as
 ``numpy.cumsum`` / ``numpy.cumprod`` - for shapes given at run time: nothing is traced, generated or compiled when they
 are called.  Inputs are float32 or float64 torch tensors on a HIP device; launches go to the current PyTorch HIP stream
-and do not synchronise.
+and do not synchronise.  ``reassociate=True`` selects the tree-shaped wavefront scan instead (not the reference's bits).
 """
 
 import ctypes
@@ -18,7 +18,10 @@ library_path = os.path.join(local.csrc_directory, 'libovl_scan.so')
 source_path = os.path.join(local.csrc_directory, 'ovl_scan.hip')
 include_directory = os.path.normpath(os.path.join(local.csrc_directory, '..', '..', 'include'))
 
-EXPORTED_SYMBOLS = ('ovl_cumsum_f32', 'ovl_cumprod_f32', 'ovl_cumsum_f64', 'ovl_cumprod_f64', 'ovl_scan_last_error')
+SCAN_SYMBOLS = ('ovl_cumsum_f32', 'ovl_cumprod_f32', 'ovl_cumsum_f64', 'ovl_cumprod_f64',
+                'ovl_cumsum_f32_reassociated', 'ovl_cumprod_f32_reassociated',
+                'ovl_cumsum_f64_reassociated', 'ovl_cumprod_f64_reassociated')
+EXPORTED_SYMBOLS = SCAN_SYMBOLS + ('ovl_scan_last_error',)
 
 
 def build(force=False):
@@ -50,7 +53,7 @@ def library():
         raise RuntimeError('The row scan library ' + library_path + ' has not been built. '
                            'Run "python -m opveclib_amd.build" first.')
     lib = ctypes.CDLL(library_path)
-    for name in EXPORTED_SYMBOLS[:4]:
+    for name in SCAN_SYMBOLS:
         fn = getattr(lib, name)
         fn.argtypes = [ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_void_p]
         fn.restype = ctypes.c_int
@@ -65,7 +68,7 @@ class RowScanError(RuntimeError):
         self.code = code
 
 
-def _scan(kind, x):
+def _scan(kind, x, reassociate=False):
     import torch
     if not isinstance(x, torch.Tensor):
         raise TypeError('x must be a torch tensor')
@@ -85,17 +88,20 @@ def _scan(kind, x):
     out = torch.empty_like(x)
     with torch.cuda.device(x.device):
         stream = torch.cuda.current_stream(x.device).cuda_stream
-        code = getattr(library(), 'ovl_' + entry)(x.data_ptr(), rows, cols, out.data_ptr(), stream)
+        entry = 'ovl_' + entry + ('_reassociated' if reassociate else '')
+        code = getattr(library(), entry)(x.data_ptr(), rows, cols, out.data_ptr(), stream)
     if code != 0:
         raise RowScanError(code, library().ovl_scan_last_error().decode('utf-8', 'replace'))
     return out
 
 
-def cumsum(x):
-    """Running sum along the last axis, accumulated strictly left to right in the dtype of ``x``."""
-    return _scan('cumsum', x)
+def cumsum(x, reassociate=False):
+    """Running sum along the last axis in the dtype of ``x``: accumulated strictly left to right (the reference's
+    bits), or with ``reassociate=True`` as a tree over the threads of a workgroup, at the speed of memory, with
+    results that differ from the sequential ones by rounding."""
+    return _scan('cumsum', x, reassociate)
 
 
-def cumprod(x):
-    """Running product along the last axis, accumulated strictly left to right in the dtype of ``x``."""
-    return _scan('cumprod', x)
+def cumprod(x, reassociate=False):
+    """Running product along the last axis in the dtype of ``x``; ``reassociate`` as for :func:`cumsum`."""
+    return _scan('cumprod', x, reassociate)

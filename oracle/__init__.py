@@ -16,6 +16,7 @@ What pins this oracle is listed in the header of :mod:`oracle.cpp_emitter`.
 import ctypes
 import hashlib
 import os
+import threading
 import subprocess
 
 import numpy as np
@@ -79,6 +80,10 @@ def hardware_threads():
     return int(driver().ovl_cpu_hardware_threads())
 
 
+_compile_locks_guard = threading.Lock()
+_compile_locks = {}
+
+
 def compile_op(dag, extra_flags=()):
     """Emit and compile one operator; returns (library path, entry name).  Cached by source text and flags."""
     name = _op_hash(dag)
@@ -87,13 +92,16 @@ def compile_op(dag, extra_flags=()):
     key = hashlib.sha224((src + ' '.join(flags)).encode('utf-8')).hexdigest()[:24]
     os.makedirs(build_directory, exist_ok=True)
     so_path = os.path.join(build_directory, 'o' + key + '_generic_cpp.so')
-    if not os.path.exists(so_path):
-        cpp_path = os.path.join(build_directory, 'o' + key + '_generic_cpp.cpp')
-        with open(cpp_path, 'w') as f:
-            f.write(src)
-        tmp = so_path + '.tmp.%d' % os.getpid()
-        _run([cxx] + flags + ['-o', tmp, cpp_path])
-        os.replace(tmp, so_path)
+    with _compile_locks_guard:
+        lock = _compile_locks.setdefault(key, threading.Lock())
+    with lock:      # threads that ask for the same operator at the same time: one compiles, the others wait
+        if not os.path.exists(so_path):
+            cpp_path = os.path.join(build_directory, 'o' + key + '_generic_cpp.cpp')
+            with open(cpp_path, 'w') as f:
+                f.write(src)
+            tmp = so_path + '.tmp.%d.%d' % (os.getpid(), threading.get_ident())
+            _run([cxx] + flags + ['-o', tmp, cpp_path])
+            os.replace(tmp, so_path)
     return so_path, name + '_generic_cpp'
 
 

@@ -34,6 +34,10 @@ def _sanitizer_runtime_directory():
     return os.path.dirname(os.path.realpath(path.strip()))
 
 
+_build_locks_guard = threading.Lock()
+_build_locks = {}
+
+
 class EmulationError(RuntimeError):
     pass
 
@@ -55,6 +59,14 @@ def build_source(source, entry, extra_flags=()):
     digest = hashlib.sha224('\0'.join(sources).encode('utf-8') + entry.encode('utf-8') + shim).hexdigest()[:32]
     os.makedirs(BUILD, exist_ok=True)
     program = os.path.join(BUILD, 'emu_' + digest)
+    with _build_locks_guard:
+        lock = _build_locks.setdefault(digest, threading.Lock())
+    with lock:      # two threads that want the same program: the second finds it built
+        _build_program(program, sources, entry, extra_flags)
+    return program
+
+
+def _build_program(program, sources, entry, extra_flags):
     if not os.path.exists(program):
         paths = []
         for k, text in enumerate(sources):
@@ -70,13 +82,18 @@ def build_source(source, entry, extra_flags=()):
         except subprocess.CalledProcessError as exception:
             raise EmulationError('host build of the generated source failed:\n' + exception.output)
         os.replace(tmp, program)
-    return program
+
+
+class _Adapter(str):
+    """Path of the hand-written kernels' program plus the adapter it is to run (see run_program)."""
+    function = None
 
 
 def build_hand_written(entry):
     """The hand-written kernel libraries (csrc/ovl_lstm.hip, csrc/ovl_scan.hip) compiled for the host together with
-    the adapters of hand_written_adapters.cpp; ``entry`` names the adapter to run.  The sources are compiled from
-    copies in the build directory, so that their ``#include "ovl_device.h"`` finds the stand-in."""
+    the adapters of hand_written_adapters.cpp, as one program for all adapters; ``entry`` names the adapter that
+    run_program is to select.  The sources are compiled from copies in the build directory, so that their
+    ``#include "ovl_device.h"`` finds the stand-in."""
     parts = []
     for name in ('ovl_lstm.hip', 'ovl_scan.hip'):
         with open(os.path.join(local.csrc_directory, name)) as f:
@@ -84,7 +101,9 @@ def build_hand_written(entry):
     with open(os.path.join(SHIM, 'hand_written_adapters.cpp')) as f:
         parts.append(f.read())
     include = os.path.normpath(os.path.join(local.csrc_directory, '..', '..', 'include'))
-    return build_source(parts, entry, ['-I' + include])
+    program = _Adapter(build_source(parts, 'emu_dispatch', ['-I' + include]))
+    program.function = entry
+    return program
 
 
 def build(op, options=None):
@@ -107,6 +126,10 @@ def run_program(program, inputs, in_types, out_types, timeout=300):
             args += [str(code), str(np.dtype(dtype).itemsize), str(int(np.prod(shape, dtype=np.int64))),
                      os.path.join(work, 'out%d' % k)]
         env = dict(os.environ, ASAN_OPTIONS='detect_leaks=0')
+        if getattr(program, 'function', None):
+            env['OVL_EMU_FUNCTION'] = program.function
+        program = str(program)
+        args[0] = program
         done = subprocess.run(args, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, universal_newlines=True,
                               timeout=timeout, env=env)
         if done.returncode != 0:

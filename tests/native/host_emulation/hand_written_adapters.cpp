@@ -42,3 +42,25 @@ OVL_EMU_SCAN(cumsum_f32, float)
 OVL_EMU_SCAN(cumprod_f32, float)
 OVL_EMU_SCAN(cumsum_f64, double)
 OVL_EMU_SCAN(cumprod_f64, double)
+OVL_EMU_SCAN(cumsum_f32_reassociated, float)
+OVL_EMU_SCAN(cumprod_f32_reassociated, float)
+OVL_EMU_SCAN(cumsum_f64_reassociated, double)
+OVL_EMU_SCAN(cumprod_f64_reassociated, double)
+
+// One program serves every adapter: the environment variable OVL_EMU_FUNCTION names the one to run.
+extern "C" int emu_dispatch(const ovl_tensor* in, uint32_t n_in, ovl_tensor* out, uint32_t n_out, void* stream) {
+    typedef int (*adapter)(const ovl_tensor*, uint32_t, ovl_tensor*, uint32_t, void*);
+    static const struct { const char* name; adapter fn; } table[] = {
+        {"emu_lstm_forward", emu_lstm_forward}, {"emu_lstm_backward", emu_lstm_backward},
+        {"emu_cumsum_f32", emu_cumsum_f32}, {"emu_cumprod_f32", emu_cumprod_f32},
+        {"emu_cumsum_f64", emu_cumsum_f64}, {"emu_cumprod_f64", emu_cumprod_f64},
+        {"emu_cumsum_f32_reassociated", emu_cumsum_f32_reassociated},
+        {"emu_cumprod_f32_reassociated", emu_cumprod_f32_reassociated},
+        {"emu_cumsum_f64_reassociated", emu_cumsum_f64_reassociated},
+        {"emu_cumprod_f64_reassociated", emu_cumprod_f64_reassociated}};
+    const char* wanted = getenv("OVL_EMU_FUNCTION");
+    for (const auto& entry : table)
+        if (wanted != nullptr && strcmp(wanted, entry.name) == 0) return entry.fn(in, n_in, out, n_out, stream);
+    fprintf(stderr, "OVL_EMU_FUNCTION names no adapter\n");
+    return OVL_EARGS;
+}

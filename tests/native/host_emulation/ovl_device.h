@@ -128,6 +128,44 @@ static inline T ovl_dpp_move(T old, T src) {
     return result;
 }
 
+// The lane-move builtin for 32-bit values with the patterns the hand-written scans use: row_shr:n (0x110 + n),
+// row_ror:1 (0x121), wave_shr:1 (0x138), row_bcast:15 (0x142), row_bcast:31 (0x143).  Rows of 16 lanes whose bit is
+// clear in row_mask, and lanes the pattern gives no source, receive `old`.
+static inline int ovl_emulated_update_dpp(int old, int src, int ctrl, int row_mask) {
+    const uint32_t t = threadIdx.x, wave = t / 64u, lane = t % 64u, row = lane / 16u, in_row = lane % 16u;
+    ovl_emulated_lane_values[t] = (uint32_t)src;
+    pthread_barrier_wait(&ovl_emulated_wave_barrier[wave]);
+    int from = -1;
+    if (ctrl > 0x110 && ctrl <= 0x11f) { if (in_row >= (uint32_t)(ctrl - 0x110)) from = (int)lane - (ctrl - 0x110); }
+    else if (ctrl == 0x121) from = (int)(row * 16u + (in_row + 15u) % 16u);
+    else if (ctrl == 0x138) { if (lane > 0u) from = (int)lane - 1; }
+    else if (ctrl == 0x142) { if (row > 0u) from = (int)(row * 16u) - 1; }
+    else if (ctrl == 0x143) { if (row > 1u) from = 31; }
+    else abort();
+    int result = old;
+    if (from >= 0 && ((row_mask >> row) & 1)) result = (int)(uint32_t)ovl_emulated_lane_values[wave * 64u + (uint32_t)from];
+    pthread_barrier_wait(&ovl_emulated_wave_barrier[wave]);
+    return result;
+}
+#define __builtin_amdgcn_update_dpp(old, src, ctrl, row_mask, bank_mask, bound_ctrl) \
+    ovl_emulated_update_dpp((old), (src), (ctrl), (row_mask))
+
+// __shfl_up: lane i receives the value of lane i - delta of its wavefront; lanes below delta keep their own.
+template <typename T>
+static inline T __shfl_up(T value, unsigned delta, int width = 64) {
+    static_assert(sizeof(T) <= 8, "shuffles carry at most 8 bytes");
+    (void)width;
+    const uint32_t t = threadIdx.x, wave = t / 64u, lane = t % 64u;
+    uint64_t bits = 0;
+    memcpy(&bits, &value, sizeof(T));
+    ovl_emulated_lane_values[t] = bits;
+    pthread_barrier_wait(&ovl_emulated_wave_barrier[wave]);
+    T result = value;
+    if (lane >= delta) memcpy(&result, &ovl_emulated_lane_values[t - delta], sizeof(T));
+    pthread_barrier_wait(&ovl_emulated_wave_barrier[wave]);
+    return result;
+}
+
 #define ovl_expf(x) ovl_math::expf_<true>((x), ovl_exp_tab)
 #define ovl_logf(x) ovl_math::logf_((x), ovl_log_tab)
 #define ovl_tanhf(x) ovl_math::tanhf_(x)

@@ -158,7 +158,7 @@ def test_scan_header_binding_and_argument_errors():
     for name in scan_declared_functions():
         assert hasattr(raw, name), name
     p = ctypes.c_void_p(64)             # never dereferenced: every call below is refused first
-    for entry in (L.ovl_cumsum_f32, L.ovl_cumprod_f32, L.ovl_cumsum_f64, L.ovl_cumprod_f64):
+    for entry in [getattr(L, name) for name in row_scan.SCAN_SYMBOLS]:
         assert entry(None, 4, 8, p, None) == launcher.OVL_EINVAL
         assert b'null' in L.ovl_scan_last_error()
         assert entry(p, 4, 8, None, None) == launcher.OVL_EINVAL

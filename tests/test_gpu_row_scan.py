@@ -70,3 +70,39 @@ def test_full_sizes_equal_the_generated_operators():
     assert torch.equal(row_scan.cumprod(xp), ovl.evaluate(cumprod(xp, axis=1)))
     xd = torch.randn((1024, 16384), device='cuda', generator=g, dtype=torch.float64)
     assert torch.equal(row_scan.cumsum(xd), ovl.evaluate(cumsum(xd, axis=1)))
+
+
+REASSOCIATED_SHAPES = [(48, 1024), (7, 256), (3, 4100), (515, 64), (4, 70, 128), (2, 16384), (5, 70), (1, 4), (4096,)]
+
+
+@pytest.mark.parametrize('dtype', [np.float32, np.float64])
+@pytest.mark.parametrize('shape', REASSOCIATED_SHAPES, ids=[str(s) for s in REASSOCIATED_SHAPES])
+def test_reassociated_scans_agree_with_the_sequential_ones_to_rounding(shape, dtype):
+    """The tree-shaped wavefront scan: not the reference's bits, but the same numbers up to rounding.  Positive
+    data, so that the relative error of the running values is meaningful."""
+    rng = np.random.default_rng(7)
+    eps = np.finfo(dtype).eps
+    for kind, fn, ref_fn in (('sum', row_scan.cumsum, np.cumsum), ('product', row_scan.cumprod, np.cumprod)):
+        x = (0.9 + 0.2 * rng.random(shape)).astype(dtype)
+        got = fn(torch.from_numpy(x).cuda(), reassociate=True).cpu().numpy()
+        ref = ref_fn(x.astype(np.float64), axis=-1)
+        assert got.dtype == x.dtype and got.shape == x.shape
+        assert np.array_equal(got[..., 0], x[..., 0])
+        # a product of n factors carries up to n roundings whatever the order; sums of positive terms far fewer
+        bound = eps * (shape[-1] if kind == 'product' else 8 * max(1.0, np.log2(shape[-1])))
+        assert np.max(np.abs(got - ref) / np.abs(ref)) <= bound, kind
+
+
+def test_reassociated_scans_at_full_size_and_their_distance_from_the_sequential_result():
+    g = torch.Generator(device='cuda')
+    g.manual_seed(3)
+    xs = torch.randn((4096, 16384), device='cuda', generator=g)
+    seq, tree = row_scan.cumsum(xs), row_scan.cumsum(xs, reassociate=True)
+    # sums of N(0, 1) values wander through zero: compare on the scale of the running sum's spread
+    assert float((seq - tree).abs().max()) <= 1e-5 * float(seq.abs().max())
+    xd = torch.randn((1024, 16384), device='cuda', generator=g, dtype=torch.float64)
+    seq, tree = row_scan.cumsum(xd), row_scan.cumsum(xd, reassociate=True)
+    assert float((seq - tree).abs().max()) <= 1e-13 * float(seq.abs().max())
+    xp = (0.99 + 0.02 * torch.rand((1024, 16384), device='cuda', generator=g, dtype=torch.float64))
+    seq, tree = row_scan.cumprod(xp), row_scan.cumprod(xp, reassociate=True)
+    assert float(((seq - tree) / seq).abs().max()) <= 1e-11

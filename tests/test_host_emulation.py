@@ -184,3 +184,26 @@ def test_hand_written_row_scans_emulated_on_the_host_equal_numpy(rows, cols, ske
         ref = (np.cumsum if 'cumsum' in name else np.cumprod)(x, axis=1, dtype=dtype)
         out = got[skew:].reshape(rows, cols)
         assert np.array_equal(out, ref) and np.array_equal(np.signbit(out), np.signbit(ref)), name
+
+
+@pytest.mark.parametrize('rows,cols,skew', [(1, 4, 0), (2, 1024, 0), (3, 2048, 0), (2, 1028, 0), (5, 4100, 0), (1, 8192, 0),
+                                            (4, 100, 0), (3, 258, 0), (2, 7, 0), (3, 64, 1)])
+def test_reassociated_row_scans_emulated_on_the_host_are_close_to_numpy(rows, cols, skew):
+    """The tree-shaped scan is not the sequential recurrence: it must agree with it to rounding (and bit for bit
+    where there is nothing to reassociate: the first column, and shapes that fall back to the sequential kernels)."""
+    rng = np.random.default_rng(rows * 1000 + cols)
+    dims = np.array([rows, cols, skew], np.uint32)
+    n = rows * cols + skew
+    for name, code, dtype, tol in (('cumsum_f32', F32, np.float32, 2e-6), ('cumprod_f32', F32, np.float32, 2e-5),
+                                   ('cumsum_f64', F64, np.float64, 1e-14), ('cumprod_f64', F64, np.float64, 1e-13)):
+        x = rng.uniform(0.9, 1.1, (rows, cols)).astype(dtype)
+        got = host_emulation.run_program(host_emulation.build_hand_written('emu_' + name + '_reassociated'),
+                                         [_skewed(x, skew), dims], [(code, dtype, [n]), (U32, np.uint32, [3])],
+                                         [(code, dtype, [n])])[0]
+        out = got[skew:].reshape(rows, cols)
+        ref = (np.cumsum if 'cumsum' in name else np.cumprod)(x.astype(np.float64), axis=1)
+        assert np.array_equal(out[:, 0], x[:, 0]), name
+        assert np.max(np.abs(out - ref) / np.abs(ref)) < tol * max(1.0, np.log2(cols)), name
+        if skew or cols % (16 // np.dtype(dtype).itemsize) != 0:
+            exact = (np.cumsum if 'cumsum' in name else np.cumprod)(x, axis=1, dtype=dtype)
+            assert np.array_equal(out, exact), name + ': sequential fallback'
