@@ -483,6 +483,10 @@ def main():
                 'max_abs_diff_over_max_abs_value': float(distance.max() / sequential.out.double().abs().max()),
                 'frac_bit_equal': float((tree.out == sequential.out).double().mean())}
             del tree, sequential, distance
+        others.append(side_workload("c3 cumsum f32[4096,16384] in the optional 'fast' math mode (generated "
+                                    "reassociating scan)", cumsum_outputs(xs), steps, args.warmup, {'math': 'fast'}))
+        others.append(side_workload("c3 cumsum f64[1024,16384] in the optional 'fast' math mode (generated "
+                                    "reassociating scan)", cumsum_outputs(xd), steps, args.warmup, {'math': 'fast'}))
         g = np.random.default_rng(4)
         concat = g.standard_normal((4096, 4096), dtype=np.float32)
         c = g.standard_normal((4096, 1024), dtype=np.float32)

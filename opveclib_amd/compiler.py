@@ -28,7 +28,7 @@ prebuild_mode = False
 #: while True, operators are compiled even when a built library exists (the "does it build" check)
 force_rebuild = False
 
-_header_paths = [os.path.join(local.csrc_directory, name) for name in ('ovl_device.h', 'ovl_math.h', 'ovl_fast_math.h')]
+_header_paths = [os.path.join(local.csrc_directory, name) for name in ('ovl_device.h', 'ovl_math.h', 'ovl_fast_math.h', 'ovl_wave_scan.h')]
 _lock = threading.Lock()
 _header_cache = []
 

@@ -12,6 +12,7 @@
 
 #include "ovl_math.h"
 #include "ovl_fast_math.h"
+#include "ovl_wave_scan.h"
 
 // Same layout as ovl_tensor in include/ovl_launch.h.
 typedef struct ovl_tensor {

@@ -198,37 +198,6 @@ int scan(const char* who, const T* x, uint32_t rows, uint32_t cols, T* out, void
 // carried in a register.  Data moves exactly once in coalesced 128-bit accesses, several steps of loads in flight, so
 // the kernel runs at the speed of memory whatever the latency of one addition; the price is the bits: results differ
 // from the sequential recurrence by rounding (the distance is reported by the tests and the benchmark).
-// Lane-to-lane move with a row mask: rows of 16 lanes whose bit is clear in ROW_MASK, and lanes the pattern gives no
-// source, receive `old`.
-template <int CTRL, int ROW_MASK, typename T>
-__device__ __forceinline__ T masked_lane_move(T old, T src) {
-    if constexpr (sizeof(T) == 8) {
-        const uint64_t o = __builtin_bit_cast(uint64_t, old), v = __builtin_bit_cast(uint64_t, src);
-        const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp((int)(uint32_t)o, (int)(uint32_t)v, CTRL, ROW_MASK, 0xf, false);
-        const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp((int)(uint32_t)(o >> 32), (int)(uint32_t)(v >> 32), CTRL,
-                                                                  ROW_MASK, 0xf, false);
-        return __builtin_bit_cast(T, ((uint64_t)hi << 32) | lo);
-    } else {
-        return __builtin_bit_cast(T, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, src),
-                                                                 CTRL, ROW_MASK, 0xf, false));
-    }
-}
-
-// Inclusive scan over the 64 lanes of a wavefront in six steps: lanes 1, 2, 4 and 8 below within each row of sixteen
-// (row_shr), then the last lane of row 0 into row 1 and of row 2 into row 3 (row_bcast:15), then lane 31 into rows 2
-// and 3 (row_bcast:31).  A lane without a partner combines with the value that leaves it unchanged.
-template <typename T, typename OP>
-__device__ __forceinline__ T wave_inclusive_scan(T v) {
-    const T unit = OP::template start<T>();
-    v = OP::apply(masked_lane_move<0x111, 0xf>(unit, v), v);
-    v = OP::apply(masked_lane_move<0x112, 0xf>(unit, v), v);
-    v = OP::apply(masked_lane_move<0x114, 0xf>(unit, v), v);
-    v = OP::apply(masked_lane_move<0x118, 0xf>(unit, v), v);
-    v = OP::apply(masked_lane_move<0x142, 0xa>(unit, v), v);
-    v = OP::apply(masked_lane_move<0x143, 0xc>(unit, v), v);
-    return v;
-}
-
 template <typename T, typename OP, int VEC, int AHEAD>
 __global__ void __launch_bounds__(BLOCK)
 reassociated_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t cols) {
@@ -265,9 +234,9 @@ reassociated_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t 
 #pragma unroll
             for (uint32_t u = 1; u < (uint32_t)VEC; ++u) mine[u] = OP::apply(mine[u - 1], mine[u]);
             // inclusive scan of the threads' totals over the wavefront
-            const T inclusive = wave_inclusive_scan<T, OP>(mine[VEC - 1]);
-            // total of the lanes below this one (wave_shr:1; lane 0 receives the unit)
-            const T before_me = masked_lane_move<0x138, 0xf>(OP::template start<T>(), inclusive);
+            const T unit = OP::template start<T>();
+            const T inclusive = ovl_wave_inclusive_scan(mine[VEC - 1], unit, [](T a, T b) { return OP::apply(a, b); });
+            const T before_me = ovl_wave_shift_up(inclusive, unit);     // total of the lanes below this one
             if (lane == WAVE - 1u) wave_totals[buffer][wave] = inclusive;
             __syncthreads();
             T base = carry, all = carry;

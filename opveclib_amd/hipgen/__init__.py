@@ -26,7 +26,7 @@ from . import tile_kernel
 from . import rowscan_kernel
 
 #: bump when generated code changes for an unchanged DAG, so cached binaries are not reused
-CODEGEN_VERSION = 24
+CODEGEN_VERSION = 25
 
 
 
@@ -58,7 +58,7 @@ def generate(expression_dag, function_name, options=None):
     """
     :param expression_dag: serialised expression DAG of one operator
     :param function_name: unique name of the operator (its content hash)
-    :param options: optional dict.  ``template``: 'auto' (default), 'map', 'transpose', 'rowscan' or 'skewscan' restricts
+    :param options: optional dict.  ``template``: 'auto' (default), 'map', 'transpose', 'rowscan', 'skewscan' or 'treescan' restricts
         the choice of kernel template (a template that does not fit the DAG falls back to 'map'); ``vec`` forces the
         map template with that vector width; ``scan_depth`` / ``scan_sets`` / ``scan_width`` / ``scan_interleave`` set the request burst (groups), the
         number of register sets, the 128-bit vectors per lane and phase and the rows per lane group of the lane-skewed scan; ``math``: 'exact'
@@ -80,7 +80,15 @@ def generate(expression_dag, function_name, options=None):
         kernel_name += '_' + info.math         # so that profiles tell the math modes of one operator apart
 
     template = options.get('template', 'auto')
-    if options.get('vec') is None and template in ('auto', 'skewscan') and rowscan_kernel.skew_plan(info) is not None:
+    tree = None
+    if options.get('vec') is None and (template == 'treescan' or (template == 'auto' and info.math == 'fast')):
+        tree = rowscan_kernel.tree_plan(info)
+        if tree is not None and (tree[0].length % tree[0].vec != 0 or tree[0].rows > MAX_GRID):
+            tree = None
+    if tree is not None:
+        # sums, products and running extrema whose order the caller has given up: the reassociating scan
+        kernel_src, launch = rowscan_kernel.generate_tree(info, kernel_name, options.get('scan_ahead') or 8)
+    elif options.get('vec') is None and template in ('auto', 'skewscan') and rowscan_kernel.skew_plan(info) is not None:
         kernel_src, launch = rowscan_kernel.generate_skewed(info, kernel_name, options.get('scan_depth'), options.get('scan_sets'), options.get('scan_nt', 's'),
                                                              options.get('scan_width'), options.get('scan_interleave'))
     elif options.get('vec') is None and template in ('auto', 'rowscan') and rowscan_kernel.plan(info) is not None:

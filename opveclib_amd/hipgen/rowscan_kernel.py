@@ -336,6 +336,156 @@ def skew_plan(info):
     return p
 
 
+TREE_OPS = (lang.ADD, lang.MULTIPLY, lang.MIN, lang.MAX)
+
+
+def tree_plan(info):
+    """
+    (ScanPlan, operation code) when the DAG is exactly ``acc = x[., 0]; out[., 0] = acc; for i in 1..n-1:
+    acc = op(acc, x[., i]); out[., i] = acc`` with op one of +, *, min, max: the scans whose operands may be
+    associated as a tree when the caller gives up the sequential order (math mode 'fast').  Else None.
+    """
+    p = plan(info)
+    if p is None:
+        return None
+    state = _carried_state(info, p)
+    if len(state) != 1:
+        return None
+    s = state[0]
+    if info.nodes[s].dtype != p.x.dtype:
+        return None
+    loads = {False: [], True: []}
+    assigns = {False: [], True: []}
+    stores = {False: [], True: []}
+    for node in info.nodes:
+        inside = bool(info.in_loop[node.idx])
+        if node.code == lang.READ_TENSOR and info.nodes[node.ops[0]].code == lang.INPUT:
+            loads[inside].append(node)
+        elif node.code == lang.ASSIGN_VARIABLE and node.ops[0] != p.counter:
+            assigns[inside].append(node)
+        elif node.code == lang.ASSIGN_TENSOR:
+            stores[inside].append(node)
+    for inside in (False, True):
+        if len(loads[inside]) != 1 or len(assigns[inside]) != 1 or len(stores[inside]) != 1:
+            return None
+        assign, store = assigns[inside][0], stores[inside][0]
+        if assign.ops[0] != s or store.ops[2] != s or store.idx < assign.idx:
+            return None
+    if assigns[False][0].ops[1] != loads[False][0].idx:         # acc = x[., 0]
+        return None
+    update = info.nodes[assigns[True][0].ops[1]]                # acc = op(acc, x[., i]) in either operand order
+    if update.code not in TREE_OPS or sorted(update.ops) != sorted([s, loads[True][0].idx]):
+        return None
+    return p, update.code
+
+
+def _tree_unit(code, dtype):
+    """C text of the value u with op(u, x) == x for every x (for the sum -0, which also keeps the sign of a zero)."""
+    floating = dtype in (lang.FLOAT32, lang.FLOAT64)
+    if code == lang.ADD:
+        return '-0.0' if floating else '0'
+    if code == lang.MULTIPLY:
+        return '1'
+    limits = {lang.INT32: ('INT32_MIN', 'INT32_MAX'), lang.INT64: ('INT64_MIN', 'INT64_MAX'),
+              lang.UINT32: ('0u', 'UINT32_MAX'), lang.UINT64: ('0ull', 'UINT64_MAX')}
+    if floating:
+        lowest, highest = '(-__builtin_inf())', '__builtin_inf()'
+    else:
+        lowest, highest = limits[dtype]
+    return highest if code == lang.MIN else lowest
+
+
+def generate_tree(info, kernel_name, ahead=8):
+    """
+    The reassociating row scan: one workgroup per row, the row in steps of 256 vectors.  Every thread scans its own
+    128-bit vector, the threads' totals are scanned over the wavefront with lane-to-lane moves, the four wavefront
+    totals go through a double-buffered LDS array (one barrier per step), the total of the steps before travels in a
+    register; ``ahead`` steps of loads stay in flight.  The kernel runs at the speed of memory, but associates the
+    operands as a tree: its results differ from the sequential recurrence by rounding, so it is only chosen in the
+    'fast' math mode.
+    """
+    from .body import binary_text
+    p, code = tree_plan(info)
+    ctype = CTYPE[p.x.dtype]
+    vec = p.vec
+    if p.length % vec != 0:
+        raise ValueError('the reassociating scan needs rows of whole vectors')
+    step_cols = BLOCK * vec
+    steps = (p.length + step_cols - 1) // step_cols
+    ahead = max(1, min(ahead, steps))
+    unit = '(%s)(%s)' % (ctype, _tree_unit(code, p.x.dtype))
+    src = []
+    src.append('typedef %s ovl_scan_vec __attribute__((ext_vector_type(%d)));' % (ctype, vec))
+    src.append('#define OVL_TREE_OP(a, b) (%s)' % binary_text(code, p.x.dtype, 'a', 'b'))
+    src.append('')
+    src.append('extern "C" __global__ void __launch_bounds__(%d)' % BLOCK)
+    src.append('%s(const %s* __restrict__ in%d, %s* __restrict__ out%d) {' % (
+        kernel_name, ctype, p.x.io_index, ctype, p.out.io_index))
+    src.append('    __shared__ %s wave_totals[2][%d];' % (ctype, BLOCK // WAVE))
+    src.append('    const uint32_t lane = threadIdx.x %% %du, wave = threadIdx.x / %du;' % (WAVE, WAVE))
+    src.append('    const %s* __restrict__ in_row = in%d + (uint64_t)blockIdx.x * %dull;' % (ctype, p.x.io_index, p.length))
+    src.append('    %s* __restrict__ out_row = out%d + (uint64_t)blockIdx.x * %dull;' % (ctype, p.out.io_index, p.length))
+    src.append('    const %s unit = %s;' % (ctype, unit))
+    src.append('    auto combine = [](%s a, %s b) -> %s { return OVL_TREE_OP(a, b); };' % (ctype, ctype, ctype))
+    src.append('    // a vector past the end of the row holds the unit and is not stored')
+    src.append('    auto fetch = [&](uint32_t step) -> ovl_scan_vec {')
+    src.append('        const uint32_t col = step * %du + threadIdx.x * %du;' % (step_cols, vec))
+    src.append('        ovl_scan_vec r;')
+    src.append('        if (step < %du && col < %du) r = *reinterpret_cast<const ovl_scan_vec*>(in_row + col);' % (steps, p.length))
+    src.append('        else')
+    src.append('            #pragma unroll')
+    src.append('            for (uint32_t u = 0; u < %du; ++u) r[u] = unit;' % vec)
+    src.append('        return r;')
+    src.append('    };')
+    src.append('    %s carry = unit;' % ctype)
+    src.append('    uint32_t buffer = 0;')
+    src.append('    // %d steps of loads are always in flight: a register is refilled as soon as its vector has been taken' % ahead)
+    src.append('    ovl_scan_vec v[%d];' % ahead)
+    src.append('    #pragma unroll')
+    src.append('    for (uint32_t a = 0; a < %du; ++a) v[a] = fetch(a);' % ahead)
+    src.append('    for (uint32_t s0 = 0; s0 < %du; s0 += %du) {' % (steps, ahead))
+    src.append('        #pragma unroll')
+    src.append('        for (uint32_t a = 0; a < %du; ++a) {' % ahead)
+    src.append('            if (s0 + a >= %du) break;        // uniform over the workgroup' % steps)
+    src.append('            const uint32_t col = (s0 + a) * %du + threadIdx.x * %du;' % (step_cols, vec))
+    src.append('            ovl_scan_vec mine = v[a];')
+    src.append('            v[a] = fetch(s0 + a + %du);' % ahead)
+    src.append('            #pragma unroll')
+    src.append('            for (uint32_t u = 1; u < %du; ++u) mine[u] = combine(mine[u - 1], mine[u]);' % vec)
+    src.append('            const %s inclusive = ovl_wave_inclusive_scan(mine[%d], unit, combine);' % (ctype, vec - 1))
+    src.append('            const %s before_me = ovl_wave_shift_up(inclusive, unit);      // total of the lanes below' % ctype)
+    src.append('            if (lane == %du) wave_totals[buffer][wave] = inclusive;' % (WAVE - 1))
+    src.append('            __syncthreads();')
+    src.append('            %s base = carry, all = carry;' % ctype)
+    src.append('            #pragma unroll')
+    src.append('            for (uint32_t w = 0; w < %du; ++w) {' % (BLOCK // WAVE))
+    src.append('                const %s t = wave_totals[buffer][w];' % ctype)
+    src.append('                if (w < wave) base = combine(base, t);')
+    src.append('                all = combine(all, t);')
+    src.append('            }')
+    src.append('            base = combine(base, before_me);')
+    src.append('            #pragma unroll')
+    src.append('            for (uint32_t u = 0; u < %du; ++u) mine[u] = combine(base, mine[u]);' % vec)
+    src.append('            if (col < %du) __builtin_nontemporal_store(mine, reinterpret_cast<ovl_scan_vec*>(out_row + col));' % p.length)
+    src.append('            carry = all;')
+    src.append('            // the next step writes the other buffer; this one is written again only behind another barrier')
+    src.append('            buffer ^= 1u;')
+    src.append('        }')
+    src.append('    }')
+    src.append('}')
+    src.append('#undef OVL_TREE_OP')
+    launch = {
+        'template': 'treescan',
+        'vec': vec,
+        'block': BLOCK,
+        'blocks_needed': p.rows,
+        'align': {('in', p.x.io_index): 16, ('out', p.out.io_index): 16},
+        'vector_loads': 1,
+        'vector_stores': 1,
+    }
+    return '\n'.join(src) + '\n', launch
+
+
 def _default_interleave(rows, vec):
     """Rows per lane group of the lane-skewed scan when the caller does not say."""
     return 1

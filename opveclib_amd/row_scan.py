@@ -27,7 +27,8 @@ EXPORTED_SYMBOLS = SCAN_SYMBOLS + ('ovl_scan_last_error',)
 def build(force=False):
     """Compile the library with hipcc next to its source (same flags as generated operators); returns its path."""
     from .compiler import HIPCC_FLAGS
-    newest = max(os.path.getmtime(p) for p in (source_path, os.path.join(local.csrc_directory, 'ovl_device.h')))
+    newest = max(os.path.getmtime(p) for p in (source_path, os.path.join(local.csrc_directory, 'ovl_device.h'),
+                                                 os.path.join(local.csrc_directory, 'ovl_wave_scan.h')))
     if not force and os.path.exists(library_path) and os.path.getmtime(library_path) >= newest:
         return library_path
     tmp = library_path + '.tmp.%d' % os.getpid()

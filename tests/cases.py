@@ -811,6 +811,10 @@ TEMPLATE_VARIANTS = [
 # fused cases also evaluated end to end in 'fast' mode (tolerance on the absolute error, see the test)
 FAST_FUSED_CASES = ['c2_chain', 'c4_lstm', 'c4_lstm_grad', 'c1_shift_expm1_log1p', 'bounded_mix']
 
+# row scans that the 'fast' math mode may run as a reassociating (tree-shaped) scan: sums, products, running extrema
+FAST_SCAN_CASES = ['c3_cumsum_f32', 'c3_cumprod_f32', 'c3_cumsum_f64', 'c3_cumprod_f64', 'c3_rowscan_shapes',
+                   'int_accumulate', 'accumulate_max', 'accumulate_axes']
+
 
 def run_variant_on_gpu(name, options):
     from opveclib_amd import runtime
@@ -851,7 +855,7 @@ def prebuild_all(cases=None, workers=8, with_oracle=True, force_benchmark=False)
             for op in _operators_of(outs, 0):
                 variants.append((op, {'math': 'fast'}))
                 oracle_ops[op.SerializeToString()] = op
-        for name in FAST_FUSED_CASES:
+        for name in FAST_FUSED_CASES + FAST_SCAN_CASES:
             for op in _operators_of(CASE_BY_NAME[name].outputs(), 3):
                 variants.append((op, {'math': 'fast'}))
         from tests import random_programs

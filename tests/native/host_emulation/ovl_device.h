@@ -149,6 +149,7 @@ static inline int ovl_emulated_update_dpp(int old, int src, int ctrl, int row_ma
 }
 #define __builtin_amdgcn_update_dpp(old, src, ctrl, row_mask, bank_mask, bound_ctrl) \
     ovl_emulated_update_dpp((old), (src), (ctrl), (row_mask))
+#include "ovl_wave_scan.h"
 
 // __shfl_up: lane i receives the value of lane i - delta of its wavefront; lanes below delta keep their own.
 template <typename T>

@@ -67,3 +67,33 @@ def test_math_mode_default_and_errors():
     exact = ovl.evaluate(cases.stdops.tanh(x), math_mode='exact')
     assert cases.ulp_distance(fast, exact).max() <= 2
     assert np.array_equal(exact, oracle.evaluate(cases.stdops.tanh(x)))
+
+
+def _assert_scan_close(name, got, ref):
+    assert got.dtype == ref.dtype and got.shape == ref.shape, name
+    if ref.dtype.kind != 'f':
+        assert np.array_equal(got, ref), name          # integer sums and extrema do not depend on the association
+        return
+    # rounding differences of a reordered sum or product, on the scale of the largest running value of the row
+    scale = np.max(np.abs(ref), axis=-1, keepdims=True) + np.finfo(ref.dtype).tiny
+    bound = np.finfo(ref.dtype).eps * 4 * ref.shape[-1]
+    assert np.max(np.abs(got.astype(np.float64) - ref.astype(np.float64)) / scale) <= bound, name
+
+
+@pytest.mark.parametrize('name', cases.FAST_SCAN_CASES)
+def test_fast_mode_scans_agree_with_the_oracle_to_rounding(name):
+    """In the 'fast' math mode sums, products and running extrema along the last axis run as the reassociating
+    wavefront scan: the same numbers as the oracle's sequential recurrence up to rounding, running extrema and
+    integer results bit for bit."""
+    import oracle
+    from opveclib_amd import runtime
+    case = cases.CASE_BY_NAME[name]
+    outs = case.outputs()
+    ref = oracle.profile(outs, 1, 0)[0]
+    got = ovl.evaluate(outs, opt_level=3, math_mode='fast')
+    got = got if isinstance(got, list) else [got]
+    for k, (g, r) in enumerate(zip(got, ref)):
+        _assert_scan_close('%s output %d' % (name, k), g, r)
+    templates = [c.lib.info['template'] for key, c in runtime._loaded.items() if "'math', 'fast'" in key[1]]
+    if name.startswith('c3_cum'):
+        assert 'treescan' in templates

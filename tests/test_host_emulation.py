@@ -207,3 +207,20 @@ def test_reassociated_row_scans_emulated_on_the_host_are_close_to_numpy(rows, co
         if skew or cols % (16 // np.dtype(dtype).itemsize) != 0:
             exact = (np.cumsum if 'cumsum' in name else np.cumprod)(x, axis=1, dtype=dtype)
             assert np.array_equal(out, exact), name + ': sequential fallback'
+
+
+@pytest.mark.parametrize('name', ['c3_cumsum_f32', 'c3_cumprod_f64', 'c3_rowscan_shapes', 'int_accumulate',
+                                  'accumulate_max'])
+def test_generated_reassociating_scans_emulated_on_the_host(name):
+    """The scans the 'fast' math mode runs as a tree (sums, products, running extrema): close to the oracle's
+    sequential results, integer sums and extrema equal to them, no access outside a tensor."""
+    outs = cases.CASE_BY_NAME[name].outputs()
+    ref = oracle.profile(outs, 1, 0)[0]
+    got = host_emulation.evaluate(outs, 3, {'math': 'fast'})
+    for g, r in zip(got, ref):
+        assert g.dtype == r.dtype and g.shape == r.shape
+        if r.dtype.kind != 'f':
+            assert np.array_equal(g, r)
+        else:
+            scale = np.max(np.abs(r), axis=-1, keepdims=True) + np.finfo(r.dtype).tiny
+            assert np.max(np.abs(g.astype(np.float64) - r.astype(np.float64)) / scale) <= np.finfo(r.dtype).eps * 4 * r.shape[-1]
