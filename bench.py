@@ -367,7 +367,9 @@ def main():
     parser.add_argument('--steps', type=int, default=100)
     parser.add_argument('--warmup', type=int, default=100)
     parser.add_argument('--no-others', action='store_true', help='skip the secondary configurations')
-    parser.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline')
+    parser.add_argument('--no-cpu', action='store_true',
+                        help='skip what starts other programs: the CPU baseline (compiler) and the clock reading '
+                             '(rocm-smi); for runs under a profiler')
     args = parser.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)' % args.gpus)
@@ -401,7 +403,7 @@ def main():
                    'algorithmic_bytes': nbytes, 'kernel': chain.kernels[0]['kernel'],
                    'pct_of_hbm_peak': round(100.0 * value / HBM_PEAK_GBPS, 2),
                    'clock_settling_launches_before_warmup': settled_after,
-                   'clocks_under_load': clocks_under_load(chain)},
+                   'clocks_under_load': None if args.no_cpu else clocks_under_load(chain)},
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
                      'frac': round(achieved / HBM_PEAK_GBPS, 4), 'traffic': CHAIN8_TRAFFIC_BYTES,
                      'kernel_us': round(event_ms * 1e3, 2), 'kernel_min_us': round(min_ms * 1e3, 2)},
