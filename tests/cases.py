@@ -877,6 +877,7 @@ def prebuild_all(cases=None, workers=8, with_oracle=True, force_benchmark=False)
             program = random_programs.scan_application(seed).expression_dag
             ops[program.SerializeToString()] = program
             oracle_ops[program.SerializeToString()] = program
+            variants.append((program, {'math': 'fast'}))
         for seed in random_programs.DAG_SEEDS:
             outs = random_programs.random_dag(seed)
             for level in (0, 3):

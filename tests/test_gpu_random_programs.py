@@ -73,6 +73,17 @@ def test_random_scan_program_equals_the_oracle(seed):
         runtime.poison_outputs = False
     assert got.dtype == ref.dtype and got.shape == ref.shape
     assert np.array_equal(got, ref, equal_nan=(ref.dtype.kind == 'f')), 'seed %d' % seed
+    # the 'fast' math mode may run plain sums, products and running extrema as a tree: integer results stay equal,
+    # floating point ones agree to rounding; every other scan body keeps its order and its bits
+    from opveclib_amd import hipgen
+    fast = ovl.evaluate(out, opt_level=3, math_mode='fast')
+    template = hipgen.generate(out.parent.expression_dag, 'f' * 57, {'math': 'fast'}).launch['template']
+    if template == 'treescan' and ref.dtype.kind == 'f':
+        scale = np.max(np.abs(ref), axis=-1, keepdims=True) + np.finfo(ref.dtype).tiny
+        assert np.max(np.abs(fast.astype(np.float64) - ref.astype(np.float64)) / scale) <= \
+            np.finfo(ref.dtype).eps * 4 * ref.shape[-1], 'seed %d fast' % seed
+    else:
+        assert np.array_equal(fast, ref, equal_nan=(ref.dtype.kind == 'f')), 'seed %d fast (%s)' % (seed, template)
 
 
 @pytest.mark.parametrize('seed', random_programs.TYPED_SEEDS)
