@@ -26,7 +26,7 @@ from . import tile_kernel
 from . import rowscan_kernel
 
 #: bump when generated code changes for an unchanged DAG, so cached binaries are not reused
-CODEGEN_VERSION = 25
+CODEGEN_VERSION = 26
 
 
 
@@ -84,6 +84,10 @@ def generate(expression_dag, function_name, options=None):
     if options.get('vec') is None and (template == 'treescan' or (template == 'auto' and info.math == 'fast')):
         tree = rowscan_kernel.tree_plan(info)
         if tree is not None and (tree[0].length % tree[0].vec != 0 or tree[0].rows > MAX_GRID):
+            tree = None
+        # one workgroup per row pays from about one full step (256 vectors) per row; shorter rows keep the lane-skewed
+        # scan, which packs sixteen rows into a workgroup
+        if tree is not None and template == 'auto' and tree[0].length < 256 * tree[0].vec:
             tree = None
     if tree is not None:
         # sums, products and running extrema whose order the caller has given up: the reassociating scan
