@@ -26,7 +26,7 @@ from . import tile_kernel
 from . import rowscan_kernel
 
 #: bump when generated code changes for an unchanged DAG, so cached binaries are not reused
-CODEGEN_VERSION = 26
+CODEGEN_VERSION = 27
 
 
 
@@ -81,8 +81,13 @@ def generate(expression_dag, function_name, options=None):
 
     template = options.get('template', 'auto')
     tree = None
-    if options.get('vec') is None and (template == 'treescan' or (template == 'auto' and info.math == 'fast')):
+    if options.get('vec') is None and template in ('auto', 'treescan'):
         tree = rowscan_kernel.tree_plan(info)
+        # integer sums, products and extrema are associative (sums and products modulo 2^n): the tree gives the
+        # reference's bits; floating point ones only when the caller has given up the order
+        if tree is not None and template == 'auto' and info.math != 'fast' and \
+                tree[0].x.dtype in (lang.FLOAT32, lang.FLOAT64):
+            tree = None
         if tree is not None and (tree[0].length % tree[0].vec != 0 or tree[0].rows > MAX_GRID):
             tree = None
         # one workgroup per row pays from about one full step (256 vectors) per row; shorter rows keep the lane-skewed

@@ -416,7 +416,14 @@ def generate_tree(info, kernel_name, ahead=8):
     unit = '(%s)(%s)' % (ctype, _tree_unit(code, p.x.dtype))
     src = []
     src.append('typedef %s ovl_scan_vec __attribute__((ext_vector_type(%d)));' % (ctype, vec))
-    src.append('#define OVL_TREE_OP(a, b) (%s)' % binary_text(code, p.x.dtype, 'a', 'b'))
+    unsigned = {lang.INT32: 'uint32_t', lang.INT64: 'uint64_t'}.get(p.x.dtype)
+    if unsigned is not None and code in (lang.ADD, lang.MULTIPLY):
+        # partial sums and products of a tree may pass the limits of a signed type where the sequential order does
+        # not: formed in the unsigned type (arithmetic modulo 2^n, always defined) they end in the same bits
+        text = '(%s)(%s)' % (ctype, binary_text(code, p.x.dtype, '(%s)(a)' % unsigned, '(%s)(b)' % unsigned))
+        src.append('#define OVL_TREE_OP(a, b) (%s)' % text)
+    else:
+        src.append('#define OVL_TREE_OP(a, b) (%s)' % binary_text(code, p.x.dtype, 'a', 'b'))
     src.append('')
     src.append('extern "C" __global__ void __launch_bounds__(%d)' % BLOCK)
     src.append('%s(const %s* __restrict__ in%d, %s* __restrict__ out%d) {' % (

@@ -491,6 +491,20 @@ def _accumulate_axes(rng):
     return outs
 
 
+def _int_tree_scans(rng):
+    """Integer sums, products, minima and maxima over rows long enough for the tree-shaped scan, values that wrap."""
+    outs = []
+    for dtype in (np.int32, np.int64, np.uint32, np.uint64):
+        info = np.iinfo(dtype)
+        big = rng.integers(info.min // 2, info.max // 2, (6, 2048), dtype=dtype)      # sums wrap around
+        small = rng.integers(0 if info.min == 0 else -3, 4, (5, 4096)).astype(dtype)
+        outs.append(cumsum(big, axis=1)[0])
+        outs.append(cumprod(small | dtype(1), axis=1)[0])                              # odd factors: products wrap
+        outs.append(accumulate(big, inner_fcn=lambda acc, x: ovl.maximum(acc, x), axis=1)[0])
+        outs.append(accumulate(big, inner_fcn=lambda acc, x: ovl.minimum(x, acc), axis=1)[0])
+    return outs
+
+
 def _accumulate_max(rng):
     a = rng.standard_normal((9, 130), dtype=np.float32)
     return [accumulate(a, inner_fcn=lambda acc, x: ovl.maximum(acc, x), axis=1)[0]]
@@ -598,6 +612,7 @@ CASES = [
     _simple('int_accumulate', _int_accumulate),
     _simple('accumulate_axes', _accumulate_axes),
     _simple('accumulate_max', _accumulate_max),
+    _simple('int_tree_scans', _int_tree_scans),
     _simple('edge_expm1_log1p', _edge_expm1_log1p, max_ulp=2, rel=1e-12),
     _simple('odd_sizes', _odd_sizes),
     _simple('adopted_position', _adopted_position),
