@@ -502,6 +502,9 @@ def _int_tree_scans(rng):
         outs.append(cumprod(small | dtype(1), axis=1)[0])                              # odd factors: products wrap
         outs.append(accumulate(big, inner_fcn=lambda acc, x: ovl.maximum(acc, x), axis=1)[0])
         outs.append(accumulate(big, inner_fcn=lambda acc, x: ovl.minimum(x, acc), axis=1)[0])
+    # rows that end inside a step of 256 vectors
+    outs.append(cumsum(rng.integers(-1000, 1000, (3, 1088)).astype(np.int32), axis=1)[0])
+    outs.append(cumsum(rng.integers(-1000, 1000, (2, 2112)).astype(np.int64), axis=1)[0])
     return outs
 
 
