@@ -351,3 +351,23 @@ def test_known_answer_fixtures():
             assert got.dtype == expected.dtype and np.array_equal(got, expected), name
         names.append(name)
     assert len(names) == 8
+
+
+def test_integer_accumulates_wrap_like_numpy():
+    """Sums and products of 32- and 64-bit integers that pass the limits of their type, running extrema: the oracle's
+    sequential C loop against numpy's accumulate in the same type (numpy wraps modulo 2^n; the generated C for signed
+    types is compiled without optimisation and wraps as well).  This pins the oracle for the cases the tree-shaped
+    integer scan is compared with."""
+    from opveclib_amd.examples import accumulate
+    rng = np.random.default_rng(17)
+    for dtype in (np.int32, np.int64, np.uint32, np.uint64):
+        info = np.iinfo(dtype)
+        big = rng.integers(info.min // 2, info.max // 2, (3, 700), dtype=dtype)
+        odd = (rng.integers(0 if info.min == 0 else -3, 4, (2, 900)).astype(dtype)) | dtype(1)
+        with np.errstate(over='ignore'):
+            assert np.array_equal(oracle.evaluate(cumsum(big, axis=1)), np.cumsum(big, axis=1, dtype=dtype))
+            assert np.array_equal(oracle.evaluate(cumprod(odd, axis=1)), np.cumprod(odd, axis=1, dtype=dtype))
+        assert np.array_equal(oracle.evaluate(accumulate(big, inner_fcn=lambda a, x: ovl.maximum(a, x), axis=1)),
+                              np.maximum.accumulate(big, axis=1))
+        assert np.array_equal(oracle.evaluate(accumulate(big, inner_fcn=lambda a, x: ovl.minimum(x, a), axis=1)),
+                              np.minimum.accumulate(big, axis=1))
