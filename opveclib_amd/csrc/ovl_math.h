@@ -319,7 +319,7 @@ OVL_HD float tanh_div_(float a, float b) {
 #ifndef OVL_TANH_DIV
 #define OVL_TANH_DIV(a, b) ((a) / (b))
 #endif
-OVL_HD float tanhf_(float x) {
+OVL_HD float tanhf_general_(float x) {
     const float one = 1.0f, two = 2.0f, tiny = 1.0e-30f;
     const float ln2_hi = 6.9313812256e-01f, ln2_lo = 9.0580006145e-06f, invln2 = 1.4426950216e+00f;
     const float Q1 = -3.3333335072e-02f, Q2 = 1.5873016091e-03f, Q3 = -7.9365076090e-05f;
@@ -384,6 +384,62 @@ OVL_HD float tanhf_(float x) {
         if (ix >= 0x41b00000u) fixed = negative ? -(one - tiny) : (one - tiny);
         if (ix >= 0x7f800000u) fixed = negative ? one / x - one : one / x + one;    // +-1 for infinities, NaN for NaN
         result = special ? fixed : result;
+    }
+    return result;
+}
+
+// tanhf_: the routine generated code calls.  For |x| < 7.5 the quotient k of the argument reduction can only
+// be 0, -1, -2 or -3 (|x| < 1) or 3 .. 22 (|x| >= 1), so of fdlibm's result formulas only four remain and the one for
+// |x| >= 1 is chosen by the comparison that is needed anyway; every other argument (NaN, infinities, large
+// magnitudes) goes to tanhf_general_ inside a block that is entered only if some lane of the wavefront needs it.
+// Same operations on the same operands as tanhf_general_ for the arguments it keeps, hence the same bits (compared
+// with the host library over all 2^32 arguments, on the host and on the GPU).
+OVL_HD float tanhf_(float x) {
+    const float one = 1.0f, two = 2.0f;
+    const float ln2_hi = 6.9313812256e-01f, ln2_lo = 9.0580006145e-06f, invln2 = 1.4426950216e+00f;
+    const float Q1 = -3.3333335072e-02f, Q2 = 1.5873016091e-03f, Q3 = -7.9365076090e-05f;
+    const float Q4 = 4.0082177293e-06f, Q5 = -2.0109921195e-07f;
+
+    uint32_t jx = as_u32(x);
+    uint32_t ix = jx & 0x7fffffffu;
+    float ax = as_f32(ix);
+    bool big = ix >= 0x3f800000u;                   // |x| >= 1
+    float a = big ? two * ax : -two * ax;           // argument of expm1
+    int32_t k = (int32_t)(invln2 * a + (big ? 0.5f : -0.5f));
+    float t = (float)k;
+    float hi = a - t * ln2_hi;
+    float lo = t * ln2_lo;
+    float xr = hi - lo;
+    float c = (hi - xr) - lo;
+
+    float hfx = 0.5f * xr;
+    float hxs = xr * hfx;
+    float r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
+    float t3 = 3.0f - r1 * hfx;
+    float e = hxs * OVL_TANH_DIV(r1 - t3, 6.0f - xr * t3);
+
+    float e2 = xr * (e - c) - c;
+    e2 -= hxs;
+    float d = e2 - xr;
+    float res0 = -d;                                // k == 0
+    float resm1 = 0.5f * (-d) - 0.5f;               // k == -1
+    // k <= -2: (1 - d) * 2^k - 1;  3 <= k < 23: ((1 - 2^-k) - d) * 2^k
+    uint32_t ks = (uint32_t)k & 31u;
+    float base = big ? as_f32(0x3f800000u - (0x1000000u >> ks)) : one;
+    float y = base - d;
+    y = as_f32(as_u32(y) + ((uint32_t)k << 23));    // add k to y's exponent
+    float small_em1 = (k == 0) ? res0 : ((k == -1) ? resm1 : y - one);
+    float em1 = big ? y : small_em1;
+
+    float q = OVL_TANH_DIV(big ? two : -em1, em1 + two);
+    float z = big ? one - q : q;
+    float result = as_f32(as_u32(z) | (jx & 0x80000000u));      // z >= +0: give it the sign of x
+    // (zero and tiny arguments need no special case: with k == 0 the formulas above return x itself, as fdlibm's
+    // x * (1 + x) does)
+    const bool special = ix >= 0x40f00000u;         // |x| >= 7.5, infinities, NaN
+    if (OVL_ANY(special)) {
+        OVL_RARE();
+        result = special ? tanhf_general_(x) : result;
     }
     return result;
 }
