@@ -56,6 +56,10 @@ def build_source(source, entry, extra_flags=()):
         shim = f.read()
     with open(os.path.join(SHIM, 'main.cpp'), 'rb') as f:
         shim += f.read()
+    for name in sorted(os.listdir(local.csrc_directory)):      # the product's own headers are compiled in as well
+        if name.endswith('.h'):
+            with open(os.path.join(local.csrc_directory, name), 'rb') as f:
+                shim += f.read()
     digest = hashlib.sha224('\0'.join(sources).encode('utf-8') + entry.encode('utf-8') + shim).hexdigest()[:32]
     os.makedirs(BUILD, exist_ok=True)
     program = os.path.join(BUILD, 'emu_' + digest)
