@@ -39,10 +39,10 @@ import numpy as np
 
 HBM_PEAK_GBPS = 8000.0
 
-# HBM bytes per launch of the chain8 kernel from rocprofv3 counters (FETCH_SIZE 262200.5, WRITE_SIZE 262144.0, each
+# HBM bytes per launch of the chain8 kernel from rocprofv3 counters (FETCH_SIZE 262207.5, WRITE_SIZE 262144.0, each
 # scaled by the same counter's reading for the copy kernel of known size: factors 1.99986 and 0.99909).
 # Source: profiles/bench_all_kernels_hbm_traffic_counters.md
-CHAIN8_TRAFFIC_BYTES = 805139592
+CHAIN8_TRAFFIC_BYTES = 805152370
 
 
 class Spec(object):
