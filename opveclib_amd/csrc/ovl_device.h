@@ -75,6 +75,18 @@ __device__ __forceinline__ T ovl_dpp_move(T old, T src) {
 #define ovl_recipf_inrange(x) ovl_math::recipf_<false>(x)
 #define ovl_divf_inrange(a, b) ovl_math::divf_inrange_((a), (b))
 
+// Once-rounded log(1 + x) and exp(x) - 1 on their checked domains, which the 'ulp2' math mode puts in place of the
+// reference's formulas for them (hipgen/accuracy.py).
+#define ovl_log1p_direct(x) ovl_math::log1p_direct_<false>((x), ovl_log_tab)
+#define ovl_log1p_direct_nan(x) ovl_math::log1p_direct_<true>((x), ovl_log_tab)
+#define ovl_expm1_direct(x) ovl_math::expm1_direct_((x), ovl_exp_tab)
+
+// The logistic function 1 / (1 + exp(-x)) for -16 <= x <= 64 (NaN propagates): hardware-based exp, the sum and the
+// correctly rounded reciprocal.  On that domain it is within two units in the last place of the same formula evaluated
+// with the host C library's expf (below -16 the exponential passes 2^24, where adding 1 rounds, and the distance can
+// reach 4); compared over every float32 argument of the domain by tests/test_gpu_math_exhaustive.py.
+#define ovl_sigmoid_ulp2(x) ovl_math::recipf_<false>(1.0f + ovl_fast::expf_<false>(-(x)))
+
 // Entry points of the optional 'fast' math mode (ovl_fast_math.h).
 #define ovl_fast_expf(x) ovl_fast::expf_<true>(x)
 #define ovl_fast_logf(x) ovl_fast::logf_<true>(x)

@@ -119,6 +119,34 @@ OVL_HD float expf_(float x, const uint64_t* tab = exp2f_tab) {
     return result;
 }
 
+// exp(x) - 1 for callers that know 2^-12 <= x <= 64, rounded once: the double precision value that expf_ forms before
+// its final conversion, minus one in the same fused multiply-add that applies the scale (so it costs what expf_
+// costs).  That value is within 2^-31 of exp(x) - 1, far below half a float32 unit in the last place for x >= 2^-12:
+// the result is the correctly rounded expm1(x) except where exp(x) - 1 lies that close to a rounding boundary.  Used
+// by the code generator's 'ulp2' math mode in place of the reference's expm1 formula
+// (e - 1) * x / log(e), e = exp(x) (opveclib/examples/test_expm1.py:22-62), from which it is at most two units in the
+// last place away on that domain (compared over every float32 argument of the domain).
+OVL_HD float expm1_direct_(float x, const uint64_t* tab = exp2f_tab) {
+    const double InvLn2N = 0x1.71547652b82fep+0 * OVL_EXP2F_N;
+    const double Shift = 0x1.8p+52;
+    const double C0 = 0x1.c6af84b912394p-5 / OVL_EXP2F_N / OVL_EXP2F_N / OVL_EXP2F_N;
+    const double C1 = 0x1.ebfce50fac4f3p-3 / OVL_EXP2F_N / OVL_EXP2F_N;
+    const double C2 = 0x1.62e42ff0c52d6p-1 / OVL_EXP2F_N;
+    double xd = (double)x;
+    double kd = __builtin_fma(InvLn2N, xd, Shift);
+    uint64_t ki = as_u64(kd);
+    kd -= Shift;
+    double r = __builtin_fma(InvLn2N, xd, -kd);
+    uint64_t t = tab[ki % OVL_EXP2F_N];
+    t += ki << (52 - OVL_EXP2F_TABLE_BITS);
+    double s = as_f64(t);
+    double z2 = __builtin_fma(C0, r, C1);
+    double r2 = r * r;
+    double y = __builtin_fma(C2, r, 1.0);
+    y = __builtin_fma(z2, r2, y);
+    return (float)__builtin_fma(y, s, -1.0);
+}
+
 // ---------------------------------------------------------------------------------------------------------------------
 // logf
 // ---------------------------------------------------------------------------------------------------------------------
@@ -209,6 +237,39 @@ OVL_HD float logf_(float x, const logf_entry* tab = logf_tab) {
         if (ix * 2 == 0) fixed = -__builtin_inff();
         result = special ? fixed : result;
     }
+    return result;
+}
+
+// log(1 + x) for callers that know 2^-10 <= x <= 2^64, rounded once: u = 1 + x is exact in double precision, and the
+// table and polynomial of logf_main_ are applied to the double u instead of a float (the table index and the exponent
+// come from the same bits, which sit in the upper word of a double).  The polynomial is within 2^-31 of log(u), so the
+// result is the correctly rounded log1p(x) except within that distance of a rounding boundary.  Used by the code
+// generator's 'ulp2' math mode in place of the reference's log1p formula log(u) * x / (u - 1), u = 1 + x rounded to
+// float (opveclib/examples/test_log1p.py:22-61), from which it is at most two units in the last place away on that
+// domain (compared over every float32 argument of the domain).
+// The common path works on the bits of u and would turn NaN into a number; with MAYBE_NAN, adding x * 0 (+-0 for every
+// number) puts the NaN back.
+template <bool MAYBE_NAN>
+OVL_HD float log1p_direct_(float x, const logf_entry* tab = logf_tab) {
+    const double Ln2 = 0x1.62e42fefa39efp-1;
+    const double A0 = -0x1.00ea348b88334p-2, A1 = 0x1.5575b0be00b6ap-2, A2 = -0x1.ffffef20a4123p-2;
+    const uint32_t Off = 0x3fe66000;            // upper word of 0.69921875, the lower end of the table's range
+    const double u = 1.0 + (double)x;
+    const uint64_t iu = as_u64(u);
+    const uint32_t tmp = (uint32_t)(iu >> 32) - Off;
+    const int i = (tmp >> (20 - OVL_LOGF_TABLE_BITS)) % OVL_LOGF_N;
+    const int k = (int32_t)tmp >> 20;
+    const double z = as_f64(iu - ((uint64_t)(tmp & 0xfff00000u) << 32));
+    const double invc = tab[i].invc;
+    const double logc = tab[i].logc;
+    double r = __builtin_fma(z, invc, -1.0);
+    double y0 = __builtin_fma((double)k, Ln2, logc);
+    double r2 = r * r;
+    double y = __builtin_fma(A1, r, A2);
+    y = __builtin_fma(A0, r2, y);
+    y = __builtin_fma(y, r2, y0 + r);
+    float result = (float)y;
+    if (MAYBE_NAN) result = __builtin_fmaf(x, 0.0f, result);
     return result;
 }
 

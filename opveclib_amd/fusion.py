@@ -411,6 +411,9 @@ class _Builder(object):
         var = lang.Expression()
         var.code = lang.VARIABLE
         var.dtype = dtype
+        # io_index has no meaning of its own on a VARIABLE: 1 marks the variable as standing for an operator's output
+        # tensor, which is where the code generator's error analysis starts a new stage (hipgen/accuracy.py)
+        var.io_index = 1
         return self.add(var, [zero_index])
 
     def add_uint64(self, value):

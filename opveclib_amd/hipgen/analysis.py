@@ -312,9 +312,17 @@ class DagInfo(object):
     # -- queries ---------------------------------------------------------------------------------------------------
     def uses_math_tables(self):
         """True when the body calls the table-driven float32 exp or log."""
-        if getattr(self, 'math', 'exact') != 'exact':
+        mode = getattr(self, 'math', 'exact')
+        if mode == 'fast':
             return False
-        return any(n.code in (lang.EXP, lang.LOG) and n.dtype == lang.FLOAT32 for n in self.nodes)
+        calls = [n for n in self.nodes if n.code in (lang.EXP, lang.LOG) and n.dtype == lang.FLOAT32]
+        if mode == 'ulp2':
+            # only the call sites that keep the bit-compatible routine
+            from . import accuracy, ranges
+            known = ranges.analyse(self) if getattr(self, 'value_ranges', True) else None
+            cheap = accuracy.select(self, known)
+            calls = [n for n in calls if n.idx not in cheap] + [k for k in cheap.values() if k in accuracy.IDIOM_DOMAIN]
+        return bool(calls)
 
     def tensor_accesses(self):
         """[(node, tensor node, affine or None)] for reads of inputs and stores to outputs, in program order."""

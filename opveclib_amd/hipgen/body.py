@@ -11,6 +11,7 @@ tiles, plain global accesses).
 
 from .. import language as lang
 from . import ranges as value_ranges
+from . import accuracy
 
 CTYPE = {
     lang.FLOAT32: 'float', lang.FLOAT64: 'double',
@@ -43,7 +44,8 @@ UNARY = {
 # Float32 math per mode: {mode: {expression code: function name}}; DIVIDE maps to a two-argument function.
 # 'exact' (the default) is the table above plus the IEEE '/' operator: the host C library's bits.  'fast' calls the
 # routines of csrc/ovl_fast_math.h (hardware exp2 / log2 / reciprocal with extended-precision range handling, each
-# within two units in the last place of the host library's result).
+# within two units in the last place of the host library's result).  The third mode, 'ulp2', has no table of its own:
+# every call site takes its routine from 'exact' or from 'fast', as accuracy.select decides.
 MATH_MODES = {
     'exact': {},
     'fast': {lang.TANH: 'ovl_fast_tanhf', lang.EXP: 'ovl_fast_expf', lang.LOG: 'ovl_fast_logf',
@@ -237,9 +239,14 @@ class BodyEmitter(object):
         """[(index of the expression that produced it, statement text)] in program order."""
         info = self.info
         math_mode = getattr(info, 'math', 'exact')
-        fast = MATH_MODES[math_mode]
-        in_range = IN_RANGE[math_mode]
         known = value_ranges.analyse(info) if getattr(info, 'value_ranges', True) else None
+        cheap_sites = accuracy.select(info, known) if math_mode == 'ulp2' else {}
+
+        def site_mode(node):
+            """The math mode of one call site."""
+            if math_mode != 'ulp2':
+                return math_mode
+            return 'fast' if node.idx in cheap_sites else 'exact'
         self._plan_if_conversion()
         names = {}
         stmts = []
@@ -341,15 +348,22 @@ class BodyEmitter(object):
                 put(CTYPE[node.dtype] + ' ' + name + ' = ' + str(known.constant(node.idx)) + ';')
             elif code in UNARY:
                 fcn = UNARY[code][node.dtype]
-                if node.dtype == lang.FLOAT32 and code in fast:
-                    fcn = fast[code]
+                mode = site_mode(node)
+                if node.dtype == lang.FLOAT32 and code in MATH_MODES[mode]:
+                    fcn = MATH_MODES[mode][code]
                 if node.dtype == lang.FLOAT32 and known is not None:
                     x = known.operand(node.idx, 0)
-                    if code == lang.EXP and value_ranges.exp_in_range(x, math_mode):
-                        fcn = in_range[code]
+                    if code == lang.EXP and value_ranges.exp_in_range(x, mode):
+                        fcn = IN_RANGE[mode][code]
                     elif code == lang.LOG and value_ranges.log_in_range(x):
-                        fcn = in_range['log nan' if x.nan else code]
+                        fcn = IN_RANGE[mode]['log nan' if x.nan else code]
                 put(CTYPE[node.dtype] + ' ' + name + ' = ' + fcn + '(' + names[ops[0]] + ');')
+            elif code == lang.DIVIDE and cheap_sites.get(node.idx) in accuracy.IDIOM_DOMAIN:
+                # the division that ends the reference's sigmoid / log1p / expm1 formula: one routine on x instead
+                kind, x, seen = accuracy.match_idiom(info, known, node)
+                fcn = {'sigmoid': 'ovl_sigmoid_ulp2', 'log1p': 'ovl_log1p_direct_nan' if seen.nan else 'ovl_log1p_direct',
+                       'expm1': 'ovl_expm1_direct'}[kind]
+                put('float ' + name + ' = ' + fcn + '(' + names[x] + ');')
             elif code == lang.DIVIDE and node.dtype == lang.FLOAT32 and self._is_constant_one(ops[0]):
                 # 1/x: the verified correctly rounded reciprocal (ovl_math.h) instead of the general division, in
                 # every math mode (it is also the cheapest form: hardware reciprocal and one refinement)
@@ -359,9 +373,11 @@ class BodyEmitter(object):
                 put('float ' + name + ' = ' + fcn + '(' + names[ops[1]] + ');')
             elif code == lang.DIVIDE and node.dtype == lang.FLOAT32 and known is not None and \
                     value_ranges.div_in_range(known.operand(node.idx, 0), known.operand(node.idx, 1)):
-                put('float ' + name + ' = ' + in_range[code] + '(' + names[ops[0]] + ', ' + names[ops[1]] + ');')
-            elif code == lang.DIVIDE and node.dtype == lang.FLOAT32 and code in fast:
-                put('float ' + name + ' = ' + fast[code] + '(' + names[ops[0]] + ', ' + names[ops[1]] + ');')
+                put('float ' + name + ' = ' + IN_RANGE[site_mode(node)][code] + '(' + names[ops[0]] + ', ' +
+                    names[ops[1]] + ');')
+            elif code == lang.DIVIDE and node.dtype == lang.FLOAT32 and code in MATH_MODES[site_mode(node)]:
+                put('float ' + name + ' = ' + MATH_MODES[site_mode(node)][code] + '(' + names[ops[0]] + ', ' +
+                    names[ops[1]] + ');')
             elif code in INFIX or code in (lang.MIN, lang.MAX, lang.POW, lang.ATAN2):
                 put(CTYPE[node.dtype] + ' ' + name + ' = ' +
                     binary_text(code, node.dtype, names[ops[0]], names[ops[1]]) + ';')

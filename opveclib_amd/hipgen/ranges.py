@@ -380,7 +380,12 @@ class RangeInfo(object):
                 r = Range(lo, hi, r.nan)
             return r
         if code in (lang.MIN, lang.MAX):
-            return hull(ops)
+            # emitted as (a < b) ? a : b and (a > b) ? a : b: the smaller (larger) of two numbers; the comparison is
+            # false when a is NaN, which selects b whatever its value, and a NaN in b comes through
+            b = ops[1]
+            pick = min if code == lang.MIN else max
+            result = Range(pick(a.lo, b.lo), pick(a.hi, b.hi), b.nan)
+            return hull([result, b]) if a.nan else result
         if code == lang.NEGATE:
             return Range(-a.hi, -a.lo, a.nan)
         if code == lang.ABS:

@@ -662,7 +662,7 @@ def _normalise_output_list(output_list):
     return list(output_list)
 
 
-MATH_MODES = ('exact', 'fast')
+MATH_MODES = ('exact', 'ulp2', 'fast')
 _default_math_mode = [None]
 
 
@@ -671,10 +671,13 @@ def set_math_mode(mode):
     Choose the float32 math library of operators evaluated from now on.
 
     'exact' (the default) reproduces the host C library's expf/logf/tanhf bit for bit and divides with IEEE rounding,
-    so results equal those of the reference's generated C++ on the same inputs.  'fast' uses the device math library
-    and a reciprocal-based division: every exp/log/tanh and every quotient is within one or two units in the last
-    place of the exact mode's, at roughly half the arithmetic cost.  The environment variable OPVECLIB_MATH sets the
-    initial mode.
+    so results equal those of the reference's generated C++ on the same inputs.  'ulp2' keeps every operator's
+    outputs within two units in the last place of the exact mode's for the same operator inputs: a static error
+    analysis (hipgen/accuracy.py) gives each exp/log/tanh/division call site the hardware-based routine where that
+    bound is proved and the bit-compatible one elsewhere.  'fast' uses the hardware-based routines and a
+    reciprocal-based division everywhere: every single exp/log/tanh and every quotient is within one or two units in
+    the last place of the exact mode's, operators composed of several calls can be further off.  The environment
+    variable OPVECLIB_MATH sets the initial mode.
     """
     if mode not in MATH_MODES:
         raise ValueError('math mode must be one of ' + str(MATH_MODES))
@@ -695,7 +698,7 @@ def evaluate(output_list, target_language='hip', opt_level=3, math_mode=None):
     :param output_list: an operator, an operator output, or a list of either
     :param target_language: must be 'hip'
     :param opt_level: operators are fused when opt_level >= 3
-    :param math_mode: 'exact' or 'fast' for this call (see :func:`set_math_mode`); None uses the current default
+    :param math_mode: 'exact', 'ulp2' or 'fast' for this call (see :func:`set_math_mode`); None uses the current default
     :return: one array for a single requested output, otherwise a list in request order.  Arrays are numpy arrays
         when every DAG input was a numpy array, otherwise torch tensors on the inputs' device.
     """

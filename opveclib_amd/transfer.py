@@ -66,6 +66,15 @@ def _stager(torch, device):
         return stager
 
 
+def shutdown():
+    """End the copy threads and drop the staging buffers (they are created again on the next large transfer)."""
+    with _lock:
+        stagers = list(_stagers.values())
+        _stagers.clear()
+    for stager in stagers:
+        stager.pool.shutdown(wait=True)
+
+
 def _torch_dtype(torch, dtype):
     return torch.from_numpy(np.empty(0, dtype=dtype)).dtype
 

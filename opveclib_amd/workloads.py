@@ -1,0 +1,163 @@
+"""
+The operator graphs of the benchmark configurations, and the step that compiles their kernels ahead of time.
+
+Each ``*_outputs`` function applies operators to its arguments and returns the requested outputs; the arguments may be
+arrays, device tensors or :class:`Spec` objects (shape and element type only), which is enough to trace, fuse,
+generate and compile an operator without allocating anything.  ``prebuild`` does that for every configuration at its
+full size and in every math mode the benchmark reports, into the package's prebuilt directory.
+"""
+
+import numpy as np
+
+
+class Spec(object):
+    """Shape and dtype of a tensor, enough to trace an operator without allocating the tensor."""
+
+    def __init__(self, shape, dtype=np.float32):
+        self.shape = list(shape)
+        self.dtype = np.dtype(dtype).type
+
+
+def uniform(rng, lo, hi, shape, dtype=np.float32):
+    """``lo + (hi - lo) * rng.random(shape)`` in ``dtype``."""
+    return (lo + (hi - lo) * rng.random(shape, dtype=dtype)).astype(dtype)
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# operator graphs
+# ----------------------------------------------------------------------------------------------------------------------
+def chain8_outputs(a, b, s):
+    """The fused 8-op chain (add, mul by scalar, tanh, sigmoid, log1p, expm1, sub, abs): its last stage."""
+    from .examples import chain8
+    return [chain8(a, b, s)[-1][0]]
+
+
+def chain8_stage_outputs(a, b, s):
+    """Every stage of the 8-op chain as a requested output (the optimizer still fuses them into one kernel)."""
+    from .examples import chain8
+    return [t[0] for t in chain8(a, b, s)]
+
+
+def copy_outputs(x):
+    """out[pos] = x[pos]: the plain copy kernel that calibrates the profiler's byte counters."""
+    import opveclib_amd as ovl
+
+    @ovl.operator()
+    def copy(arg):
+        pos = ovl.position_in(arg.shape)
+        out = ovl.output_like(arg)
+        out[pos] = arg[pos]
+        return out
+
+    return [copy(x)[0]]
+
+
+def c1_outputs(x):
+    from .examples import shift_cyclic, expm1, log1p
+    return [log1p(expm1(shift_cyclic(x)))[0]]
+
+
+def cumsum_outputs(x, axis=1):
+    from .examples import cumsum
+    return [cumsum(x, axis=axis)[0]]
+
+
+def cumprod_outputs(x, axis=1):
+    from .examples import cumprod
+    return [cumprod(x, axis=axis)[0]]
+
+
+def lstm_outputs(concat, c):
+    from .lstm import lstm
+    op = lstm(concat, c, forget_bias=1.0)
+    return [op[0], op[1]]
+
+
+def lstm_grad_outputs(concat, c, dc, dh):
+    from .lstm import lstm_grad
+    op = lstm_grad(concat, c, dc, dh, forget_bias=1.0)
+    return [op[0], op[1]]
+
+
+def gather_outputs(a, b_flat):
+    from .examples import gather_transpose
+    return [gather_transpose(a, b_flat, alpha=0.5, stride=7919)[0]]
+
+
+#: the LSTM cell sizes the reference's profiler runs (lstm/profile_lstm.py:41-51): batch 20, these unit counts
+REFERENCE_LSTM_BATCH = 20
+REFERENCE_LSTM_UNITS = (200, 650, 1500)
+#: the shape of the reference's accumulate timing (opveclib/examples/test_perf_accumulate.py:35-47): float64, axis 0
+REFERENCE_CUMSUM_SHAPE = (10000, 1000)
+
+
+def all_workload_outputs():
+    """Operator outputs of every benchmark workload at full size, built from shape specs."""
+    f32, f64 = np.float32, np.float64
+    yield chain8_outputs(Spec((8192, 8192)), Spec((8192, 8192)), Spec((1,)))
+    yield chain8_stage_outputs(Spec((8192, 8192)), Spec((8192, 8192)), Spec((1,)))
+    yield copy_outputs(Spec((8192, 8192)))
+    yield c1_outputs(Spec((1 << 20,)))
+    yield cumsum_outputs(Spec((4096, 16384), f32))
+    yield cumprod_outputs(Spec((4096, 16384), f32))
+    yield cumsum_outputs(Spec((1024, 16384), f64))
+    yield cumprod_outputs(Spec((1024, 16384), f64))
+    yield lstm_outputs(Spec((4096, 4096)), Spec((4096, 1024)))
+    yield lstm_grad_outputs(Spec((4096, 4096)), Spec((4096, 1024)), Spec((4096, 1024)), Spec((4096, 1024)))
+    yield gather_outputs(Spec((16384, 16384)), Spec((16384 * 16384,)))
+    yield cumsum_outputs(Spec(REFERENCE_CUMSUM_SHAPE, f64), axis=0)
+    for units in REFERENCE_LSTM_UNITS:
+        batch = REFERENCE_LSTM_BATCH
+        yield lstm_outputs(Spec((batch, 4 * units)), Spec((batch, units)))
+        yield lstm_grad_outputs(Spec((batch, 4 * units)), Spec((batch, units)), Spec((batch, units)),
+                                Spec((batch, units)))
+
+
+def fused_operators(outputs):
+    """The operators of the fused DAG behind ``outputs``."""
+    from .operator import _build_op_dag
+    from .fusion import _merge_op_dag
+    dag, _ = _merge_op_dag(_build_op_dag(*outputs).proto_dag, None)
+    return list(dag.operators)
+
+
+def unfused_operators(outputs):
+    """The operators behind ``outputs`` as written, one kernel each."""
+    from .operator import _build_op_dag
+    return list(_build_op_dag(*outputs).proto_dag.operators)
+
+
+def prebuild(force=False, workers=8):
+    """
+    Compile the kernels of every benchmark workload into the package's prebuilt directory: each in the default
+    'exact' math mode, and those that call exp, log, tanh or divide also in the 'ulp2' and 'fast' modes.  Needs
+    hipcc, not a GPU.  ``force`` compiles even where a built library exists.  Returns the number of libraries.
+    """
+    from concurrent.futures import ThreadPoolExecutor
+    from . import compiler, runtime
+    from . import language as lang
+
+    jobs = {}
+    for outputs in all_workload_outputs():
+        for op in fused_operators(outputs):
+            key = op.SerializeToString()
+            jobs[(key, 'exact')] = (op, None)
+            if any(e.code in (lang.EXP, lang.LOG, lang.TANH, lang.DIVIDE) for e in op.expressions):
+                for mode in ('ulp2', 'fast'):
+                    jobs[(key, mode)] = (op, {'math': mode})
+            elif op.name == 'accumulate':
+                jobs[(key, 'fast')] = (op, {'math': 'fast'})       # the reassociating scan
+    # the single operators of the chain at full size, bit-exact: what the benchmark compares each stage with
+    headline = chain8_stage_outputs(Spec((8192, 8192)), Spec((8192, 8192)), Spec((1,)))
+    for op in unfused_operators(headline):
+        jobs[(op.SerializeToString(), 'exact')] = (op, None)
+    previous = compiler.prebuild_mode, compiler.force_rebuild
+    compiler.prebuild_mode, compiler.force_rebuild = True, bool(force)
+    try:
+        with ThreadPoolExecutor(max_workers=workers) as pool:
+            list(pool.map(lambda job: runtime.build_operator(*job), jobs.values()))
+    finally:
+        compiler.prebuild_mode, compiler.force_rebuild = previous
+        if force:
+            runtime._generated.clear()
+    return len(jobs)

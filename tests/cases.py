@@ -11,7 +11,7 @@ import numpy as np
 import opveclib_amd as ovl
 from opveclib_amd import stdops
 from opveclib_amd import language as lang
-from opveclib_amd.examples import (shift_cyclic, cumsum, cumprod, accumulate, expm1, log1p, absolute,
+from opveclib_amd.examples import (chain8, shift_cyclic, cumsum, cumprod, accumulate, expm1, log1p, absolute,
                                    gather_transpose)
 from opveclib_amd.lstm import lstm, lstm_grad
 
@@ -52,19 +52,6 @@ def all_outputs(op):
 # ----------------------------------------------------------------------------------------------------------------------
 # the five benchmark configurations, at sizes the oracle finishes in well under a second
 # ----------------------------------------------------------------------------------------------------------------------
-def chain8(a, b, s):
-    """The fused 8-op chain: add, mul by scalar, tanh, sigmoid, log1p, expm1, sub, abs; returns every stage."""
-    t1 = stdops.add(a, b)
-    t2 = stdops.mul(t1, s)
-    t3 = stdops.tanh(t2)
-    t4 = stdops.sigmoid(t3)
-    t5 = log1p(t4)
-    t6 = expm1(t5)
-    t7 = stdops.sub(t6, b)
-    y = absolute(t7)
-    return [t1, t2, t3, t4, t5, t6, t7, y]
-
-
 def c1_shift_expm1_log1p(rng, n=1 << 14):
     x = uniform(rng, -0.9, 0.9, n)
     return [log1p(expm1(shift_cyclic(x)))[0]]
@@ -782,12 +769,13 @@ FAST_CASES = [
 ]
 
 
-def run_fast_case_on_gpu(case):
-    """The case's operators unfused in 'fast' mode against the oracle (exact by construction); returns the distances."""
+def run_fast_case_on_gpu(case, math_mode='fast'):
+    """The case's operators unfused in ``math_mode`` against the oracle (exact by construction); returns the
+    distances."""
     import oracle
     outs = case.outputs()
     ref = oracle.profile(outs, 1, 0)[0]
-    got = ovl.evaluate(outs, target_language='hip', opt_level=0, math_mode='fast')
+    got = ovl.evaluate(outs, target_language='hip', opt_level=0, math_mode=math_mode)
     got = got if isinstance(got, list) else [got]
     dists = []
     for g, r in zip(got, ref):
@@ -796,6 +784,45 @@ def run_fast_case_on_gpu(case):
         assert np.array_equal(np.isnan(g), nan), case.name + ': NaN pattern differs'
         dists.append(ulp_distance(np.where(nan, 0, g).astype(r.dtype), np.where(nan, 0, r).astype(r.dtype)))
     return dists
+
+
+# ----------------------------------------------------------------------------------------------------------------------
+# 'ulp2' math mode at the benchmark's full size
+# ----------------------------------------------------------------------------------------------------------------------
+CHAIN8_SHAPE = (8192, 8192)
+CHAIN8_STAGES = ('add', 'mul', 'tanh', 'sigmoid', 'log1p', 'expm1', 'sub', 'abs')
+#: value ranges of the chain's stage inputs (what the code generator derives in the fused kernel, rounded outward)
+CHAIN8_STAGE_INPUT_RANGE = {'log1p': (0.25, 0.75), 'expm1': (0.2, 0.6)}
+
+
+@ovl.operator()
+def clip(x, lo=0.0, hi=1.0):
+    """min(max(x, lo), hi): leaves every value inside [lo, hi] untouched and tells the code generator the range."""
+    out = ovl.output_like(x)
+    pos = ovl.position_in(x.shape)
+    out[pos] = ovl.minimum(ovl.maximum(x[pos], lo), hi)
+    return out
+
+
+def chain8_single_stage(name, x, with_range=False):
+    """Operator output of one transcendental stage of the chain applied to ``x``; with ``with_range`` behind a clip
+    to the stage's input range, which the optimizer fuses in (so the stage sees the range it sees inside the chain)."""
+    fcn = {'tanh': stdops.tanh, 'sigmoid': stdops.sigmoid, 'log1p': log1p, 'expm1': expm1}[name]
+    if with_range and name in CHAIN8_STAGE_INPUT_RANGE:
+        lo, hi = CHAIN8_STAGE_INPUT_RANGE[name]
+        x = clip(x, lo=lo, hi=hi)
+    return fcn(x)[0]
+
+
+def ulp2_full_size_operators():
+    """[(operator, options)] of tests/test_gpu_ulp2.py that the benchmark's own prebuild step does not cover."""
+    from opveclib_amd import workloads
+    spec = workloads.Spec(CHAIN8_SHAPE)
+    jobs = []
+    for name in ('tanh', 'sigmoid', 'log1p', 'expm1'):
+        for op in _operators_of([chain8_single_stage(name, spec, with_range=True)], 3):
+            jobs.append((op, {'math': 'ulp2'}))
+    return jobs
 
 
 # (case, code generator options): the same cases through kernel templates the generator would not pick by itself
@@ -843,12 +870,12 @@ def run_variant_on_gpu(name, options):
         runtime.codegen_options = {}
 
 
-def prebuild_all(cases=None, workers=8, with_oracle=True, force_benchmark=False):
+def prebuild_all(cases=None, workers=8, with_oracle=True):
     """Compile the HIP library (and the oracle library) of every operator used by the cases and the benchmark."""
     from concurrent.futures import ThreadPoolExecutor
     from opveclib_amd import compiler, runtime
     import oracle
-    import bench
+    from opveclib_amd import workloads
 
     ops = {}
     oracle_ops = {}
@@ -859,9 +886,18 @@ def prebuild_all(cases=None, workers=8, with_oracle=True, force_benchmark=False)
                 ops[op.SerializeToString()] = op
         for op in _operators_of(outs, 0):
             oracle_ops[op.SerializeToString()] = op
-    for outs in bench.all_workload_outputs():
+    oracle_o2 = {}
+    for outs in workloads.all_workload_outputs():
         for op in _operators_of(outs, 3):
             ops[op.SerializeToString()] = op
+        # the benchmark's CPU legs: every workload as written, the headline also fused, with and without -O2
+        for op in _operators_of(outs, 0):
+            oracle_ops[op.SerializeToString()] = op
+    headline = workloads.chain8_outputs(workloads.Spec((8192, 8192)), workloads.Spec((8192, 8192)),
+                                        workloads.Spec((1,)))
+    for op in _operators_of(headline, 3):
+        oracle_ops[op.SerializeToString()] = op
+        oracle_o2[op.SerializeToString()] = op
 
     variants = []
     if cases is None:
@@ -872,10 +908,24 @@ def prebuild_all(cases=None, workers=8, with_oracle=True, force_benchmark=False)
             outs = case.outputs()
             for op in _operators_of(outs, 0):
                 variants.append((op, {'math': 'fast'}))
+                variants.append((op, {'math': 'ulp2'}))
                 oracle_ops[op.SerializeToString()] = op
         for name in FAST_FUSED_CASES + FAST_SCAN_CASES:
             for op in _operators_of(CASE_BY_NAME[name].outputs(), 3):
                 variants.append((op, {'math': 'fast'}))
+        for name in FAST_FUSED_CASES + ['c2_chain_stages']:
+            for op in _operators_of(CASE_BY_NAME[name].outputs(), 3):
+                variants.append((op, {'math': 'ulp2'}))
+        variants.extend(ulp2_full_size_operators())
+        # tests/test_gpu_ulp2.py: the oracle on slices of 64 rows of the full-size chain and on the small chain's stages
+        rows = np.zeros((64, CHAIN8_SHAPE[1]), np.float32)
+        small = np.zeros((96, 256), np.float32)
+        for x in (rows, small):
+            for name in ('tanh', 'sigmoid', 'log1p', 'expm1'):
+                for op in _operators_of([chain8_single_stage(name, x)], 0):
+                    oracle_ops[op.SerializeToString()] = op
+        for op in _operators_of(workloads.chain8_stage_outputs(rows, rows, np.ones(1, np.float32)), 0):
+            oracle_ops[op.SerializeToString()] = op
         from tests import random_programs
         for seed in random_programs.GPU_SEEDS:
             program = random_programs.application(seed).expression_dag
@@ -928,31 +978,19 @@ def prebuild_all(cases=None, workers=8, with_oracle=True, force_benchmark=False)
             for level in (0, 3):
                 for op in _operators_of(outs, level):
                     ops[op.SerializeToString()] = op
-        for outs in bench.all_workload_outputs():
+        for outs in workloads.all_workload_outputs():
             for op in _operators_of(outs, 3):
                 if any(e.code in (lang.EXP, lang.LOG, lang.TANH, lang.DIVIDE) for e in op.expressions):
                     variants.append((op, {'math': 'fast'}))
 
     compiler.prebuild_mode = True
     try:
-        if force_benchmark:
-            # the benchmark's and the smoke check's kernels are compiled again even when built libraries exist
-            forced = {}
-            for outs in list(bench.all_workload_outputs()) + [CASE_BY_NAME[n].outputs() for n in SMOKE_CASES]:
-                for op in _operators_of(outs, 3):
-                    forced[op.SerializeToString()] = op
-            compiler.force_rebuild = True
-            try:
-                with ThreadPoolExecutor(max_workers=workers) as pool:
-                    list(pool.map(runtime.build_operator, forced.values()))
-            finally:
-                compiler.force_rebuild = False
-            runtime._generated.clear()
         with ThreadPoolExecutor(max_workers=workers) as pool:
             list(pool.map(runtime.build_operator, ops.values()))
             list(pool.map(lambda v: runtime.build_operator(*v), variants))
             if with_oracle:
                 list(pool.map(oracle.compile_op, oracle_ops.values()))
+                list(pool.map(lambda op: oracle.compile_op(op, ('-O2',)), oracle_o2.values()))
     finally:
         compiler.prebuild_mode = False
     return len(ops), len(oracle_ops)

@@ -4,6 +4,8 @@
 //                          call them) against the host C library's expf / logf / tanhf / (1.0f / x) on this machine
 //                          (function 4 evaluates the device math library's own expf instead: a self-test of the
 //                          checker, which must report differences for it)
+//   ovl_exh_ulp_in_range   the once-rounded log1p / expm1 of the 'ulp2' math mode against the reference's formulas for
+//                          them evaluated with the host C library, on every float of a range of bit patterns
 //   ovl_exh_tanh_division  device tanhf with its shortened divisions against the same code with IEEE divisions
 //   ovl_exh_in_range       the variants without a rare-argument block (expf, logf, reciprocal, division) against the
 //                          full routines / the '/' operator, on every argument the code generator may hand them
@@ -32,7 +34,8 @@ using namespace ovl_math;
 namespace {
 
 enum { FN_EXP = 0, FN_LOG = 1, FN_TANH = 2, FN_RECIP = 3, FN_DEVICE_LIBRARY_EXP = 4,
-       FN_FAST_EXP = 5, FN_FAST_LOG = 6, FN_FAST_TANH = 7, FN_FAST_RECIP = 8 };
+       FN_FAST_EXP = 5, FN_FAST_LOG = 6, FN_FAST_TANH = 7, FN_FAST_RECIP = 8,
+       FN_LOG1P_DIRECT = 9, FN_EXPM1_DIRECT = 10, FN_SIGMOID_ULP2 = 11 };
 
 __global__ void __launch_bounds__(256) eval_kernel(int fn, uint32_t first, uint32_t count, float* __restrict__ out) {
     OVL_DECLARE_MATH_TABLES();
@@ -48,6 +51,9 @@ __global__ void __launch_bounds__(256) eval_kernel(int fn, uint32_t first, uint3
         else if (fn == FN_FAST_LOG) y = ovl_fast_logf(x);
         else if (fn == FN_FAST_TANH) y = ovl_fast_tanhf(x);
         else if (fn == FN_FAST_RECIP) y = ovl_fast_divf(1.0f, x);
+        else if (fn == FN_LOG1P_DIRECT) y = ovl_log1p_direct_nan(x);
+        else if (fn == FN_EXPM1_DIRECT) y = ovl_expm1_direct(x);
+        else if (fn == FN_SIGMOID_ULP2) y = ovl_sigmoid_ulp2(x);
         else y = expf(x);            // the device math library's own expf: differs from the host's in the last place
         out[i] = y;
     }
@@ -132,7 +138,41 @@ __global__ void __launch_bounds__(256) in_range_kernel(int which, unsigned long 
     atomicAdd(compared, done);
 }
 
+// The reference's log1p and expm1 operators (opveclib/examples/test_log1p.py:22-61, test_expm1.py:22-62) as the
+// generated C++ evaluates them: every operation in float, exp and log from the host C library.
+float host_log1p_formula(float x) {
+    volatile float u = 1.0f + x;
+    volatile float d = u - 1.0f;
+    if (isinf(x) && x > 0.0f) return x;
+    if (d == 0.0f) return x;
+    volatile float l = logf(u);
+    volatile float p = l * x;
+    return p / d;
+}
+
+float host_expm1_formula(float x) {
+    volatile float e = expf(x);
+    if (isinf(x) && x > 0.0f) return x;
+    if (e == 1.0f) return x;
+    volatile float em = e - 1.0f;
+    if (em == -1.0f) return -1.0f;
+    volatile float p = em * x;
+    volatile float l = logf(e);
+    return p / l;
+}
+
+// The reference's sigmoid (opveclib/stdops/math.py:93): 1 / (1 + exp(-x)) in float.
+float host_sigmoid_formula(float x) {
+    volatile float e = expf(-x);
+    volatile float s = 1.0f + e;
+    volatile float one = 1.0f;
+    return one / s;
+}
+
 float host_value(int fn, float x) {
+    if (fn == FN_SIGMOID_ULP2) return host_sigmoid_formula(x);
+    if (fn == FN_LOG1P_DIRECT) return host_log1p_formula(x);
+    if (fn == FN_EXPM1_DIRECT) return host_expm1_formula(x);
     if (fn == FN_EXP || fn == FN_DEVICE_LIBRARY_EXP || fn == FN_FAST_EXP) return expf(x);
     if (fn == FN_LOG || fn == FN_FAST_LOG) return logf(x);
     if (fn == FN_TANH || fn == FN_FAST_TANH) return tanhf(x);
@@ -190,7 +230,8 @@ extern "C" int ovl_exh_in_range(int which, uint64_t* mismatches, uint64_t* compa
 // Compare fn over the bit patterns first, first + step, ... (count of them) with the host C library.
 // step = 1 and count = 2^32 is the exhaustive run.  threads = host threads used for the host side.
 static int against_host(int fn, uint64_t count, uint32_t step, uint32_t threads, uint64_t* mismatches,
-                        uint32_t* first_bad, uint64_t* beyond_two_ulp, uint32_t* max_ulp, uint32_t* worst_bits);
+                        uint32_t* first_bad, uint64_t* beyond_two_ulp, uint32_t* max_ulp, uint32_t* worst_bits,
+                        uint64_t first_pattern = 0, uint64_t end_pattern = 1ull << 32);
 
 extern "C" int ovl_exh_against_host(int fn, uint64_t count, uint32_t step, uint32_t threads, uint64_t* mismatches,
                                     uint32_t* first_bad) {
@@ -212,8 +253,20 @@ static int64_t ordered(uint32_t bits) {       // float bit pattern -> integer th
     return (bits & 0x80000000u) ? -(int64_t)(bits & 0x7fffffffu) : (int64_t)bits;
 }
 
+// Every float whose bit pattern lies in [first_bits, last_bits] (a range of one sign: consecutive patterns are
+// consecutive floats): fn against its host counterpart, distances in units in the last place.
+extern "C" int ovl_exh_ulp_in_range(int fn, uint32_t first_bits, uint32_t last_bits, uint32_t threads,
+                                    uint64_t* compared, uint64_t* mismatches, uint64_t* beyond_two_ulp,
+                                    uint32_t* max_ulp, uint32_t* worst_bits) {
+    uint32_t first = 0;
+    *compared = (uint64_t)last_bits - first_bits + 1;
+    return against_host(fn, 1ull << 32, 1, threads, mismatches, &first, beyond_two_ulp, max_ulp, worst_bits,
+                        first_bits, (uint64_t)last_bits + 1);
+}
+
 static int against_host(int fn, uint64_t count, uint32_t step, uint32_t threads, uint64_t* mismatches,
-                        uint32_t* first_bad, uint64_t* beyond_two_ulp, uint32_t* max_ulp, uint32_t* worst_bits) {
+                        uint32_t* first_bad, uint64_t* beyond_two_ulp, uint32_t* max_ulp, uint32_t* worst_bits,
+                        uint64_t first_pattern, uint64_t end_pattern) {
     const uint32_t chunk = 1u << 26;
     float* d_out = nullptr;
     float* h_out = nullptr;
@@ -225,7 +278,8 @@ static int against_host(int fn, uint64_t count, uint32_t step, uint32_t threads,
     uint32_t lowest = 0xffffffffu, largest = 0, largest_at = 0;
     if (threads == 0) threads = 1;
     // with step > 1 the device still evaluates whole chunks; the host then samples every step-th pattern
-    for (uint64_t base = 0; base < (1ull << 32) && base / step < count; base += chunk) {
+    for (uint64_t base = first_pattern & ~(uint64_t)(chunk - 1); base < end_pattern && base / step < count;
+         base += chunk) {
         hipLaunchKernelGGL(eval_kernel, dim3(2048), dim3(256), 0, 0, fn, (uint32_t)base, chunk, d_out);
         err = hipMemcpy(h_out, d_out, (size_t)chunk * sizeof(float), hipMemcpyDeviceToHost);
         if (err != hipSuccess) break;
@@ -239,6 +293,7 @@ static int against_host(int fn, uint64_t count, uint32_t step, uint32_t threads,
                 uint32_t i = begin + (step - (base + begin) % step) % step;
                 for (; i < end; i += step) {
                     const uint32_t bits = (uint32_t)base + i;
+                    if (bits < first_pattern || bits >= end_pattern) continue;
                     float x;
                     memcpy(&x, &bits, 4);
                     const float want = host_value(fn, x);

@@ -1,0 +1,214 @@
+"""
+The 'ulp2' math mode on the CPU: which routine every call site gets (hipgen/accuracy.py), and the once-rounded
+log1p / expm1 routines of csrc/ovl_math.h compiled for the host against the reference's formulas
+(opveclib/examples/test_log1p.py:22-61, test_expm1.py:22-62) evaluated with the host C library.
+
+The header is plain IEEE double arithmetic, so the host build returns the bits the GPU returns; the sweep here takes
+every 31st float32 of the domain on which the code generator uses the routines (the GPU test takes every one).
+"""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+import opveclib_amd as ovl
+from opveclib_amd import language as lang
+from opveclib_amd import stdops, workloads
+from opveclib_amd.examples import log1p, expm1
+from opveclib_amd.hipgen import accuracy, ranges
+from opveclib_amd.hipgen.analysis import DagInfo
+from opveclib_amd.workloads import Spec
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(os.path.dirname(HERE), 'opveclib_amd', 'csrc')
+
+
+def selection(operator_dag):
+    """{expression code or idiom name: [cheap?]} in program order for one operator."""
+    info = DagInfo(operator_dag)
+    info.math = 'ulp2'
+    known = ranges.analyse(info)
+    cheap = accuracy.select(info, known)
+    kinds = accuracy.candidate_sites(info, known)
+    return [(kinds[idx], idx in cheap) for idx in sorted(kinds)]
+
+
+def test_fused_chain_uses_cheap_routines_where_two_ulp_are_proved():
+    outs = workloads.chain8_outputs(Spec((64, 256)), Spec((64, 256)), Spec((1,)))
+    op, = workloads.fused_operators(outs)
+    chosen = selection(op)
+    cheap = [kind for kind, is_cheap in chosen if is_cheap]
+    # tanh directly; the three composite formulas as one routine each
+    assert lang.TANH in cheap and 'sigmoid' in cheap and 'log1p' in cheap and 'expm1' in cheap
+    assert [kind for kind, is_cheap in chosen if kind in accuracy.IDIOM_DOMAIN and not is_cheap] == []
+
+
+def test_unfused_formulas_keep_the_bit_compatible_log_and_exp():
+    """Without a known argument range the formulas are not replaced; their log and exp feed a product and a quotient,
+    which can double an error twice, so they stay exact, while the final division (1 ulp) may be the cheap one."""
+    x = Spec((1024,))
+    chosen = dict(selection(workloads.unfused_operators([log1p(x)[0]])[0]))
+    assert chosen[lang.LOG] is False and chosen[lang.DIVIDE] is True
+    chosen = dict(selection(workloads.unfused_operators([expm1(x)[0]])[0]))
+    assert chosen[lang.EXP] is False and chosen[lang.LOG] is False and chosen[lang.DIVIDE] is True
+
+
+def test_single_calls_are_cheap_and_cancelling_sums_are_not():
+    x = Spec((1024,))
+    assert selection(workloads.unfused_operators([stdops.tanh(x)[0]])[0]) == [(lang.TANH, True)]
+    # 1 / (1 + e): an inexact e loses a step in the sum and up to twice that in the reciprocal; without a known
+    # argument range the formula is not replaced either
+    assert selection(workloads.unfused_operators([stdops.sigmoid(x)[0]])[0]) == [(lang.EXP, False)]
+    # the LSTM cell adds products of either sign: a distance in the operands is unbounded in ulp of the sum
+    outs = workloads.lstm_outputs(Spec((8, 64)), Spec((8, 16)))
+    assert all(not is_cheap for _, is_cheap in selection(workloads.fused_operators(outs)[0]))
+
+
+def test_an_inexact_value_never_decides_a_branch_or_an_index():
+    @ovl.operator()
+    def branchy(x):
+        out = ovl.output_like(x)
+        pos = ovl.position_in(x.shape)
+        e = ovl.exp(x[pos])
+        with ovl.if_(e > 2.0):
+            out[pos] = e
+        with ovl.else_():
+            out[pos] = x[pos]
+        return out
+
+    chosen = selection(workloads.unfused_operators([branchy(Spec((256,)))[0]])[0])
+    assert chosen == [(lang.EXP, False)]
+
+
+def test_stage_variables_are_marked_by_the_optimizer():
+    outs = workloads.chain8_outputs(Spec((64, 256)), Spec((64, 256)), Spec((1,)))
+    op, = workloads.fused_operators(outs)
+    marked = [e for e in op.expressions if e.code == lang.VARIABLE and e.io_index == accuracy.STAGE_VARIABLE]
+    assert len(marked) == 7         # every internalised edge of the eight-operator chain
+
+
+def test_generated_text_names_the_chosen_routines():
+    from opveclib_amd import hipgen
+    outs = workloads.chain8_outputs(Spec((64, 256)), Spec((64, 256)), Spec((1,)))
+    op, = workloads.fused_operators(outs)
+    text = hipgen.generate(op, 'f' + '0' * 56, {'math': 'ulp2'}).source
+    for wanted in ('ovl_fast_tanhf(', 'ovl_sigmoid_ulp2(', 'ovl_log1p_direct', 'ovl_expm1_direct('):
+        assert wanted in text
+    assert 'ovl_tanhf(' not in text
+    exact = hipgen.generate(op, 'f' + '0' * 56, None).source
+    assert 'ovl_fast' not in exact and '_direct' not in exact
+
+
+PROGRAM = r'''
+#include <math.h>
+#include <stdio.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#include "ovl_math.h"
+static int32_t ordered(float f) { int32_t i; memcpy(&i, &f, 4); return i < 0 ? (int32_t)0x80000000 - i : i; }
+static float log1p_formula(float x) {
+    volatile float u = 1.0f + x; volatile float d = u - 1.0f;
+    if (isinf(x) && x > 0) return x;
+    if (d == 0) return x;
+    volatile float l = logf(u); volatile float p = l * x; return p / d;
+}
+static float expm1_formula(float x) {
+    volatile float e = expf(x);
+    if (isinf(x) && x > 0) return x;
+    if (e == 1.0f) return x;
+    volatile float em = e - 1.0f;
+    if (em == -1.0f) return -1.0f;
+    volatile float p = em * x; volatile float l = logf(e); return p / l;
+}
+int main(int argc, char** argv) {
+    int which = atoi(argv[1]); float lo = strtof(argv[2], 0), hi = strtof(argv[3], 0); uint32_t step = atoi(argv[4]);
+    uint32_t a, b; memcpy(&a, &lo, 4); memcpy(&b, &hi, 4);
+    long total = 0, differing = 0; int worst = 0;
+    for (uint64_t i = a; i <= b; i += step) {
+        uint32_t bits = (uint32_t)i; float x; memcpy(&x, &bits, 4);
+        float want = which ? expm1_formula(x) : log1p_formula(x);
+        float got = which ? ovl_math::expm1_direct_(x) : ovl_math::log1p_direct_<true>(x);
+        int d = abs(ordered(want) - ordered(got));
+        ++total; if (d) ++differing; if (d > worst) worst = d;
+    }
+    float nan_result = which ? ovl_math::expm1_direct_(NAN) : ovl_math::log1p_direct_<true>(NAN);
+    printf("%ld %ld %d %d\n", total, differing, worst, nan_result != nan_result ? 1 : 0);
+    return 0;
+}
+'''
+
+
+@pytest.fixture(scope='module')
+def sweep(tmp_path_factory):
+    directory = tmp_path_factory.mktemp('once_rounded')
+    src = directory / 'sweep.cpp'
+    src.write_text(PROGRAM)
+    exe = directory / 'sweep'
+    subprocess.check_call(['g++', '-O2', '-ffp-contract=off', '-mfma', '-std=c++17', '-I' + CSRC, str(src), '-o',
+                           str(exe)])
+    return exe
+
+
+@pytest.mark.parametrize('kind', ['log1p', 'expm1'])
+def test_once_rounded_routines_within_two_ulp_of_the_reference_formulas_on_the_host(sweep, kind):
+    lo, hi = accuracy.IDIOM_DOMAIN[kind]
+    out = subprocess.check_output([str(sweep), '01'[kind == 'expm1'], repr(lo), repr(hi), '31'],
+                                  universal_newlines=True).split()
+    total, differing, worst, nan_kept = (int(v) for v in out)
+    assert total > 4 << 20
+    assert worst <= accuracy.ROUTINE_ULPS[kind] == accuracy.TOLERANCE
+    assert 0 < differing < total // 2
+    assert nan_kept == 1
+
+
+@pytest.mark.parametrize('kind,outside', [('log1p', (8e37, 3e38)), ('expm1', (70.0, 88.0))])
+def test_the_domain_limits_are_needed(sweep, kind, outside):
+    """Towards overflow the reference's formulas (whose 1 + x and exp(x) become infinite early) leave the once-rounded
+    values far behind, which is why the code generator keeps the formula outside the domains."""
+    out = subprocess.check_output([str(sweep), '01'[kind == 'expm1'], repr(outside[0]), repr(outside[1]), '1'],
+                                  universal_newlines=True).split()
+    assert int(out[2]) > accuracy.TOLERANCE
+
+
+def test_formula_outside_the_domain_is_not_replaced():
+    """A consumer of raw input (range unknown) keeps the formula; one behind a clip into the domain gets the
+    routine."""
+    @ovl.operator()
+    def clipped(x):
+        out = ovl.output_like(x)
+        pos = ovl.position_in(x.shape)
+        out[pos] = ovl.minimum(ovl.maximum(x[pos], 0.25), 0.75)
+        return out
+
+    raw = dict(selection(workloads.fused_operators([log1p(Spec((1024,)))[0]])[0]))
+    assert 'log1p' not in raw
+    fused, = workloads.fused_operators([log1p(clipped(Spec((1024,))))[0]])
+    assert dict(selection(fused)).get('log1p') is True
+    too_wide, = workloads.fused_operators([expm1(stdops.mul(clipped(Spec((1024,))), np.array([200.0], np.float32)))[0]])
+    assert 'expm1' not in dict(selection(too_wide))
+    fused, = workloads.fused_operators([stdops.sigmoid(clipped(Spec((1024,))))[0]])
+    assert dict(selection(fused)).get('sigmoid') is True
+
+
+def test_rounding_operations_after_an_inexact_value_cost_a_step():
+    """exp(x) + 1 stored: the cheap exp is one ulp off and the rounding of the sum can add another: still two.
+    (exp(x) + 1) * 3 stored: up to twice that plus one: the exp must be the bit-compatible one."""
+    @ovl.operator()
+    def exp_plus_one(x):
+        out = ovl.output_like(x)
+        pos = ovl.position_in(x.shape)
+        out[pos] = ovl.exp(x[pos]) + 1.0
+        return out
+
+    @ovl.operator()
+    def exp_plus_one_times_three(x):
+        out = ovl.output_like(x)
+        pos = ovl.position_in(x.shape)
+        out[pos] = (ovl.exp(x[pos]) + 1.0) * 3.0
+        return out
+
+    x = Spec((256,))
+    assert selection(workloads.unfused_operators([exp_plus_one(x)[0]])[0]) == [(lang.EXP, True)]
+    assert selection(workloads.unfused_operators([exp_plus_one_times_three(x)[0]])[0]) == [(lang.EXP, False)]

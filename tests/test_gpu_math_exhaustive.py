@@ -10,6 +10,9 @@ exponents and both signs); OVL_EXHAUSTIVE=1 compares all 2^32 (about 10 s per fu
 argument the code generator may hand them (division: 2^32 operand pairs), device against device.
 `test_fast_mode_routines_*`: the optional fast routines against the host C library, largest distance in units in the
 last place (measured over all 2^32 arguments: expf 1, logf 2, tanhf 2, reciprocal 0).
+`test_formula_routines_*`: the sigmoid / log1p / expm1 routines that the 'ulp2' math mode puts in place of the
+reference's formulas, against those formulas evaluated with the host C library, on every float32 of the domain on which the code
+generator uses them: at most 2 units in the last place.
 """
 import ctypes
 import os
@@ -103,3 +106,33 @@ def test_in_range_variants_equal_the_full_routines(lib, name):
     assert compared.value >= at_least, 'only %d arguments were compared' % compared.value
     assert bad.value == 0, '%s: %d of %d arguments differ, first at 0x%08x' % (name, bad.value, compared.value,
                                                                                first.value)
+
+
+def _bits(value):
+    import struct
+    return struct.unpack('<I', struct.pack('<f', value))[0]
+
+
+@pytest.mark.parametrize('kind', ['sigmoid', 'log1p', 'expm1'])
+def test_formula_routines_within_two_ulp_of_the_reference_formulas(lib, kind):
+    """Every float32 argument of the domain the code generator allows (hipgen/accuracy.py: IDIOM_DOMAIN)."""
+    from opveclib_amd.hipgen import accuracy
+    lib.ovl_exh_ulp_in_range.argtypes = [ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32] + \
+        [ctypes.POINTER(ctypes.c_uint64)] * 3 + [ctypes.POINTER(ctypes.c_uint32)] * 2
+    lo, hi = accuracy.IDIOM_DOMAIN[kind]
+    # ranges of bit patterns of one sign each: consecutive patterns are consecutive floats
+    spans = [(_bits(lo), _bits(hi))] if lo > 0 else [(_bits(-0.0), _bits(lo)), (_bits(0.0), _bits(hi))]
+    total = total_differing = 0
+    for first, last in spans:
+        compared, differing, beyond = ctypes.c_uint64(0), ctypes.c_uint64(0), ctypes.c_uint64(0)
+        largest, where = ctypes.c_uint32(0), ctypes.c_uint32(0)
+        err = lib.ovl_exh_ulp_in_range({'log1p': 9, 'expm1': 10, 'sigmoid': 11}[kind], first, last,
+                                       min(16, os.cpu_count() or 1), ctypes.byref(compared), ctypes.byref(differing),
+                                       ctypes.byref(beyond), ctypes.byref(largest), ctypes.byref(where))
+        assert err == 0, 'HIP error %d' % err
+        assert beyond.value == 0 and largest.value <= accuracy.ROUTINE_ULPS[kind], \
+            '%s: %d ulp at bits 0x%08x, %d arguments beyond 2 ulp' % (kind, largest.value, where.value, beyond.value)
+        total += compared.value
+        total_differing += differing.value
+    assert total > 140 << 20
+    assert total_differing > 0          # it is not the formula itself

@@ -1,0 +1,148 @@
+"""
+The 'ulp2' float32 math mode on the GPU.
+
+Promise of the mode: every operator's outputs are within two float32 units in the last place (ulp) of what the
+reference's generated C++ computes from the same operator inputs (the tolerance stated for transcendental operators);
+in a fused chain the promise holds for every operator of the chain.  The CPU oracle is that reference; the 'exact'
+mode returns the oracle's bits (tests/test_gpu_parity.py, tests/test_gpu_configs.py), so at sizes the oracle would
+need minutes for, the exact mode stands in for it and the oracle itself is applied to a slice of rows.
+
+  * all eight stages of the benchmark chain at full size [8192, 8192], two ways: each stage of the fused kernel
+    against the exact operator applied to the same stage input, and each stage's operator fed the exact mode's
+    stage input (the oracle's bits) against the exact mode's stage output;
+  * the same on a slice of rows against the oracle itself;
+  * every transcendental operator on its own, on chain-like inputs and on wide sweeps, against the oracle;
+  * fused test cases end to end: absolute error of a few ulp of the O(1) intermediates, NaN / infinity patterns equal;
+  * operators without exp / log / tanh / division do not change with the mode.
+"""
+import numpy as np
+import pytest
+
+import opveclib_amd as ovl
+import oracle
+from opveclib_amd import workloads
+from tests import cases
+
+pytestmark = pytest.mark.gpu
+
+TOLERANCE = 2
+MATH_STAGES = ('tanh', 'sigmoid', 'log1p', 'expm1')
+
+
+def _ulps(x, y):
+    import torch
+    xi, yi = x.view(torch.int32).long(), y.view(torch.int32).long()
+    xi = torch.where(xi < 0, -(xi & 0x7fffffff), xi)
+    yi = torch.where(yi < 0, -(yi & 0x7fffffff), yi)
+    return (xi - yi).abs()
+
+
+@pytest.fixture(scope='module')
+def chain_inputs():
+    import torch
+    rng = np.random.default_rng(2)
+    a = torch.from_numpy(workloads.uniform(rng, -1, 1, cases.CHAIN8_SHAPE)).cuda()
+    b = torch.from_numpy(workloads.uniform(rng, -1, 1, cases.CHAIN8_SHAPE)).cuda()
+    s = torch.tensor([1.0001], dtype=torch.float32).cuda()
+    return a, b, s
+
+
+def test_every_stage_of_the_fused_chain_at_full_size(chain_inputs):
+    """One launch of the fused kernel in 'ulp2' mode with every stage requested; stage k is compared with the exact
+    operator applied to the kernel's own stage k-1 output (sub also reads B).  add, mul, sub and abs must be exact."""
+    import torch
+    a, b, s = chain_inputs
+    outs = workloads.chain8_stage_outputs(a, b, s)
+    assert len(workloads.fused_operators(outs)) == 1
+    stages = ovl.evaluate(outs, opt_level=3, math_mode='ulp2')
+    exact_ops = {'add': lambda prev: cases.stdops.add(a, b), 'mul': lambda prev: cases.stdops.mul(prev, s),
+                 'sub': lambda prev: cases.stdops.sub(prev, b), 'abs': lambda prev: cases.absolute(prev)}
+    for k, name in enumerate(cases.CHAIN8_STAGES):
+        prev = stages[k - 1] if k else None
+        if name in MATH_STAGES:
+            ref = ovl.evaluate(cases.chain8_single_stage(name, prev), opt_level=0, math_mode='exact')
+            worst = int(_ulps(stages[k], ref).max())
+            assert worst <= TOLERANCE, 'stage %s: %d ulp' % (name, worst)
+        else:
+            ref = ovl.evaluate(exact_ops[name](prev)[0], opt_level=0, math_mode='exact')
+            assert torch.equal(stages[k], ref), 'stage %s is not exact' % name
+        del ref
+    # the oracle itself on a slice of rows of every transcendental stage
+    rows = slice(4000, 4064)
+    for k, name in enumerate(cases.CHAIN8_STAGES):
+        if name in MATH_STAGES:
+            x = stages[k - 1][rows].cpu().numpy()
+            want = oracle.evaluate(cases.chain8_single_stage(name, x))
+            got = stages[k][rows].cpu().numpy()
+            assert cases.ulp_distance(got, want).max() <= TOLERANCE, name
+
+
+def test_every_stage_on_the_exact_stage_inputs_at_full_size(chain_inputs):
+    """Each stage's operator in 'ulp2' mode is fed the exact mode's stage input (the oracle's bits) and compared with
+    the exact mode's stage output.  log1p and expm1 sit behind a clip to their stage's input range, as they sit behind
+    sigmoid and log1p in the chain, so that the code generator makes the choices it makes in the fused kernel."""
+    import torch
+    from opveclib_amd import runtime
+    a, b, s = chain_inputs
+    exact = ovl.evaluate(workloads.chain8_stage_outputs(a, b, s), opt_level=0, math_mode='exact')
+    rows = slice(100, 164)
+    want = oracle.evaluate(workloads.chain8_stage_outputs(a[rows].cpu().numpy(), b[rows].cpu().numpy(),
+                                                          s.cpu().numpy()))
+    for k, name in enumerate(cases.CHAIN8_STAGES):
+        assert np.array_equal(exact[k][rows].cpu().numpy(), want[k]), 'exact mode differs from the oracle at ' + name
+        if name not in MATH_STAGES:
+            continue
+        x = exact[k - 1]
+        if name in cases.CHAIN8_STAGE_INPUT_RANGE:
+            lo, hi = cases.CHAIN8_STAGE_INPUT_RANGE[name]
+            assert float(x.min()) >= lo and float(x.max()) <= hi     # the clip changes nothing
+        got = ovl.evaluate(cases.chain8_single_stage(name, x, with_range=True), opt_level=3, math_mode='ulp2')
+        worst = int(_ulps(got, exact[k]).max())
+        assert worst <= TOLERANCE, 'stage %s: %d ulp' % (name, worst)
+        del got
+    # the kernels that ran are the ones with the cheap routines, not the exact ones
+    sources = [c.gen.source for key, c in runtime._loaded.items() if "'math', 'ulp2'" in key[1]]
+    assert any('ovl_log1p_direct' in text for text in sources)
+    assert any('ovl_expm1_direct' in text for text in sources)
+    assert any('ovl_fast_tanhf' in text for text in sources)
+
+
+@pytest.mark.parametrize('case', cases.FAST_CASES, ids=[c.name for c in cases.FAST_CASES])
+def test_single_operators_within_two_ulp_of_the_oracle(case):
+    for dist in cases.run_fast_case_on_gpu(case, 'ulp2'):
+        assert dist.max() <= TOLERANCE, '%s: %d ulp' % (case.name, int(dist.max()))
+
+
+@pytest.mark.parametrize('name', cases.FAST_FUSED_CASES)
+def test_fused_cases_stay_close_end_to_end(name):
+    case = cases.CASE_BY_NAME[name]
+    outs = case.outputs()
+    ref = oracle.profile(outs, 1, 0)[0]
+    got = ovl.evaluate(outs, opt_level=3, math_mode='ulp2')
+    got = got if isinstance(got, list) else [got]
+    for g, r in zip(got, ref):
+        finite = np.isfinite(r)
+        assert np.array_equal(g[~finite], r[~finite], equal_nan=True), name + ': NaN / infinity pattern differs'
+        scale = max(1.0, float(np.abs(r[finite]).max()))
+        assert float(np.abs(g[finite].astype(np.float64) - r[finite]).max()) <= 8 * np.finfo(np.float32).eps * scale
+
+
+def test_small_chain_stagewise_against_the_oracle():
+    """The chain at a size the oracle finishes at once: every stage of the fused 'ulp2' kernel against the oracle's
+    operator on the same stage input."""
+    outs = cases.CASE_BY_NAME['c2_chain_stages'].outputs()
+    stages = ovl.evaluate(outs, opt_level=3, math_mode='ulp2')
+    for k, name in enumerate(cases.CHAIN8_STAGES):
+        if name in MATH_STAGES:
+            want = oracle.evaluate(cases.chain8_single_stage(name, stages[k - 1]))
+            assert cases.ulp_distance(stages[k], want).max() <= TOLERANCE, name
+
+
+def test_lstm_keeps_the_oracle_bits_in_ulp2_mode():
+    """The LSTM cell adds products of either sign, so no call site of it may be inexact: the mode changes nothing."""
+    for name in ('c4_lstm', 'c4_lstm_grad'):
+        outs = cases.CASE_BY_NAME[name].outputs()
+        ref = oracle.profile(outs, 1, 0)[0]
+        got = ovl.evaluate(outs, opt_level=3, math_mode='ulp2')
+        for g, r in zip(got, ref):
+            assert np.array_equal(g, r, equal_nan=True), name
