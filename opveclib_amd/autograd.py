@@ -91,9 +91,23 @@ def build_backward(op_dag, wanted):
 
     leaf_slot = dict((id(leaf), n) for n, leaf in enumerate(op_dag.inputs))
     leaf_contributions = [[] for _ in op_dag.inputs]
+    # operators and leaves that a gradient reaches only to stop at an operator without a gradient definition
+    blocked_ops = {}        # id(operator) -> name of the operator that stops the gradient
+    blocked_leaves = {}     # leaf slot -> the same
 
     for op in reversed(ops):            # operators are sorted by depth, so consumers come before producers here
         received = [pending.get((id(op), k), []) for k in range(len(op.output_types))]
+        stopped_by = blocked_ops.get(id(op))
+        if op.grad_dag is None and any(received):
+            stopped_by = op.name
+        if stopped_by is not None:
+            for cur_input in op.inputs:
+                try:
+                    resolved = _resolve_output(cur_input)
+                except TypeError:
+                    blocked_leaves.setdefault(leaf_slot[id(cur_input)], stopped_by)
+                else:
+                    blocked_ops.setdefault(id(resolved.parent), stopped_by)
         if op.grad_dag is None or not any(received):
             continue
         grad_inputs = list(op.inputs) + [_total(c, t) for c, t in zip(received, op.output_types)]
@@ -108,6 +122,9 @@ def build_backward(op_dag, wanted):
 
     leaf_grads = []
     for n, leaf in enumerate(op_dag.inputs):
+        if wanted[n] and n in blocked_leaves:
+            raise ValueError('the gradient of input %d passes through operator "%s", which has no gradient defined'
+                             % (n, blocked_leaves[n]))
         if wanted[n] and leaf_contributions[n]:
             leaf_grads.append(_total(leaf_contributions[n], TensorType.like(leaf)))
         else:
@@ -134,10 +151,10 @@ def as_torch(output_list, opt_level=3, math_mode=None):
     :param output_list: an operator, an operator output, or a list of either; the DAG's leaf inputs are torch tensors
         on a HIP device (differentiable where they require grad) or numpy arrays (copied to the device, constant)
     :param opt_level: operators are fused when opt_level >= 3 (forward and backward)
-    :param math_mode: 'exact' or 'fast'; None uses the current default
+    :param math_mode: 'exact', 'ulp2' or 'fast'; None uses the current default
     :return: one tensor for a single requested output, otherwise a list in request order
-    :raises ValueError: if a gradient is requested through an operator that has no gradient defined - raised by
-        autograd at ``backward()`` time as for any non-differentiable function (the gradient is None)
+    :raises ValueError: at ``backward()`` time, if the gradient of an input that requires one passes through an
+        operator that has no gradient defined
     """
     import torch
 

@@ -86,8 +86,8 @@ lstm_forward_kernel(const float* __restrict__ concat, const float* __restrict__ 
         const uint64_t at = (uint64_t)row * units + elem;
         const vec vi = load_nt<vec>(gates);
         const vec vj = load_nt<vec>(gates + units);
-        const vec vf = load_nt<vec>(gates + 2u * units);
-        const vec vo = load_nt<vec>(gates + 3u * units);
+        const vec vf = load_nt<vec>(gates + (uint64_t)2 * units);
+        const vec vo = load_nt<vec>(gates + (uint64_t)3 * units);
         const vec vc = load_nt<vec>(c + at);
         vec out_c, out_h;
 #pragma unroll
@@ -126,8 +126,8 @@ lstm_backward_kernel(const float* __restrict__ concat, const float* __restrict__
         const float* gates = concat + gate_at;
         const vec vi = load_nt<vec>(gates);
         const vec vj = load_nt<vec>(gates + units);
-        const vec vf = load_nt<vec>(gates + 2u * units);
-        const vec vo = load_nt<vec>(gates + 3u * units);
+        const vec vf = load_nt<vec>(gates + (uint64_t)2 * units);
+        const vec vo = load_nt<vec>(gates + (uint64_t)3 * units);
         const vec vc = load_nt<vec>(c + at);
         const vec vdc = load_nt<vec>(d_new_c + at);
         const vec vdh = load_nt<vec>(d_new_h + at);
@@ -153,8 +153,8 @@ lstm_backward_kernel(const float* __restrict__ concat, const float* __restrict__
         float* grads = d_concat + gate_at;
         __builtin_nontemporal_store(out_i, reinterpret_cast<vec*>(grads));
         __builtin_nontemporal_store(out_j, reinterpret_cast<vec*>(grads + units));
-        __builtin_nontemporal_store(out_f, reinterpret_cast<vec*>(grads + 2u * units));
-        __builtin_nontemporal_store(out_o, reinterpret_cast<vec*>(grads + 3u * units));
+        __builtin_nontemporal_store(out_f, reinterpret_cast<vec*>(grads + (uint64_t)2 * units));
+        __builtin_nontemporal_store(out_o, reinterpret_cast<vec*>(grads + (uint64_t)3 * units));
         __builtin_nontemporal_store(out_c, reinterpret_cast<vec*>(d_c + at));
     }
 }

@@ -19,6 +19,38 @@
 // The file compiles as plain C++ for the host as well (no HIP headers needed), which is how the routines are checked
 // against the host C library over all 2^32 float arguments.  All arithmetic must be compiled without contraction
 // (-ffp-contract=off); fused operations are spelled out with __builtin_fma.
+//
+// Third-party notices.  The algorithms, lookup tables and polynomial coefficients of expf_ / logf_ (and of the
+// once-rounded expm1 / log1p built on them) come from Arm Optimized Routines (math/expf.c, math/logf.c,
+// math/exp2f_data.c, math/logf_data.c), which the GNU C library adopted:
+//
+//   Copyright (c) 2017-2018, Arm Limited.
+//   SPDX-License-Identifier: MIT
+//
+//   Permission is hereby granted, free of charge, to any person obtaining a copy of this software and associated
+//   documentation files (the "Software"), to deal in the Software without restriction, including without limitation
+//   the rights to use, copy, modify, merge, publish, distribute, sublicense, and/or sell copies of the Software, and
+//   to permit persons to whom the Software is furnished to do so, subject to the following conditions:
+//
+//   The above copyright notice and this permission notice shall be included in all copies or substantial portions of
+//   the Software.
+//
+//   THE SOFTWARE IS PROVIDED "AS IS", WITHOUT WARRANTY OF ANY KIND, EXPRESS OR IMPLIED, INCLUDING BUT NOT LIMITED TO
+//   THE WARRANTIES OF MERCHANTABILITY, FITNESS FOR A PARTICULAR PURPOSE AND NONINFRINGEMENT.  IN NO EVENT SHALL THE
+//   AUTHORS OR COPYRIGHT HOLDERS BE LIABLE FOR ANY CLAIM, DAMAGES OR OTHER LIABILITY, WHETHER IN AN ACTION OF
+//   CONTRACT, TORT OR OTHERWISE, ARISING FROM, OUT OF OR IN CONNECTION WITH THE SOFTWARE OR THE USE OR OTHER DEALINGS
+//   IN THE SOFTWARE.
+//
+// expm1f_ and the tanh routines follow fdlibm's s_expm1f.c and s_tanhf.c (constants and evaluation order):
+//
+//   ====================================================
+//   Copyright (C) 1993 by Sun Microsystems, Inc. All rights reserved.
+//
+//   Developed at SunPro, a Sun Microsystems, Inc. business.
+//   Permission to use, copy, modify, and distribute this
+//   software is freely granted, provided that this notice
+//   is preserved.
+//   ====================================================
 #ifndef OVL_MATH_H_
 #define OVL_MATH_H_
 

@@ -103,6 +103,21 @@ def _same_subtree(dag0, index0, dag1, index1):
     return True
 
 
+def _reads_tensor_data(dag, index):
+    """True when the sub-DAG of ``index`` reads an operator input (an index that depends on tensor contents)."""
+    pending = [index]
+    seen = set()
+    while pending:
+        cur = pending.pop()
+        if cur in seen:
+            continue
+        seen.add(cur)
+        if dag.expressions[cur].code in (lang.INPUT, lang.OUTPUT):
+            return True
+        pending.extend(dag.references[cur].operand_indices)
+    return False
+
+
 def _constant_int(dag, index):
     """Value of an integer literal (through casts)."""
     expr = dag.expressions[index]
@@ -292,11 +307,20 @@ def _edge_kind(ops, to_op_index, to_in_arg_index, in_ref):
     first_index = from_dag.references[writes[0]].operand_indices[1]
     if _depends_on_variable(from_dag, first_index):
         return None, 'Write index depends on a variable for '
+    # An index computed from tensor contents never qualifies.  Input numbers are local to each operator, so equal
+    # sub-DAGs of two operators may read different tensors (out[idx1[p]] = x[p] followed by y[p] = t[idx2[p]]); and
+    # even with one index tensor the store need not be one-to-one, in which case the element a consumer reads was
+    # written by another worker.
+    if _reads_tensor_data(from_dag, first_index):
+        return None, 'Write index depends on tensor contents for '
     for other in writes[1:]:
         if not _same_subtree(from_dag, first_index, from_dag, from_dag.references[other].operand_indices[1]):
             return None, 'Multiple write patterns to the producer output for '
     for read in _accesses(to_dag, lang.READ_TENSOR, in_expr_index):
-        if not _same_subtree(from_dag, first_index, to_dag, to_dag.references[read].operand_indices[1]):
+        read_index = to_dag.references[read].operand_indices[1]
+        if _reads_tensor_data(to_dag, read_index):
+            return None, 'Read index depends on tensor contents for '
+        if not _same_subtree(from_dag, first_index, to_dag, read_index):
             return adopted('No-matching read/write index pattern for ')
     return 'same', None
 

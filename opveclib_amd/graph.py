@@ -22,7 +22,7 @@ class CapturedDag(object):
         contiguous torch tensor on one HIP device whose data pointer is 16-byte aligned; these tensors are the graph's
         input buffers.
     :param opt_level: operators are fused when opt_level >= 3
-    :param math_mode: 'exact' or 'fast'; None uses the current default
+    :param math_mode: 'exact', 'ulp2' or 'fast'; None uses the current default
     """
 
     def __init__(self, output_list, opt_level=3, math_mode=None):

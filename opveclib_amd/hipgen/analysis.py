@@ -334,6 +334,24 @@ class DagInfo(object):
                 found.append((node, self.nodes[node.ops[0]], self.affine[node.ops[1]]))
         return found
 
+    def bufferable_outputs(self):
+        """
+        Output node indices whose stores may be held in registers (or an LDS tile) until the end of the worker's
+        iteration: every store to the tensor is outside loops and uses one affine index.  A store that a template
+        cannot buffer (inside a loop, through a computed index) is written at once; buffering another store to the
+        same tensor would write it later and so reverse the program's order whenever both hit one element.
+        """
+        signatures = {}
+        refused = set()
+        for node, tensor, aff in self.tensor_accesses():
+            if node.code != lang.ASSIGN_TENSOR:
+                continue
+            if aff is None or self.in_loop[node.idx]:
+                refused.add(tensor.idx)
+            else:
+                signatures.setdefault(tensor.idx, set()).add(aff.signature())
+        return set(idx for idx, found in signatures.items() if len(found) == 1 and idx not in refused)
+
     def definitely_stores(self, keys):
         """
         Subset of ``keys`` (each a (output node index, affine signature)) that every worker is certain to store on

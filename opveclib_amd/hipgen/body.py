@@ -104,7 +104,7 @@ def binary_text(code, dtype, a, b):
     if code == lang.POW:
         return ('powf(' if dtype == lang.FLOAT32 else 'pow(') + a + ',' + b + ')'
     if code == lang.ATAN2:
-        return ('atan2f(' if dtype == lang.FLOAT32 else 'atan2(') + a + ',' + b + ')'
+        return ('ovl_atan2f(' if dtype == lang.FLOAT32 else 'atan2(') + a + ',' + b + ')'
     if code == lang.MODULO and dtype == lang.FLOAT32:
         return 'fmodf(' + a + ',' + b + ')'
     if code == lang.MODULO and dtype == lang.FLOAT64:

@@ -130,8 +130,9 @@ def generate(info, kernel_name, vec=None, nt=None, grid_cap=None):
             if key not in unaligned:
                 unaligned[key] = Access(tensor, aff, 'lu%d' % len(unaligned))
     certain = info.definitely_stores(store_keys)
+    bufferable = info.bufferable_outputs()
     for node, tensor, aff in accesses:
-        if node.code == lang.ASSIGN_TENSOR and aff is not None:
+        if node.code == lang.ASSIGN_TENSOR and aff is not None and tensor.idx in bufferable:
             key = (tensor.idx, aff.signature())
             if key in certain and key not in stores and vec > 1 and _is_vector_access(info, node, tensor, aff, vec):
                 stores[key] = Access(tensor, aff, 'st%d' % len(stores))

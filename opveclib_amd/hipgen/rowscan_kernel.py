@@ -54,6 +54,15 @@ def plan(info, rows_per_block=None, chunk=None):
     if len(loops) != 1 or any(item.kind == 'if' for item in info.tree):
         return None
     loop = loops[0]
+    # the shape the scan generators rely on: what sets up the first column (at most one store), then the loop, then
+    # nothing; anything else (a store after the loop, two stores before it) runs on the map template
+    if info.tree[-1] is not loop:
+        return None
+    stores_before = [item for item in info.tree[:-1] if item.kind == 'stmt' and
+                     info.nodes[item.node].code == lang.ASSIGN_TENSOR and
+                     info.nodes[info.nodes[item.node].ops[0]].code == lang.OUTPUT]
+    if len(stores_before) > 1:
+        return None
     range_node = info.nodes[loop.node]
     counter = range_node.ops[0]
     if counter not in info.loop_counters:

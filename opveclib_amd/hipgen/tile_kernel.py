@@ -56,7 +56,8 @@ def applicable(info):
     keys = [(t.idx, a.signature()) for n, t, a in stores if _is_transposed_store(info, n, t, a, vec)]
     if not keys:
         return None
-    certain = info.definitely_stores(keys)
+    bufferable = info.bufferable_outputs()
+    certain = set(key for key in info.definitely_stores(keys) if key[0] in bufferable)
     if not certain:
         return None
     # all transposed outputs share one element width so one tile geometry serves them all
@@ -96,8 +97,9 @@ def generate(info, kernel_name, tile_i=None, tile_j=None, nt='ls'):
             elif _is_transposed_store(info, node, tensor, aff, vec):
                 tkeys.append((tensor.idx, aff.signature()))
     certain = info.definitely_stores(store_keys + tkeys)
+    bufferable = info.bufferable_outputs()
     for node, tensor, aff in accesses:
-        if node.code != lang.ASSIGN_TENSOR or aff is None:
+        if node.code != lang.ASSIGN_TENSOR or aff is None or tensor.idx not in bufferable:
             continue
         key = (tensor.idx, aff.signature())
         if key not in certain:

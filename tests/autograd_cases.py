@@ -245,7 +245,8 @@ def graphs_to_build():
         outputs = [_resolve_output(o) for o in case.graph(*leaves)]
         built.append(outputs)
         op_dag = _build_op_dag(*outputs)
-        wanted = [any(leaf is leaves[k] for k in case.differentiable) for leaf in op_dag.inputs]
+        differentiable = [1] if case is NO_GRADIENT else case.differentiable
+        wanted = [any(leaf is leaves[k] for k in differentiable) for leaf in op_dag.inputs]
         leaf_grads, _ = autograd.build_backward(op_dag, wanted)
         backward = [g for g in leaf_grads if g is not None]
         if backward:

@@ -562,6 +562,52 @@ def _adopted_position(rng):
             stdops.tanh(stdops.add(transpose_scaled(m), v))[0]]
 
 
+@ovl.operator()
+def store_then_loop_store(x):
+    """One element stored at the top level and again, with another value, inside a loop: the last store must win."""
+    out = ovl.output_like(x)
+    pos = ovl.position_in(x.shape)
+    out[pos] = x[pos]
+    acc = ovl.variable(0, x.dtype)
+    for _ in ovl.arange(3):
+        acc <<= acc + x[pos]
+        out[pos] = acc
+    return out
+
+
+@ovl.operator()
+def scan_late_store(x):
+    """A row scan that stores its first column after the loop instead of before it."""
+    out = ovl.output_like(x)
+    pos = ovl.position_in([x.shape[0]])
+    acc = ovl.variable(x[pos[0], 0], x.dtype)
+    for i in ovl.arange(1, x.shape[1]):
+        acc <<= acc + x[pos[0], i]
+        out[pos[0], i] = acc
+    out[pos[0], 0] = x[pos[0], 0] * 2
+    return out
+
+
+@ovl.operator()
+def scan_two_stores(x):
+    """A row scan whose first column is stored twice before the loop."""
+    out = ovl.output_like(x)
+    pos = ovl.position_in([x.shape[0]])
+    acc = ovl.variable(x[pos[0], 0], x.dtype)
+    out[pos[0], 0] = acc * 3
+    out[pos[0], 0] = acc
+    for i in ovl.arange(1, x.shape[1]):
+        acc <<= acc + x[pos[0], i]
+        out[pos[0], i] = acc
+    return out
+
+
+def _store_order(rng):
+    x = rng.standard_normal((64, 256), dtype=np.float32)
+    return [store_then_loop_store(rng.standard_normal(1024, dtype=np.float32))[0], scan_late_store(x)[0],
+            scan_two_stores(x)[0]]
+
+
 def _odd_sizes(rng):
     # sizes that are not multiples of the vector width, rank 1 and rank 3
     a = rng.standard_normal(1001, dtype=np.float32)
@@ -585,6 +631,7 @@ CASES = [
     Case('c4_lstm_grad', c4_lstm_grad, seed=4),
     Case('c5_gather_transpose', c5_gather_transpose, seed=5),
     Case('c5_variants', c5_variants, seed=5),
+    _simple('store_order', _store_order),
     _simple('clip', lambda rng: [clip(rng.random(1000), threshold1=0.1, threshold2=0.9)[0]]),
     _simple('limits_f32', lambda rng: [set_limits(np.array([0], np.float32))[0]]),
     _simple('limits_f64', lambda rng: [set_limits(np.array([0], np.float64))[0]]),
@@ -787,6 +834,42 @@ def run_fast_case_on_gpu(case, math_mode='fast'):
 
 
 # ----------------------------------------------------------------------------------------------------------------------
+# strided sweeps of the float32 functions that come from the device math library
+# ----------------------------------------------------------------------------------------------------------------------
+LIBRARY_SWEEP_STEP = 4099       # every 4099th float32 bit pattern: about one million arguments over all exponents
+LIBRARY_UNARY = [('sin', ovl.sin), ('cos', ovl.cos), ('tan', ovl.tan), ('arcsin', ovl.arcsin),
+                 ('arccos', ovl.arccos), ('arctan', ovl.arctan), ('sinh', ovl.sinh), ('cosh', ovl.cosh),
+                 ('log10', ovl.log10), ('sqrt', ovl.sqrt)]
+LIBRARY_BINARY = [('power', ovl.power), ('arctan2', ovl.arctan2)]
+
+
+def library_sweep_arguments():
+    """Every LIBRARY_SWEEP_STEP-th float32 bit pattern (both signs, subnormals, infinities, NaNs included)."""
+    bits = np.arange(0, 1 << 32, LIBRARY_SWEEP_STEP, dtype=np.uint64).astype(np.uint32)
+    return bits.view(np.float32)
+
+
+def library_sweep_pairs(n=1 << 20):
+    """Operand pairs with magnitudes spread over binades 2^-40 .. 2^40, both signs, some exact small integers."""
+    rng = np.random.default_rng(11)
+    sign = lambda: np.where(rng.random(n) < 0.5, -1.0, 1.0).astype(np.float32)
+    a = sign() * _log_uniform(rng, -40, 40, n)
+    b = sign() * _log_uniform(rng, -40, 40, n)
+    b[::5] = rng.integers(-8, 9, size=b[::5].size).astype(np.float32)
+    a[::7] = sign()[::7] * _log_uniform(rng, -3, 3, a[::7].size)
+    return a, b
+
+
+def library_sweep_outputs():
+    """[(name, operator output)] of the sweeps (tests/test_gpu_library_math.py)."""
+    x = library_sweep_arguments()
+    a, b = library_sweep_pairs()
+    found = [(name, _unary_op(fcn)(x)[0]) for name, fcn in LIBRARY_UNARY]
+    found += [(name, _binary_op(fcn)(a, b)[0]) for name, fcn in LIBRARY_BINARY]
+    return found
+
+
+# ----------------------------------------------------------------------------------------------------------------------
 # 'ulp2' math mode at the benchmark's full size
 # ----------------------------------------------------------------------------------------------------------------------
 CHAIN8_SHAPE = (8192, 8192)
@@ -796,7 +879,7 @@ CHAIN8_STAGE_INPUT_RANGE = {'log1p': (0.25, 0.75), 'expm1': (0.2, 0.6)}
 
 
 @ovl.operator()
-def clip(x, lo=0.0, hi=1.0):
+def clip_to_range(x, lo=0.0, hi=1.0):
     """min(max(x, lo), hi): leaves every value inside [lo, hi] untouched and tells the code generator the range."""
     out = ovl.output_like(x)
     pos = ovl.position_in(x.shape)
@@ -810,7 +893,7 @@ def chain8_single_stage(name, x, with_range=False):
     fcn = {'tanh': stdops.tanh, 'sigmoid': stdops.sigmoid, 'log1p': log1p, 'expm1': expm1}[name]
     if with_range and name in CHAIN8_STAGE_INPUT_RANGE:
         lo, hi = CHAIN8_STAGE_INPUT_RANGE[name]
-        x = clip(x, lo=lo, hi=hi)
+        x = clip_to_range(x, lo=lo, hi=hi)
     return fcn(x)[0]
 
 
@@ -917,6 +1000,10 @@ def prebuild_all(cases=None, workers=8, with_oracle=True):
             for op in _operators_of(CASE_BY_NAME[name].outputs(), 3):
                 variants.append((op, {'math': 'ulp2'}))
         variants.extend(ulp2_full_size_operators())
+        for _name, out in library_sweep_outputs():
+            for op in _operators_of([out], 0):
+                ops[op.SerializeToString()] = op
+                oracle_ops[op.SerializeToString()] = op
         # tests/test_gpu_ulp2.py: the oracle on slices of 64 rows of the full-size chain and on the small chain's stages
         rows = np.zeros((64, CHAIN8_SHAPE[1]), np.float32)
         small = np.zeros((96, 256), np.float32)

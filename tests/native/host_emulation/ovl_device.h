@@ -176,6 +176,7 @@ static inline T __shfl_up(T value, unsigned delta, int width = 64) {
 #define ovl_logf_inrange_nan(x) ovl_math::logf_inrange_<true>((x), ovl_log_tab)
 #define ovl_recipf_inrange(x) (1.0f / (x))
 #define ovl_divf_inrange(a, b) ((a) / (b))
+#define ovl_atan2f(a, b) atan2f((a), (b))
 
 // The 'fast' math mode is built on device instructions; sources that also instantiate it (the hand-written LSTM
 // cell) compile against the exact routines here, and the emulation tests never select it.

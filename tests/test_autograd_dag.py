@@ -64,11 +64,19 @@ def test_unwanted_and_gradient_free_leaves_get_none():
     by_leaf = dict((id(leaf), g) for leaf, g in zip(op_dag.inputs, grads))
     assert by_leaf[id(leaves[0])] is not None and by_leaf[id(leaves[1])] is None
 
-    leaves, op_dag, grads, _ = _backward(ac.NO_GRADIENT)
-    by_leaf = dict((id(leaf), g) for leaf, g in zip(op_dag.inputs, grads))
     # no gradient is defined for the operator that consumes leaf 0; leaf 1 is reached through mul
+    leaves, op_dag, grads, _ = _backward(ac.NO_GRADIENT, wanted_leaves=[1])
+    by_leaf = dict((id(leaf), g) for leaf, g in zip(op_dag.inputs, grads))
     assert by_leaf[id(leaves[0])] is None and by_leaf[id(leaves[1])] is not None
     assert 'no_gradient_scale' in '_'.join(_names([by_leaf[id(leaves[1])]], merged=False))
+
+
+def test_wanted_gradient_through_an_operator_without_gradient_is_an_error():
+    """A missing gradient definition must not turn into a silent None (which autograd reads as zero)."""
+    with pytest.raises(ValueError, match='no_gradient_scale'):
+        _backward(ac.NO_GRADIENT, wanted_leaves=[0, 1])
+    with pytest.raises(ValueError, match='no_gradient_scale'):
+        _backward(ac.NO_GRADIENT, wanted_leaves=[0])
 
 
 def test_unused_output_gets_a_zero_gradient_operator():

@@ -268,3 +268,25 @@ def test_missing_operators_of_a_dag_are_built_side_by_side(tmp_path, monkeypatch
     seen_threads.clear()
     runtime._build_missing(dag.operators, None)
     assert not seen_threads
+
+
+def test_clear_op_cache_removes_cached_operators_only(tmp_path, monkeypatch):
+    """`clear_op_cache` (the reference's local.py:43-50) deletes what was compiled on demand in the per-user cache
+    and nothing else: other files there and the prebuilt operators of the package stay."""
+    from opveclib_amd import local
+    cache = tmp_path / 'cache'
+    cache.mkdir()
+    prebuilt = tmp_path / 'prebuilt'
+    prebuilt.mkdir()
+    for name in ('f0123_generic_hip.so', 'f0123_generic_hip.hip', 'fabc_generic_hip.so'):
+        (cache / name).write_text('x')
+        (prebuilt / name).write_text('x')
+    (cache / 'notes.txt').write_text('keep')
+    monkeypatch.setattr(local, 'cache_directory', str(cache))
+    monkeypatch.setattr(local, 'prebuilt_directory', str(prebuilt))
+    local.clear_op_cache()
+    assert sorted(p.name for p in cache.iterdir()) == ['notes.txt']
+    assert len(list(prebuilt.iterdir())) == 3
+    local.clear_op_cache()                      # an empty cache is fine
+    monkeypatch.setattr(local, 'cache_directory', str(tmp_path / 'missing'))
+    local.clear_op_cache()                      # and so is a cache that does not exist yet

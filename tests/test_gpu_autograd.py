@@ -66,14 +66,18 @@ def test_values_and_gradients_match_torch(case):
             assert torch.equal(got.detach(), ref.detach()), case.name + ': fused and unfused results differ'
 
 
-def test_leaf_behind_an_operator_without_gradient_gets_none():
+def test_leaf_behind_an_operator_without_gradient():
+    """Asking for the gradient raises; not asking for it (the leaf does not require grad) works."""
     import torch
     case = ac.NO_GRADIENT
     a, b = (torch.from_numpy(x).cuda().requires_grad_(True) for x in case.leaves())
     y = ovl.as_torch(case.graph(a, b))
-    ga, gb = torch.autograd.grad(y, [a, b], torch.ones_like(y), allow_unused=True)
-    assert ga is None
-    assert torch.equal(gb, 2 * a.detach())
+    with pytest.raises(ValueError, match='no_gradient_scale'):
+        torch.autograd.grad(y, [a, b], torch.ones_like(y), allow_unused=True)
+    a = a.detach()
+    y = ovl.as_torch(case.graph(a, b))
+    gb, = torch.autograd.grad(y, [b], torch.ones_like(y))
+    assert torch.equal(gb, 2 * a)
 
 
 def test_backward_through_surrounding_torch_graph_and_numpy_constants():
