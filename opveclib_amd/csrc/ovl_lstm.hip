@@ -64,9 +64,11 @@ __device__ __forceinline__ float sig_grad_(float x, float e) {
     return (x > -50.0f && x < 50.0f) ? q : 0.0f;
 }
 
+// Plain loads and non-temporal stores: measured fastest for these kernels' five to seven load streams
+// (forward 26.5 us against 27.2 with the hint on the loads too, gradient 36.4 against 41.7).
 template <typename V>
-__device__ __forceinline__ V load_nt(const float* p) {
-    return __builtin_nontemporal_load(reinterpret_cast<const V*>(p));
+__device__ __forceinline__ V load_vec(const float* p) {
+    return *reinterpret_cast<const V*>(p);
 }
 
 template <bool FAST, int VEC>
@@ -84,11 +86,11 @@ lstm_forward_kernel(const float* __restrict__ concat, const float* __restrict__ 
         const uint32_t elem = (v - row * vectors_per_row.divisor) * VEC;
         const float* gates = concat + (uint64_t)row * 4u * units + elem;
         const uint64_t at = (uint64_t)row * units + elem;
-        const vec vi = load_nt<vec>(gates);
-        const vec vj = load_nt<vec>(gates + units);
-        const vec vf = load_nt<vec>(gates + (uint64_t)2 * units);
-        const vec vo = load_nt<vec>(gates + (uint64_t)3 * units);
-        const vec vc = load_nt<vec>(c + at);
+        const vec vi = load_vec<vec>(gates);
+        const vec vj = load_vec<vec>(gates + units);
+        const vec vf = load_vec<vec>(gates + (uint64_t)2 * units);
+        const vec vo = load_vec<vec>(gates + (uint64_t)3 * units);
+        const vec vc = load_vec<vec>(c + at);
         vec out_c, out_h;
 #pragma unroll
         for (int u = 0; u < VEC; ++u) {
@@ -124,13 +126,13 @@ lstm_backward_kernel(const float* __restrict__ concat, const float* __restrict__
         const uint64_t gate_at = (uint64_t)row * 4u * units + elem;
         const uint64_t at = (uint64_t)row * units + elem;
         const float* gates = concat + gate_at;
-        const vec vi = load_nt<vec>(gates);
-        const vec vj = load_nt<vec>(gates + units);
-        const vec vf = load_nt<vec>(gates + (uint64_t)2 * units);
-        const vec vo = load_nt<vec>(gates + (uint64_t)3 * units);
-        const vec vc = load_nt<vec>(c + at);
-        const vec vdc = load_nt<vec>(d_new_c + at);
-        const vec vdh = load_nt<vec>(d_new_h + at);
+        const vec vi = load_vec<vec>(gates);
+        const vec vj = load_vec<vec>(gates + units);
+        const vec vf = load_vec<vec>(gates + (uint64_t)2 * units);
+        const vec vo = load_vec<vec>(gates + (uint64_t)3 * units);
+        const vec vc = load_vec<vec>(c + at);
+        const vec vdc = load_vec<vec>(d_new_c + at);
+        const vec vdh = load_vec<vec>(d_new_h + at);
         vec out_i, out_j, out_f, out_o, out_c;
 #pragma unroll
         for (int u = 0; u < VEC; ++u) {

@@ -26,7 +26,7 @@ from . import tile_kernel
 from . import rowscan_kernel
 
 #: bump when generated code changes for an unchanged DAG, so cached binaries are not reused
-CODEGEN_VERSION = 27
+CODEGEN_VERSION = 28
 
 
 
@@ -60,9 +60,9 @@ def generate(expression_dag, function_name, options=None):
     :param function_name: unique name of the operator (its content hash)
     :param options: optional dict.  ``template``: 'auto' (default), 'map', 'transpose', 'rowscan', 'skewscan' or 'treescan' restricts
         the choice of kernel template (a template that does not fit the DAG falls back to 'map'); ``vec`` forces the
-        map template with that vector width; ``scan_depth`` / ``scan_sets`` / ``scan_width`` / ``scan_interleave`` set the request burst (groups), the
+        map template with that vector width, ``per_thread`` its vectors per thread (1 or 2); ``scan_depth`` / ``scan_sets`` / ``scan_width`` / ``scan_interleave`` set the request burst (groups), the
         number of register sets, the 128-bit vectors per lane and phase and the rows per lane group of the lane-skewed scan; ``math``: 'exact'
-        or 'fast'; ``if_conversion`` / ``value_ranges``: False switches that transformation off; ``scan_rows`` / ``scan_chunk`` the LDS tile of the row scan; ``nt`` /
+        or 'fast'; ``if_conversion`` / ``value_ranges`` / ``cse``: False switches that transformation off; ``scan_rows`` / ``scan_chunk`` the LDS tile of the row scan, ``scan_batch`` the vectors per register set of its scanning wavefront; ``nt`` /
         ``scan_nt`` which vector accesses carry the non-temporal hint ('l' loads, 's' stores, 'ls', ''); ``grid_cap``
         the largest grid of the map and transpose templates (their kernels then stride over the rest)
     :return: a :class:`GeneratedOperator`
@@ -75,6 +75,7 @@ def generate(expression_dag, function_name, options=None):
     info.math = options.get('math', 'exact')
     info.if_conversion = options.get('if_conversion', True)
     info.value_ranges = options.get('value_ranges', True)
+    info.cse = options.get('cse', True)
     kernel_name = 'ovl_' + _kernel_label(info.name) + '_' + function_name[1:9]
     if info.math != 'exact':
         kernel_name += '_' + info.math         # so that profiles tell the math modes of one operator apart
@@ -102,13 +103,13 @@ def generate(expression_dag, function_name, options=None):
                                                              options.get('scan_width'), options.get('scan_interleave'))
     elif options.get('vec') is None and template in ('auto', 'rowscan') and rowscan_kernel.plan(info) is not None:
         kernel_src, launch = rowscan_kernel.generate(info, kernel_name, options.get('scan_rows'),
-                                                     options.get('scan_chunk'))
+                                                     options.get('scan_chunk'), options.get('scan_batch'))
     elif options.get('vec') is None and template in ('auto', 'transpose') and tile_kernel.applicable(info) is not None:
         kernel_src, launch = tile_kernel.generate(info, kernel_name, options.get('tile_i'), options.get('tile_j'),
                                                   options.get('nt', 'ls'))
     else:
         kernel_src, launch = map_kernel.generate(info, kernel_name, options.get('vec'), options.get('nt'),
-                                                 options.get('grid_cap'))
+                                                 options.get('grid_cap'), options.get('per_thread'))
 
     num_inputs = len(info.inputs)
     num_outputs = len(info.outputs)

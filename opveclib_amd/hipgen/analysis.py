@@ -334,23 +334,20 @@ class DagInfo(object):
                 found.append((node, self.nodes[node.ops[0]], self.affine[node.ops[1]]))
         return found
 
-    def bufferable_outputs(self):
+    def bufferable_outputs(self, buffers):
         """
         Output node indices whose stores may be held in registers (or an LDS tile) until the end of the worker's
-        iteration: every store to the tensor is outside loops and uses one affine index.  A store that a template
-        cannot buffer (inside a loop, through a computed index) is written at once; buffering another store to the
-        same tensor would write it later and so reverse the program's order whenever both hit one element.
+        iteration.  ``buffers(node, tensor, affine) -> bool`` says whether the template would buffer that one store;
+        a tensor qualifies when it says so for every store to it.  A store that is not buffered (inside a loop,
+        through a computed index, under a condition that not every path takes) is written at once; buffering another
+        store to the same tensor would write it later and so reverse the program's order whenever both hit one element.
         """
-        signatures = {}
-        refused = set()
+        verdict = {}
         for node, tensor, aff in self.tensor_accesses():
-            if node.code != lang.ASSIGN_TENSOR:
-                continue
-            if aff is None or self.in_loop[node.idx]:
-                refused.add(tensor.idx)
-            else:
-                signatures.setdefault(tensor.idx, set()).add(aff.signature())
-        return set(idx for idx, found in signatures.items() if len(found) == 1 and idx not in refused)
+            if node.code == lang.ASSIGN_TENSOR:
+                ok = aff is not None and not self.in_loop[node.idx] and bool(buffers(node, tensor, aff))
+                verdict[tensor.idx] = verdict.get(tensor.idx, True) and ok
+        return set(idx for idx, ok in verdict.items() if ok)
 
     def definitely_stores(self, keys):
         """

@@ -250,6 +250,37 @@ class BodyEmitter(object):
         self._plan_if_conversion()
         names = {}
         stmts = []
+        # Common subexpressions.  The worker functions of the reference repeat whole sub-expressions (its LSTM gradient
+        # evaluates sigmoid(i), sigmoid(f + bias), tanh(j) and tanh(new_c) once for the forward recomputation and again
+        # inside every gate's derivative, lstm/lstm.py:84-103); the same operation on the same operands gives the same
+        # bits, so a repeated expression takes the name of its first evaluation at the top level of the worker.  The
+        # C++ compiler finds only some of these across the rare-argument blocks of the math routines.
+        value_key = {}          # node index -> hashable description of a pure expression, or None
+        first_value = {}        # description -> name of its first unconditional evaluation
+        cse = getattr(info, 'cse', True)
+
+        def describe(node):
+            code = node.code
+            if code == lang.CONST_SCALAR:
+                return ('const', node.dtype, repr(node.data[0]))
+            if code in LIMITS:
+                return ('limit', code, node.dtype)
+            operands = tuple(value_key.get(o) for o in node.ops)
+            if code == lang.READ_TENSOR:
+                tensor = info.nodes[node.ops[0]]
+                if tensor.code == lang.POSITION and operands[1] is not None:
+                    return ('position', operands[1])
+                if tensor.code == lang.INPUT and operands[1] is not None and not info.in_loop[node.idx]:
+                    return ('read', tensor.io_index, operands[1])
+                return None
+            if any(o is None for o in operands) or not operands:
+                return None
+            if code == lang.CAST:
+                return ('cast', node.dtype, operands[0])
+            if code in UNARY or code in INFIX or code in (lang.MIN, lang.MAX, lang.POW, lang.ATAN2):
+                return (code, node.dtype, site_mode(node) if code in accuracy.ROUTINE_ULPS else None) + operands
+            return None
+
         indent = 0
         current = [0]
         open_chains = []        # True for a converted chain, False for one emitted as branches
@@ -269,6 +300,13 @@ class BodyEmitter(object):
             code = node.code
             ops = node.ops
             name = 'e' + str(node.idx) + self.suffix
+            key = value_key[node.idx] = describe(node) if cse else None
+            if key is not None and code not in (lang.CONST_SCALAR,) and code not in LIMITS:
+                if key in first_value:
+                    names[node.idx] = first_value[key]
+                    continue
+                if info.depth[node.idx] == 0:
+                    first_value[key] = name
             if code in (lang.INPUT, lang.OUTPUT):
                 name = self.tensor_name(node)
             elif code == lang.POSITION:

@@ -11,8 +11,8 @@ threads per block, expression.py:696-698 and operator.py:30).  For gfx950 the te
   buffers the stores in registers until the end of the iteration;
 * launches one 256-thread workgroup (four wavefronts) per 256 vectors, in address order, so that at any time the
   whole chip streams through one neighbourhood of each tensor (measured on MI355X: 6.85 TB/s for a three-stream
-  float32 add, against 5.3 TB/s for a grid-stride loop over 8 workgroups per CU); vector stores, and for streams
-  with more loads than stores also the loads, carry the non-temporal hint (every element is touched exactly once);
+  float32 add, against 5.3 TB/s for a grid-stride loop over 8 workgroups per CU); the vector stores or the vector
+  loads carry the non-temporal hint, whichever was measured to be faster for the kernel's mix of streams;
 * keeps every other access (gathers, scatters, accesses inside loops or behind non-exhaustive conditions) as the
   scalar access the worker function asked for.
 
@@ -101,8 +101,23 @@ def contiguous_unaligned(info, node, tensor, aff, vec):
     return not _is_vector_access(info, node, tensor, aff, vec)
 
 
-def generate(info, kernel_name, vec=None, nt=None, grid_cap=None):
+def _arithmetic_weight(info):
+    """Rough count of expensive float operations per worker (transcendental calls and divisions)."""
+    heavy = (lang.EXP, lang.LOG, lang.TANH, lang.DIVIDE, lang.SIN, lang.COS, lang.TAN, lang.POW, lang.SQRT,
+             lang.SINH, lang.COSH, lang.ASIN, lang.ACOS, lang.ATAN, lang.ATAN2, lang.LOG10)
+    return sum(1 for n in info.nodes if n.code in heavy and n.dtype in (lang.FLOAT32, lang.FLOAT64))
+
+
+def generate(info, kernel_name, vec=None, nt=None, grid_cap=None, per_thread=None):
     """
+    :param per_thread: vectors per thread (1 or 2; None chooses).  Two vectors, 256 apart so that every request of a
+        wavefront stays one contiguous run, are requested together before the arithmetic of either: a wavefront then
+        has twice the bytes in flight while it waits and the workgroup's set-up (math tables, barrier) is paid once
+        for twice the work.  Measured on MI355X, interleaved runs: the 8-op chain in the 'ulp2' math mode, where
+        arithmetic and memory time are about equal, 148.7 -> 142.4 us; the same chain in the 'exact' mode, which is
+        bound by arithmetic alone, 252 -> 255 us; the LSTM cell with its five to seven load streams 27.8 -> 30.4 us
+        (forward) and 36.2 -> 39.9 us (gradient).  So it is chosen for bodies with few streams and some arithmetic,
+        outside the 'exact' mode.
     :return: (kernel source text, launch description dict) for the map template.
     """
     rank = len(info.workgroup_shape)
@@ -130,18 +145,25 @@ def generate(info, kernel_name, vec=None, nt=None, grid_cap=None):
             if key not in unaligned:
                 unaligned[key] = Access(tensor, aff, 'lu%d' % len(unaligned))
     certain = info.definitely_stores(store_keys)
-    bufferable = info.bufferable_outputs()
+    bufferable = info.bufferable_outputs(
+        lambda node, tensor, aff: vec > 1 and (tensor.idx, aff.signature()) in certain and
+        _is_vector_access(info, node, tensor, aff, vec))
     for node, tensor, aff in accesses:
         if node.code == lang.ASSIGN_TENSOR and aff is not None and tensor.idx in bufferable:
             key = (tensor.idx, aff.signature())
             if key in certain and key not in stores and vec > 1 and _is_vector_access(info, node, tensor, aff, vec):
                 stores[key] = Access(tensor, aff, 'st%d' % len(stores))
 
-    # Non-temporal hints, measured on MI355X: a stream with as many stores as loads (copy 83 -> 74 us, row scan
-    # 100 -> 85 us) is fastest with the hint on the stores only, a stream with more loads than stores (three-operand
-    # add 136 -> 124 us, gather + transposed store) with the hint on both.
+    # Non-temporal hints, measured on MI355X (every element is touched exactly once in all of these):
+    #   copy, 1 load : 1 store             hint on the stores 75 us, on neither 84
+    #   three-operand add, 2 : 1           hint on the loads 116 us, on both 124, on the stores 135, on neither 138
+    #   LSTM cell forward, 5 : 2           stores 26.5 us, both 27.2, neither 27.2, loads 29.7
+    #   LSTM cell gradient, 7 : 5          stores 36.4 us, neither 38.1, loads 40.5, both 41.7
+    # so: on the stores when there are at least as many stores as loads or many load streams, on the loads when two
+    # or three load streams feed fewer stores.
     if nt is None:
-        nt = 's' if len(loads) + len(unaligned) <= len(stores) else 'ls'
+        streams = len(loads) + len(unaligned)
+        nt = 's' if (streams <= len(stores) or streams >= 4) else 'l'
     load_fn = 'OVL_LOAD_NT' if 'l' in nt else 'OVL_LOAD_PLAIN'
     store_fn = 'OVL_STORE_NT' if 's' in nt else 'OVL_STORE_PLAIN'
 
@@ -161,12 +183,40 @@ def generate(info, kernel_name, vec=None, nt=None, grid_cap=None):
                 return acc.reg + '[lane] = ' + value_name + ';'
         return None
 
-    pos_names = ['p%d' % k for k in range(rank)]
-    lane_position = list(pos_names)
-    lane_position[last] = pos_names[last] + ' + lane' if vec > 1 else pos_names[last]
-    body = BodyEmitter(info, lane_position, read_hook, store_hook).emit()
-
     num_vectors = info.num_workers // vec
+    single_grid = (num_vectors + BLOCK - 1) // BLOCK <= min(grid_cap or MAX_GRID, MAX_GRID)
+    if per_thread is None:
+        few_streams = len(loads) + len(unaligned) + len(stores) <= 3
+        per_thread = 2 if (vec > 1 and few_streams and _arithmetic_weight(info) >= 4 and
+                           getattr(info, 'math', 'exact') != 'exact') else 1
+    if per_thread > 1 and not (single_grid and num_vectors % (BLOCK * per_thread) == 0 and
+                               not any(info.in_loop.values())):
+        per_thread = 1
+    # names of the registers of one of the thread's vectors: '' for a single vector, else '_0', '_1', ...
+    reps = [''] if per_thread == 1 else ['_%d' % r for r in range(per_thread)]
+
+    def hooks(sfx):
+        def read_rep(node, tensor, index_name):
+            text = read_hook(node, tensor, index_name)
+            return text.replace('[lane]', sfx + '[lane]') if text else text
+
+        def store_rep(node, tensor, index_name, value_name):
+            text = store_hook(node, tensor, index_name, value_name)
+            return text.replace('[lane] = ', sfx + '[lane] = ', 1) if text else text
+        return read_rep, store_rep
+
+    def names_of(sfx):
+        return ['p%d%s' % (k, sfx) for k in range(rank)]
+
+    bodies = {}
+    for sfx in reps:
+        lane_position = names_of(sfx)
+        if vec > 1:
+            lane_position[last] = lane_position[last] + ' + lane'
+        read_rep, store_rep = hooks(sfx)
+        bodies[sfx] = BodyEmitter(info, lane_position, read_rep, store_rep).emit()
+    pos_names = names_of(reps[0])
+
     args = []
     for i in range(len(info.inputs)):
         args.append('const ' + CTYPE[info.inputs[i].dtype] + '* __restrict__ in' + str(i))
@@ -185,15 +235,19 @@ def generate(info, kernel_name, vec=None, nt=None, grid_cap=None):
     src.append('')
     src.append('extern "C" __global__ void __launch_bounds__(%d)' % BLOCK)
     src.append(kernel_name + '(' + ', '.join(args) + ') {')
-    blocks_needed = (num_vectors + BLOCK - 1) // BLOCK
+    blocks_needed = (num_vectors + BLOCK * per_thread - 1) // (BLOCK * per_thread)
     # When the grid covers every vector (always, unless the workgroup has more than 2^32 - 256 workers at VEC = 1 or
-    # the caller caps the grid) a thread runs one vector without a loop.  Kernels that use the LDS math tables then
+    # the caller caps the grid) a thread runs its vectors without a loop.  Kernels that use the LDS math tables then
     # request their operands first and copy the tables (with the barrier that implies) while they are in flight,
     # instead of waiting for the tables before the first request.
     covers = blocks_needed <= min(grid_cap or MAX_GRID, MAX_GRID)
     single_pass = info.uses_math_tables() and covers
     src.append('    const uint32_t num_vectors = %du;' % num_vectors)
-    if single_pass:
+    if per_thread > 1:
+        # the grid covers the vectors exactly: no idle threads
+        src.append('    const uint32_t v = blockIdx.x * %du + threadIdx.x;' % (BLOCK * per_thread))
+        src.append('    {')
+    elif single_pass:
         src.append('    const uint32_t v_raw = blockIdx.x * %du + threadIdx.x;' % BLOCK)
         src.append('    const bool active = v_raw < num_vectors;')
         src.append('    // idle threads of the last workgroup request vector 0 and store nothing')
@@ -209,51 +263,56 @@ def generate(info, kernel_name, vec=None, nt=None, grid_cap=None):
         src.append('    const uint32_t stride = gridDim.x * %du;' % BLOCK)
         src.append('    for (uint32_t v = blockIdx.x * %du + threadIdx.x; v < num_vectors;' % BLOCK)
         src.append('         v = (num_vectors - v > stride) ? v + stride : num_vectors) {')
-    src.append('        const uint32_t worker0 = v * %du;' % vec)
-    # position of the first of this thread's workers
+    # position of the first worker of each of this thread's vectors
     block = 1
     blocks = [1] * rank
     for k in range(rank - 2, -1, -1):
         block *= info.workgroup_shape[k + 1]
         blocks[k] = block
-    for k in range(rank):
-        expr = 'worker0'
-        if k > 0:
-            expr = '(worker0 % ' + str(blocks[k - 1]) + 'u)'
-        src.append('        const uint32_t %s = %s / %du;' % (pos_names[k], expr, blocks[k]))
-
-    for acc in loads.values():
-        vname = vec_types[CTYPE[acc.tensor.dtype]]
-        wide = acc.aff.hi >= 2 ** 32
-        src.append('        const %s %s = %s(reinterpret_cast<const %s*>(in%d + (%s)));' % (
-            vname, acc.reg, load_fn, vname, acc.tensor.io_index, _index_expr(acc.aff, pos_names, wide)))
-    for acc in unaligned.values():
-        vname = vec_types[CTYPE[acc.tensor.dtype]]
-        wide = acc.aff.hi >= 2 ** 32
-        src.append('        const %s %s = *reinterpret_cast<const %s_u*>(in%d + (%s));' % (
-            vname, acc.reg, vname, acc.tensor.io_index, _index_expr(acc.aff, pos_names, wide)))
+    for r, sfx in enumerate(reps):
+        names = names_of(sfx)
+        src.append('        const uint32_t worker0%s = (v + %du) * %du;' % (sfx, r * BLOCK, vec))
+        for k in range(rank):
+            expr = 'worker0' + sfx
+            if k > 0:
+                expr = '(worker0' + sfx + ' % ' + str(blocks[k - 1]) + 'u)'
+            src.append('        const uint32_t %s = %s / %du;' % (names[k], expr, blocks[k]))
+    for sfx in reps:
+        names = names_of(sfx)
+        for acc in loads.values():
+            vname = vec_types[CTYPE[acc.tensor.dtype]]
+            wide = acc.aff.hi >= 2 ** 32
+            src.append('        const %s %s = %s(reinterpret_cast<const %s*>(in%d + (%s)));' % (
+                vname, acc.reg + sfx, load_fn, vname, acc.tensor.io_index, _index_expr(acc.aff, names, wide)))
+        for acc in unaligned.values():
+            vname = vec_types[CTYPE[acc.tensor.dtype]]
+            wide = acc.aff.hi >= 2 ** 32
+            src.append('        const %s %s = *reinterpret_cast<const %s_u*>(in%d + (%s));' % (
+                vname, acc.reg + sfx, vname, acc.tensor.io_index, _index_expr(acc.aff, names, wide)))
     if single_pass:
         src.append('        OVL_DECLARE_MATH_TABLES();')
-        src.append('        if (active) {')
-    for acc in stores.values():
-        src.append('        %s %s;' % (vec_types[CTYPE[acc.tensor.dtype]], acc.reg))
-
-    if vec > 1:
-        src.append('        #pragma unroll')
-        src.append('        for (uint32_t lane = 0; lane < %du; ++lane) {' % vec)
-        pad = '            '
-    else:
+        if per_thread == 1:
+            src.append('        if (active) {')
+    for sfx in reps:
+        names = names_of(sfx)
         src.append('        {')
-        pad = '            '
-    for stmt in body:
-        src.append(pad + stmt)
-    src.append('        }')
-    for acc in stores.values():
-        vname = vec_types[CTYPE[acc.tensor.dtype]]
-        wide = acc.aff.hi >= 2 ** 32
-        src.append('        %s(%s, reinterpret_cast<%s*>(out%d + (%s)));' % (
-            store_fn, acc.reg, vname, acc.tensor.io_index, _index_expr(acc.aff, pos_names, wide)))
-    if single_pass:
+        for acc in stores.values():
+            src.append('        %s %s;' % (vec_types[CTYPE[acc.tensor.dtype]], acc.reg + sfx))
+        if vec > 1:
+            src.append('        #pragma unroll')
+            src.append('        for (uint32_t lane = 0; lane < %du; ++lane) {' % vec)
+        else:
+            src.append('        {')
+        for stmt in bodies[sfx]:
+            src.append('            ' + stmt)
+        src.append('        }')
+        for acc in stores.values():
+            vname = vec_types[CTYPE[acc.tensor.dtype]]
+            wide = acc.aff.hi >= 2 ** 32
+            src.append('        %s(%s, reinterpret_cast<%s*>(out%d + (%s)));' % (
+                store_fn, acc.reg + sfx, vname, acc.tensor.io_index, _index_expr(acc.aff, names, wide)))
+        src.append('        }')
+    if single_pass and per_thread == 1:
         src.append('        }')
     src.append('    }')
     src.append('}')
@@ -269,6 +328,7 @@ def generate(info, kernel_name, vec=None, nt=None, grid_cap=None):
     launch = {
         'template': 'map',
         'vec': vec,
+        'per_thread': per_thread,
         'block': BLOCK,
         'blocks_needed': blocks_needed,
         'align': align,

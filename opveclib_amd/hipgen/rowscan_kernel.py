@@ -115,7 +115,8 @@ def plan(info, rows_per_block=None, chunk=None):
     rows_per_block = forced_rows or max(1, min(WAVE, (rows + NUM_CU - 1) // NUM_CU))
     chunk = None
     for cand in ((forced_chunk,) if forced_chunk else (1024, 512, 256, 128, 64)):
-        if length % cand == 0 and 3 * rows_per_block * (cand + vec) * itemsize <= LDS_BUDGET:
+        if length % cand == 0 and cand % (2 * vec) == 0 and \
+                3 * rows_per_block * (cand + vec) * itemsize <= LDS_BUDGET:
             chunk = cand
             break
     if chunk is None:
@@ -123,9 +124,14 @@ def plan(info, rows_per_block=None, chunk=None):
     return ScanPlan(loop, counter, length, rows, x, out, vec, rows_per_block, chunk)
 
 
-def generate(info, kernel_name, rows_per_block=None, chunk=None):
+def generate(info, kernel_name, rows_per_block=None, chunk=None, batch=None):
     p = plan(info, rows_per_block, chunk)
     assert p is not None
+    # vectors per register set of the scanning wavefront: two sets must fit a chunk a whole number of times
+    batch = batch or 8
+    while p.chunk % (2 * batch * p.vec) != 0:
+        batch //= 2
+    assert batch >= 1
     ctype = CTYPE[p.x.dtype]
     vec, chunk, rpb = p.vec, p.chunk, p.rows_per_block
     row_stride = chunk + vec        # keeps 128-bit alignment; lanes of the scanning wavefront fall in different banks
@@ -243,17 +249,31 @@ def generate(info, kernel_name, rows_per_block=None, chunk=None):
         src.append('        step(%du, set_b);' % (num_chunks - 1))
     src.append('        store_chunk(%du, m);' % (num_chunks - 1))
     src.append('    } else {')
-    src.append('        // The scanning wavefront: lane r owns row row0 + r.  Surplus lanes shadow the last row of the tile: they')
-    src.append('        // compute and write the same values to the same LDS words as its owner, which keeps the loop branch free')
-    src.append('        // (masking them off instead was measured to be slower).')
+    src.append('        // The scanning wavefront: lane r owns row row0 + r; surplus lanes are switched off for the LDS accesses')
+    src.append('        // (an LDS instruction costs by the lanes that take part).')
+    src.append('        // The row travels through two register sets of %d vectors: while one set runs the recurrence, the' % batch)
+    src.append('        // other is being read from LDS, so the latency of an LDS read is paid once per chunk and not once per')
+    src.append('        // vector; what remains on the critical path is the recurrence itself.')
     src.append('        const uint32_t r = lane < %du ? lane : %du;' % (rpb, rpb - 1))
     src.append('        const uint32_t row = (row0 + r < %du) ? row0 + r : %du;' % (p.rows, p.rows - 1))
     src.append('        __syncthreads();')
     src.append('        %s* rowp = &tile[0][r][0];' % ctype)
-    src.append('        %s xv = *reinterpret_cast<const %s*>(rowp);' % (vname, vname))
+    src.append('        %s set_a[%d], set_b[%d];' % (vname, batch, batch))
+    src.append('        auto fetch = [&](%s (&set)[%d], const %s* from) {' % (vname, batch, ctype))
+    src.append('            #pragma unroll')
+    src.append('            for (uint32_t v = 0; v < %du; ++v) set[v] = *reinterpret_cast<const %s*>(from + v * %du);' % (
+        batch, vname, vec))
+    src.append('        };')
+    src.append('        const bool owner = lane < %du;' % rpb)
+    src.append('        auto put_back = [&](const %s (&set)[%d], %s* to) {' % (vname, batch, ctype))
+    src.append('            #pragma unroll')
+    src.append('            for (uint32_t v = 0; v < %du; ++v) *reinterpret_cast<%s*>(to + v * %du) = set[v];' % (
+        batch, vname, vec))
+    src.append('        };')
+    src.append('        if (owner) fetch(set_a, rowp);')
     src.append('        // first column: the statements the worker runs before its loop')
-    src.append('#define OVL_SCAN_IN xv[0]')
-    src.append('#define OVL_SCAN_OUT(value) xv[0] = (value)')
+    src.append('#define OVL_SCAN_IN set_a[0][0]')
+    src.append('#define OVL_SCAN_OUT(value) set_a[0][0] = (value)')
     for stmt in prologue:
         src.append('        ' + stmt)
     src.append('#undef OVL_SCAN_IN')
@@ -262,22 +282,31 @@ def generate(info, kernel_name, rows_per_block=None, chunk=None):
     src.append('#define OVL_SCAN_OUT(value) xv[u] = (value)')
     src.append('#define OVL_SCAN_STEP(column) { %s = (%s)(column); %s }' % (
         counter_name, counter_type, ' '.join(body)))
-    src.append('        #pragma unroll')
-    src.append('        for (uint32_t u = 1; u < %du; ++u) OVL_SCAN_STEP(u)' % vec)
-    src.append('        *reinterpret_cast<%s*>(rowp) = xv;' % vname)
+    src.append('        // the recurrence over one register set; `first` skips the row\'s first column, which is done above')
+    src.append('        auto run = [&](%s (&set)[%d], uint32_t column0, bool first) {' % (vname, batch))
+    src.append('            #pragma unroll')
+    src.append('            for (uint32_t v = 0; v < %du; ++v) {' % batch)
+    src.append('                %s& xv = set[v];' % vname)
+    src.append('                #pragma unroll')
+    src.append('                for (uint32_t u = 0; u < %du; ++u) {' % vec)
+    src.append('                    if (v == 0u && u == 0u && first) continue;')
+    src.append('                    OVL_SCAN_STEP(column0 + v * %du + u)' % vec)
+    src.append('                }')
+    src.append('            }')
+    src.append('        };')
     src.append('        for (uint32_t k = 0; k < %du; ++k) {' % num_chunks)
     src.append('            rowp = &tile[k % 3u][r][0];')
-    src.append('            uint32_t c = (k == 0u) ? %du : 0u;' % vec)
-    src.append('            // the next vector is read from LDS while the current one is being accumulated')
-    src.append('            %s next = *reinterpret_cast<const %s*>(rowp + c);' % (vname, vname))
-    src.append('            #pragma unroll 8')
-    src.append('            for (; c < %du; c += %du) {' % (chunk, vec))
-    src.append('                xv = next;')
-    src.append('                next = *reinterpret_cast<const %s*>(rowp + (c + %du < %du ? c + %du : c));' % (
-        vname, vec, chunk, vec))
-    src.append('                #pragma unroll')
-    src.append('                for (uint32_t u = 0; u < %du; ++u) OVL_SCAN_STEP(k * %du + c + u)' % (vec, chunk))
-    src.append('                *reinterpret_cast<%s*>(rowp + c) = xv;' % vname)
+    src.append('            if (owner) {')
+    src.append('            if (k != 0u) fetch(set_a, rowp);')
+    src.append('            #pragma unroll 1')
+    src.append('            for (uint32_t c = 0; c < %du; c += %du) {' % (chunk, 2 * batch * vec))
+    src.append('                fetch(set_b, rowp + c + %du);' % (batch * vec))
+    src.append('                run(set_a, k * %du + c, k == 0u && c == 0u);' % chunk)
+    src.append('                put_back(set_a, rowp + c);')
+    src.append('                if (c + %du < %du) fetch(set_a, rowp + c + %du);' % (2 * batch * vec, chunk, 2 * batch * vec))
+    src.append('                run(set_b, k * %du + c + %du, false);' % (chunk, batch * vec))
+    src.append('                put_back(set_b, rowp + c + %du);' % (batch * vec))
+    src.append('            }')
     src.append('            }')
     src.append('            __syncthreads();')
     src.append('        }')

@@ -56,8 +56,11 @@ def applicable(info):
     keys = [(t.idx, a.signature()) for n, t, a in stores if _is_transposed_store(info, n, t, a, vec)]
     if not keys:
         return None
-    bufferable = info.bufferable_outputs()
-    certain = set(key for key in info.definitely_stores(keys) if key[0] in bufferable)
+    certain = info.definitely_stores(keys)
+    bufferable = info.bufferable_outputs(
+        lambda node, tensor, aff: (tensor.idx, aff.signature()) in certain and
+        _is_transposed_store(info, node, tensor, aff, vec))
+    certain = set(key for key in certain if key[0] in bufferable)
     if not certain:
         return None
     # all transposed outputs share one element width so one tile geometry serves them all
@@ -97,7 +100,9 @@ def generate(info, kernel_name, tile_i=None, tile_j=None, nt='ls'):
             elif _is_transposed_store(info, node, tensor, aff, vec):
                 tkeys.append((tensor.idx, aff.signature()))
     certain = info.definitely_stores(store_keys + tkeys)
-    bufferable = info.bufferable_outputs()
+    bufferable = info.bufferable_outputs(
+        lambda node, tensor, aff: (tensor.idx, aff.signature()) in certain and
+        (_is_vector_access(info, node, tensor, aff, vec) or _is_transposed_store(info, node, tensor, aff, vec)))
     for node, tensor, aff in accesses:
         if node.code != lang.ASSIGN_TENSOR or aff is None or tensor.idx not in bufferable:
             continue

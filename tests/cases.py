@@ -602,10 +602,22 @@ def scan_two_stores(x):
     return out
 
 
+@ovl.operator()
+def diagonal_overwrite(x):
+    """Every element stored through the worker's own position, the diagonal stored again through the transposed
+    index under a condition: on the diagonal both stores of one worker hit one element, and the second must win."""
+    out = ovl.output_like(x)
+    pos = ovl.position_in(x.shape)
+    out[pos] = x[pos]
+    with ovl.if_(pos[0] == pos[1]):
+        out[pos[1], pos[0]] = x[pos] * 2
+    return out
+
+
 def _store_order(rng):
     x = rng.standard_normal((64, 256), dtype=np.float32)
     return [store_then_loop_store(rng.standard_normal(1024, dtype=np.float32))[0], scan_late_store(x)[0],
-            scan_two_stores(x)[0]]
+            scan_two_stores(x)[0], diagonal_overwrite(rng.standard_normal((64, 64), dtype=np.float32))[0]]
 
 
 def _odd_sizes(rng):

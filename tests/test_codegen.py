@@ -290,3 +290,33 @@ def test_clear_op_cache_removes_cached_operators_only(tmp_path, monkeypatch):
     local.clear_op_cache()                      # an empty cache is fine
     monkeypatch.setattr(local, 'cache_directory', str(tmp_path / 'missing'))
     local.clear_op_cache()                      # and so is a cache that does not exist yet
+
+
+def test_repeated_subexpressions_are_evaluated_once():
+    """The reference's LSTM gradient repeats sigmoid(i), sigmoid(f + bias), tanh(j) and tanh(new_c) inside every
+    gate's derivative (lstm/lstm.py:84-103): the emitted body evaluates three exponentials and two tanh, as a
+    hand-written kernel would, and the operands of a repeated read are requested once."""
+    from opveclib_amd import hipgen, workloads
+    from opveclib_amd.workloads import Spec
+    op, = workloads.fused_operators(workloads.lstm_grad_outputs(Spec((64, 256)), Spec((64, 64)), Spec((64, 64)),
+                                                                Spec((64, 64))))
+    merged = hipgen.generate(op, 'f' + '0' * 56, {'per_thread': 1}).source
+    repeated = hipgen.generate(op, 'f' + '0' * 56, {'cse': False, 'per_thread': 1}).source
+    assert (merged.count('ovl_expf'), merged.count('ovl_tanhf(')) == (3, 2)
+    assert repeated.count('ovl_expf') > 3 and repeated.count('ovl_tanhf(') > 2
+    # a value computed under a condition is not reused outside it
+    import opveclib_amd as ovl
+
+    @ovl.operator()
+    def guarded(x):
+        out = ovl.output_like(x)
+        pos = ovl.position_in(x.shape)
+        y = ovl.variable(0, x.dtype)
+        with ovl.if_(x[pos] > 0):
+            y <<= ovl.exp(x[pos])
+        out[pos] = y + ovl.exp(x[pos])
+        return out
+
+    text = hipgen.generate(guarded(Spec((256,))).expression_dag, 'f' + '1' * 56,
+                           {'if_conversion': False, 'per_thread': 1}).source
+    assert text.count('ovl_expf') == 2
