@@ -7,8 +7,9 @@ CUDA text built around a one-thread-per-worker template.  Here the DAG is analys
 
 * :mod:`.map_kernel` - vectorised map (any DAG; vector width 1 is the general fallback);
 * :mod:`.tile_kernel` - rank-2 workgroups with transposed stores: LDS-tiled so reads and writes are both coalesced;
-* :mod:`.rowscan_kernel` - loop-carried accumulation along the last tensor axis: order-preserving row scan fed
-  through LDS by dedicated data-moving wavefronts.
+* :mod:`.rowscan_kernel` - loop-carried accumulation along the last tensor axis: order-preserving row scans
+  (lane-skewed out of registers; lane-skewed or lane = row out of LDS, fed by dedicated data-moving wavefronts) and
+  the reassociating wavefront scan.
 
 Every library exports ``<name>_generic_hip(in, n_in, out, n_out, stream)``: it validates tensor counts, lengths,
 dtypes (the reference's ``*err = 1`` checks, expression.py:621-646, 662-663) and pointer alignment, enqueues the
@@ -58,7 +59,7 @@ def generate(expression_dag, function_name, options=None):
     """
     :param expression_dag: serialised expression DAG of one operator
     :param function_name: unique name of the operator (its content hash)
-    :param options: optional dict.  ``template``: 'auto' (default), 'map', 'transpose', 'rowscan', 'skewscan' or 'treescan' restricts
+    :param options: optional dict.  ``template``: 'auto' (default), 'map', 'transpose', 'rowscan', 'skewscan', 'fedscan' or 'treescan' restricts
         the choice of kernel template (a template that does not fit the DAG falls back to 'map'); ``vec`` forces the
         map template with that vector width, ``per_thread`` its vectors per thread (1 or 2); ``scan_depth`` / ``scan_sets`` / ``scan_width`` / ``scan_interleave`` set the request burst (groups), the
         number of register sets, the 128-bit vectors per lane and phase and the rows per lane group of the lane-skewed scan; ``math``: 'exact'
@@ -98,6 +99,12 @@ def generate(expression_dag, function_name, options=None):
     if tree is not None:
         # sums, products and running extrema whose order the caller has given up: the reassociating scan
         kernel_src, launch = rowscan_kernel.generate_tree(info, kernel_name, options.get('scan_ahead') or 8)
+    elif options.get('vec') is None and template in ('auto', 'fedscan') and \
+            rowscan_kernel.fed_plan(info, options.get('scan_width'), options.get('scan_chunk')) is not None and \
+            (template == 'fedscan' or rowscan_kernel.fed_plan(info)[0].vec == 2):
+        # 8-byte elements run at the latency of their recurrence: the LDS-fed variant halves the hand-overs
+        kernel_src, launch = rowscan_kernel.generate_fed(info, kernel_name, options.get('scan_width'),
+                                                         options.get('scan_chunk'))
     elif options.get('vec') is None and template in ('auto', 'skewscan') and rowscan_kernel.skew_plan(info) is not None:
         kernel_src, launch = rowscan_kernel.generate_skewed(info, kernel_name, options.get('scan_depth'), options.get('scan_sets'), options.get('scan_nt', 's'),
                                                              options.get('scan_width'), options.get('scan_interleave'))

@@ -124,6 +124,93 @@ def plan(info, rows_per_block=None, chunk=None):
     return ScanPlan(loop, counter, length, rows, x, out, vec, rows_per_block, chunk)
 
 
+def _emit_movers(src, p, ctype, vname, vec, chunk, rpb, num_chunks, lds_column=None):
+    """
+    Source of the data-moving wavefronts (threads 64..255) of the LDS-fed scans, up to and including their branch of
+    the kernel: they stream chunks of ``chunk`` columns of the workgroup's ``rpb`` rows from global memory into three
+    rotating LDS buffers ``tile[3][rpb][...]`` and the scanned chunks back, with coalesced 128-bit accesses, one
+    barrier per chunk.  ``lds_column(text)`` maps the C expression of a column (a multiple of ``vec``) to the column
+    of the LDS row that holds it (identity by default; the lane-skewed scanner pads its segments).
+    """
+    if lds_column is None:
+        lds_column = lambda text: text
+    vectors_per_row = chunk // vec
+    tile_vectors = rpb * vectors_per_row
+    vpt = (tile_vectors + MOVERS - 1) // MOVERS      # vectors each mover thread handles per chunk
+    src.append('    // Movers (threads 64..255): every thread owns up to %d vectors of each chunk.  A vector that does not exist' % vpt)
+    src.append('    // (past the tile or past the last row) is redirected to the thread\'s first vector for loading and skipped')
+    src.append('    // when writing, so the loops are branch free and all loads of a chunk are in flight together.')
+    src.append('    struct MoverRegs { %s v[%d]; };' % (vname, vpt))
+    src.append('    auto slot = [&](uint32_t m, uint32_t i, uint32_t& r, uint32_t& cv) -> bool {')
+    src.append('        const uint32_t v = m + i * %du;' % MOVERS)
+    src.append('        r = v / %du; cv = (v %% %du) * %du;' % (vectors_per_row, vectors_per_row, vec))
+    src.append('        return v < %du && row0 + r < %du;' % (tile_vectors, p.rows))
+    src.append('    };')
+    src.append('    auto issue_loads = [&](uint32_t k, uint32_t m, MoverRegs& regs) {')
+    src.append('        #pragma unroll')
+    src.append('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
+    src.append('            uint32_t r, cv;')
+    src.append('            if (!slot(m, i, r, cv)) { r = 0; cv = 0; }')
+    src.append('            const uint32_t gr = (row0 + r < %du) ? row0 + r : %du;' % (p.rows, p.rows - 1))
+    src.append('            const uint64_t g = (uint64_t)gr * %dull + k * %du + cv;' % (p.length, chunk))
+    src.append('            regs.v[i] = __builtin_nontemporal_load(reinterpret_cast<const %s*>(gin + g));' % vname)
+    src.append('        }')
+    src.append('    };')
+    src.append('    auto write_lds = [&](uint32_t k, uint32_t m, const MoverRegs& regs) {')
+    src.append('        #pragma unroll')
+    src.append('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
+    src.append('            uint32_t r, cv;')
+    src.append('            if (slot(m, i, r, cv)) *reinterpret_cast<%s*>(&tile[k %% 3u][r][%s]) = regs.v[i];' % (
+        vname, lds_column('cv')))
+    src.append('        }')
+    src.append('    };')
+    src.append('    auto store_chunk = [&](uint32_t k, uint32_t m) {')
+    src.append('        MoverRegs regs;')
+    src.append('        #pragma unroll')
+    src.append('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
+    src.append('            uint32_t r, cv;')
+    src.append('            if (!slot(m, i, r, cv)) { r = 0; cv = 0; }')
+    src.append('            regs.v[i] = *reinterpret_cast<const %s*>(&tile[k %% 3u][r][%s]);' % (
+        vname, lds_column('cv')))
+    src.append('        }')
+    src.append('        #pragma unroll')
+    src.append('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
+    src.append('            uint32_t r, cv;')
+    src.append('            if (slot(m, i, r, cv)) {')
+    src.append('                const uint64_t g = (uint64_t)(row0 + r) * %dull + k * %du + cv;' % (p.length, chunk))
+    src.append('                __builtin_nontemporal_store(regs.v[i], reinterpret_cast<%s*>(gout + g));' % vname)
+    src.append('            }')
+    src.append('        }')
+    src.append('    };')
+    src.append('')
+    src.append('    if (threadIdx.x >= %du) {' % WAVE)
+    src.append('        const uint32_t m = threadIdx.x - %du;' % WAVE)
+    src.append('        // Two register sets keep two chunks of loads in flight: while chunk k is being scanned, chunk k+1 is')
+    src.append('        // written to LDS from the set requested two iterations ago, and chunk k+3 is requested into that set.')
+    src.append('        MoverRegs set_a, set_b;')
+    src.append('        issue_loads(0u, m, set_a);')
+    src.append('        write_lds(0u, m, set_a);')
+    if num_chunks > 1:
+        src.append('        issue_loads(1u, m, set_b);')
+    if num_chunks > 2:
+        src.append('        issue_loads(2u, m, set_a);')
+    src.append('        __syncthreads();')
+    src.append('        auto step = [&](uint32_t k, MoverRegs& regs) {')
+    src.append('            if (k + 1u < %du) write_lds(k + 1u, m, regs);' % num_chunks)
+    src.append('            if (k + 3u < %du) issue_loads(k + 3u, m, regs);' % num_chunks)
+    src.append('            if (k >= 1u) store_chunk(k - 1u, m);')
+    src.append('            __syncthreads();')
+    src.append('        };')
+    src.append('        #pragma unroll 1')
+    src.append('        for (uint32_t k = 0; k + 1u < %du; k += 2u) {' % num_chunks)
+    src.append('            step(k, set_b);             // chunks 1, 3, 5, ... travel through set_b')
+    src.append('            step(k + 1u, set_a);        // chunks 2, 4, 6, ... travel through set_a')
+    src.append('        }')
+    if num_chunks % 2 == 1:
+        src.append('        step(%du, set_b);' % (num_chunks - 1))
+    src.append('        store_chunk(%du, m);' % (num_chunks - 1))
+
+
 def generate(info, kernel_name, rows_per_block=None, chunk=None, batch=None):
     p = plan(info, rows_per_block, chunk)
     assert p is not None
@@ -177,77 +264,7 @@ def generate(info, kernel_name, rows_per_block=None, chunk=None, batch=None):
     src.append('    const %s* __restrict__ gin = in%d;' % (ctype, p.x.io_index))
     src.append('    %s* __restrict__ gout = out%d;' % (ctype, p.out.io_index))
     src.append('')
-    vpt = (tile_vectors + MOVERS - 1) // MOVERS      # vectors each mover thread handles per chunk
-    src.append('    // Movers (threads 64..255): every thread owns up to %d vectors of each chunk.  A vector that does not exist' % vpt)
-    src.append('    // (past the tile or past the last row) is redirected to the thread\'s first vector for loading and skipped')
-    src.append('    // when writing, so the loops are branch free and all loads of a chunk are in flight together.')
-    src.append('    struct MoverRegs { %s v[%d]; };' % (vname, vpt))
-    src.append('    auto slot = [&](uint32_t m, uint32_t i, uint32_t& r, uint32_t& cv) -> bool {')
-    src.append('        const uint32_t v = m + i * %du;' % MOVERS)
-    src.append('        r = v / %du; cv = (v %% %du) * %du;' % (vectors_per_row, vectors_per_row, vec))
-    src.append('        return v < %du && row0 + r < %du;' % (tile_vectors, p.rows))
-    src.append('    };')
-    src.append('    auto issue_loads = [&](uint32_t k, uint32_t m, MoverRegs& regs) {')
-    src.append('        #pragma unroll')
-    src.append('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
-    src.append('            uint32_t r, cv;')
-    src.append('            if (!slot(m, i, r, cv)) { r = 0; cv = 0; }')
-    src.append('            const uint32_t gr = (row0 + r < %du) ? row0 + r : %du;' % (p.rows, p.rows - 1))
-    src.append('            const uint64_t g = (uint64_t)gr * %dull + k * %du + cv;' % (p.length, chunk))
-    src.append('            regs.v[i] = __builtin_nontemporal_load(reinterpret_cast<const %s*>(gin + g));' % vname)
-    src.append('        }')
-    src.append('    };')
-    src.append('    auto write_lds = [&](uint32_t k, uint32_t m, const MoverRegs& regs) {')
-    src.append('        #pragma unroll')
-    src.append('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
-    src.append('            uint32_t r, cv;')
-    src.append('            if (slot(m, i, r, cv)) *reinterpret_cast<%s*>(&tile[k %% 3u][r][cv]) = regs.v[i];' % vname)
-    src.append('        }')
-    src.append('    };')
-    src.append('    auto store_chunk = [&](uint32_t k, uint32_t m) {')
-    src.append('        MoverRegs regs;')
-    src.append('        #pragma unroll')
-    src.append('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
-    src.append('            uint32_t r, cv;')
-    src.append('            if (!slot(m, i, r, cv)) { r = 0; cv = 0; }')
-    src.append('            regs.v[i] = *reinterpret_cast<const %s*>(&tile[k %% 3u][r][cv]);' % vname)
-    src.append('        }')
-    src.append('        #pragma unroll')
-    src.append('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
-    src.append('            uint32_t r, cv;')
-    src.append('            if (slot(m, i, r, cv)) {')
-    src.append('                const uint64_t g = (uint64_t)(row0 + r) * %dull + k * %du + cv;' % (p.length, chunk))
-    src.append('                __builtin_nontemporal_store(regs.v[i], reinterpret_cast<%s*>(gout + g));' % vname)
-    src.append('            }')
-    src.append('        }')
-    src.append('    };')
-    src.append('')
-    src.append('    if (threadIdx.x >= %du) {' % WAVE)
-    src.append('        const uint32_t m = threadIdx.x - %du;' % WAVE)
-    src.append('        // Two register sets keep two chunks of loads in flight: while chunk k is being scanned, chunk k+1 is')
-    src.append('        // written to LDS from the set requested two iterations ago, and chunk k+3 is requested into that set.')
-    src.append('        MoverRegs set_a, set_b;')
-    src.append('        issue_loads(0u, m, set_a);')
-    src.append('        write_lds(0u, m, set_a);')
-    if num_chunks > 1:
-        src.append('        issue_loads(1u, m, set_b);')
-    if num_chunks > 2:
-        src.append('        issue_loads(2u, m, set_a);')
-    src.append('        __syncthreads();')
-    src.append('        auto step = [&](uint32_t k, MoverRegs& regs) {')
-    src.append('            if (k + 1u < %du) write_lds(k + 1u, m, regs);' % num_chunks)
-    src.append('            if (k + 3u < %du) issue_loads(k + 3u, m, regs);' % num_chunks)
-    src.append('            if (k >= 1u) store_chunk(k - 1u, m);')
-    src.append('            __syncthreads();')
-    src.append('        };')
-    src.append('        #pragma unroll 1')
-    src.append('        for (uint32_t k = 0; k + 1u < %du; k += 2u) {' % num_chunks)
-    src.append('            step(k, set_b);             // chunks 1, 3, 5, ... travel through set_b')
-    src.append('            step(k + 1u, set_a);        // chunks 2, 4, 6, ... travel through set_a')
-    src.append('        }')
-    if num_chunks % 2 == 1:
-        src.append('        step(%du, set_b);' % (num_chunks - 1))
-    src.append('        store_chunk(%du, m);' % (num_chunks - 1))
+    _emit_movers(src, p, ctype, vname, vec, chunk, rpb, num_chunks)
     src.append('    } else {')
     src.append('        // The scanning wavefront: lane r owns row row0 + r; surplus lanes are switched off for the LDS accesses')
     src.append('        // (an LDS instruction costs by the lanes that take part).')
@@ -372,6 +389,187 @@ def skew_plan(info):
         if info.nodes[idx].dtype not in CTYPE:
             return None
     return p
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# The LDS-fed lane-skewed variant, for recurrences that run at their own latency (8-byte elements, few rows).
+#
+# The lane-skewed scan above pays a hand-over between neighbouring lanes once per VEC * width columns, and its width
+# is limited by the memory pipeline: a lane that owns more than 32 consecutive bytes makes the wavefront's requests
+# sparse (float64 [1024, 16384]: 75 us with 32 bytes per lane, 126 us with 64).  Here the requests are made by other
+# wavefronts: three of the workgroup's four wavefronts stream the rows through LDS with dense 128-bit accesses (as in
+# the lane = row variant), and the fourth runs the skewed recurrence out of LDS, where a lane can own a segment of any
+# length at no cost: with 16 columns per lane and phase the hand-over is paid once per 16 additions.  Segments are
+# padded by one vector in LDS so that the sixteen lanes of a group read and write without bank conflicts.
+# Measured on MI355X, float64, against the lane-skewed scan: [1024, 16384] 60 us against 74, [512, 16384] 55 / 73,
+# [2048, 16384] 111 / 119, [4096, 4096] 51 / 75, [8192, 2048] 51 / 69, [256, 65536] 203 / 279.  The recurrence alone
+# (no memory traffic at all, segments in registers) takes 45 us for 16384 columns, fed from LDS 52 us.  float32,
+# whose lane-skewed scan already runs at the speed of memory, loses with it (108 us against 85).
+# ---------------------------------------------------------------------------------------------------------------------
+FED_ROWS = WAVE // GROUP_LANES      # rows per workgroup: one group of sixteen lanes of the scanning wavefront each
+
+
+def fed_plan(info, width=None, chunk=None):
+    """(ScanPlan, width, chunk) when the LDS-fed lane-skewed variant can run this DAG, else None."""
+    p = skew_plan(info)
+    if p is None:
+        return None
+    itemsize = ITEMSIZE[p.x.dtype]
+    width = width or 8
+    while width > 1 and p.length % (GROUP_LANES * p.vec * width) != 0:
+        width //= 2
+    group_cols = GROUP_LANES * p.vec * width
+    if p.length % group_cols != 0:
+        return None
+    # (float64 [1024, 16384]: chunks of 512 and 1024 columns run alike; 512 lets two workgroups share a CU's LDS,
+    # which is what tensors with more rows than CUs times four need)
+    for cand in ((chunk,) if chunk else (512, 1024, 256, 128, 64)):
+        padded = cand + (cand // (p.vec * width)) * p.vec
+        if cand % group_cols == 0 and p.length % cand == 0 and 3 * FED_ROWS * padded * itemsize <= LDS_BUDGET:
+            return p, width, cand
+    return None
+
+
+def generate_fed(info, kernel_name, width=None, chunk=None):
+    p, width, chunk = fed_plan(info, width, chunk)
+    ctype = CTYPE[p.x.dtype]
+    vec = p.vec
+    rpb = FED_ROWS
+    seg = vec * width                       # columns a lane owns per group
+    group_cols = GROUP_LANES * seg
+    groups = chunk // group_cols            # groups per chunk
+    num_chunks = p.length // chunk
+    row_stride = chunk + (chunk // seg) * vec
+
+    rank = len(info.workgroup_shape)
+    pos_exprs = []
+    stride = 1
+    strides = [1] * rank
+    for k in range(rank - 2, -1, -1):
+        stride *= info.workgroup_shape[k + 1]
+        strides[k] = stride
+    for k in range(rank):
+        expr = 'row'
+        if k > 0:
+            expr = '(row % ' + str(strides[k - 1]) + 'u)'
+        pos_exprs.append(expr + ' / ' + str(strides[k]) + 'u')
+    emitter = BodyEmitter(info, pos_exprs,
+                          read_hook=lambda node, tensor, idx: 'OVL_SCAN_IN',
+                          store_hook=lambda node, tensor, idx, value: 'OVL_SCAN_OUT(' + value + ');')
+    tagged = emitter.emit_tagged()
+    range_idx = p.loop_item.node
+    end_idx = max(i for i, _ in tagged)
+    prologue = [t for i, t in tagged if i < range_idx]
+    body = [t.strip() for i, t in tagged if range_idx < i < end_idx]
+    counter_name = 'e' + str(p.counter)
+    counter_type = CTYPE[info.nodes[p.counter].dtype]
+    state = [('e' + str(idx), CTYPE[info.nodes[idx].dtype]) for idx in _carried_state(info, p)]
+
+    vname = 'ovl_scan_vec'
+    src = []
+    src.append('typedef %s %s __attribute__((ext_vector_type(%d)));' % (ctype, vname, vec))
+    src.append('')
+    src.append('extern "C" __global__ void __launch_bounds__(%d)' % BLOCK)
+    src.append('%s(const %s* __restrict__ in%d, %s* __restrict__ out%d) {' % (
+        kernel_name, ctype, p.x.io_index, ctype, p.out.io_index))
+    if info.uses_math_tables():
+        src.append('    OVL_DECLARE_MATH_TABLES();')
+    src.append('    __shared__ __attribute__((aligned(16))) %s tile[3][%d][%d];' % (ctype, rpb, row_stride))
+    src.append('    const uint32_t row0 = blockIdx.x * %du;' % rpb)
+    src.append('    const uint32_t lane = threadIdx.x %% %du;' % WAVE)
+    src.append('    const %s* __restrict__ gin = in%d;' % (ctype, p.x.io_index))
+    src.append('    %s* __restrict__ gout = out%d;' % (ctype, p.out.io_index))
+    src.append('')
+    # column cv of a chunk lives at cv + (cv / seg) * vec of the LDS row: every segment is followed by one spare vector
+    _emit_movers(src, p, ctype, vname, vec, chunk, rpb, num_chunks,
+                 lds_column=lambda cv: '%s + (%s / %du) * %du' % (cv, cv, seg, vec))
+    src.append('    } else {')
+    src.append('        // The scanning wavefront: sixteen lanes per row, lane `part` of a group owns columns')
+    src.append('        // [part * %d, part * %d + %d) of every group of %d columns.  A group past the last row shadows it.' % (
+        seg, seg, seg, group_cols))
+    src.append('        const uint32_t part = lane %% %du;' % GROUP_LANES)
+    src.append('        const uint32_t q = lane / %du;' % GROUP_LANES)
+    src.append('        const uint32_t row = (row0 + q < %du) ? row0 + q : %du;' % (p.rows, p.rows - 1))
+    src.append('        // first column: the statements the worker runs before its loop, in every lane')
+    src.append('        %s first_out;' % ctype)
+    src.append('#define OVL_SCAN_IN (in%d[(uint64_t)row * %dull])' % (p.x.io_index, p.length))
+    src.append('#define OVL_SCAN_OUT(value) first_out = (value)')
+    for stmt in prologue:
+        src.append('        ' + stmt)
+    src.append('#undef OVL_SCAN_IN')
+    src.append('#undef OVL_SCAN_OUT')
+    for name, stype in state:
+        src.append('        %s carry_%s = %s;' % (stype, name, name))
+    src.append('#define OVL_SCAN_IN xv[u]')
+    src.append('#define OVL_SCAN_OUT(value) ov[w][u] = (value)')
+    src.append('#define OVL_SCAN_STEP(column) { %s = (%s)(column); %s }' % (
+        counter_name, counter_type, ' '.join(body)))
+    src.append('        %s set_a[%d], set_b[%d];' % (vname, width, width))
+    src.append('        auto fetch = [&](%s (&set)[%d], const %s* from) {' % (vname, width, ctype))
+    src.append('            #pragma unroll')
+    src.append('            for (uint32_t w = 0; w < %du; ++w) set[w] = *reinterpret_cast<const %s*>(from + w * %du);' % (
+        width, vname, vec))
+    src.append('        };')
+    src.append('        // one group: in phase p every lane runs the recurrence over its segment from the state it holds and')
+    src.append('        // hands its final state to its right neighbour; after phase p lanes 0..p are exact')
+    src.append('        auto run = [&](%s (&set)[%d], %s* to, uint32_t column0, bool first_group) {' % (vname, width, ctype))
+    src.append('            %s ov[%d];' % (vname, width))
+    src.append('            const uint32_t col0 = column0 + part * %du;' % seg)
+    src.append('            const bool first_column = first_group && part == 0u;')
+    src.append('            #pragma unroll')
+    src.append('            for (uint32_t phase = 0; phase < %du; ++phase) {' % GROUP_LANES)
+    for name, _ in state:
+        src.append('                %s = carry_%s;' % (name, name))
+    src.append('                #pragma unroll')
+    src.append('                for (uint32_t w = 0; w < %du; ++w) {' % width)
+    src.append('                    const %s xv = set[w];' % vname)
+    src.append('                    #pragma unroll')
+    src.append('                    for (uint32_t u = 0; u < %du; ++u) {' % vec)
+    src.append('                        if (w == 0u && u == 0u && first_column) ov[0][0] = first_out;')
+    src.append('                        else OVL_SCAN_STEP(col0 + w * %du + u)' % vec)
+    src.append('                    }')
+    src.append('                }')
+    for name, _ in state:
+        src.append('                carry_%s = ovl_dpp_move<OVL_DPP_ROW_SHR1>(carry_%s, %s);' % (name, name, name))
+    src.append('            }')
+    src.append('            // the last lane of the group finished the group: its state is the carry into the next one')
+    for name, _ in state:
+        src.append('            carry_%s = ovl_dpp_move<OVL_DPP_ROW_ROR1>(carry_%s, %s);' % (name, name, name))
+    src.append('            #pragma unroll')
+    src.append('            for (uint32_t w = 0; w < %du; ++w) *reinterpret_cast<%s*>(to + w * %du) = ov[w];' % (
+        width, vname, vec))
+    src.append('        };')
+    src.append('        __syncthreads();')
+    src.append('        for (uint32_t k = 0; k < %du; ++k) {' % num_chunks)
+    src.append('            %s* segp = &tile[k %% 3u][q][part * %du];' % (ctype, seg + vec))
+    src.append('            fetch(set_a, segp);')
+    src.append('            #pragma unroll 1')
+    src.append('            for (uint32_t g = 0; g < %du; g += 2u) {' % groups)
+    src.append('                %s* here = segp + g * %du;' % (ctype, GROUP_LANES * (seg + vec)))
+    src.append('                if (g + 1u < %du) fetch(set_b, here + %du);' % (groups, GROUP_LANES * (seg + vec)))
+    src.append('                run(set_a, here, k * %du + g * %du, k == 0u && g == 0u);' % (chunk, group_cols))
+    src.append('                if (g + 2u < %du) fetch(set_a, here + %du);' % (groups, 2 * GROUP_LANES * (seg + vec)))
+    src.append('                if (g + 1u < %du) run(set_b, here + %du, k * %du + (g + 1u) * %du, false);' % (
+        groups, GROUP_LANES * (seg + vec), chunk, group_cols))
+    src.append('            }')
+    src.append('            __syncthreads();')
+    src.append('        }')
+    src.append('#undef OVL_SCAN_STEP')
+    src.append('#undef OVL_SCAN_IN')
+    src.append('#undef OVL_SCAN_OUT')
+    src.append('    }')
+    src.append('}')
+
+    launch = {
+        'template': 'fedscan',
+        'vec': vec,
+        'block': BLOCK,
+        'blocks_needed': (p.rows + rpb - 1) // rpb,
+        'align': {('in', p.x.io_index): 16, ('out', p.out.io_index): 16},
+        'vector_loads': 1,
+        'vector_stores': 1,
+    }
+    return '\n'.join(src) + '\n', launch
 
 
 TREE_OPS = (lang.ADD, lang.MULTIPLY, lang.MIN, lang.MAX)

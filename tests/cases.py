@@ -922,18 +922,26 @@ def ulp2_full_size_operators():
 
 # (case, code generator options): the same cases through kernel templates the generator would not pick by itself
 TEMPLATE_VARIANTS = [
+    ('c3_rowscan_shapes', {'template': 'fedscan'}),
+    ('c3_cumsum_f64', {'template': 'fedscan'}),
+    ('c3_cumprod_f64', {'template': 'fedscan', 'scan_width': 2}),
+    ('c3_cumsum_f32', {'template': 'fedscan', 'scan_width': 4, 'scan_chunk': 256}),
     ('c3_rowscan_shapes', {'template': 'rowscan'}),
     ('c3_cumsum_f32', {'template': 'rowscan'}),
     ('c3_cumprod_f64', {'template': 'rowscan'}),
     ('c3_rowscan_shapes', {'template': 'map'}),
-    ('c3_rowscan_shapes', {'scan_depth': 1, 'scan_sets': 3}),
-    ('c3_cumsum_f32', {'scan_depth': 2, 'scan_sets': 2}),
-    ('c3_cumsum_f32', {'scan_width': 2}),
-    ('c3_cumprod_f64', {'scan_width': 1}),
-    ('c3_rowscan_shapes', {'scan_width': 4, 'scan_depth': 1}),
-    ('c3_rowscan_shapes', {'scan_interleave': 2}),
-    ('c3_cumprod_f64', {'scan_interleave': 3, 'scan_sets': 3}),
-    ('accumulate_max', {'scan_interleave': 4}),
+    ('c3_cumsum_f64', {'template': 'skewscan'}),
+    ('c2_chain', {'per_thread': 2}),
+    ('c4_lstm_grad', {'per_thread': 2}),
+    ('c4_lstm_grad', {'cse': False}),
+    ('c3_rowscan_shapes', {'template': 'skewscan', 'scan_depth': 1, 'scan_sets': 3}),
+    ('c3_cumsum_f32', {'template': 'skewscan', 'scan_depth': 2, 'scan_sets': 2}),
+    ('c3_cumsum_f32', {'template': 'skewscan', 'scan_width': 2}),
+    ('c3_cumprod_f64', {'template': 'skewscan', 'scan_width': 1}),
+    ('c3_rowscan_shapes', {'template': 'skewscan', 'scan_width': 4, 'scan_depth': 1}),
+    ('c3_rowscan_shapes', {'template': 'skewscan', 'scan_interleave': 2}),
+    ('c3_cumprod_f64', {'template': 'skewscan', 'scan_interleave': 3, 'scan_sets': 3}),
+    ('accumulate_max', {'template': 'skewscan', 'scan_interleave': 4}),
     ('c5_variants', {'template': 'map'}),
     ('c2_chain', {'vec': 2}),
     ('c2_chain', {'value_ranges': False}),

@@ -84,12 +84,6 @@ def test_every_parity_case_emulated_on_the_host_equals_the_oracle():
 def test_forced_templates_emulated_on_the_host_equal_the_oracle():
     jobs = []
     for name, options in cases.TEMPLATE_VARIANTS:
-        if options.get('template') == 'rowscan':
-            # The LDS row scan lets the surplus lanes of its scanning wavefront shadow the last row of the tile: they
-            # read, compute and write the same LDS words as the row's owner, instruction by instruction.  That is
-            # harmless only because the 64 lanes of a wavefront run in lockstep (all reads of an instruction precede
-            # the writes of the next), which independent host threads do not model.
-            continue
         jobs.append(('%s %r' % (name, options), cases.CASE_BY_NAME[name].outputs(), 3, options))
     assert _run_all(jobs) == []
 
