@@ -58,7 +58,7 @@ HBM_PEAK_GBPS = 8000.0
 
 # HBM bytes per launch of the chain8 kernel from rocprofv3 counters (FETCH_SIZE, WRITE_SIZE, each scaled by the same
 # counter's reading for the copy kernel of known size).  Source: profiles/bench_all_kernels_hbm_traffic_counters.md
-CHAIN8_TRAFFIC_BYTES = {'exact': 805152370, 'ulp2': 805152370}
+CHAIN8_TRAFFIC_BYTES = {'exact': 805201832, 'ulp2': 805156198}
 
 CHAIN8_STAGES = ('add', 'mul', 'tanh', 'sigmoid', 'log1p', 'expm1', 'sub', 'abs')
 
@@ -134,13 +134,20 @@ class Prepared(object):
         return [self.buffers[ref.op_index][ref.op_output_index] for ref in self.dag.dag_outputs]
 
 
-def settle(prepared, busy_ms=40.0, limit_ms=250.0, window=8, tolerance=0.02):
+SETTLE_MS = [40.0]      # --settle-ms
+
+
+def settle(prepared, busy_ms=None, limit_ms=250.0, window=8, tolerance=0.02):
     """
     Launch until the GPU's clocks have settled under this kernel: for at least ``busy_ms`` of kernel time and until
     the last ``window`` launch times lie within ``tolerance`` of each other, at most ``limit_ms``.  Untimed
     conditioning before the warm-up; returns the number of launches it took.
     """
     import torch
+    if busy_ms is None:
+        busy_ms = SETTLE_MS[0]
+    if busy_ms <= 0:
+        return 0
     stream_obj = torch.cuda.current_stream()
     stream = stream_obj.cuda_stream
     recent = []
@@ -260,16 +267,23 @@ def side_workload(name, outputs, steps, warmup, options=None, reference=None):
     if reference is not None:
         line['cpu_reference'] = {'ms': reference['ms'], 'cores': reference['cores'], 'sample': reference['sample'],
                                  'bit_exact': same_bits(prepared.results(), reference['results'])}
+    sys.stderr.write('done: %s\n' % name)      # progress, so that a long run is seen to be alive
+    sys.stderr.flush()
     return line
 
 
 def _read_sysfs_mhz(pattern):
-    """Current frequency in MHz from the first readable hwmon file matching ``pattern`` (hertz inside), else None."""
+    """The clock level marked as current ("1: 2392Mhz *") in the first readable sysfs file matching ``pattern``, in
+    MHz, else None."""
     for path in sorted(glob.glob(pattern)):
         try:
             with open(path) as f:
-                return float(f.read().strip()) / 1e6
-        except (OSError, ValueError):
+                for line in f:
+                    if '*' in line:
+                        digits = ''.join(ch for ch in line.split(':', 1)[1] if ch.isdigit() or ch == '.')
+                        if digits:
+                            return float(digits)
+        except (OSError, ValueError, IndexError):
             continue
     return None
 
@@ -285,8 +299,8 @@ def clocks_under_load(prepared, seconds=1.5, per_launch_ms=0.15):
     readings = {'sclk_mhz': [], 'mclk_mhz': []}
     time.sleep(1.0)
     for _ in range(3):
-        for key, name in (('sclk_mhz', 'freq1_input'), ('mclk_mhz', 'freq2_input')):
-            value = _read_sysfs_mhz('/sys/class/drm/card*/device/hwmon/hwmon*/' + name)
+        for key, name in (('sclk_mhz', 'pp_dpm_sclk'), ('mclk_mhz', 'pp_dpm_mclk')):
+            value = _read_sysfs_mhz('/sys/class/drm/card*/device/' + name)
             if value:
                 readings[key].append(value)
         time.sleep(0.05)
@@ -335,7 +349,11 @@ def main():
     parser.add_argument('--no-others', action='store_true', help='skip the secondary configurations')
     parser.add_argument('--no-cpu', action='store_true',
                         help='skip the CPU oracle (baseline, reference times, bit-exact checks)')
+    parser.add_argument('--settle-ms', type=float, default=40.0,
+                        help='kernel time spent on untimed launches before each warm-up so that the clocks settle; '
+                             '0 skips them (for counter collection, where every launch is slow and only counted)')
     args = parser.parse_args()
+    SETTLE_MS[0] = args.settle_ms
     if args.gpus != 1:
         sys.exit('bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)' % args.gpus)
 

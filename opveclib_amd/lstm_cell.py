@@ -78,7 +78,9 @@ def _fast(math_mode):
         math_mode = get_math_mode()
     if math_mode not in MATH_MODES:
         raise ValueError('math_mode must be one of ' + str(MATH_MODES))
-    return 0 if math_mode == 'exact' else 1
+    # the cell adds products of either sign, so only the 'fast' mode, which promises nothing per operator, may use the
+    # hardware-based routines; 'ulp2' keeps the bit-compatible ones here, as the code generator does for this operator
+    return 1 if math_mode == 'fast' else 0
 
 
 def _prepare(torch, tensors, names):

@@ -78,7 +78,10 @@ def test_template_selection():
     # last-axis accumulation with a chunkable row length: the order-preserving row scan
     scan = template(cumsum(np.zeros((48, 1024), np.float32), axis=1))
     assert scan['template'] == 'skewscan' and scan['blocks_needed'] == 3       # 16 rows per workgroup
-    assert template(cumsum(np.zeros((1024, 16384), np.float64), axis=1))['blocks_needed'] == 64
+    # 8-byte elements: the lane-skewed recurrence fed from LDS, four rows per workgroup
+    fed = template(cumsum(np.zeros((1024, 16384), np.float64), axis=1))
+    assert fed['template'] == 'fedscan' and fed['blocks_needed'] == 256
+    assert template(cumsum(np.zeros((1024, 16384), np.float64), axis=1), {'template': 'skewscan'})['blocks_needed'] == 64
     lds = template(cumsum(np.zeros((48, 1024), np.float32), axis=1), {'template': 'rowscan'})
     assert lds['template'] == 'rowscan' and lds['blocks_needed'] == 48
     assert template(cumsum(np.zeros((48, 1024), np.float32), axis=1), {'template': 'map'})['template'] == 'map'

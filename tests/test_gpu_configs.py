@@ -100,11 +100,10 @@ def test_c4_lstm_full():
 
 def test_c5_gather_transpose_full():
     import torch
-    g = torch.Generator(device='cuda')
-    g.manual_seed(5)
     n = 16384
-    a = torch.randn((n, n), device='cuda', generator=g)
-    b = torch.randn((n * n,), device='cuda', generator=g)
+    g = np.random.default_rng(5)                # inputs drawn on the host and copied once, as for the other configurations
+    a = torch.from_numpy(g.standard_normal((n, n), dtype=np.float32)).cuda()
+    b = torch.from_numpy(g.standard_normal(n * n, dtype=np.float32)).cuda()
     out = ovl.evaluate(gather_transpose(a, b, alpha=0.5, stride=7919))
     assert out.shape == (n, n)
     # every element, in row blocks to bound memory: out[j, i] == 0.5*a[i, j] + b[i*7919 + j] in float32
@@ -119,3 +118,37 @@ def test_c5_gather_transpose_full():
     small_gpu = ovl.evaluate(gather_transpose(a[:rows].contiguous(), b[:rows * n].contiguous(), alpha=0.5,
                                               stride=7919))
     assert np.array_equal(small_gpu.cpu().numpy(), small)
+
+
+def test_reference_timing_cumsum_float64_along_axis_0():
+    """The shape the reference times (opveclib/examples/test_perf_accumulate.py:35-47): float64 [10000, 1000] along
+    axis 0, against numpy's sequential accumulate and against the oracle, every element."""
+    from opveclib_amd import workloads
+    x = np.random.default_rng(6).standard_normal(workloads.REFERENCE_CUMSUM_SHAPE)
+    got = ovl.evaluate(cumsum(x, axis=0))
+    assert np.array_equal(got, np.cumsum(x, axis=0))
+    assert np.array_equal(got, oracle.evaluate(cumsum(x, axis=0)))
+
+
+@pytest.mark.parametrize('units', [200, 650, 1500])
+def test_reference_timing_lstm_cell_batch_20(units):
+    """The cell sizes the reference's profiler runs (lstm/profile_lstm.py:41-51): batch 20 with 200, 650 and 1500
+    units, forward and gradient, generated operators and hand-written run-time-shape kernels (650 units are not a
+    multiple of the vector width: the scalar kernels) against the oracle, bit for bit."""
+    import torch
+    from opveclib_amd import lstm_cell, workloads
+    batch = workloads.REFERENCE_LSTM_BATCH
+    g = np.random.default_rng(6 + units)
+    concat = g.standard_normal((batch, 4 * units), dtype=np.float32)
+    c, dc, dh = (g.standard_normal((batch, units), dtype=np.float32) for _ in range(3))
+    want_fwd = oracle.evaluate(cases.all_outputs(lstm(concat, c, forget_bias=1.0)))
+    want_grad = oracle.evaluate(cases.all_outputs(lstm_grad(concat, c, dc, dh, forget_bias=1.0)))
+    got_fwd = ovl.evaluate(cases.all_outputs(lstm(concat, c, forget_bias=1.0)))
+    got_grad = ovl.evaluate(cases.all_outputs(lstm_grad(concat, c, dc, dh, forget_bias=1.0)))
+    t = [torch.from_numpy(v).cuda() for v in (concat, c, dc, dh)]
+    hand_fwd = lstm_cell.lstm_cell(t[0], t[1], 1.0)
+    hand_grad = lstm_cell.lstm_cell_grad(t[0], t[1], t[2], t[3], 1.0)
+    for got, hand, want in zip(list(got_fwd) + list(got_grad), list(hand_fwd) + list(hand_grad),
+                               list(want_fwd) + list(want_grad)):
+        assert np.array_equal(got, want)
+        assert np.array_equal(hand.cpu().numpy(), want)
