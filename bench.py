@@ -523,6 +523,9 @@ def main():
         del fast, exact_y, fast_y, ulps
         others.append(side_workload('copy f32[8192,8192] (counter calibration, plain copy bandwidth)',
                                     copy_outputs(leaves[0]), steps, warm))
+        others.append(side_workload('launch floor: copy of 1024 floats, one workgroup (what the clock around a launch '
+                                    'reads for a kernel with nothing to do)',
+                                    copy_outputs(np.zeros(1024, np.float32)), steps, warm))
         others.append(side_workload('c1 shift_cyclic -> expm1 -> log1p, f32[2^20]', c1_outputs(data['c1']), steps,
                                     warm, reference=cpu.get('c1')))
         del chain, exact, leaves

@@ -97,6 +97,7 @@ def all_workload_outputs():
     yield chain8_outputs(Spec((8192, 8192)), Spec((8192, 8192)), Spec((1,)))
     yield chain8_stage_outputs(Spec((8192, 8192)), Spec((8192, 8192)), Spec((1,)))
     yield copy_outputs(Spec((8192, 8192)))
+    yield copy_outputs(Spec((1024,)))               # one workgroup: the floor of a launch
     yield c1_outputs(Spec((1 << 20,)))
     yield cumsum_outputs(Spec((4096, 16384), f32))
     yield cumprod_outputs(Spec((4096, 16384), f32))

@@ -164,6 +164,19 @@ def c3_rowscan_shapes(rng):
     return outs
 
 
+def c3_colscan_shapes(rng):
+    """Scans along an axis other than the last: partial strips, a partial last chunk of rows, dimensions before the
+    axis, 4- and 8-byte elements, a single short chunk, more chunks than register sets with and without a remainder."""
+    return [cumsum(rng.standard_normal((200, 100)), axis=0)[0],
+            cumsum(rng.standard_normal((700, 30)), axis=0)[0],
+            cumsum(rng.standard_normal((1100, 20), dtype=np.float32), axis=0)[0],
+            cumprod(uniform(rng, 0.9, 1.1, (130, 70), np.float32), axis=0)[0],
+            cumsum(rng.standard_normal((3, 65, 40), dtype=np.float32), axis=1)[0],
+            cumsum(rng.integers(-1000, 1000, size=(64, 5)).astype(np.int32), axis=0)[0],
+            accumulate(rng.standard_normal((2, 3, 129, 7)), inner_fcn=lambda acc, x: ovl.maximum(acc, x), axis=2)[0],
+            cumsum(rng.standard_normal((10, 33)), axis=0)[0]]
+
+
 def c4_lstm(rng, batch=32, units=128):
     concat = rng.standard_normal((batch, 4 * units), dtype=np.float32)
     c = rng.standard_normal((batch, units), dtype=np.float32)
@@ -639,6 +652,7 @@ CASES = [
     Case('c3_cumsum_f64', c3_cumsum_f64, seed=3),
     Case('c3_cumprod_f64', c3_cumprod_f64, seed=3),
     Case('c3_rowscan_shapes', c3_rowscan_shapes, seed=3),
+    Case('c3_colscan_shapes', c3_colscan_shapes, seed=3),
     Case('c4_lstm', c4_lstm, seed=4),
     Case('c4_lstm_grad', c4_lstm_grad, seed=4),
     Case('c5_gather_transpose', c5_gather_transpose, seed=5),
@@ -922,6 +936,10 @@ def ulp2_full_size_operators():
 
 # (case, code generator options): the same cases through kernel templates the generator would not pick by itself
 TEMPLATE_VARIANTS = [
+    ('c3_colscan_shapes', {'template': 'colscan'}),
+    ('c3_colscan_shapes', {'template': 'colscan', 'scan_rows': 32, 'scan_batch': 2}),
+    ('c3_colscan_shapes', {'template': 'colscan', 'scan_sets': 3}),
+    ('c3_colscan_shapes', {'template': 'map'}),
     ('c3_rowscan_shapes', {'template': 'fedscan'}),
     ('c3_cumsum_f64', {'template': 'fedscan'}),
     ('c3_cumprod_f64', {'template': 'fedscan', 'scan_width': 2}),

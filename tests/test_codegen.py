@@ -87,7 +87,13 @@ def test_template_selection():
     assert template(cumsum(np.zeros((48, 1024), np.float32), axis=1), {'template': 'map'})['template'] == 'map'
     # rows that are not a multiple of 64 long, other axes, and loop bodies with branches use the general template
     assert template(cumsum(np.zeros((48, 1000), np.float32), axis=1))['template'] == 'map'
+    # along another axis: a short axis keeps one worker per thread, a long one with few lines gets strips of 64 lines
     assert template(cumsum(np.zeros((48, 1024), np.float32), axis=0))['template'] == 'map'
+    col = template(cumsum(np.zeros((1000, 200), np.float64), axis=0))
+    assert col['template'] == 'colscan' and col['blocks_needed'] == 4 and col['block'] == 1024
+    mid = template(cumsum(np.zeros((3, 500, 96), np.float32), axis=1))
+    assert mid['template'] == 'colscan' and mid['blocks_needed'] == 3 * 2
+    assert template(cumsum(np.zeros((128, 1 << 17), np.float32), axis=0))['template'] == 'map'    # enough wavefronts
     assert template(cases.dot(np.zeros((16, 64)), np.zeros((16, 64))))['template'] == 'map'
     # transposed store of a rank-2 workgroup: LDS tiles; the gather is one dword-aligned 128-bit load per thread
     tr = template(gather_transpose(np.zeros((192, 320), np.float32), np.zeros(192 * 320, np.float32),
