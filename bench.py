@@ -288,23 +288,42 @@ def _read_sysfs_mhz(pattern):
     return None
 
 
-def clocks_under_load(prepared, seconds=1.5, per_launch_ms=0.15):
-    """Shader and memory clock (MHz) read from sysfs while a queue of launches of the workload runs: the median of
-    three readings taken after the first second (the power management needs that long to settle under this kernel);
-    None where the files are missing.  Outside every timed region, no other program is started."""
+def _read_sysfs_watts(pattern):
+    """Board power in watts from the first readable hwmon file matching ``pattern`` (microwatts), else None."""
+    for path in sorted(glob.glob(pattern)):
+        try:
+            with open(path) as f:
+                return int(f.read().strip()) / 1e6
+        except (OSError, ValueError):
+            continue
+    return None
+
+
+def clocks_under_load(prepared, seconds=3.0, batch=300):
+    """Shader clock, memory clock (MHz) and board power (W) read from sysfs while the workload runs back to back:
+    launches go out in batches, a reading is taken every half second right after a batch has been queued (so the GPU
+    is busy with it), and the median of the readings after the first second is reported (the power management needs
+    about that long to settle under this kernel).  None where the files are missing.  Outside every timed region, no
+    other program is started."""
     import torch
     stream = torch.cuda.current_stream(prepared.device).cuda_stream
-    for _ in range(int(seconds * 1e3 / per_launch_ms)):
-        prepared.launch(stream)
-    readings = {'sclk_mhz': [], 'mclk_mhz': []}
-    time.sleep(1.0)
-    for _ in range(3):
-        for key, name in (('sclk_mhz', 'pp_dpm_sclk'), ('mclk_mhz', 'pp_dpm_mclk')):
-            value = _read_sysfs_mhz('/sys/class/drm/card*/device/' + name)
-            if value:
-                readings[key].append(value)
-        time.sleep(0.05)
-    torch.cuda.synchronize(prepared.device)
+    readings = {'sclk_mhz': [], 'mclk_mhz': [], 'power_w': []}
+    start = time.time()
+    next_reading = 1.0
+    while time.time() - start < seconds:
+        for _ in range(batch):
+            prepared.launch(stream)
+        if time.time() - start >= next_reading:
+            next_reading += 0.5
+            for key, name in (('sclk_mhz', 'pp_dpm_sclk'), ('mclk_mhz', 'pp_dpm_mclk')):
+                value = _read_sysfs_mhz('/sys/class/drm/card*/device/' + name)
+                if value:
+                    readings[key].append(value)
+            watts = (_read_sysfs_watts('/sys/class/drm/card*/device/hwmon/hwmon*/power1_average') or
+                     _read_sysfs_watts('/sys/class/drm/card*/device/hwmon/hwmon*/power1_input'))
+            if watts:
+                readings['power_w'].append(round(watts))
+        torch.cuda.synchronize(prepared.device)       # bounds the queue; the next batch follows at once
     found = dict((k, sorted(v)[len(v) // 2]) for k, v in readings.items() if v)
     return found or None
 
@@ -503,7 +522,8 @@ def main():
                        'cpu_reference': None if 'chain8' not in cpu else {
                            'ms': cpu['chain8']['ms'], 'cores': cpu['chain8']['cores'],
                            'sample': cpu['chain8']['sample'],
-                           'bit_exact': parity['exact_mode_vs_cpu_oracle']['bit_exact']}})
+                           'bit_exact': parity['exact_mode_vs_cpu_oracle']['bit_exact']},
+                       'clocks_under_load': clocks_under_load(exact, seconds=2.5)})
         # The 'fast' math mode (hardware-based routines everywhere): no promise per operator beyond 4 ulp, reported
         # with its distance from the exact result.
         fast = Prepared(chain8_outputs(*leaves), {'math': 'fast'})
@@ -523,6 +543,9 @@ def main():
         del fast, exact_y, fast_y, ulps
         others.append(side_workload('copy f32[8192,8192] (counter calibration, plain copy bandwidth)',
                                     copy_outputs(leaves[0]), steps, warm))
+        # the same readings under a kernel that only moves data: what the clocks and the board power are when the
+        # arithmetic is absent
+        others[-1]['clocks_under_load'] = clocks_under_load(Prepared(copy_outputs(leaves[0])), seconds=2.5)
         others.append(side_workload('launch floor: copy of 1024 floats, one workgroup (what the clock around a launch '
                                     'reads for a kernel with nothing to do)',
                                     copy_outputs(np.zeros(1024, np.float32)), steps, warm))

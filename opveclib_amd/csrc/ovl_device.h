@@ -86,6 +86,9 @@ __device__ __forceinline__ float ovl_atan2f(float a, float b) { return (float)at
 #define ovl_log1p_direct(x) ovl_math::log1p_direct_<false>((x), ovl_log_tab)
 #define ovl_log1p_direct_nan(x) ovl_math::log1p_direct_<true>((x), ovl_log_tab)
 #define ovl_expm1_direct(x) ovl_math::expm1_direct_((x), ovl_exp_tab)
+// The same for arguments whose value range is known to be narrow: 2^-4 <= x < 1 resp. 2^-12 <= x <= 0.68.
+#define ovl_log1p_unit(x) ovl_math::log1p_unit_((x), ovl_log_unit_tab)
+#define ovl_expm1_small(x) ovl_math::expm1_small_((x), ovl_exp_plain_tab)
 
 // The logistic function 1 / (1 + exp(-x)) for -16 <= x <= 64 (NaN propagates): hardware-based exp, the sum and the
 // correctly rounded reciprocal.  On that domain it is within two units in the last place of the same formula evaluated
@@ -106,6 +109,8 @@ __device__ __forceinline__ float ovl_atan2f(float a, float b) { return (float)at
     __shared__ ovl_math::lds_tables ovl_lds_tables;                            \
     ovl_math::load_tables(ovl_lds_tables);                                     \
     const uint64_t* const ovl_exp_tab = ovl_lds_tables.exp2f;                  \
-    const ovl_math::logf_entry* const ovl_log_tab = ovl_lds_tables.logf
+    const ovl_math::logf_entry* const ovl_log_tab = ovl_lds_tables.logf;       \
+    const uint64_t* const ovl_exp_plain_tab = ovl_lds_tables.exp2_plain;       \
+    const ovl_math::logf_entry* const ovl_log_unit_tab = ovl_lds_tables.log_unit
 
 #endif  // OVL_DEVICE_H_

@@ -179,6 +179,35 @@ OVL_HD float expm1_direct_(float x, const uint64_t* tab = exp2f_tab) {
     return (float)__builtin_fma(y, s, -1.0);
 }
 
+// exp(x) - 1 for 2^-12 <= x <= 0.68, where the scaled argument x * 32 / ln 2 rounds to 0 ... 31: the same arithmetic as
+// expm1_direct_, but the table entry is 2^(i/32) itself and needs no exponent added.  On the device `plain` is that
+// table (a copy in LDS, built from exp2f_tab when the tables are loaded); on the host the entry is computed here.
+// NaN gives NaN; the index is masked, so an argument outside the domain reads inside the table (and gets a wrong
+// value: the code generator uses the routine only where the value range of the argument lies in the domain).
+OVL_HD float expm1_small_(float x, const uint64_t* plain = nullptr) {
+    const double InvLn2N = 0x1.71547652b82fep+0 * OVL_EXP2F_N;
+    const double Shift = 0x1.8p+52;
+    const double C0 = 0x1.c6af84b912394p-5 / OVL_EXP2F_N / OVL_EXP2F_N / OVL_EXP2F_N;
+    const double C1 = 0x1.ebfce50fac4f3p-3 / OVL_EXP2F_N / OVL_EXP2F_N;
+    const double C2 = 0x1.62e42ff0c52d6p-1 / OVL_EXP2F_N;
+    double xd = (double)x;
+    double kd = __builtin_fma(InvLn2N, xd, Shift);
+    const uint32_t i = (uint32_t)as_u64(kd) % OVL_EXP2F_N;
+    kd -= Shift;
+    double r = __builtin_fma(InvLn2N, xd, -kd);
+#if defined(__HIP_DEVICE_COMPILE__)
+    const uint64_t t = plain[i];
+#else
+    const uint64_t t = plain ? plain[i] : exp2f_tab[i] + ((uint64_t)i << (52 - OVL_EXP2F_TABLE_BITS));
+#endif
+    double s = as_f64(t);
+    double z2 = __builtin_fma(C0, r, C1);
+    double r2 = r * r;
+    double y = __builtin_fma(C2, r, 1.0);
+    y = __builtin_fma(z2, r2, y);
+    return (float)__builtin_fma(y, s, -1.0);
+}
+
 // ---------------------------------------------------------------------------------------------------------------------
 // logf
 // ---------------------------------------------------------------------------------------------------------------------
@@ -207,18 +236,49 @@ struct logf_entry { double invc, logc; };
 
 OVL_TABLE logf_entry logf_tab[OVL_LOGF_N] = OVL_LOGF_TABLE;
 
+// For arguments in [1, 2): entry i belongs to [1 + i/16, 1 + (i+1)/16), c = 1 + (2 i + 1)/32 is its centre,
+// { 1/c, log(c) } rounded to double.
+#define OVL_LOG_UNIT_TABLE { \
+    { 0x1.f07c1f07c1f08p-1, 0x1.f829b0e783300p-6 }, \
+    { 0x1.d41d41d41d41dp-1, 0x1.6f0d28ae56b4cp-4 }, \
+    { 0x1.bacf914c1bad0p-1, 0x1.29552f81ff523p-3 }, \
+    { 0x1.a41a41a41a41ap-1, 0x1.9525a9cf456b4p-3 }, \
+    { 0x1.8f9c18f9c18fap-1, 0x1.fb9186d5e3e2bp-3 }, \
+    { 0x1.7d05f417d05f4p-1, 0x1.2e8e2bae11d31p-2 }, \
+    { 0x1.6c16c16c16c17p-1, 0x1.5d1bdbf5809cap-2 }, \
+    { 0x1.5c9882b931057p-1, 0x1.89a3386c1425bp-2 }, \
+    { 0x1.4e5e0a72f0539p-1, 0x1.b44f77bcc8f63p-2 }, \
+    { 0x1.4141414141414p-1, 0x1.dd46a04c1c4a1p-2 }, \
+    { 0x1.3521cfb2b78c1p-1, 0x1.02552a5a5d0ffp-1 }, \
+    { 0x1.29e4129e4129ep-1, 0x1.154c3d2f4d5eap-1 }, \
+    { 0x1.1f7047dc11f70p-1, 0x1.2795e1289b11bp-1 }, \
+    { 0x1.15b1e5f75270dp-1, 0x1.393e0d3562a1ap-1 }, \
+    { 0x1.0c9714fbcda3bp-1, 0x1.4a4f85db03ebbp-1 }, \
+    { 0x1.0410410410410p-1, 0x1.5ad404c359f2dp-1 } }
+
+OVL_TABLE logf_entry log_unit_tab[OVL_LOGF_N] = OVL_LOG_UNIT_TABLE;
+
 #if defined(__HIPCC__)
-// Copies of both lookup tables in LDS.  Table lookups are per-lane gathers; served from LDS they cost a few cycles,
+// Copies of the lookup tables in LDS.  Table lookups are per-lane gathers; served from LDS they cost a few cycles,
 // while gathers from global memory occupy the vector memory pipeline that the kernel needs for streaming its tensors.
 struct lds_tables {
     uint64_t exp2f[OVL_EXP2F_N];
     logf_entry logf[OVL_LOGF_N];
+    uint64_t exp2_plain[OVL_EXP2F_N];       // bits of 2^(i/32): exp2f[i] with the exponent part of i/32 put back
+    logf_entry log_unit[OVL_LOGF_N];
 };
 
 // Must be called by every thread of the workgroup before any divergent control flow.
 __device__ __forceinline__ void load_tables(lds_tables& t) {
-    if (threadIdx.x < OVL_EXP2F_N) t.exp2f[threadIdx.x] = exp2f_tab[threadIdx.x];
-    if (threadIdx.x < OVL_LOGF_N) t.logf[threadIdx.x] = logf_tab[threadIdx.x];
+    if (threadIdx.x < OVL_EXP2F_N) {
+        const uint64_t entry = exp2f_tab[threadIdx.x];
+        t.exp2f[threadIdx.x] = entry;
+        t.exp2_plain[threadIdx.x] = entry + ((uint64_t)threadIdx.x << (52 - OVL_EXP2F_TABLE_BITS));
+    }
+    if (threadIdx.x < OVL_LOGF_N) {
+        t.logf[threadIdx.x] = logf_tab[threadIdx.x];
+        t.log_unit[threadIdx.x] = log_unit_tab[threadIdx.x];
+    }
     __syncthreads();
 }
 #endif
@@ -303,6 +363,24 @@ OVL_HD float log1p_direct_(float x, const logf_entry* tab = logf_tab) {
     float result = (float)y;
     if (MAYBE_NAN) result = __builtin_fmaf(x, 0.0f, result);
     return result;
+}
+
+// log(1 + x) for 2^-4 <= x < 1: u = 1 + x (exact in double precision) lies in [1, 2), so its exponent is known, the
+// table is indexed by the top four fraction bits of u itself and neither the exponent's share k * ln 2 nor the
+// re-centring of u is needed.  Same polynomial as logf_; |u / c - 1| <= 1/33.  NaN gives NaN (u is used as it is).
+// The lower end of the domain keeps log(c) + log1p(u / c - 1) away from cancellation.
+OVL_HD float log1p_unit_(float x, const logf_entry* tab = log_unit_tab) {
+    const double A0 = -0x1.00ea348b88334p-2, A1 = 0x1.5575b0be00b6ap-2, A2 = -0x1.ffffef20a4123p-2;
+    const double u = 1.0 + (double)x;
+    const uint32_t i = ((uint32_t)(as_u64(u) >> 32) >> (20 - OVL_LOGF_TABLE_BITS)) % OVL_LOGF_N;
+    const double invc = tab[i].invc;
+    const double logc = tab[i].logc;
+    double r = __builtin_fma(u, invc, -1.0);
+    double r2 = r * r;
+    double y = __builtin_fma(A1, r, A2);
+    y = __builtin_fma(A0, r2, y);
+    y = __builtin_fma(y, r2, logc + r);
+    return (float)y;
 }
 
 // ---------------------------------------------------------------------------------------------------------------------

@@ -923,6 +923,40 @@ def chain8_single_stage(name, x, with_range=False):
     return fcn(x)[0]
 
 
+#: (formula, lower and upper end of the clip in front of it, the routine the 'ulp2' mode must choose): the general
+#: once-rounded routines on wide ranges, their shorter forms on narrow ones, the formula itself where the range leaves
+#: the compared domain
+ULP2_CLIPPED_FORMULAS = [
+    ('log1p', 2.0 ** -9, 1.0e6, 'ovl_log1p_direct'),
+    ('log1p', 0.0625, 0.999, 'ovl_log1p_unit'),
+    ('log1p', 1.0e-5, 0.5, 'ovl_logf_inrange'),
+    ('expm1', 0.001, 50.0, 'ovl_expm1_direct'),
+    ('expm1', 0.001, 0.68, 'ovl_expm1_small'),
+    ('expm1', -1.0, 0.5, 'ovl_expf_inrange'),
+    ('sigmoid', -15.0, 60.0, 'ovl_sigmoid_ulp2'),
+]
+ULP2_CLIPPED_COUNT = 1 << 20
+
+
+def ulp2_clipped_formula(kind, lo, hi, x):
+    fcn = {'sigmoid': stdops.sigmoid, 'log1p': log1p, 'expm1': expm1}[kind]
+    return fcn(clip_to_range(x, lo=lo, hi=hi))[0]
+
+
+def ulp2_clipped_arguments(lo, hi):
+    """Arguments spread evenly over the binades of [lo, hi] (both signs where the range has both), some beyond the
+    ends (the clip brings them back), the ends themselves."""
+    rng = np.random.default_rng(12)
+    n = ULP2_CLIPPED_COUNT
+    top = max(abs(lo), abs(hi)) * 2.0
+    bottom = min(abs(lo), abs(hi)) / 2.0 if lo * hi > 0 else top * 2.0 ** -30
+    x = _log_uniform(rng, np.log2(bottom), np.log2(top), n)
+    if lo < 0:
+        x = x * np.where(rng.random(n) < 0.5, -1.0, 1.0).astype(np.float32)
+    x[:2] = (lo, hi)
+    return x.astype(np.float32)
+
+
 def ulp2_full_size_operators():
     """[(operator, options)] of tests/test_gpu_ulp2.py that the benchmark's own prebuild step does not cover."""
     from opveclib_amd import workloads
@@ -931,6 +965,10 @@ def ulp2_full_size_operators():
     for name in ('tanh', 'sigmoid', 'log1p', 'expm1'):
         for op in _operators_of([chain8_single_stage(name, spec, with_range=True)], 3):
             jobs.append((op, {'math': 'ulp2'}))
+    for kind, lo, hi, _routine in ULP2_CLIPPED_FORMULAS:
+        for op in _operators_of([ulp2_clipped_formula(kind, lo, hi, workloads.Spec((ULP2_CLIPPED_COUNT,)))], 3):
+            jobs.append((op, {'math': 'ulp2'}))
+            jobs.append((op, None))
     return jobs
 
 

@@ -4,8 +4,9 @@
 //                          call them) against the host C library's expf / logf / tanhf / (1.0f / x) on this machine
 //                          (function 4 evaluates the device math library's own expf instead: a self-test of the
 //                          checker, which must report differences for it)
-//   ovl_exh_ulp_in_range   the once-rounded log1p / expm1 of the 'ulp2' math mode against the reference's formulas for
-//                          them evaluated with the host C library, on every float of a range of bit patterns
+//   ovl_exh_ulp_in_range   the once-rounded log1p / expm1 of the 'ulp2' math mode (and their shorter forms for narrow
+//                          argument ranges) against the reference's formulas for them evaluated with the host C
+//                          library, on every float of a range of bit patterns
 //   ovl_exh_tanh_division  device tanhf with its shortened divisions against the same code with IEEE divisions
 //   ovl_exh_in_range       the variants without a rare-argument block (expf, logf, reciprocal, division) against the
 //                          full routines / the '/' operator, on every argument the code generator may hand them
@@ -35,7 +36,7 @@ namespace {
 
 enum { FN_EXP = 0, FN_LOG = 1, FN_TANH = 2, FN_RECIP = 3, FN_DEVICE_LIBRARY_EXP = 4,
        FN_FAST_EXP = 5, FN_FAST_LOG = 6, FN_FAST_TANH = 7, FN_FAST_RECIP = 8,
-       FN_LOG1P_DIRECT = 9, FN_EXPM1_DIRECT = 10, FN_SIGMOID_ULP2 = 11 };
+       FN_LOG1P_DIRECT = 9, FN_EXPM1_DIRECT = 10, FN_SIGMOID_ULP2 = 11, FN_LOG1P_UNIT = 12, FN_EXPM1_SMALL = 13 };
 
 __global__ void __launch_bounds__(256) eval_kernel(int fn, uint32_t first, uint32_t count, float* __restrict__ out) {
     OVL_DECLARE_MATH_TABLES();
@@ -54,6 +55,8 @@ __global__ void __launch_bounds__(256) eval_kernel(int fn, uint32_t first, uint3
         else if (fn == FN_LOG1P_DIRECT) y = ovl_log1p_direct_nan(x);
         else if (fn == FN_EXPM1_DIRECT) y = ovl_expm1_direct(x);
         else if (fn == FN_SIGMOID_ULP2) y = ovl_sigmoid_ulp2(x);
+        else if (fn == FN_LOG1P_UNIT) y = ovl_log1p_unit(x);
+        else if (fn == FN_EXPM1_SMALL) y = ovl_expm1_small(x);
         else y = expf(x);            // the device math library's own expf: differs from the host's in the last place
         out[i] = y;
     }
@@ -171,8 +174,8 @@ float host_sigmoid_formula(float x) {
 
 float host_value(int fn, float x) {
     if (fn == FN_SIGMOID_ULP2) return host_sigmoid_formula(x);
-    if (fn == FN_LOG1P_DIRECT) return host_log1p_formula(x);
-    if (fn == FN_EXPM1_DIRECT) return host_expm1_formula(x);
+    if (fn == FN_LOG1P_DIRECT || fn == FN_LOG1P_UNIT) return host_log1p_formula(x);
+    if (fn == FN_EXPM1_DIRECT || fn == FN_EXPM1_SMALL) return host_expm1_formula(x);
     if (fn == FN_EXP || fn == FN_DEVICE_LIBRARY_EXP || fn == FN_FAST_EXP) return expf(x);
     if (fn == FN_LOG || fn == FN_FAST_LOG) return logf(x);
     if (fn == FN_TANH || fn == FN_FAST_TANH) return tanhf(x);

@@ -93,11 +93,61 @@ def test_generated_text_names_the_chosen_routines():
     outs = workloads.chain8_outputs(Spec((64, 256)), Spec((64, 256)), Spec((1,)))
     op, = workloads.fused_operators(outs)
     text = hipgen.generate(op, 'f' + '0' * 56, {'math': 'ulp2'}).source
-    for wanted in ('ovl_fast_tanhf(', 'ovl_sigmoid_ulp2(', 'ovl_log1p_direct', 'ovl_expm1_direct('):
+    # behind the tanh and the sigmoid the arguments of log1p and expm1 lie in the narrow domains
+    for wanted in ('ovl_fast_tanhf(', 'ovl_sigmoid_ulp2(', 'ovl_log1p_unit(', 'ovl_expm1_small('):
         assert wanted in text
     assert 'ovl_tanhf(' not in text
     exact = hipgen.generate(op, 'f' + '0' * 56, None).source
-    assert 'ovl_fast' not in exact and '_direct' not in exact
+    for unwanted in ('ovl_fast', '_direct', '_unit', '_small'):
+        assert unwanted not in exact
+
+
+def test_narrow_routines_only_where_the_range_allows():
+    from opveclib_amd import hipgen
+
+    def clip_op(lo, hi):
+        @ovl.operator()
+        def clipped(x):
+            out = ovl.output_like(x)
+            pos = ovl.position_in(x.shape)
+            out[pos] = ovl.minimum(ovl.maximum(x[pos], lo), hi)
+            return out
+        return clipped
+
+    def text(outputs):
+        op, = workloads.fused_operators(outputs)
+        return hipgen.generate(op, 'f' + '0' * 56, {'math': 'ulp2'}).source
+
+    x = Spec((1024,))
+    assert 'ovl_log1p_unit(' in text([log1p(clip_op(0.0625, 0.99)(x))[0]])
+    wide = text([log1p(clip_op(0.01, 0.99)(x))[0]])            # below 2^-4: the general once-rounded routine
+    assert 'ovl_log1p_direct' in wide and '_unit' not in wide
+    reaches_one = text([log1p(clip_op(0.5, 1.0)(x))[0]])        # 1 + 1 = 2 has another exponent
+    assert 'ovl_log1p_direct' in reaches_one and '_unit' not in reaches_one
+    assert 'ovl_expm1_small(' in text([expm1(clip_op(0.001, 0.68)(x))[0]])
+    large = text([expm1(clip_op(0.001, 0.7)(x))[0]])
+    assert 'ovl_expm1_direct(' in large and '_small' not in large
+
+
+def test_formula_results_are_bounded_by_the_function():
+    """log1p of [0.25, 0.75] lies in [0.22, 0.56], not in the [0.07, 1.7] that interval arithmetic over
+    log(u) * x / (u - 1) gives: the expm1 behind it sees an argument in its narrow domain."""
+    from opveclib_amd.hipgen import analysis, ranges
+
+    @ovl.operator()
+    def clipped(x):
+        out = ovl.output_like(x)
+        pos = ovl.position_in(x.shape)
+        out[pos] = ovl.minimum(ovl.maximum(x[pos], 0.25), 0.75)
+        return out
+
+    op, = workloads.fused_operators([log1p(clipped(Spec((1024,))))[0]])
+    info = analysis.DagInfo(op)
+    known = ranges.analyse(info)
+    quotients = [n for n in info.nodes if n.code == lang.DIVIDE and accuracy.match_idiom(info, known, n)]
+    assert len(quotients) == 1
+    r = known.ranges[quotients[0].idx]
+    assert 0.2231 < r.lo < 0.2232 and 0.5596 < r.hi < 0.5597
 
 
 PROGRAM = r'''
@@ -128,12 +178,14 @@ int main(int argc, char** argv) {
     long total = 0, differing = 0; int worst = 0;
     for (uint64_t i = a; i <= b; i += step) {
         uint32_t bits = (uint32_t)i; float x; memcpy(&x, &bits, 4);
-        float want = which ? expm1_formula(x) : log1p_formula(x);
-        float got = which ? ovl_math::expm1_direct_(x) : ovl_math::log1p_direct_<true>(x);
+        float want = (which & 1) ? expm1_formula(x) : log1p_formula(x);
+        float got = which == 1 ? ovl_math::expm1_direct_(x) : which == 0 ? ovl_math::log1p_direct_<true>(x)
+                  : which == 3 ? ovl_math::expm1_small_(x) : ovl_math::log1p_unit_(x);
         int d = abs(ordered(want) - ordered(got));
         ++total; if (d) ++differing; if (d > worst) worst = d;
     }
-    float nan_result = which ? ovl_math::expm1_direct_(NAN) : ovl_math::log1p_direct_<true>(NAN);
+    float nan_result = which == 1 ? ovl_math::expm1_direct_(NAN) : which == 0 ? ovl_math::log1p_direct_<true>(NAN)
+                     : which == 3 ? ovl_math::expm1_small_(NAN) : ovl_math::log1p_unit_(NAN);
     printf("%ld %ld %d %d\n", total, differing, worst, nan_result != nan_result ? 1 : 0);
     return 0;
 }
@@ -161,6 +213,28 @@ def test_once_rounded_routines_within_two_ulp_of_the_reference_formulas_on_the_h
     assert worst <= accuracy.ROUTINE_ULPS[kind] == accuracy.TOLERANCE
     assert 0 < differing < total // 2
     assert nan_kept == 1
+
+
+@pytest.mark.parametrize('kind', ['log1p', 'expm1'])
+def test_narrow_routines_within_two_ulp_of_the_reference_formulas_on_the_host(sweep, kind):
+    """Every seventh argument of the narrow domains (all of them: tests/test_gpu_math_exhaustive.py on the GPU)."""
+    lo, hi = accuracy.NARROW_DOMAIN[kind]
+    out = subprocess.check_output([str(sweep), '23'[kind == 'expm1'], repr(lo), repr(hi), '7'],
+                                  universal_newlines=True).split()
+    total, differing, worst, nan_kept = (int(v) for v in out)
+    assert total > 4 << 20
+    assert worst <= accuracy.TOLERANCE
+    assert 0 < differing < total // 2
+    assert nan_kept == 1
+
+
+@pytest.mark.parametrize('kind,outside', [('log1p', (2.0 ** -6, 2.0 ** -4)), ('expm1', (0.6824, 0.69))])
+def test_the_narrow_domain_limits_are_needed(sweep, kind, outside):
+    """Below 2^-4 the table entry's logarithm and the polynomial cancel too far; past 0.682 the scaled argument
+    rounds to 32 and the table index wraps."""
+    out = subprocess.check_output([str(sweep), '23'[kind == 'expm1'], repr(outside[0]), repr(outside[1]), '1'],
+                                  universal_newlines=True).split()
+    assert int(out[2]) > accuracy.TOLERANCE
 
 
 @pytest.mark.parametrize('kind,outside', [('log1p', (8e37, 3e38)), ('expm1', (70.0, 88.0))])

@@ -113,26 +113,30 @@ def _bits(value):
     return struct.unpack('<I', struct.pack('<f', value))[0]
 
 
-@pytest.mark.parametrize('kind', ['sigmoid', 'log1p', 'expm1'])
+@pytest.mark.parametrize('kind', ['sigmoid', 'log1p', 'expm1', 'log1p_unit', 'expm1_small'])
 def test_formula_routines_within_two_ulp_of_the_reference_formulas(lib, kind):
-    """Every float32 argument of the domain the code generator allows (hipgen/accuracy.py: IDIOM_DOMAIN)."""
+    """Every float32 argument of the domain the code generator allows (hipgen/accuracy.py: IDIOM_DOMAIN, and
+    NARROW_DOMAIN for the shorter forms `_unit` / `_small`)."""
     from opveclib_amd.hipgen import accuracy
     lib.ovl_exh_ulp_in_range.argtypes = [ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32] + \
         [ctypes.POINTER(ctypes.c_uint64)] * 3 + [ctypes.POINTER(ctypes.c_uint32)] * 2
-    lo, hi = accuracy.IDIOM_DOMAIN[kind]
+    narrow = {'log1p_unit': 'log1p', 'expm1_small': 'expm1'}.get(kind)
+    lo, hi = accuracy.NARROW_DOMAIN[narrow] if narrow else accuracy.IDIOM_DOMAIN[kind]
+    bound = accuracy.TOLERANCE if narrow else accuracy.ROUTINE_ULPS[kind]
     # ranges of bit patterns of one sign each: consecutive patterns are consecutive floats
     spans = [(_bits(lo), _bits(hi))] if lo > 0 else [(_bits(-0.0), _bits(lo)), (_bits(0.0), _bits(hi))]
     total = total_differing = 0
     for first, last in spans:
         compared, differing, beyond = ctypes.c_uint64(0), ctypes.c_uint64(0), ctypes.c_uint64(0)
         largest, where = ctypes.c_uint32(0), ctypes.c_uint32(0)
-        err = lib.ovl_exh_ulp_in_range({'log1p': 9, 'expm1': 10, 'sigmoid': 11}[kind], first, last,
-                                       min(16, os.cpu_count() or 1), ctypes.byref(compared), ctypes.byref(differing),
-                                       ctypes.byref(beyond), ctypes.byref(largest), ctypes.byref(where))
+        fn = {'log1p': 9, 'expm1': 10, 'sigmoid': 11, 'log1p_unit': 12, 'expm1_small': 13}[kind]
+        err = lib.ovl_exh_ulp_in_range(fn, first, last, min(16, os.cpu_count() or 1), ctypes.byref(compared),
+                                       ctypes.byref(differing), ctypes.byref(beyond), ctypes.byref(largest),
+                                       ctypes.byref(where))
         assert err == 0, 'HIP error %d' % err
-        assert beyond.value == 0 and largest.value <= accuracy.ROUTINE_ULPS[kind], \
+        assert beyond.value == 0 and largest.value <= bound, \
             '%s: %d ulp at bits 0x%08x, %d arguments beyond 2 ulp' % (kind, largest.value, where.value, beyond.value)
         total += compared.value
         total_differing += differing.value
-    assert total > 140 << 20
+    assert total >= {'log1p_unit': 32 << 20, 'expm1_small': 90 << 20}.get(kind, 140 << 20)
     assert total_differing > 0          # it is not the formula itself

@@ -102,9 +102,28 @@ def test_every_stage_on_the_exact_stage_inputs_at_full_size(chain_inputs):
         del got
     # the kernels that ran are the ones with the cheap routines, not the exact ones
     sources = [c.gen.source for key, c in runtime._loaded.items() if "'math', 'ulp2'" in key[1]]
-    assert any('ovl_log1p_direct' in text for text in sources)
-    assert any('ovl_expm1_direct' in text for text in sources)
+    # (the chain's stage ranges lie in the narrow domains: the shorter forms of the once-rounded routines)
+    assert any('ovl_log1p_unit' in text for text in sources)
+    assert any('ovl_expm1_small' in text for text in sources)
     assert any('ovl_fast_tanhf' in text for text in sources)
+
+
+@pytest.mark.parametrize('kind,lo,hi,routine', cases.ULP2_CLIPPED_FORMULAS,
+                         ids=['%s_%g_%g' % f[:3] for f in cases.ULP2_CLIPPED_FORMULAS])
+def test_formulas_behind_a_clip_use_the_routine_their_range_allows(kind, lo, hi, routine):
+    """The clip is exact in every mode, so the formula's stage sees the same input in both runs and the distance of
+    the results is the stage's own."""
+    from opveclib_amd import runtime
+    x = cases.ulp2_clipped_arguments(lo, hi)
+    out = cases.ulp2_clipped_formula(kind, lo, hi, x)
+    want = ovl.evaluate(out, opt_level=3, math_mode='exact')
+    got = ovl.evaluate(out, opt_level=3, math_mode='ulp2')
+    assert not np.isnan(want).any() and not np.isnan(got).any()
+    worst = int(cases.ulp_distance(got, want).max())
+    assert worst <= TOLERANCE, '%s on [%g, %g]: %d ulp' % (kind, lo, hi, worst)
+    sources = [c.gen.source for key, c in runtime._loaded.items()
+               if "'math', 'ulp2'" in key[1] and c.gen.source.count('ovl_') and 'clip_to_range' in c.gen.source]
+    assert any(routine + '(' in text or routine + '_nan(' in text for text in sources)
 
 
 @pytest.mark.parametrize('case', cases.FAST_CASES, ids=[c.name for c in cases.FAST_CASES])
