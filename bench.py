@@ -593,6 +593,10 @@ def main():
                                     reference=cpu.get('lstm')))
         others.append(side_workload('c4 lstm cell gradient [4096, 4x1024]', lstm_grad_outputs(concat, c, dc, dh),
                                     steps, warm, reference=cpu.get('lstm_grad')))
+        # these two also run at the board's power limit: the readings say so
+        others[-2]['clocks_under_load'] = clocks_under_load(Prepared(lstm_outputs(concat, c)), seconds=2.5)
+        others[-1]['clocks_under_load'] = clocks_under_load(Prepared(lstm_grad_outputs(concat, c, dc, dh)),
+                                                            seconds=2.5)
         others.append(side_workload('c4 lstm cell forward, hand-written kernel (run-time shape, same bits)',
                                     HandWrittenLstm(concat, c), steps, warm, reference=cpu.get('lstm')))
         others.append(side_workload('c4 lstm cell gradient, hand-written kernel (run-time shape, same bits)',
