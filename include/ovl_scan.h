@@ -17,9 +17,11 @@
  * Kernel: the lane-skewed order-preserving scan.  Sixteen neighbouring lanes share a row; a lane owns a run of
  * consecutive columns of the current group (one 128-bit access for float32, two for float64), runs the recurrence
  * over its run from the carried state it holds and hands its state to its right neighbour with a lane-to-lane move;
- * after sixteen such phases the group is exact and the last lane's state is the carry into the next group.  Column
- * counts that are not a multiple of the group (64 columns for float32, 64 for float64) or unaligned tensors take a
- * plain kernel with one lane per row.
+ * after sixteen such phases the group is exact and the last lane's state is the carry into the next group.  float64
+ * rows whose length is a multiple of 512 columns run the same recurrence fed from LDS (three wavefronts of the
+ * workgroup stream four rows through LDS, the fourth scans them, a lane owning 16 columns per phase), which pays the
+ * hand-over between lanes four times less often.  Column counts that are not a multiple of the group (64 columns) or
+ * unaligned tensors take a plain kernel with one lane per row.  The result is the same bits whichever kernel runs.
  *
  * Conventions: tensor memory belongs to the caller and must be device accessible; `out` may not overlap `x`; the
  * functions enqueue one kernel on `hip_stream` (a hipStream_t; NULL is the default stream), return without
