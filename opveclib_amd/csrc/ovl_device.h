@@ -62,16 +62,17 @@ __device__ __forceinline__ T ovl_dpp_move(T old, T src) {
 
 // float32 transcendental entry points used by generated code: bit-compatible with the host C library's
 // expf/logf/tanhf (see ovl_math.h).  ovl_exp_tab / ovl_log_tab name the lookup tables in scope: kernels that call
-// exp or log declare them with OVL_DECLARE_MATH_TABLES at their top, pointing at copies in LDS.
-#define ovl_expf(x) ovl_math::expf_<true>((x), ovl_exp_tab)
-#define ovl_logf(x) ovl_math::logf_((x), ovl_log_tab)
+// exp or log declare them with OVL_DECLARE_MATH_TABLES at their top, pointing at copies in LDS, together with
+// ovl_f64, the routines' float64 constants held in scalar registers.
+#define ovl_expf(x) ovl_math::expf_<true>((x), ovl_exp_tab, ovl_f64)
+#define ovl_logf(x) ovl_math::logf_((x), ovl_log_tab, ovl_f64)
 #define ovl_tanhf(x) ovl_math::tanhf_(x)
 #define ovl_recipf(x) ovl_math::recipf_<true>(x)
 // Variants for arguments that the code generator has proved to lie where the routine's common path is valid
 // (hipgen/ranges.py): no rare-argument block.
-#define ovl_expf_inrange(x) ovl_math::expf_<false>((x), ovl_exp_tab)
-#define ovl_logf_inrange(x) ovl_math::logf_inrange_<false>((x), ovl_log_tab)
-#define ovl_logf_inrange_nan(x) ovl_math::logf_inrange_<true>((x), ovl_log_tab)
+#define ovl_expf_inrange(x) ovl_math::expf_<false>((x), ovl_exp_tab, ovl_f64)
+#define ovl_logf_inrange(x) ovl_math::logf_inrange_<false>((x), ovl_log_tab, ovl_f64)
+#define ovl_logf_inrange_nan(x) ovl_math::logf_inrange_<true>((x), ovl_log_tab, ovl_f64)
 #define ovl_recipf_inrange(x) ovl_math::recipf_<false>(x)
 #define ovl_divf_inrange(a, b) ovl_math::divf_inrange_((a), (b))
 
@@ -83,12 +84,12 @@ __device__ __forceinline__ float ovl_atan2f(float a, float b) { return (float)at
 
 // Once-rounded log(1 + x) and exp(x) - 1 on their checked domains, which the 'ulp2' math mode puts in place of the
 // reference's formulas for them (hipgen/accuracy.py).
-#define ovl_log1p_direct(x) ovl_math::log1p_direct_<false>((x), ovl_log_tab)
-#define ovl_log1p_direct_nan(x) ovl_math::log1p_direct_<true>((x), ovl_log_tab)
-#define ovl_expm1_direct(x) ovl_math::expm1_direct_((x), ovl_exp_tab)
+#define ovl_log1p_direct(x) ovl_math::log1p_direct_<false>((x), ovl_log_tab, ovl_f64)
+#define ovl_log1p_direct_nan(x) ovl_math::log1p_direct_<true>((x), ovl_log_tab, ovl_f64)
+#define ovl_expm1_direct(x) ovl_math::expm1_direct_((x), ovl_exp_tab, ovl_f64)
 // The same for arguments whose value range is known to be narrow: 2^-4 <= x < 1 resp. 2^-12 <= x <= 0.68.
-#define ovl_log1p_unit(x) ovl_math::log1p_unit_((x), ovl_log_unit_tab)
-#define ovl_expm1_small(x) ovl_math::expm1_small_((x), ovl_exp_plain_tab)
+#define ovl_log1p_unit(x) ovl_math::log1p_unit_((x), ovl_log_unit_tab, ovl_f64)
+#define ovl_expm1_small(x) ovl_math::expm1_small_((x), ovl_exp_plain_tab, ovl_f64)
 
 // The logistic function 1 / (1 + exp(-x)) for -16 <= x <= 64 (NaN propagates): hardware-based exp, the sum and the
 // correctly rounded reciprocal.  On that domain it is within two units in the last place of the same formula evaluated
@@ -111,6 +112,7 @@ __device__ __forceinline__ float ovl_atan2f(float a, float b) { return (float)at
     const uint64_t* const ovl_exp_tab = ovl_lds_tables.exp2f;                  \
     const ovl_math::logf_entry* const ovl_log_tab = ovl_lds_tables.logf;       \
     const uint64_t* const ovl_exp_plain_tab = ovl_lds_tables.exp2_plain;       \
-    const ovl_math::logf_entry* const ovl_log_unit_tab = ovl_lds_tables.log_unit
+    const ovl_math::logf_entry* const ovl_log_unit_tab = ovl_lds_tables.log_unit; \
+    const ovl_math::f64_constants ovl_f64 = ovl_math::pinned_constants()
 
 #endif  // OVL_DEVICE_H_

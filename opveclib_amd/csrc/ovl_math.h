@@ -92,6 +92,22 @@ OVL_HD float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
 OVL_HD uint64_t as_u64(double f) { return __builtin_bit_cast(uint64_t, f); }
 OVL_HD double as_f64(uint64_t u) { return __builtin_bit_cast(double, u); }
 
+// The float64 constants of the table-driven routines below.  A float64 operand cannot be written into a vector
+// instruction as a literal, so the compiler moves each half into a scalar register first, and in straight-line code
+// it does that again at every use: a kernel with twelve inlined exponentials issued 116 scalar moves per wavefront
+// for their five constants, a tenth of all its instructions.  Kernels therefore set the constants up once
+// (pinned_constants: the values pass through an empty assembly statement, after which the compiler cannot recreate
+// them and keeps them in scalar registers) and hand them to every call.
+struct f64_constants {
+    double InvLn2N, Shift, C0, C1, C2;      // expf: N / ln 2, 1.5 * 2^52, the polynomial of 2^(r/N)
+    double Ln2, A0, A1, A2;                 // logf: ln 2, the polynomial of log1p(r)
+};
+#define OVL_F64_CONSTANTS {                                                                      \
+    0x1.71547652b82fep+0 * OVL_EXP2F_N, 0x1.8p+52,                                                 \
+    0x1.c6af84b912394p-5 / OVL_EXP2F_N / OVL_EXP2F_N / OVL_EXP2F_N,                               \
+    0x1.ebfce50fac4f3p-3 / OVL_EXP2F_N / OVL_EXP2F_N, 0x1.62e42ff0c52d6p-1 / OVL_EXP2F_N,          \
+    0x1.62e42fefa39efp-1, -0x1.00ea348b88334p-2, 0x1.5575b0be00b6ap-2, -0x1.ffffef20a4123p-2 }
+
 // ---------------------------------------------------------------------------------------------------------------------
 // expf
 // ---------------------------------------------------------------------------------------------------------------------
@@ -116,12 +132,8 @@ OVL_HD uint32_t top12(float x) { return as_u32(x) >> 20; }
 // CHECKED = false leaves out the repair of |x| >= 88 and NaN: for callers that know -88 < x < 88 (NaN still gives
 // NaN, through the polynomial in r).
 template <bool CHECKED = true>
-OVL_HD float expf_(float x, const uint64_t* tab = exp2f_tab) {
-    const double InvLn2N = 0x1.71547652b82fep+0 * OVL_EXP2F_N;
-    const double Shift = 0x1.8p+52;
-    const double C0 = 0x1.c6af84b912394p-5 / OVL_EXP2F_N / OVL_EXP2F_N / OVL_EXP2F_N;
-    const double C1 = 0x1.ebfce50fac4f3p-3 / OVL_EXP2F_N / OVL_EXP2F_N;
-    const double C2 = 0x1.62e42ff0c52d6p-1 / OVL_EXP2F_N;
+OVL_HD float expf_(float x, const uint64_t* tab = exp2f_tab, const f64_constants& f64 = f64_constants OVL_F64_CONSTANTS) {
+    const double InvLn2N = f64.InvLn2N, Shift = f64.Shift, C0 = f64.C0, C1 = f64.C1, C2 = f64.C2;
 
     double xd = (double)x;
     uint32_t abstop = top12(x) & 0x7ff;
@@ -158,12 +170,9 @@ OVL_HD float expf_(float x, const uint64_t* tab = exp2f_tab) {
 // by the code generator's 'ulp2' math mode in place of the reference's expm1 formula
 // (e - 1) * x / log(e), e = exp(x) (opveclib/examples/test_expm1.py:22-62), from which it is at most two units in the
 // last place away on that domain (compared over every float32 argument of the domain).
-OVL_HD float expm1_direct_(float x, const uint64_t* tab = exp2f_tab) {
-    const double InvLn2N = 0x1.71547652b82fep+0 * OVL_EXP2F_N;
-    const double Shift = 0x1.8p+52;
-    const double C0 = 0x1.c6af84b912394p-5 / OVL_EXP2F_N / OVL_EXP2F_N / OVL_EXP2F_N;
-    const double C1 = 0x1.ebfce50fac4f3p-3 / OVL_EXP2F_N / OVL_EXP2F_N;
-    const double C2 = 0x1.62e42ff0c52d6p-1 / OVL_EXP2F_N;
+OVL_HD float expm1_direct_(float x, const uint64_t* tab = exp2f_tab,
+                           const f64_constants& f64 = f64_constants OVL_F64_CONSTANTS) {
+    const double InvLn2N = f64.InvLn2N, Shift = f64.Shift, C0 = f64.C0, C1 = f64.C1, C2 = f64.C2;
     double xd = (double)x;
     double kd = __builtin_fma(InvLn2N, xd, Shift);
     uint64_t ki = as_u64(kd);
@@ -184,12 +193,9 @@ OVL_HD float expm1_direct_(float x, const uint64_t* tab = exp2f_tab) {
 // table (a copy in LDS, built from exp2f_tab when the tables are loaded); on the host the entry is computed here.
 // NaN gives NaN; the index is masked, so an argument outside the domain reads inside the table (and gets a wrong
 // value: the code generator uses the routine only where the value range of the argument lies in the domain).
-OVL_HD float expm1_small_(float x, const uint64_t* plain = nullptr) {
-    const double InvLn2N = 0x1.71547652b82fep+0 * OVL_EXP2F_N;
-    const double Shift = 0x1.8p+52;
-    const double C0 = 0x1.c6af84b912394p-5 / OVL_EXP2F_N / OVL_EXP2F_N / OVL_EXP2F_N;
-    const double C1 = 0x1.ebfce50fac4f3p-3 / OVL_EXP2F_N / OVL_EXP2F_N;
-    const double C2 = 0x1.62e42ff0c52d6p-1 / OVL_EXP2F_N;
+OVL_HD float expm1_small_(float x, const uint64_t* plain = nullptr,
+                          const f64_constants& f64 = f64_constants OVL_F64_CONSTANTS) {
+    const double InvLn2N = f64.InvLn2N, Shift = f64.Shift, C0 = f64.C0, C1 = f64.C1, C2 = f64.C2;
     double xd = (double)x;
     double kd = __builtin_fma(InvLn2N, xd, Shift);
     const uint32_t i = (uint32_t)as_u64(kd) % OVL_EXP2F_N;
@@ -268,6 +274,16 @@ struct lds_tables {
     logf_entry log_unit[OVL_LOGF_N];
 };
 
+// The float64 constants in scalar registers for the rest of the kernel (see f64_constants).
+__device__ __forceinline__ f64_constants pinned_constants() {
+    f64_constants k = OVL_F64_CONSTANTS;
+    // (an instruction reads at most one scalar operand: the second constant of Shift + InvLn2N * x, C1 + C0 * r and
+    // A2 + A1 * r lives in vector registers)
+    asm volatile("" : "+s"(k.InvLn2N), "+v"(k.Shift), "+s"(k.C0), "+v"(k.C1), "+s"(k.C2),
+                      "+s"(k.Ln2), "+s"(k.A0), "+s"(k.A1), "+v"(k.A2));
+    return k;
+}
+
 // Must be called by every thread of the workgroup before any divergent control flow.
 __device__ __forceinline__ void load_tables(lds_tables& t) {
     if (threadIdx.x < OVL_EXP2F_N) {
@@ -283,9 +299,8 @@ __device__ __forceinline__ void load_tables(lds_tables& t) {
 }
 #endif
 
-OVL_HD float logf_main_(uint32_t ix, const logf_entry* tab) {
-    const double Ln2 = 0x1.62e42fefa39efp-1;
-    const double A0 = -0x1.00ea348b88334p-2, A1 = 0x1.5575b0be00b6ap-2, A2 = -0x1.ffffef20a4123p-2;
+OVL_HD float logf_main_(uint32_t ix, const logf_entry* tab, const f64_constants& f64) {
+    const double Ln2 = f64.Ln2, A0 = f64.A0, A1 = f64.A1, A2 = f64.A2;
     const uint32_t Off = 0x3f330000;
     // x = 2^k z; z in [Off, 2*Off) is exact; the range is split into N subintervals, c is near the centre of z's
     uint32_t tmp = ix - Off;
@@ -308,22 +323,23 @@ OVL_HD float logf_main_(uint32_t ix, const logf_entry* tab) {
 // logf_inrange_: for callers that know x is a positive normal number or, with MAYBE_NAN, possibly NaN.  The common
 // path works on the bits of x and would turn NaN into a number; adding x * 0 (+0 for every number) puts the NaN back.
 template <bool MAYBE_NAN>
-OVL_HD float logf_inrange_(float x, const logf_entry* tab = logf_tab) {
-    float result = logf_main_(as_u32(x), tab);
+OVL_HD float logf_inrange_(float x, const logf_entry* tab = logf_tab,
+                           const f64_constants& f64 = f64_constants OVL_F64_CONSTANTS) {
+    float result = logf_main_(as_u32(x), tab, f64);
     if (MAYBE_NAN) result = __builtin_fmaf(x, 0.0f, result);
     return result;
 }
 
-OVL_HD float logf_(float x, const logf_entry* tab = logf_tab) {
+OVL_HD float logf_(float x, const logf_entry* tab = logf_tab, const f64_constants& f64 = f64_constants OVL_F64_CONSTANTS) {
     uint32_t ix = as_u32(x);
     // log(1) needs no special case in round-to-nearest: the table entry around 1 has invc = 1 and logc = 0, so the
     // common path returns +0 (the exhaustive comparison with the host library covers it)
-    float result = logf_main_(ix, tab);
+    float result = logf_main_(ix, tab, f64);
     const bool special = ix - 0x00800000 >= 0x7f800000 - 0x00800000;    // x < 0x1p-126 or inf or nan
     if (OVL_ANY(special)) {
         // subnormal arguments are normalised and evaluated again
         uint32_t scaled = as_u32(x * 0x1p23f) - (23u << 23);
-        float fixed = logf_main_(scaled, tab);
+        float fixed = logf_main_(scaled, tab, f64);
         if ((ix & 0x80000000) || ix * 2 >= 0xff000000) fixed = __builtin_nanf("");
         if (ix == 0x7f800000) fixed = x;
         if (ix * 2 == 0) fixed = -__builtin_inff();
@@ -342,9 +358,9 @@ OVL_HD float logf_(float x, const logf_entry* tab = logf_tab) {
 // The common path works on the bits of u and would turn NaN into a number; with MAYBE_NAN, adding x * 0 (+-0 for every
 // number) puts the NaN back.
 template <bool MAYBE_NAN>
-OVL_HD float log1p_direct_(float x, const logf_entry* tab = logf_tab) {
-    const double Ln2 = 0x1.62e42fefa39efp-1;
-    const double A0 = -0x1.00ea348b88334p-2, A1 = 0x1.5575b0be00b6ap-2, A2 = -0x1.ffffef20a4123p-2;
+OVL_HD float log1p_direct_(float x, const logf_entry* tab = logf_tab,
+                           const f64_constants& f64 = f64_constants OVL_F64_CONSTANTS) {
+    const double Ln2 = f64.Ln2, A0 = f64.A0, A1 = f64.A1, A2 = f64.A2;
     const uint32_t Off = 0x3fe66000;            // upper word of 0.69921875, the lower end of the table's range
     const double u = 1.0 + (double)x;
     const uint64_t iu = as_u64(u);
@@ -369,8 +385,9 @@ OVL_HD float log1p_direct_(float x, const logf_entry* tab = logf_tab) {
 // table is indexed by the top four fraction bits of u itself and neither the exponent's share k * ln 2 nor the
 // re-centring of u is needed.  Same polynomial as logf_; |u / c - 1| <= 1/33.  NaN gives NaN (u is used as it is).
 // The lower end of the domain keeps log(c) + log1p(u / c - 1) away from cancellation.
-OVL_HD float log1p_unit_(float x, const logf_entry* tab = log_unit_tab) {
-    const double A0 = -0x1.00ea348b88334p-2, A1 = 0x1.5575b0be00b6ap-2, A2 = -0x1.ffffef20a4123p-2;
+OVL_HD float log1p_unit_(float x, const logf_entry* tab = log_unit_tab,
+                         const f64_constants& f64 = f64_constants OVL_F64_CONSTANTS) {
+    const double A0 = f64.A0, A1 = f64.A1, A2 = f64.A2;
     const double u = 1.0 + (double)x;
     const uint32_t i = ((uint32_t)(as_u64(u) >> 32) >> (20 - OVL_LOGF_TABLE_BITS)) % OVL_LOGF_N;
     const double invc = tab[i].invc;
