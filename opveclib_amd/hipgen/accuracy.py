@@ -447,6 +447,24 @@ def candidate_sites(info, known):
     return kinds
 
 
+def formula_sites(info, known):
+    """{node index: kind} of the divisions that end a recognised sigmoid / log1p / expm1 formula whose argument lies
+    in the compared domain.  The 'fast' math mode replaces these too: the one routine is both closer to the reference
+    and shorter than the formula composed of cheap routines."""
+    return dict((idx, kind) for idx, kind in candidate_sites(info, known).items() if kind in IDIOM_DOMAIN)
+
+
+def cheap_sites(info, known):
+    """The call sites that do not use the bit-compatible routine, by math mode: none ('exact'), those `select` allows
+    ('ulp2'); for 'fast', where every routine is the cheap one anyway, the recognised formulas."""
+    mode = getattr(info, 'math', 'exact')
+    if mode == 'ulp2':
+        return select(info, known)
+    if mode == 'fast':
+        return formula_sites(info, known)
+    return {}
+
+
 def select(info, known):
     """
     ``{node index: kind}`` of the call sites that may use the cheap routine while every operator output stays within

@@ -313,15 +313,15 @@ class DagInfo(object):
     def uses_math_tables(self):
         """True when the body calls the table-driven float32 exp or log."""
         mode = getattr(self, 'math', 'exact')
-        if mode == 'fast':
-            return False
         calls = [n for n in self.nodes if n.code in (lang.EXP, lang.LOG) and n.dtype == lang.FLOAT32]
-        if mode == 'ulp2':
-            # only the call sites that keep the bit-compatible routine
+        if mode in ('ulp2', 'fast'):
+            # the call sites that keep the bit-compatible routine (none in 'fast' mode) and the once-rounded
+            # log1p / expm1 that stand in for the reference's formulas
             from . import accuracy, ranges
             known = ranges.analyse(self) if getattr(self, 'value_ranges', True) else None
-            cheap = accuracy.select(self, known)
-            calls = [n for n in calls if n.idx not in cheap] + [k for k in cheap.values() if k in accuracy.IDIOM_DOMAIN]
+            cheap = accuracy.cheap_sites(self, known)
+            calls = [] if mode == 'fast' else [n for n in calls if n.idx not in cheap]
+            calls += [k for k in cheap.values() if k in ('log1p', 'expm1')]
         return bool(calls)
 
     def tensor_accesses(self):

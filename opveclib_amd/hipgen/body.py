@@ -240,7 +240,7 @@ class BodyEmitter(object):
         info = self.info
         math_mode = getattr(info, 'math', 'exact')
         known = value_ranges.analyse(info) if getattr(info, 'value_ranges', True) else None
-        cheap_sites = accuracy.select(info, known) if math_mode == 'ulp2' else {}
+        cheap_sites = accuracy.cheap_sites(info, known)
 
         def site_mode(node):
             """The math mode of one call site."""
