@@ -110,14 +110,15 @@ def _arithmetic_weight(info):
 
 def generate(info, kernel_name, vec=None, nt=None, grid_cap=None, per_thread=None):
     """
-    :param per_thread: vectors per thread (1 or 2; None chooses).  Two vectors, 256 apart so that every request of a
-        wavefront stays one contiguous run, are requested together before the arithmetic of either: a wavefront then
-        has twice the bytes in flight while it waits and the workgroup's set-up (math tables, barrier) is paid once
-        for twice the work.  Measured on MI355X, interleaved runs: the 8-op chain in the 'ulp2' math mode, where
-        arithmetic and memory time are about equal, 148.7 -> 142.4 us; the same chain in the 'exact' mode, which is
-        bound by arithmetic alone, 252 -> 255 us; the LSTM cell with its five to seven load streams 27.8 -> 30.4 us
-        (forward) and 36.2 -> 39.9 us (gradient).  So it is chosen for bodies with few streams and some arithmetic,
-        outside the 'exact' mode.
+    :param per_thread: vectors per thread (None chooses 1, 2 or 4).  The vectors, 256 apart so that every request of a
+        wavefront stays one contiguous run, are requested together before the arithmetic of any: a wavefront then
+        has several times the bytes in flight while it waits and the workgroup's set-up (math tables, barrier) is paid
+        once for that much more work.  Measured on MI355X, interleaved runs: the 8-op chain in the 'ulp2' math mode,
+        where arithmetic and memory time are about equal, 148.7 -> 142.4 us with two, and in steady state at the
+        power limit 138.3 -> 133.1 us with four instead of two (eight: 138.3, sixteen: 162); the same chain in the
+        'exact' mode, which is bound by arithmetic alone, 252 -> 255 us; the LSTM cell with its five to seven load
+        streams 27.8 -> 30.4 us (forward) and 36.2 -> 39.9 us (gradient).  So it is chosen for bodies with few
+        streams and some arithmetic, outside the 'exact' mode.
     :return: (kernel source text, launch description dict) for the map template.
     """
     rank = len(info.workgroup_shape)
@@ -187,8 +188,10 @@ def generate(info, kernel_name, vec=None, nt=None, grid_cap=None, per_thread=Non
     single_grid = (num_vectors + BLOCK - 1) // BLOCK <= min(grid_cap or MAX_GRID, MAX_GRID)
     if per_thread is None:
         few_streams = len(loads) + len(unaligned) + len(stores) <= 3
-        per_thread = 2 if (vec > 1 and few_streams and _arithmetic_weight(info) >= 4 and
+        per_thread = 4 if (vec > 1 and few_streams and _arithmetic_weight(info) >= 4 and
                            getattr(info, 'math', 'exact') != 'exact') else 1
+        while per_thread > 1 and num_vectors % (BLOCK * per_thread) != 0:
+            per_thread //= 2
     if per_thread > 1 and not (single_grid and num_vectors % (BLOCK * per_thread) == 0 and
                                not any(info.in_loop.values())):
         per_thread = 1

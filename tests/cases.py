@@ -988,6 +988,7 @@ TEMPLATE_VARIANTS = [
     ('c3_rowscan_shapes', {'template': 'map'}),
     ('c3_cumsum_f64', {'template': 'skewscan'}),
     ('c2_chain', {'per_thread': 2}),
+    ('c2_chain', {'per_thread': 4}),
     ('c4_lstm_grad', {'per_thread': 2}),
     ('c4_lstm_grad', {'cse': False}),
     ('c3_rowscan_shapes', {'template': 'skewscan', 'scan_depth': 1, 'scan_sets': 3}),
