@@ -61,14 +61,16 @@ __device__ __forceinline__ float tanhf_(float x) {
     p = __builtin_fmaf(p, u, -3.333329618e-01f);
     const float small = __builtin_fmaf(ax * u, p, ax);
     // exp(2|x|), with the rounding error of the product 2|x| log2(e) put back in (as in expf_)
-    // (arguments above 10, where tanh rounds to 1, are clamped so that the exponential stays finite; NaN passes)
+    // (arguments above 10, where tanh rounds to 1, are clamped so that the exponential stays finite)
     const float c = 0x1.715476p+1f;
-    const float ac = ax > 10.0f ? 10.0f : ax;
+    // (one median-of-three instruction instead of a compare and a select; for NaN it gives a number, and the
+    // selection below then takes the polynomial's NaN)
+    const float ac = __builtin_amdgcn_fmed3f(ax, 0.0f, 10.0f);
     const float e2 = ac * c;
     float t = __builtin_amdgcn_exp2f(e2);
     t = __builtin_fmaf(t, __builtin_fmaf(ac, c, -e2) * 0x1.62e43p-1f, t);
     const float big = __builtin_fmaf(-2.0f, __builtin_amdgcn_rcpf(t + 1.0f), 1.0f);
-    const float z = ax < 0.6f ? small : big;
+    const float z = ax >= 0.6f ? big : small;
     return __builtin_copysignf(z, x);
 }
 
