@@ -1097,6 +1097,7 @@ def prebuild_all(cases=None, workers=8, with_oracle=True):
             oracle_ops[program.SerializeToString()] = program
             variants.append((program, {'value_ranges': False}))
             variants.append((program, {'math': 'fast'}))
+            variants.append((program, {'math': 'ulp2'}))
         for seed in random_programs.INDEX_SEEDS:
             program = random_programs.index_application(seed).expression_dag
             ops[program.SerializeToString()] = program
