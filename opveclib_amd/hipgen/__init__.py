@@ -10,7 +10,8 @@ CUDA text built around a one-thread-per-worker template.  Here the DAG is analys
 * :mod:`.rowscan_kernel` - loop-carried accumulation along the last tensor axis: order-preserving row scans
   (lane-skewed out of registers; lane-skewed or lane = row out of LDS, fed by dedicated data-moving wavefronts) and
   the reassociating wavefront scan;
-* :mod:`.colscan_kernel` - the same accumulation along another axis: lane = line, rows streamed through LDS.
+* :mod:`.colscan_kernel` - the same accumulation along another axis: rows streamed through LDS, lane-skewed over
+  sixteen lanes per line for tensors with up to 32768 lines ('colskew'), lane = line beyond ('colscan').
 
 Every library exports ``<name>_generic_hip(in, n_in, out, n_out, stream)``: it validates tensor counts, lengths,
 dtypes (the reference's ``*err = 1`` checks, expression.py:621-646, 662-663) and pointer alignment, enqueues the
@@ -61,7 +62,7 @@ def generate(expression_dag, function_name, options=None):
     """
     :param expression_dag: serialised expression DAG of one operator
     :param function_name: unique name of the operator (its content hash)
-    :param options: optional dict.  ``template``: 'auto' (default), 'map', 'transpose', 'rowscan', 'skewscan', 'fedscan', 'treescan' or 'colscan' restricts
+    :param options: optional dict.  ``template``: 'auto' (default), 'map', 'transpose', 'rowscan', 'skewscan', 'fedscan', 'treescan', 'colscan' or 'colskew' restricts
         the choice of kernel template (a template that does not fit the DAG falls back to 'map'); ``vec`` forces the
         map template with that vector width, ``per_thread`` its vectors per thread (1 or 2); ``scan_depth`` / ``scan_sets`` / ``scan_width`` / ``scan_interleave`` set the request burst (groups), the
         number of register sets, the 128-bit vectors per lane and phase and the rows per lane group of the lane-skewed scan; ``math``: 'exact'
@@ -113,6 +114,11 @@ def generate(expression_dag, function_name, options=None):
     elif options.get('vec') is None and template in ('auto', 'rowscan') and rowscan_kernel.plan(info) is not None:
         kernel_src, launch = rowscan_kernel.generate(info, kernel_name, options.get('scan_rows'),
                                                      options.get('scan_chunk'), options.get('scan_batch'))
+    elif options.get('vec') is None and template in ('auto', 'colskew') and colscan_kernel.plan(info) is not None and \
+            (template == 'colskew' or (colscan_kernel.worthwhile(info, colscan_kernel.plan(info)) and
+                                       colscan_kernel.prefers_skew(info, colscan_kernel.plan(info)))):
+        kernel_src, launch = colscan_kernel.generate_skewed(info, kernel_name, options.get('scan_sets'),
+                                                            options.get('scan_strip'))
     elif options.get('vec') is None and template in ('auto', 'colscan') and \
             colscan_kernel.plan(info, options.get('scan_rows'), options.get('scan_batch'),
                                 options.get('scan_sets')) is not None and \

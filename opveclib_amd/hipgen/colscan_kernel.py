@@ -349,3 +349,280 @@ def _emit_movers(a, sets, num_chunks):
         a('        step(%du, sets[%d]);' % (k, (k + 1) % sets))
     a('        store_chunk(%du, m);' % (num_chunks - 1))
 
+
+# ---------------------------------------------------------------------------------------------------------------------
+# The lane-skewed column scan: every wavefront of the workgroup scans.
+#
+# In the kernel above one wavefront runs the recurrence for the 64 lines of a strip, one LDS access per two or four
+# rows, and sets the pace: about 45 clocks per row.  A tensor with few lines has few strips, and the order-preserving
+# recurrence leaves no other parallelism between rows.  But a wavefront need not own 64 lines: here a wavefront owns
+# four lines, sixteen lanes per line, and the rows of a chunk are spread over the sixteen lanes of a line as in the
+# lane-skewed row scans (rowscan_kernel.py): lane `part` owns SEG consecutive rows, runs the recurrence over them from
+# the state it holds and hands its final state to its right neighbour; after sixteen such phases the chunk is exact.
+# A chunk of 16 * SEG rows then costs a wavefront sixteen times (SEG steps + one hand-over), and a workgroup is a strip
+# of 8 to 64 lines (2 to 16 wavefronts), chosen so that the tensor gives a few hundred workgroups: the instructions a
+# wavefront issues are sixteen times redundant, so the gain is there only while the wavefronts have SIMDs to
+# themselves (sixteen wavefronts on one CU's four SIMDs scan a strip of 64 lines no faster than the kernel above).
+# All threads move data: they load their share of the chunks ahead into registers (row-major, sixteen lanes read
+# neighbouring lines of one row), write it transposed into LDS (line-major, so that a lane's rows are adjacent, whole
+# 128-bit words), and after the scan read the results back and store them.  Two LDS buffers alternate; two barriers
+# per chunk.
+# ---------------------------------------------------------------------------------------------------------------------
+SKEW_GROUP = 16                 # lanes per line
+SKEW_SEG_VECTORS = 2            # 128-bit vectors a lane owns per phase (32 bytes: 4 float64 or 8 float32 rows)
+SKEW_SETS = 8                   # chunks of loads in flight per workgroup
+
+
+#: with more lines than this the strips of 64 lines of the kernel above already give every CU several workgroups
+SKEW_MAX_LINES = 1 << 15
+
+
+def skew_strip(info, p):
+    """Lines per workgroup of the lane-skewed column scan: a power of two between 8 and 64 that gives about 256
+    workgroups.  Measured on MI355X, microseconds with strips of 4 / 8 / 16 / 32 / 64 lines (and the kernel above):
+    float64 [10000, 1000] 85 / 79 / 91 / 141 / 257 (191); float32 [10000, 1000] 82 / 56 / 61 / 72 / 120 (117);
+    float64 [5000, 300] 41 / 42 / 48 / 74 / 131 (97); float64 [4096, 4096] 177 / 70 / 41 / 61 / 108 (82);
+    float32 [4096, 8192] 356 / 195 / 66 / 46 / 54 (77); float32 [1000, 16384] 182 / 105 / 36 / 26 / 23 (31);
+    float64 [1000, 16384] 193 / 67 / 46 / 46 / 50 (43)."""
+    lines = p.outer * p.inner
+    strip = 8
+    while strip < 64 and lines > 256 * strip:
+        strip *= 2
+    return strip
+
+
+def prefers_skew(info, p):
+    """Few enough lines that the lane-skewed kernel's small strips pay (see `skew_strip`)."""
+    from .rowscan_kernel import _carried_state
+    if p.outer * p.inner > SKEW_MAX_LINES:
+        return False
+    return all(info.nodes[idx].dtype in CTYPE for idx in _carried_state(info, p))
+
+
+def generate_skewed(info, kernel_name, sets=None, strip=None):
+    from .rowscan_kernel import _carried_state
+    p = plan(info)
+    assert p is not None
+    STRIP = strip or skew_strip(info, p)            # lines per workgroup
+    BLOCK = STRIP * SKEW_GROUP                      # sixteen lanes per line
+    ctype = CTYPE[p.x.dtype]
+    per = p.per
+    seg = SKEW_SEG_VECTORS * per                    # rows a lane owns per phase
+    rc = SKEW_GROUP * seg                           # rows per chunk
+    seg_stride = seg + per                          # a segment and its padding vector (bank conflicts)
+    line_stride = SKEW_GROUP * seg_stride + per     # a line and its padding vector
+    num_chunks = (p.length + rc - 1) // rc
+    strips = (p.inner + STRIP - 1) // STRIP
+    rows_per_pass = BLOCK // STRIP                  # rows covered by one load instruction of the workgroup
+    ipt = rc // rows_per_pass                       # elements each thread moves per chunk
+    vpt = ipt // per                                # ... as 128-bit vectors of consecutive rows of one line
+    sets = max(2, min(int(sets or SKEW_SETS), 16, max(2, num_chunks)))
+    lines_per_wave = WAVE // SKEW_GROUP
+
+    wg = list(info.workgroup_shape)
+    rank = len(wg)
+    wg_strides = [1] * rank
+    for k in range(rank - 2, -1, -1):
+        wg_strides[k] = wg_strides[k + 1] * wg[k + 1]
+    pos_exprs = []
+    for k in range(rank):
+        expr = 'line'
+        if k > 0:
+            expr = '(line % ' + str(wg_strides[k - 1]) + 'u)'
+        pos_exprs.append(expr + ' / ' + str(wg_strides[k]) + 'u')
+    emitter = BodyEmitter(info, pos_exprs,
+                          read_hook=lambda node, tensor, idx: 'OVL_SCAN_IN',
+                          store_hook=lambda node, tensor, idx, value: 'OVL_SCAN_OUT(' + value + ');')
+    tagged = emitter.emit_tagged()
+    range_idx = p.loop_item.node
+    end_idx = max(i for i, _ in tagged)
+    prologue = [t for i, t in tagged if i < range_idx]
+    body = [t.strip() for i, t in tagged if range_idx < i < end_idx]
+    counter_name = 'e' + str(p.counter)
+    counter_type = CTYPE[info.nodes[p.counter].dtype]
+    state = [('e' + str(idx), CTYPE[info.nodes[idx].dtype]) for idx in _carried_state(info, p)]
+
+    vname = 'ovl_scan_vec'
+    src = []
+    a = src.append
+    a('typedef %s %s __attribute__((ext_vector_type(%d)));' % (ctype, vname, per))
+    a('')
+    a('extern "C" __global__ void __launch_bounds__(%d)' % BLOCK)
+    a('%s(const %s* __restrict__ in%d, %s* __restrict__ out%d) {' % (
+        kernel_name, ctype, p.x.io_index, ctype, p.out.io_index))
+    if info.uses_math_tables():
+        a('    OVL_DECLARE_MATH_TABLES();')
+    a('    // tile[buffer][line][row]: a line holds the %d rows of a chunk as 16 segments of %d rows, each followed by one' % (rc, seg))
+    a('    // spare vector, and one more at its end')
+    a('    __shared__ __attribute__((aligned(16))) %s tile[2][%d][%d];' % (ctype, STRIP, line_stride))
+    a('    const uint32_t strip = blockIdx.x %% %du;' % strips)
+    a('    const uint32_t o = blockIdx.x / %du;                 // index over the dimensions before the scanned axis' % strips)
+    a('    const uint32_t c0 = strip * %du;                      // first line of the strip within its row' % STRIP)
+    a('    const uint64_t obase = (uint64_t)o * %dull + c0;      // element of row 0, first line of the strip' % (
+        p.length * p.inner))
+    a('    const %s* __restrict__ gin = in%d + obase;' % (ctype, p.x.io_index))
+    a('    %s* __restrict__ gout = out%d + obase;' % (ctype, p.out.io_index))
+    a('')
+    a('    // Moving data: thread t owns line t %% %d of rows t / %d, t / %d + %d, ... of every chunk (%d elements).' % (
+        STRIP, STRIP, STRIP, rows_per_pass, ipt))
+    a('    // An element that does not exist (past the last row, past the last line) is replaced by the nearest one that')
+    a('    // does: it is loaded, and later stored, a second time with the same value.  Without conditions around the')
+    a('    // memory instructions the compiler can count them, and waits for the loads of exactly the chunk it needs while')
+    a('    // those of the chunks after it stay in flight (with conditional stores it waited for all but the last dozen')
+    a('    // requests: float64 [10000, 1000] 264 us).')
+    a('    const uint32_t lines_here = (%du - c0 < %du) ? %du - c0 : %du;' % (p.inner, STRIP, p.inner, STRIP))
+    a('    const uint32_t mc = (threadIdx.x %% %du < lines_here) ? threadIdx.x %% %du : lines_here - 1u;' % (STRIP, STRIP))
+    a('    const uint32_t mv = threadIdx.x / %du;               // first of the vectors (%d consecutive rows) the thread owns' % (
+        STRIP, per))
+    a('    struct MoverRegs { %s v[%d]; };' % (vname, vpt))
+    a('    auto chunk_row = [&](uint32_t k, uint32_t i, uint32_t u) -> uint32_t {     // clamped to the chunk\'s last row')
+    a('        const uint32_t r = (mv + i * %du) * %du + u;' % (BLOCK // STRIP, per))
+    a('        const uint32_t rows_here = (%du - k * %du < %du) ? %du - k * %du : %du;' % (
+        p.length, rc, rc, p.length, rc, rc))
+    a('        return r < rows_here ? r : rows_here - 1u;')
+    a('    };')
+    a('    // (a thread writes and reads whole 128-bit words of LDS: lanes on neighbouring lines are %d words apart, an odd' % (
+        line_stride // per))
+    a('    // number, so eight of them cover all banks; 64-bit accesses at that stride ran into 8-way conflicts: 257 us)')
+    a('    auto lds_at = [&](uint32_t k, uint32_t i) -> %s* {' % vname)
+    a('        const uint32_t r = (mv + i * %du) * %du;' % (BLOCK // STRIP, per))
+    a('        return reinterpret_cast<%s*>(&tile[k %% 2u][mc][(r / %du) * %du + r %% %du]);' % (vname, seg, seg_stride, seg))
+    a('    };')
+    a('    auto issue_loads = [&](uint32_t k, MoverRegs& regs) {')
+    a('        #pragma unroll')
+    a('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
+    a('            #pragma unroll')
+    a('            for (uint32_t u = 0; u < %du; ++u)' % per)
+    a('                regs.v[i][u] = gin[(uint64_t)(k * %du + chunk_row(k, i, u)) * %dull + mc];' % (rc, p.inner))
+    a('        }')
+    a('    };')
+    a('    auto write_lds = [&](uint32_t k, const MoverRegs& regs) {')
+    a('        #pragma unroll')
+    a('        for (uint32_t i = 0; i < %du; ++i) *lds_at(k, i) = regs.v[i];' % vpt)
+    a('    };')
+    a('    auto store_chunk = [&](uint32_t k) {')
+    a('        // (a row past the chunk\'s last one is stored as that last row once more: its value comes from the word that')
+    a('        // holds the last row)')
+    a('        const uint32_t last = ((%du - k * %du < %du) ? %du - k * %du : %du) - 1u;' % (
+        p.length, rc, rc, p.length, rc, rc))
+    a('        MoverRegs regs;')
+    a('        #pragma unroll')
+    a('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
+    a('            const uint32_t word = mv + i * %du;' % (BLOCK // STRIP))
+    a('            const uint32_t r = (word < last / %du ? word : last / %du) * %du;' % (per, per, per))
+    a('            regs.v[i] = *reinterpret_cast<const %s*>(&tile[k %% 2u][mc][(r / %du) * %du + r %% %du]);' % (
+        vname, seg, seg_stride, seg))
+    a('        }')
+    a('        #pragma unroll')
+    a('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
+    a('            %s of_last = regs.v[i][0];' % ctype)
+    a('            #pragma unroll')
+    a('            for (uint32_t u = 1; u < %du; ++u) of_last = (last %% %du == u) ? regs.v[i][u] : of_last;' % (per, per))
+    a('            #pragma unroll')
+    a('            for (uint32_t u = 0; u < %du; ++u) {' % per)
+    a('                const uint32_t r = (mv + i * %du) * %du + u;' % (BLOCK // STRIP, per))
+    a('                __builtin_nontemporal_store(r <= last ? regs.v[i][u] : of_last,')
+    a('                                            gout + (uint64_t)(k * %du + (r <= last ? r : last)) * %dull + mc);' % (
+        rc, p.inner))
+    a('            }')
+    a('        }')
+    a('    };')
+    a('')
+    a('    // Scanning: wavefront w owns lines %d w ... %d w + %d of the strip, sixteen lanes each; lane `part` of a line owns' % (
+        lines_per_wave, lines_per_wave, lines_per_wave - 1))
+    a('    // rows [part * %d, part * %d + %d) of every chunk.  A line past the last one shadows it.' % (seg, seg, seg))
+    a('    const uint32_t lane = threadIdx.x %% %du;' % WAVE)
+    a('    const uint32_t part = lane %% %du;' % SKEW_GROUP)
+    a('    const uint32_t sl = threadIdx.x / %du * %du + lane / %du;      // line of the strip' % (
+        WAVE, lines_per_wave, SKEW_GROUP))
+    a('    const uint32_t c = (c0 + sl < %du) ? sl : %du - c0;' % (p.inner, p.inner - 1))
+    a('    const uint32_t line = o * %du + c0 + c;' % p.inner)
+    a('    // first row: the statements the worker runs before its loop, in every lane')
+    a('    %s first_out;' % ctype)
+    a('#define OVL_SCAN_IN (gin[c])')
+    a('#define OVL_SCAN_OUT(value) first_out = (value)')
+    for stmt in prologue:
+        a('    ' + stmt)
+    a('#undef OVL_SCAN_IN')
+    a('#undef OVL_SCAN_OUT')
+    for name, stype in state:
+        a('    %s carry_%s = %s;' % (stype, name, name))
+    a('#define OVL_SCAN_IN xv[u]')
+    a('#define OVL_SCAN_OUT(value) ov[w][u] = (value)')
+    a('#define OVL_SCAN_STEP(row) { %s = (%s)(row); %s }' % (counter_name, counter_type, ' '.join(body)))
+    a('    // one chunk: in phase p every lane runs the recurrence over its rows from the state it holds and hands its')
+    a('    // final state to its right neighbour; after phase p lanes 0..p are exact')
+    a('    auto scan_chunk = [&](uint32_t k) {')
+    a('        %s* segp = &tile[k %% 2u][sl][part * %du];' % (ctype, seg_stride))
+    a('        %s set[%d], ov[%d];' % (vname, SKEW_SEG_VECTORS, SKEW_SEG_VECTORS))
+    a('        #pragma unroll')
+    a('        for (uint32_t w = 0; w < %du; ++w) set[w] = *reinterpret_cast<const %s*>(segp + w * %du);' % (
+        SKEW_SEG_VECTORS, vname, per))
+    a('        const uint32_t row0 = k * %du + part * %du;' % (rc, seg))
+    a('        const bool first_row = k == 0u && part == 0u;')
+    a('        #pragma unroll')
+    a('        for (uint32_t phase = 0; phase < %du; ++phase) {' % SKEW_GROUP)
+    for name, _ in state:
+        a('            %s = carry_%s;' % (name, name))
+    a('            #pragma unroll')
+    a('            for (uint32_t w = 0; w < %du; ++w) {' % SKEW_SEG_VECTORS)
+    a('                const %s xv = set[w];' % vname)
+    a('                #pragma unroll')
+    a('                for (uint32_t u = 0; u < %du; ++u) {' % per)
+    a('                    if (w == 0u && u == 0u && first_row) ov[0][0] = first_out;')
+    a('                    else OVL_SCAN_STEP(row0 + w * %du + u)' % per)
+    a('                }')
+    a('            }')
+    for name, _ in state:
+        a('            carry_%s = ovl_dpp_move<OVL_DPP_ROW_SHR1>(carry_%s, %s);' % (name, name, name))
+    a('        }')
+    a('        // the last lane of the line finished the chunk: its state is the carry into the next one')
+    for name, _ in state:
+        a('        carry_%s = ovl_dpp_move<OVL_DPP_ROW_ROR1>(carry_%s, %s);' % (name, name, name))
+    a('        #pragma unroll')
+    a('        for (uint32_t w = 0; w < %du; ++w) *reinterpret_cast<%s*>(segp + w * %du) = ov[w];' % (
+        SKEW_SEG_VECTORS, vname, per))
+    a('    };')
+    a('')
+    a('    // %d register sets keep %d chunks of loads in flight: chunk j travels through set j %% %d' % (sets, sets, sets))
+    a('    MoverRegs sets[%d];' % sets)
+    for j in range(min(sets, num_chunks)):
+        a('    issue_loads(%du, sets[%d]);' % (j, j))
+    a('    write_lds(0u, sets[0]);')
+    if sets < num_chunks:
+        a('    issue_loads(%du, sets[0]);' % sets)
+    a('    __syncthreads();')
+    a('    // step k: chunk k is scanned in place; then its results go out while chunk k + 1 comes into the other buffer')
+    a('    auto step = [&](uint32_t k, MoverRegs& regs) {')
+    a('        scan_chunk(k);')
+    a('        __syncthreads();')
+    a('        store_chunk(k);')
+    a('        if (k + 1u < %du) write_lds(k + 1u, regs);' % num_chunks)
+    a('        if (k + 1u + %du < %du) issue_loads(k + 1u + %du, regs);' % (sets, num_chunks, sets))
+    a('        __syncthreads();')
+    a('    };')
+    full = num_chunks // sets
+    if full:
+        a('    #pragma unroll 1')
+        a('    for (uint32_t k0 = 0; k0 < %du; k0 += %du) {' % (full * sets, sets))
+        for d in range(sets):
+            a('        step(k0 + %du, sets[%d]);' % (d, (d + 1) % sets))
+        a('    }')
+    for k in range(full * sets, num_chunks):
+        a('    step(%du, sets[%d]);' % (k, (k + 1) % sets))
+    a('#undef OVL_SCAN_STEP')
+    a('#undef OVL_SCAN_IN')
+    a('#undef OVL_SCAN_OUT')
+    a('}')
+
+    itemsize = ITEMSIZE[p.x.dtype]
+    launch = {
+        'template': 'colskew',
+        'vec': 1,
+        'block': BLOCK,
+        'blocks_needed': p.outer * strips,
+        'align': {('in', p.x.io_index): itemsize, ('out', p.out.io_index): itemsize},
+        'vector_loads': 1,
+        'vector_stores': 1,
+    }
+    return '\n'.join(src) + '\n', launch

@@ -974,6 +974,9 @@ def ulp2_full_size_operators():
 
 # (case, code generator options): the same cases through kernel templates the generator would not pick by itself
 TEMPLATE_VARIANTS = [
+    ('c3_colscan_shapes', {'template': 'colskew', 'scan_strip': 64}),
+    ('c3_colscan_shapes', {'template': 'colskew', 'scan_strip': 4, 'scan_sets': 3}),
+    ('c3_colscan_shapes', {'template': 'colskew', 'scan_strip': 16, 'scan_sets': 2}),
     ('c3_colscan_shapes', {'template': 'colscan'}),
     ('c3_colscan_shapes', {'template': 'colscan', 'scan_rows': 32, 'scan_batch': 2}),
     ('c3_colscan_shapes', {'template': 'colscan', 'scan_sets': 3}),

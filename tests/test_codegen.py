@@ -89,10 +89,15 @@ def test_template_selection():
     assert template(cumsum(np.zeros((48, 1000), np.float32), axis=1))['template'] == 'map'
     # along another axis: a short axis keeps one worker per thread, a long one with few lines gets strips of 64 lines
     assert template(cumsum(np.zeros((48, 1024), np.float32), axis=0))['template'] == 'map'
+    # (up to 32768 lines: sixteen lanes per line, strips of 8 to 64 lines for about 256 workgroups)
     col = template(cumsum(np.zeros((1000, 200), np.float64), axis=0))
-    assert col['template'] == 'colscan' and col['blocks_needed'] == 4 and col['block'] == 1024
+    assert col['template'] == 'colskew' and col['blocks_needed'] == 25 and col['block'] == 128
     mid = template(cumsum(np.zeros((3, 500, 96), np.float32), axis=1))
-    assert mid['template'] == 'colscan' and mid['blocks_needed'] == 3 * 2
+    assert mid['template'] == 'colskew' and mid['blocks_needed'] == 3 * 12
+    wide = template(cumsum(np.zeros((200, 16384), np.float32), axis=0))
+    assert wide['template'] == 'colskew' and wide['blocks_needed'] == 256 and wide['block'] == 1024
+    many = template(cumsum(np.zeros((200, 65536), np.float32), axis=0))
+    assert many['template'] == 'colscan' and many['blocks_needed'] == 1024 and many['block'] == 1024
     assert template(cumsum(np.zeros((128, 1 << 17), np.float32), axis=0))['template'] == 'map'    # enough wavefronts
     assert template(cases.dot(np.zeros((16, 64)), np.zeros((16, 64))))['template'] == 'map'
     # transposed store of a rank-2 workgroup: LDS tiles; the gather is one dword-aligned 128-bit load per thread
