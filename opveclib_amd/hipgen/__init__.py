@@ -118,7 +118,7 @@ def generate(expression_dag, function_name, options=None):
             (template == 'colskew' or (colscan_kernel.worthwhile(info, colscan_kernel.plan(info)) and
                                        colscan_kernel.prefers_skew(info, colscan_kernel.plan(info)))):
         kernel_src, launch = colscan_kernel.generate_skewed(info, kernel_name, options.get('scan_sets'),
-                                                            options.get('scan_strip'))
+                                                            options.get('scan_strip'), options.get('scan_width'))
     elif options.get('vec') is None and template in ('auto', 'colscan') and \
             colscan_kernel.plan(info, options.get('scan_rows'), options.get('scan_batch'),
                                 options.get('scan_sets')) is not None and \

@@ -370,6 +370,7 @@ def _emit_movers(a, sets, num_chunks):
 # ---------------------------------------------------------------------------------------------------------------------
 SKEW_GROUP = 16                 # lanes per line
 SKEW_SEG_VECTORS = 2            # 128-bit vectors a lane owns per phase (32 bytes: 4 float64 or 8 float32 rows)
+SKEW_SEG_VECTORS_NARROW = 8     # ... in strips of 8 lines
 SKEW_SETS = 8                   # chunks of loads in flight per workgroup
 
 
@@ -399,7 +400,7 @@ def prefers_skew(info, p):
     return all(info.nodes[idx].dtype in CTYPE for idx in _carried_state(info, p))
 
 
-def generate_skewed(info, kernel_name, sets=None, strip=None):
+def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None):
     from .rowscan_kernel import _carried_state
     p = plan(info)
     assert p is not None
@@ -407,7 +408,15 @@ def generate_skewed(info, kernel_name, sets=None, strip=None):
     BLOCK = STRIP * SKEW_GROUP                      # sixteen lanes per line
     ctype = CTYPE[p.x.dtype]
     per = p.per
-    seg = SKEW_SEG_VECTORS * per                    # rows a lane owns per phase
+    if seg_vectors is None:
+        # the narrowest strips are chosen for tensors with few lines, whose time is the latency of the recurrence:
+        # there a lane owns 128 bytes of rows, so that a hand-over is paid once per 16 (32) steps, and four chunks of
+        # loads stay in flight (float64 [10000, 1000]: 79 us with 32 bytes, 65 with 64, 59 with 128; with wider strips
+        # the longer segments lose: float64 [4096, 4096] 41 -> 45 us)
+        seg_vectors = SKEW_SEG_VECTORS_NARROW if STRIP <= 8 else SKEW_SEG_VECTORS
+        if sets is None and STRIP <= 8:
+            sets = 4
+    seg = seg_vectors * per                         # rows a lane owns per phase
     rc = SKEW_GROUP * seg                           # rows per chunk
     seg_stride = seg + per                          # a segment and its padding vector (bank conflicts)
     line_stride = SKEW_GROUP * seg_stride + per     # a line and its padding vector
@@ -554,10 +563,10 @@ def generate_skewed(info, kernel_name, sets=None, strip=None):
     a('    // final state to its right neighbour; after phase p lanes 0..p are exact')
     a('    auto scan_chunk = [&](uint32_t k) {')
     a('        %s* segp = &tile[k %% 2u][sl][part * %du];' % (ctype, seg_stride))
-    a('        %s set[%d], ov[%d];' % (vname, SKEW_SEG_VECTORS, SKEW_SEG_VECTORS))
+    a('        %s set[%d], ov[%d];' % (vname, seg_vectors, seg_vectors))
     a('        #pragma unroll')
     a('        for (uint32_t w = 0; w < %du; ++w) set[w] = *reinterpret_cast<const %s*>(segp + w * %du);' % (
-        SKEW_SEG_VECTORS, vname, per))
+        seg_vectors, vname, per))
     a('        const uint32_t row0 = k * %du + part * %du;' % (rc, seg))
     a('        const bool first_row = k == 0u && part == 0u;')
     a('        #pragma unroll')
@@ -565,7 +574,7 @@ def generate_skewed(info, kernel_name, sets=None, strip=None):
     for name, _ in state:
         a('            %s = carry_%s;' % (name, name))
     a('            #pragma unroll')
-    a('            for (uint32_t w = 0; w < %du; ++w) {' % SKEW_SEG_VECTORS)
+    a('            for (uint32_t w = 0; w < %du; ++w) {' % seg_vectors)
     a('                const %s xv = set[w];' % vname)
     a('                #pragma unroll')
     a('                for (uint32_t u = 0; u < %du; ++u) {' % per)
@@ -581,7 +590,7 @@ def generate_skewed(info, kernel_name, sets=None, strip=None):
         a('        carry_%s = ovl_dpp_move<OVL_DPP_ROW_ROR1>(carry_%s, %s);' % (name, name, name))
     a('        #pragma unroll')
     a('        for (uint32_t w = 0; w < %du; ++w) *reinterpret_cast<%s*>(segp + w * %du) = ov[w];' % (
-        SKEW_SEG_VECTORS, vname, per))
+        seg_vectors, vname, per))
     a('    };')
     a('')
     a('    // %d register sets keep %d chunks of loads in flight: chunk j travels through set j %% %d' % (sets, sets, sets))
