@@ -464,8 +464,22 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None):
     a('    // tile[buffer][line][row]: a line holds the %d rows of a chunk as 16 segments of %d rows, each followed by one' % (rc, seg))
     a('    // spare vector, and one more at its end')
     a('    __shared__ __attribute__((aligned(16))) %s tile[2][%d][%d];' % (ctype, STRIP, line_stride))
-    a('    const uint32_t strip = blockIdx.x %% %du;' % strips)
-    a('    const uint32_t o = blockIdx.x / %du;                 // index over the dimensions before the scanned axis' % strips)
+    # A strip narrower than a 128-byte line shares the lines of every row with its neighbours.  Workgroups go to the
+    # eight XCDs (each with its own L2) in turn, so neighbouring strips are given to workgroups 8 apart: they land on
+    # one XCD at about the same time and the line is fetched from memory once (float64 [10000, 1000] in strips of 8
+    # lines read its input twice).
+    share = max(1, 128 // (STRIP * ITEMSIZE[p.x.dtype]))
+    total = p.outer * strips
+    if share > 1 and total >= 8 * share:
+        whole = total // (8 * share) * (8 * share)
+        a('    // workgroups b and b + 8 (same XCD) take neighbouring strips, which share the cache lines of every row')
+        a('    const uint32_t wg = blockIdx.x < %du' % whole)
+        a('        ? blockIdx.x / %du * %du + blockIdx.x %% 8u * %du + blockIdx.x / 8u %% %du : blockIdx.x;' % (
+            8 * share, 8 * share, share, share))
+    else:
+        a('    const uint32_t wg = blockIdx.x;')
+    a('    const uint32_t strip = wg %% %du;' % strips)
+    a('    const uint32_t o = wg / %du;                         // index over the dimensions before the scanned axis' % strips)
     a('    const uint32_t c0 = strip * %du;                      // first line of the strip within its row' % STRIP)
     a('    const uint64_t obase = (uint64_t)o * %dull + c0;      // element of row 0, first line of the strip' % (
         p.length * p.inner))
