@@ -342,12 +342,12 @@ class DagInfo(object):
         through a computed index, under a condition that not every path takes) is written at once; buffering another
         store to the same tensor would write it later and so reverse the program's order whenever both hit one element.
         """
-        verdict = {}
+        allowed = {}
         for node, tensor, aff in self.tensor_accesses():
             if node.code == lang.ASSIGN_TENSOR:
                 ok = aff is not None and not self.in_loop[node.idx] and bool(buffers(node, tensor, aff))
-                verdict[tensor.idx] = verdict.get(tensor.idx, True) and ok
-        return set(idx for idx, ok in verdict.items() if ok)
+                allowed[tensor.idx] = allowed.get(tensor.idx, True) and ok
+        return set(idx for idx, ok in allowed.items() if ok)
 
     def definitely_stores(self, keys):
         """
