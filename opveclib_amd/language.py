@@ -208,9 +208,8 @@ class Message(object):
         f = type(self)._by_name.get(key)
         if f is None:
             raise AttributeError('%s has no field "%s"' % (type(self).__name__, key))
-        value = self._default(f)
-        self.__dict__[key] = value
-        return value
+        # (setdefault: when two threads materialise the same field, both get the one container that is kept)
+        return self.__dict__.setdefault(key, self._default(f))
 
     def __setattr__(self, key, value):
         f = self._by_name.get(key)
@@ -251,7 +250,9 @@ class Message(object):
                     mine[name].Clear()
                 else:
                     del mine[name]
-        for name, src in theirs.items():
+        # (a snapshot: traced DAGs are shared between threads, and a reader of `other` in another thread may materialise
+        # a default there meanwhile)
+        for name, src in list(theirs.items()):
             f = self._by_name[name]
             if f.repeated:
                 dst = getattr(self, name)

@@ -191,3 +191,49 @@ def test_sparse_storage_keeps_message_semantics():
     dag = sample_dag()
     assert copy.deepcopy(dag) == dag
     assert pickle.loads(pickle.dumps(dag)) == dag
+
+
+def test_copy_from_a_message_that_another_thread_is_reading():
+    # Traced DAGs are shared between threads.  Reading an unset field materialises its default in the message's
+    # storage, so a reader in one thread changes the dictionary that CopyFrom in another thread walks.
+    import threading
+    names = [f.name for f in lang.Expression._fields]
+    messages = []
+    for k in range(4000):
+        m = lang.Expression()
+        m.code = lang.CONST_SCALAR
+        m.double_data.append(float(k))
+        messages.append(m)
+    errors = []
+    position = [0]
+
+    def reader():
+        while position[0] < len(messages):
+            m = messages[min(position[0], len(messages) - 1)]
+            for name in names:
+                getattr(m, name)
+
+    def copier():
+        try:
+            for k, m in enumerate(messages):
+                position[0] = k
+                target = lang.Expression()
+                target.CopyFrom(m)
+                assert target == m
+        except Exception as exception:      # noqa: B902 - reported by the main thread
+            errors.append(exception)
+        finally:
+            position[0] = len(messages)
+
+    import sys
+    threads = [threading.Thread(target=reader) for _ in range(3)] + [threading.Thread(target=copier)]
+    interval = sys.getswitchinterval()
+    sys.setswitchinterval(1e-6)             # hand the interpreter from thread to thread as often as possible
+    try:
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+    finally:
+        sys.setswitchinterval(interval)
+    assert errors == []
