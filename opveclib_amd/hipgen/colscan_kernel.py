@@ -363,15 +363,23 @@ def _emit_movers(a, sets, num_chunks):
 # of 8 to 64 lines (2 to 16 wavefronts), chosen so that the tensor gives a few hundred workgroups: the instructions a
 # wavefront issues are sixteen times redundant, so the gain is there only while the wavefronts have SIMDs to
 # themselves (sixteen wavefronts on one CU's four SIMDs scan a strip of 64 lines no faster than the kernel above).
-# All threads move data: they load their share of the chunks ahead into registers (row-major, sixteen lanes read
-# neighbouring lines of one row), write it transposed into LDS (line-major, so that a lane's rows are adjacent, whole
-# 128-bit words), and after the scan read the results back and store them.  Two LDS buffers alternate; two barriers
-# per chunk.
+# Moving data: the chunks ahead are loaded into registers (row-major, sixteen lanes read neighbouring lines of one
+# row), written transposed into LDS (line-major, so that a lane's rows are adjacent, whole 128-bit words), and after
+# the scan the results are read back and stored.  In strips of 16 lines and more the scanning wavefronts do this
+# themselves between two chunks (two LDS buffers alternate, two barriers per chunk).  The narrowest strips belong to
+# tensors with few lines, where most SIMDs are idle and the time is the length of one wavefront's instruction stream:
+# there four more wavefronts of the workgroup do nothing but move data through three rotating buffers (one barrier per
+# chunk) and the scanning wavefronts only read their segments, run the recurrence and write them back (float64
+# [10000, 1000] 58 -> 40 us, float32 47 -> 33 us, float64 [5000, 300] 32 -> 23 us; in strips of 16 lines the extra
+# wavefronts lose: float64 [4096, 4096] 41 -> 45 us).  What is left there is the recurrence: 0.86 us per chunk of 256
+# rows, of which the sixteen phases of sixteen dependent float64 additions and a hand-over are 0.70.
 # ---------------------------------------------------------------------------------------------------------------------
 SKEW_GROUP = 16                 # lanes per line
 SKEW_SEG_VECTORS = 2            # 128-bit vectors a lane owns per phase (32 bytes: 4 float64 or 8 float32 rows)
 SKEW_SEG_VECTORS_NARROW = 8     # ... in strips of 8 lines
 SKEW_SETS = 8                   # chunks of loads in flight per workgroup
+SKEW_MOVERS = 256               # threads that only move data, in strips of at most ...
+SKEW_MOVERS_MAX_STRIP = 8       # ... this many lines (128, 256 and 512 threads measured the same)
 
 
 #: with more lines than this the strips of 64 lines of the kernel above already give every CU several workgroups
@@ -380,7 +388,8 @@ SKEW_MAX_LINES = 1 << 15
 
 def skew_strip(info, p):
     """Lines per workgroup of the lane-skewed column scan: a power of two between 8 and 64 that gives about 256
-    workgroups.  Measured on MI355X, microseconds with strips of 4 / 8 / 16 / 32 / 64 lines (and the kernel above):
+    workgroups.  Measured on MI355X with every wavefront moving data, 32-byte segments and eight register sets,
+    microseconds with strips of 4 / 8 / 16 / 32 / 64 lines (and the kernel above):
     float64 [10000, 1000] 85 / 79 / 91 / 141 / 257 (191); float32 [10000, 1000] 82 / 56 / 61 / 72 / 120 (117);
     float64 [5000, 300] 41 / 42 / 48 / 74 / 131 (97); float64 [4096, 4096] 177 / 70 / 41 / 61 / 108 (82);
     float32 [4096, 8192] 356 / 195 / 66 / 46 / 54 (77); float32 [1000, 16384] 182 / 105 / 36 / 26 / 23 (31);
@@ -400,29 +409,42 @@ def prefers_skew(info, p):
     return all(info.nodes[idx].dtype in CTYPE for idx in _carried_state(info, p))
 
 
-def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None):
+def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, movers=None):
     from .rowscan_kernel import _carried_state
     p = plan(info)
     assert p is not None
     STRIP = strip or skew_strip(info, p)            # lines per workgroup
-    BLOCK = STRIP * SKEW_GROUP                      # sixteen lanes per line
+    SCAN_THREADS = STRIP * SKEW_GROUP               # sixteen lanes per line
     ctype = CTYPE[p.x.dtype]
     per = p.per
+    narrow = STRIP <= 8
     if seg_vectors is None:
         # the narrowest strips are chosen for tensors with few lines, whose time is the latency of the recurrence:
-        # there a lane owns 128 bytes of rows, so that a hand-over is paid once per 16 (32) steps, and four chunks of
-        # loads stay in flight (float64 [10000, 1000]: 79 us with 32 bytes, 65 with 64, 59 with 128; with wider strips
-        # the longer segments lose: float64 [4096, 4096] 41 -> 45 us)
-        seg_vectors = SKEW_SEG_VECTORS_NARROW if STRIP <= 8 else SKEW_SEG_VECTORS
-        if sets is None and STRIP <= 8:
-            sets = 4
+        # there a lane owns 128 bytes of rows, so that a hand-over is paid once per 16 (32) steps (float64
+        # [10000, 1000] without separate movers: 79 us with 32 bytes, 65 with 64, 59 with 128; with wider strips the
+        # longer segments lose: float64 [4096, 4096] 41 -> 45 us)
+        seg_vectors = SKEW_SEG_VECTORS_NARROW if narrow else SKEW_SEG_VECTORS
     seg = seg_vectors * per                         # rows a lane owns per phase
     rc = SKEW_GROUP * seg                           # rows per chunk
+    if movers is None:
+        movers = SKEW_MOVERS if STRIP <= SKEW_MOVERS_MAX_STRIP else 0
+    if movers and (movers % WAVE or movers % STRIP or (rc // per) % (movers // STRIP) or
+                   SCAN_THREADS + movers > 1024):
+        movers = 0
+    if sets is None:
+        # chunks of loads in flight.  With separate movers two are enough and more lose (float32 [10000, 1000]: 33 us
+        # with two, 37 with four, 55 with eight: neighbouring strips share the cache lines of a row, and the further
+        # the workgroups run ahead of each other the more often a line is fetched twice); without them the narrow
+        # strips take four
+        sets = 2 if movers else 4 if narrow else SKEW_SETS
+    BLOCK = SCAN_THREADS + movers
+    MOVE = movers or BLOCK                          # threads that move data
+    NBUF = 3 if movers else 2
     seg_stride = seg + per                          # a segment and its padding vector (bank conflicts)
     line_stride = SKEW_GROUP * seg_stride + per     # a line and its padding vector
     num_chunks = (p.length + rc - 1) // rc
     strips = (p.inner + STRIP - 1) // STRIP
-    rows_per_pass = BLOCK // STRIP                  # rows covered by one load instruction of the workgroup
+    rows_per_pass = MOVE // STRIP                   # vectors of a line covered by one load instruction of the movers
     ipt = rc // rows_per_pass                       # elements each thread moves per chunk
     vpt = ipt // per                                # ... as 128-bit vectors of consecutive rows of one line
     sets = max(2, min(int(sets or SKEW_SETS), 16, max(2, num_chunks)))
@@ -463,7 +485,7 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None):
         a('    OVL_DECLARE_MATH_TABLES();')
     a('    // tile[buffer][line][row]: a line holds the %d rows of a chunk as 16 segments of %d rows, each followed by one' % (rc, seg))
     a('    // spare vector, and one more at its end')
-    a('    __shared__ __attribute__((aligned(16))) %s tile[2][%d][%d];' % (ctype, STRIP, line_stride))
+    a('    __shared__ __attribute__((aligned(16))) %s tile[%d][%d][%d];' % (ctype, NBUF, STRIP, line_stride))
     # A strip narrower than a 128-byte line shares the lines of every row with its neighbours.  Workgroups go to the
     # eight XCDs (each with its own L2) in turn, so neighbouring strips are given to workgroups 8 apart: they land on
     # one XCD at about the same time and the line is fetched from memory once (float64 [10000, 1000] in strips of 8
@@ -486,7 +508,12 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None):
     a('    const %s* __restrict__ gin = in%d + obase;' % (ctype, p.x.io_index))
     a('    %s* __restrict__ gout = out%d + obase;' % (ctype, p.out.io_index))
     a('')
-    a('    // Moving data: thread t owns line t %% %d of rows t / %d, t / %d + %d, ... of every chunk (%d elements).' % (
+    if movers:
+        a('    // Threads %d and up move data, the others scan.' % SCAN_THREADS)
+        a('    const uint32_t mt = threadIdx.x - %du;' % SCAN_THREADS)
+    else:
+        a('    const uint32_t mt = threadIdx.x;')
+    a('    // Moving data: thread mt owns line mt %% %d of vectors mt / %d, mt / %d + %d, ... of every chunk (%d elements).' % (
         STRIP, STRIP, STRIP, rows_per_pass, ipt))
     a('    // An element that does not exist (past the last row, past the last line) is replaced by the nearest one that')
     a('    // does: it is loaded, and later stored, a second time with the same value.  Without conditions around the')
@@ -494,12 +521,12 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None):
     a('    // those of the chunks after it stay in flight (with conditional stores it waited for all but the last dozen')
     a('    // requests: float64 [10000, 1000] 264 us).')
     a('    const uint32_t lines_here = (%du - c0 < %du) ? %du - c0 : %du;' % (p.inner, STRIP, p.inner, STRIP))
-    a('    const uint32_t mc = (threadIdx.x %% %du < lines_here) ? threadIdx.x %% %du : lines_here - 1u;' % (STRIP, STRIP))
-    a('    const uint32_t mv = threadIdx.x / %du;               // first of the vectors (%d consecutive rows) the thread owns' % (
+    a('    const uint32_t mc = (mt %% %du < lines_here) ? mt %% %du : lines_here - 1u;' % (STRIP, STRIP))
+    a('    const uint32_t mv = mt / %du;                        // first of the vectors (%d consecutive rows) the thread owns' % (
         STRIP, per))
     a('    struct MoverRegs { %s v[%d]; };' % (vname, vpt))
     a('    auto chunk_row = [&](uint32_t k, uint32_t i, uint32_t u) -> uint32_t {     // clamped to the chunk\'s last row')
-    a('        const uint32_t r = (mv + i * %du) * %du + u;' % (BLOCK // STRIP, per))
+    a('        const uint32_t r = (mv + i * %du) * %du + u;' % (rows_per_pass, per))
     a('        const uint32_t rows_here = (%du - k * %du < %du) ? %du - k * %du : %du;' % (
         p.length, rc, rc, p.length, rc, rc))
     a('        return r < rows_here ? r : rows_here - 1u;')
@@ -508,8 +535,8 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None):
         line_stride // per))
     a('    // number, so eight of them cover all banks; 64-bit accesses at that stride ran into 8-way conflicts: 257 us)')
     a('    auto lds_at = [&](uint32_t k, uint32_t i) -> %s* {' % vname)
-    a('        const uint32_t r = (mv + i * %du) * %du;' % (BLOCK // STRIP, per))
-    a('        return reinterpret_cast<%s*>(&tile[k %% 2u][mc][(r / %du) * %du + r %% %du]);' % (vname, seg, seg_stride, seg))
+    a('        const uint32_t r = (mv + i * %du) * %du;' % (rows_per_pass, per))
+    a('        return reinterpret_cast<%s*>(&tile[k %% %du][mc][(r / %du) * %du + r %% %du]);' % (vname, NBUF, seg, seg_stride, seg))
     a('    };')
     a('    auto issue_loads = [&](uint32_t k, MoverRegs& regs) {')
     a('        #pragma unroll')
@@ -531,10 +558,10 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None):
     a('        MoverRegs regs;')
     a('        #pragma unroll')
     a('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
-    a('            const uint32_t word = mv + i * %du;' % (BLOCK // STRIP))
+    a('            const uint32_t word = mv + i * %du;' % rows_per_pass)
     a('            const uint32_t r = (word < last / %du ? word : last / %du) * %du;' % (per, per, per))
-    a('            regs.v[i] = *reinterpret_cast<const %s*>(&tile[k %% 2u][mc][(r / %du) * %du + r %% %du]);' % (
-        vname, seg, seg_stride, seg))
+    a('            regs.v[i] = *reinterpret_cast<const %s*>(&tile[k %% %du][mc][(r / %du) * %du + r %% %du]);' % (
+        vname, NBUF, seg, seg_stride, seg))
     a('        }')
     a('        #pragma unroll')
     a('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
@@ -543,7 +570,7 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None):
     a('            for (uint32_t u = 1; u < %du; ++u) of_last = (last %% %du == u) ? regs.v[i][u] : of_last;' % (per, per))
     a('            #pragma unroll')
     a('            for (uint32_t u = 0; u < %du; ++u) {' % per)
-    a('                const uint32_t r = (mv + i * %du) * %du + u;' % (BLOCK // STRIP, per))
+    a('                const uint32_t r = (mv + i * %du) * %du + u;' % (rows_per_pass, per))
     a('                __builtin_nontemporal_store(r <= last ? regs.v[i][u] : of_last,')
     a('                                            gout + (uint64_t)(k * %du + (r <= last ? r : last)) * %dull + mc);' % (
         rc, p.inner))
@@ -575,12 +602,16 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None):
     a('#define OVL_SCAN_STEP(row) { %s = (%s)(row); %s }' % (counter_name, counter_type, ' '.join(body)))
     a('    // one chunk: in phase p every lane runs the recurrence over its rows from the state it holds and hands its')
     a('    // final state to its right neighbour; after phase p lanes 0..p are exact')
-    a('    auto scan_chunk = [&](uint32_t k) {')
-    a('        %s* segp = &tile[k %% 2u][sl][part * %du];' % (ctype, seg_stride))
-    a('        %s set[%d], ov[%d];' % (vname, seg_vectors, seg_vectors))
+    a('    struct Segment { %s v[%d]; };' % (vname, seg_vectors))
+    a('    auto fetch_segment = [&](uint32_t k, Segment& segment) {')
+    a('        const %s* segp = &tile[k %% %du][sl][part * %du];' % (ctype, NBUF, seg_stride))
     a('        #pragma unroll')
-    a('        for (uint32_t w = 0; w < %du; ++w) set[w] = *reinterpret_cast<const %s*>(segp + w * %du);' % (
+    a('        for (uint32_t w = 0; w < %du; ++w) segment.v[w] = *reinterpret_cast<const %s*>(segp + w * %du);' % (
         seg_vectors, vname, per))
+    a('    };')
+    a('    auto scan_segment = [&](uint32_t k, const Segment& segment) {')
+    a('        %s* segp = &tile[k %% %du][sl][part * %du];' % (ctype, NBUF, seg_stride))
+    a('        %s ov[%d];' % (vname, seg_vectors))
     a('        const uint32_t row0 = k * %du + part * %du;' % (rc, seg))
     a('        const bool first_row = k == 0u && part == 0u;')
     a('        #pragma unroll')
@@ -589,7 +620,7 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None):
         a('            %s = carry_%s;' % (name, name))
     a('            #pragma unroll')
     a('            for (uint32_t w = 0; w < %du; ++w) {' % seg_vectors)
-    a('                const %s xv = set[w];' % vname)
+    a('                const %s xv = segment.v[w];' % vname)
     a('                #pragma unroll')
     a('                for (uint32_t u = 0; u < %du; ++u) {' % per)
     a('                    if (w == 0u && u == 0u && first_row) ov[0][0] = first_out;')
@@ -606,33 +637,96 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None):
     a('        for (uint32_t w = 0; w < %du; ++w) *reinterpret_cast<%s*>(segp + w * %du) = ov[w];' % (
         seg_vectors, vname, per))
     a('    };')
+    a('    auto scan_chunk = [&](uint32_t k) {')
+    a('        Segment segment;')
+    a('        fetch_segment(k, segment);')
+    a('        scan_segment(k, segment);')
+    a('    };')
     a('')
     a('    // %d register sets keep %d chunks of loads in flight: chunk j travels through set j %% %d' % (sets, sets, sets))
     a('    MoverRegs sets[%d];' % sets)
-    for j in range(min(sets, num_chunks)):
-        a('    issue_loads(%du, sets[%d]);' % (j, j))
-    a('    write_lds(0u, sets[0]);')
-    if sets < num_chunks:
-        a('    issue_loads(%du, sets[0]);' % sets)
-    a('    __syncthreads();')
-    a('    // step k: chunk k is scanned in place; then its results go out while chunk k + 1 comes into the other buffer')
-    a('    auto step = [&](uint32_t k, MoverRegs& regs) {')
-    a('        scan_chunk(k);')
-    a('        __syncthreads();')
-    a('        store_chunk(k);')
-    a('        if (k + 1u < %du) write_lds(k + 1u, regs);' % num_chunks)
-    a('        if (k + 1u + %du < %du) issue_loads(k + 1u + %du, regs);' % (sets, num_chunks, sets))
-    a('        __syncthreads();')
-    a('    };')
     full = num_chunks // sets
-    if full:
-        a('    #pragma unroll 1')
-        a('    for (uint32_t k0 = 0; k0 < %du; k0 += %du) {' % (full * sets, sets))
-        for d in range(sets):
-            a('        step(k0 + %du, sets[%d]);' % (d, (d + 1) % sets))
+    if movers:
+        # Three buffers rotate: while chunk k is scanned in place, the movers bring chunk k + 1 into the next buffer and
+        # take the results of chunk k - 1 out of the one before; one barrier per chunk.  (A fourth buffer, the movers one
+        # chunk further ahead and the scanning wavefronts reading the segments of chunk k + 1 into a second register
+        # set before they start on chunk k gained 0.4 us of 40 on float64 [10000, 1000]: not kept.)
+        ahead = 1
+        a('    if (threadIdx.x >= %du) {' % SCAN_THREADS)
+        for j in range(min(sets, num_chunks)):
+            a('        issue_loads(%du, sets[%d]);' % (j, j))
+        for j in range(ahead):
+            if j < num_chunks:
+                a('        write_lds(%du, sets[%d]);' % (j, j % sets))
+                if j + sets < num_chunks:
+                    a('        issue_loads(%du, sets[%d]);' % (j + sets, j % sets))
+            a('        __syncthreads();')
+        # Step k: chunk k + ahead goes to LDS, its register set is refilled with chunk k + ahead + sets, chunk k - 1 goes
+        # out.  The steps in which all three happen run in a loop without conditions; the first step and the last ones
+        # are written out.  (With the conditions inside the loop the compiler merges the paths that skip the loads and
+        # stores into its count of outstanding requests and then waits for all of them before every write to LDS:
+        # float64 [10000, 1000] 40 us.)
+        def emit_step(k, indent, k_static=None):
+            # k: the chunk index as source text; k_static: its value when known here
+            regs = 'sets[%d]' % ((k_static + ahead) % sets) if k_static is not None else None
+            if k_static is None or k_static + ahead < num_chunks:
+                a(indent + 'write_lds(%s + %du, %s);' % (k, ahead, regs or 'REGS'))
+            if k_static is None or k_static + ahead + sets < num_chunks:
+                a(indent + 'issue_loads(%s + %du, %s);' % (k, ahead + sets, regs or 'REGS'))
+            if k_static is None or k_static >= 1:
+                a(indent + 'store_chunk(%s - 1u);' % k)
+            a(indent + '__syncthreads();')
+        # (the loop is entered after one full round of complete steps, so that the requests outstanding at its entry are
+        # those outstanding at its end: otherwise the compiler counts with the fewer of the two)
+        steady_first = 1 + sets
+        steady_end = max(steady_first, num_chunks - ahead - sets)       # steps [steady_first, steady_end) are complete
+        groups = (steady_end - steady_first) // sets
+        for k in range(0, min(steady_first, num_chunks)):
+            emit_step('%du' % k, '        ', k)
+        if groups:
+            a('        #pragma unroll 1')
+            a('        for (uint32_t k0 = %du; k0 < %du; k0 += %du) {' % (steady_first, steady_first + groups * sets, sets))
+            for d in range(sets):
+                a('            write_lds(k0 + %du, sets[%d]);' % (d + ahead, (steady_first + d + ahead) % sets))
+                a('            issue_loads(k0 + %du, sets[%d]);' % (d + ahead + sets, (steady_first + d + ahead) % sets))
+                a('            store_chunk(k0 + %du - 1u);' % d)
+                a('            __syncthreads();')
+            a('        }')
+        for k in range(steady_first + groups * sets, num_chunks):
+            emit_step('%du' % k, '        ', k)
+        a('        store_chunk(%du);' % (num_chunks - 1))
+        a('    } else {')
+        a('        __syncthreads();')
+        a('        #pragma unroll 1')
+        a('        for (uint32_t k = 0; k < %du; ++k) {' % num_chunks)
+        a('            scan_chunk(k);')
+        a('            __syncthreads();')
+        a('        }')
         a('    }')
-    for k in range(full * sets, num_chunks):
-        a('    step(%du, sets[%d]);' % (k, (k + 1) % sets))
+    else:
+        for j in range(min(sets, num_chunks)):
+            a('    issue_loads(%du, sets[%d]);' % (j, j))
+        a('    write_lds(0u, sets[0]);')
+        if sets < num_chunks:
+            a('    issue_loads(%du, sets[0]);' % sets)
+        a('    __syncthreads();')
+        a('    // step k: chunk k is scanned in place; then its results go out while chunk k + 1 comes into the other buffer')
+        a('    auto step = [&](uint32_t k, MoverRegs& regs) {')
+        a('        scan_chunk(k);')
+        a('        __syncthreads();')
+        a('        store_chunk(k);')
+        a('        if (k + 1u < %du) write_lds(k + 1u, regs);' % num_chunks)
+        a('        if (k + 1u + %du < %du) issue_loads(k + 1u + %du, regs);' % (sets, num_chunks, sets))
+        a('        __syncthreads();')
+        a('    };')
+        if full:
+            a('    #pragma unroll 1')
+            a('    for (uint32_t k0 = 0; k0 < %du; k0 += %du) {' % (full * sets, sets))
+            for d in range(sets):
+                a('        step(k0 + %du, sets[%d]);' % (d, (d + 1) % sets))
+            a('    }')
+        for k in range(full * sets, num_chunks):
+            a('    step(%du, sets[%d]);' % (k, (k + 1) % sets))
     a('#undef OVL_SCAN_STEP')
     a('#undef OVL_SCAN_IN')
     a('#undef OVL_SCAN_OUT')

@@ -978,6 +978,10 @@ TEMPLATE_VARIANTS = [
     ('c3_colscan_shapes', {'template': 'colskew', 'scan_strip': 4, 'scan_sets': 3}),
     ('c3_colscan_shapes', {'template': 'colskew', 'scan_strip': 16, 'scan_sets': 2}),
     ('c3_colscan_shapes', {'template': 'colskew', 'scan_width': 4, 'scan_sets': 5}),
+    ('c3_colscan_shapes', {'template': 'colskew', 'scan_movers': 0}),
+    ('c3_colscan_shapes', {'template': 'colskew', 'scan_movers': 512, 'scan_sets': 3}),
+    ('c3_colscan_shapes', {'template': 'colskew', 'scan_sets': 5}),
+    ('c3_colscan_shapes', {'template': 'colskew', 'scan_movers': 128, 'scan_strip': 16}),
     ('c3_colscan_shapes', {'template': 'colscan'}),
     ('c3_colscan_shapes', {'template': 'colscan', 'scan_rows': 32, 'scan_batch': 2}),
     ('c3_colscan_shapes', {'template': 'colscan', 'scan_sets': 3}),

@@ -91,7 +91,10 @@ def test_template_selection():
     assert template(cumsum(np.zeros((48, 1024), np.float32), axis=0))['template'] == 'map'
     # (up to 32768 lines: sixteen lanes per line, strips of 8 to 64 lines for about 256 workgroups)
     col = template(cumsum(np.zeros((1000, 200), np.float64), axis=0))
-    assert col['template'] == 'colskew' and col['blocks_needed'] == 25 and col['block'] == 128
+    # (strips of 8 lines: two scanning wavefronts and four that only move data)
+    assert col['template'] == 'colskew' and col['blocks_needed'] == 25 and col['block'] == 128 + 256
+    old = template(cumsum(np.zeros((1000, 200), np.float64), axis=0), {'scan_movers': 0})
+    assert old['template'] == 'colskew' and old['block'] == 128
     mid = template(cumsum(np.zeros((3, 500, 96), np.float32), axis=1))
     assert mid['template'] == 'colskew' and mid['blocks_needed'] == 3 * 12
     wide = template(cumsum(np.zeros((200, 16384), np.float32), axis=0))
