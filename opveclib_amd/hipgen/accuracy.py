@@ -68,11 +68,13 @@ IDIOM_DOMAIN = {'sigmoid': (-16.0, 64.0), 'log1p': (2.0 ** -10, 2.0 ** 64), 'exp
 
 #: narrower argument ranges on which shorter forms of the once-rounded routines hold the same bound (also compared
 #: with the formulas on every argument): for 2^-4 <= x < 1 the sum 1 + x has a known exponent (`ovl_log1p_unit`), up
-#: to 0.68 the exponential's table entry needs no exponent (`ovl_expm1_small`).  About a tenth fewer instructions in
-#: the 8-op chain; that kernel runs at the board's power limit, so its time follows the instruction count
-#: (143-147 -> 133-137 us on one box).
+#: to 0.68 the exponential's table entry needs no exponent (`ovl_expm1_small`), from -1 on the sigmoid's exponential
+#: needs no second term for the rounding of its scaled argument (`ovl_sigmoid_small`).  About a tenth fewer
+#: instructions in the 8-op chain; that kernel runs at the board's power limit, so its time follows the instruction
+#: count (143-147 -> 133-137 us on one box).
 NARROW_DOMAIN = {'log1p': (2.0 ** -4, float(np.nextafter(np.float32(1.0), np.float32(0.0)))),
-                 'expm1': (2.0 ** -12, float(np.float32(0.68)))}
+                 'expm1': (2.0 ** -12, float(np.float32(0.68))),
+                 'sigmoid': (-1.0, 64.0)}
 
 
 def in_narrow_domain(kind, seen):

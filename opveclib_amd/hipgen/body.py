@@ -402,7 +402,7 @@ class BodyEmitter(object):
                 fcn = {'sigmoid': 'ovl_sigmoid_ulp2', 'log1p': 'ovl_log1p_direct_nan' if seen.nan else 'ovl_log1p_direct',
                        'expm1': 'ovl_expm1_direct'}[kind]
                 if accuracy.in_narrow_domain(kind, seen):
-                    fcn = {'log1p': 'ovl_log1p_unit', 'expm1': 'ovl_expm1_small'}[kind]
+                    fcn = {'log1p': 'ovl_log1p_unit', 'expm1': 'ovl_expm1_small', 'sigmoid': 'ovl_sigmoid_small'}[kind]
                 put('float ' + name + ' = ' + fcn + '(' + names[x] + ');')
             elif code == lang.DIVIDE and node.dtype == lang.FLOAT32 and self._is_constant_one(ops[0]):
                 # 1/x: the verified correctly rounded reciprocal (ovl_math.h) instead of the general division, in

@@ -934,6 +934,7 @@ ULP2_CLIPPED_FORMULAS = [
     ('expm1', 0.001, 0.68, 'ovl_expm1_small'),
     ('expm1', -1.0, 0.5, 'ovl_expf_inrange'),
     ('sigmoid', -15.0, 60.0, 'ovl_sigmoid_ulp2'),
+    ('sigmoid', -1.0, 60.0, 'ovl_sigmoid_small'),
 ]
 ULP2_CLIPPED_COUNT = 1 << 20
 

@@ -36,7 +36,8 @@ namespace {
 
 enum { FN_EXP = 0, FN_LOG = 1, FN_TANH = 2, FN_RECIP = 3, FN_DEVICE_LIBRARY_EXP = 4,
        FN_FAST_EXP = 5, FN_FAST_LOG = 6, FN_FAST_TANH = 7, FN_FAST_RECIP = 8,
-       FN_LOG1P_DIRECT = 9, FN_EXPM1_DIRECT = 10, FN_SIGMOID_ULP2 = 11, FN_LOG1P_UNIT = 12, FN_EXPM1_SMALL = 13 };
+       FN_LOG1P_DIRECT = 9, FN_EXPM1_DIRECT = 10, FN_SIGMOID_ULP2 = 11, FN_LOG1P_UNIT = 12, FN_EXPM1_SMALL = 13,
+       FN_SIGMOID_SMALL = 14 };
 
 __global__ void __launch_bounds__(256) eval_kernel(int fn, uint32_t first, uint32_t count, float* __restrict__ out) {
     OVL_DECLARE_MATH_TABLES();
@@ -57,6 +58,7 @@ __global__ void __launch_bounds__(256) eval_kernel(int fn, uint32_t first, uint3
         else if (fn == FN_SIGMOID_ULP2) y = ovl_sigmoid_ulp2(x);
         else if (fn == FN_LOG1P_UNIT) y = ovl_log1p_unit(x);
         else if (fn == FN_EXPM1_SMALL) y = ovl_expm1_small(x);
+        else if (fn == FN_SIGMOID_SMALL) y = ovl_sigmoid_small(x);
         else y = expf(x);            // the device math library's own expf: differs from the host's in the last place
         out[i] = y;
     }
@@ -173,7 +175,7 @@ float host_sigmoid_formula(float x) {
 }
 
 float host_value(int fn, float x) {
-    if (fn == FN_SIGMOID_ULP2) return host_sigmoid_formula(x);
+    if (fn == FN_SIGMOID_ULP2 || fn == FN_SIGMOID_SMALL) return host_sigmoid_formula(x);
     if (fn == FN_LOG1P_DIRECT || fn == FN_LOG1P_UNIT) return host_log1p_formula(x);
     if (fn == FN_EXPM1_DIRECT || fn == FN_EXPM1_SMALL) return host_expm1_formula(x);
     if (fn == FN_EXP || fn == FN_DEVICE_LIBRARY_EXP || fn == FN_FAST_EXP) return expf(x);

@@ -93,8 +93,8 @@ def test_generated_text_names_the_chosen_routines():
     outs = workloads.chain8_outputs(Spec((64, 256)), Spec((64, 256)), Spec((1,)))
     op, = workloads.fused_operators(outs)
     text = hipgen.generate(op, 'f' + '0' * 56, {'math': 'ulp2'}).source
-    # behind the tanh and the sigmoid the arguments of log1p and expm1 lie in the narrow domains
-    for wanted in ('ovl_fast_tanhf(', 'ovl_sigmoid_ulp2(', 'ovl_log1p_unit(', 'ovl_expm1_small('):
+    # behind the tanh and the sigmoid the arguments of sigmoid, log1p and expm1 lie in the narrow domains
+    for wanted in ('ovl_fast_tanhf(', 'ovl_sigmoid_small(', 'ovl_log1p_unit(', 'ovl_expm1_small('):
         assert wanted in text
     assert 'ovl_tanhf(' not in text
     exact = hipgen.generate(op, 'f' + '0' * 56, None).source
@@ -127,6 +127,9 @@ def test_narrow_routines_only_where_the_range_allows():
     assert 'ovl_expm1_small(' in text([expm1(clip_op(0.001, 0.68)(x))[0]])
     large = text([expm1(clip_op(0.001, 0.7)(x))[0]])
     assert 'ovl_expm1_direct(' in large and '_small' not in large
+    assert 'ovl_sigmoid_small(' in text([stdops.sigmoid(clip_op(-1.0, 5.0)(x))])
+    below = text([stdops.sigmoid(clip_op(-1.5, 5.0)(x))])
+    assert 'ovl_sigmoid_ulp2(' in below and '_small' not in below
 
 
 def test_formula_results_are_bounded_by_the_function():

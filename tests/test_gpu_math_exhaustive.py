@@ -113,14 +113,14 @@ def _bits(value):
     return struct.unpack('<I', struct.pack('<f', value))[0]
 
 
-@pytest.mark.parametrize('kind', ['sigmoid', 'log1p', 'expm1', 'log1p_unit', 'expm1_small'])
+@pytest.mark.parametrize('kind', ['sigmoid', 'log1p', 'expm1', 'log1p_unit', 'expm1_small', 'sigmoid_small'])
 def test_formula_routines_within_two_ulp_of_the_reference_formulas(lib, kind):
     """Every float32 argument of the domain the code generator allows (hipgen/accuracy.py: IDIOM_DOMAIN, and
     NARROW_DOMAIN for the shorter forms `_unit` / `_small`)."""
     from opveclib_amd.hipgen import accuracy
     lib.ovl_exh_ulp_in_range.argtypes = [ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32] + \
         [ctypes.POINTER(ctypes.c_uint64)] * 3 + [ctypes.POINTER(ctypes.c_uint32)] * 2
-    narrow = {'log1p_unit': 'log1p', 'expm1_small': 'expm1'}.get(kind)
+    narrow = {'log1p_unit': 'log1p', 'expm1_small': 'expm1', 'sigmoid_small': 'sigmoid'}.get(kind)
     lo, hi = accuracy.NARROW_DOMAIN[narrow] if narrow else accuracy.IDIOM_DOMAIN[kind]
     bound = accuracy.TOLERANCE if narrow else accuracy.ROUTINE_ULPS[kind]
     # ranges of bit patterns of one sign each: consecutive patterns are consecutive floats
@@ -129,7 +129,7 @@ def test_formula_routines_within_two_ulp_of_the_reference_formulas(lib, kind):
     for first, last in spans:
         compared, differing, beyond = ctypes.c_uint64(0), ctypes.c_uint64(0), ctypes.c_uint64(0)
         largest, where = ctypes.c_uint32(0), ctypes.c_uint32(0)
-        fn = {'log1p': 9, 'expm1': 10, 'sigmoid': 11, 'log1p_unit': 12, 'expm1_small': 13}[kind]
+        fn = {'log1p': 9, 'expm1': 10, 'sigmoid': 11, 'log1p_unit': 12, 'expm1_small': 13, 'sigmoid_small': 14}[kind]
         err = lib.ovl_exh_ulp_in_range(fn, first, last, min(16, os.cpu_count() or 1), ctypes.byref(compared),
                                        ctypes.byref(differing), ctypes.byref(beyond), ctypes.byref(largest),
                                        ctypes.byref(where))

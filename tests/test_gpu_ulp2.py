@@ -105,6 +105,7 @@ def test_every_stage_on_the_exact_stage_inputs_at_full_size(chain_inputs):
     # (the chain's stage ranges lie in the narrow domains: the shorter forms of the once-rounded routines)
     assert any('ovl_log1p_unit' in text for text in sources)
     assert any('ovl_expm1_small' in text for text in sources)
+    assert any('ovl_sigmoid_small' in text for text in sources)
     assert any('ovl_fast_tanhf' in text for text in sources)
 
 
