@@ -662,27 +662,27 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
                     a('        issue_loads(%du, sets[%d]);' % (j + sets, j % sets))
             a('        __syncthreads();')
         # Step k: chunk k + ahead goes to LDS, its register set is refilled with chunk k + ahead + sets, chunk k - 1 goes
-        # out.  The steps in which all three happen run in a loop without conditions; the first step and the last ones
+        # out.  The steps in which all three happen run in a loop without conditions; the first steps and the last ones
         # are written out.  (With the conditions inside the loop the compiler merges the paths that skip the loads and
-        # stores into its count of outstanding requests and then waits for all of them before every write to LDS:
-        # float64 [10000, 1000] 40 us.)
-        def emit_step(k, indent, k_static=None):
-            # k: the chunk index as source text; k_static: its value when known here
-            regs = 'sets[%d]' % ((k_static + ahead) % sets) if k_static is not None else None
-            if k_static is None or k_static + ahead < num_chunks:
-                a(indent + 'write_lds(%s + %du, %s);' % (k, ahead, regs or 'REGS'))
-            if k_static is None or k_static + ahead + sets < num_chunks:
-                a(indent + 'issue_loads(%s + %du, %s);' % (k, ahead + sets, regs or 'REGS'))
-            if k_static is None or k_static >= 1:
-                a(indent + 'store_chunk(%s - 1u);' % k)
-            a(indent + '__syncthreads();')
+        # stores into its count of outstanding requests and then waits for all of them before every write to LDS.
+        # On float64 [10000, 1000] both forms take 40 us, because there the scanning wavefronts set the pace; the
+        # loads in flight are what keeps the movers ahead of them.)
+        def emit_step(k):
+            regs = 'sets[%d]' % ((k + ahead) % sets)
+            if k + ahead < num_chunks:
+                a('        write_lds(%du, %s);' % (k + ahead, regs))
+            if k + ahead + sets < num_chunks:
+                a('        issue_loads(%du, %s);' % (k + ahead + sets, regs))
+            if k >= 1:
+                a('        store_chunk(%du);' % (k - 1))
+            a('        __syncthreads();')
         # (the loop is entered after one full round of complete steps, so that the requests outstanding at its entry are
         # those outstanding at its end: otherwise the compiler counts with the fewer of the two)
         steady_first = 1 + sets
         steady_end = max(steady_first, num_chunks - ahead - sets)       # steps [steady_first, steady_end) are complete
         groups = (steady_end - steady_first) // sets
         for k in range(0, min(steady_first, num_chunks)):
-            emit_step('%du' % k, '        ', k)
+            emit_step(k)
         if groups:
             a('        #pragma unroll 1')
             a('        for (uint32_t k0 = %du; k0 < %du; k0 += %du) {' % (steady_first, steady_first + groups * sets, sets))
@@ -693,7 +693,7 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
                 a('            __syncthreads();')
             a('        }')
         for k in range(steady_first + groups * sets, num_chunks):
-            emit_step('%du' % k, '        ', k)
+            emit_step(k)
         a('        store_chunk(%du);' % (num_chunks - 1))
         a('    } else {')
         a('        __syncthreads();')
