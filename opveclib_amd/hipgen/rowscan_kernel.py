@@ -137,22 +137,29 @@ def _emit_movers(src, p, ctype, vname, vec, chunk, rpb, num_chunks, lds_column=N
     vectors_per_row = chunk // vec
     tile_vectors = rpb * vectors_per_row
     vpt = (tile_vectors + MOVERS - 1) // MOVERS      # vectors each mover thread handles per chunk
-    src.append('    // Movers (threads 64..255): every thread owns up to %d vectors of each chunk.  A vector that does not exist' % vpt)
-    src.append('    // (past the tile or past the last row) is redirected to the thread\'s first vector for loading and skipped')
-    src.append('    // when writing, so the loops are branch free and all loads of a chunk are in flight together.')
+    ragged_rows = p.rows % rpb != 0
+    src.append('    // Movers (threads 64..255): every thread owns %d vectors of each chunk.  A vector that does not exist (past' % vpt)
+    src.append('    // the tile, past the last row) is replaced by the nearest one that does: it is loaded, written to LDS and')
+    src.append('    // later stored a second time with the same value.  No memory instruction sits under a condition, so the')
+    src.append('    // compiler can count them and waits for the loads of exactly the chunk it needs while those of the chunks')
+    src.append('    // after it stay in flight.')
     src.append('    struct MoverRegs { %s v[%d]; };' % (vname, vpt))
-    src.append('    auto slot = [&](uint32_t m, uint32_t i, uint32_t& r, uint32_t& cv) -> bool {')
-    src.append('        const uint32_t v = m + i * %du;' % MOVERS)
+    if ragged_rows:
+        src.append('    const uint32_t rows_here = (%du - row0 < %du) ? %du - row0 : %du;' % (p.rows, rpb, p.rows, rpb))
+    src.append('    auto slot = [&](uint32_t m, uint32_t i, uint32_t& r, uint32_t& cv) {')
+    src.append('        uint32_t v = m + i * %du;' % MOVERS)
+    if vpt * MOVERS > tile_vectors:
+        src.append('        v = v < %du ? v : %du;' % (tile_vectors, tile_vectors - 1))
     src.append('        r = v / %du; cv = (v %% %du) * %du;' % (vectors_per_row, vectors_per_row, vec))
-    src.append('        return v < %du && row0 + r < %du;' % (tile_vectors, p.rows))
+    if ragged_rows:
+        src.append('        r = r < rows_here ? r : rows_here - 1u;')
     src.append('    };')
     src.append('    auto issue_loads = [&](uint32_t k, uint32_t m, MoverRegs& regs) {')
     src.append('        #pragma unroll')
     src.append('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
     src.append('            uint32_t r, cv;')
-    src.append('            if (!slot(m, i, r, cv)) { r = 0; cv = 0; }')
-    src.append('            const uint32_t gr = (row0 + r < %du) ? row0 + r : %du;' % (p.rows, p.rows - 1))
-    src.append('            const uint64_t g = (uint64_t)gr * %dull + k * %du + cv;' % (p.length, chunk))
+    src.append('            slot(m, i, r, cv);')
+    src.append('            const uint64_t g = (uint64_t)(row0 + r) * %dull + k * %du + cv;' % (p.length, chunk))
     src.append('            regs.v[i] = __builtin_nontemporal_load(reinterpret_cast<const %s*>(gin + g));' % vname)
     src.append('        }')
     src.append('    };')
@@ -160,8 +167,8 @@ def _emit_movers(src, p, ctype, vname, vec, chunk, rpb, num_chunks, lds_column=N
     src.append('        #pragma unroll')
     src.append('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
     src.append('            uint32_t r, cv;')
-    src.append('            if (slot(m, i, r, cv)) *reinterpret_cast<%s*>(&tile[k %% 3u][r][%s]) = regs.v[i];' % (
-        vname, lds_column('cv')))
+    src.append('            slot(m, i, r, cv);')
+    src.append('            *reinterpret_cast<%s*>(&tile[k %% 3u][r][%s]) = regs.v[i];' % (vname, lds_column('cv')))
     src.append('        }')
     src.append('    };')
     src.append('    auto store_chunk = [&](uint32_t k, uint32_t m) {')
@@ -169,45 +176,61 @@ def _emit_movers(src, p, ctype, vname, vec, chunk, rpb, num_chunks, lds_column=N
     src.append('        #pragma unroll')
     src.append('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
     src.append('            uint32_t r, cv;')
-    src.append('            if (!slot(m, i, r, cv)) { r = 0; cv = 0; }')
-    src.append('            regs.v[i] = *reinterpret_cast<const %s*>(&tile[k %% 3u][r][%s]);' % (
-        vname, lds_column('cv')))
+    src.append('            slot(m, i, r, cv);')
+    src.append('            regs.v[i] = *reinterpret_cast<const %s*>(&tile[k %% 3u][r][%s]);' % (vname, lds_column('cv')))
     src.append('        }')
     src.append('        #pragma unroll')
     src.append('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
     src.append('            uint32_t r, cv;')
-    src.append('            if (slot(m, i, r, cv)) {')
-    src.append('                const uint64_t g = (uint64_t)(row0 + r) * %dull + k * %du + cv;' % (p.length, chunk))
-    src.append('                __builtin_nontemporal_store(regs.v[i], reinterpret_cast<%s*>(gout + g));' % vname)
-    src.append('            }')
+    src.append('            slot(m, i, r, cv);')
+    src.append('            const uint64_t g = (uint64_t)(row0 + r) * %dull + k * %du + cv;' % (p.length, chunk))
+    src.append('            __builtin_nontemporal_store(regs.v[i], reinterpret_cast<%s*>(gout + g));' % vname)
     src.append('        }')
     src.append('    };')
     src.append('')
     src.append('    if (threadIdx.x >= %du) {' % WAVE)
     src.append('        const uint32_t m = threadIdx.x - %du;' % WAVE)
-    src.append('        // Two register sets keep two chunks of loads in flight: while chunk k is being scanned, chunk k+1 is')
-    src.append('        // written to LDS from the set requested two iterations ago, and chunk k+3 is requested into that set.')
-    src.append('        MoverRegs set_a, set_b;')
-    src.append('        issue_loads(0u, m, set_a);')
-    src.append('        write_lds(0u, m, set_a);')
-    if num_chunks > 1:
-        src.append('        issue_loads(1u, m, set_b);')
-    if num_chunks > 2:
-        src.append('        issue_loads(2u, m, set_a);')
+    src.append('        // Two register sets keep two chunks of loads in flight: chunk j travels through set j %% 2, is requested two')
+    src.append('        // steps before it is written to LDS, and is written one step before the scanning wavefront needs it.')
+    src.append('        MoverRegs sets[2];')
+    sets = 2
+    for j in range(min(sets, num_chunks)):
+        src.append('        issue_loads(%du, m, sets[%d]);' % (j, j))
+    src.append('        write_lds(0u, m, sets[0]);')
+    if sets < num_chunks:
+        src.append('        issue_loads(%du, m, sets[0]);' % sets)
     src.append('        __syncthreads();')
-    src.append('        auto step = [&](uint32_t k, MoverRegs& regs) {')
-    src.append('            if (k + 1u < %du) write_lds(k + 1u, m, regs);' % num_chunks)
-    src.append('            if (k + 3u < %du) issue_loads(k + 3u, m, regs);' % num_chunks)
-    src.append('            if (k >= 1u) store_chunk(k - 1u, m);')
-    src.append('            __syncthreads();')
-    src.append('        };')
-    src.append('        #pragma unroll 1')
-    src.append('        for (uint32_t k = 0; k + 1u < %du; k += 2u) {' % num_chunks)
-    src.append('            step(k, set_b);             // chunks 1, 3, 5, ... travel through set_b')
-    src.append('            step(k + 1u, set_a);        // chunks 2, 4, 6, ... travel through set_a')
-    src.append('        }')
-    if num_chunks % 2 == 1:
-        src.append('        step(%du, set_b);' % (num_chunks - 1))
+
+    # Step k: chunk k is being scanned; chunk k + 1 goes to LDS, its register set is refilled with chunk k + 3, chunk
+    # k - 1 goes out.  The steps in which all three happen run in a loop without conditions, entered after one full
+    # round of them (the compiler counts outstanding requests along the cheapest path into a join: with the first
+    # and last steps' conditions inside the loop it waits for every outstanding request before each write to LDS).
+    def emit_step(k):
+        regs = 'sets[%d]' % ((k + 1) % sets)
+        if k + 1 < num_chunks:
+            src.append('        write_lds(%du, m, %s);' % (k + 1, regs))
+        if k + 1 + sets < num_chunks:
+            src.append('        issue_loads(%du, m, %s);' % (k + 1 + sets, regs))
+        if k >= 1:
+            src.append('        store_chunk(%du, m);' % (k - 1))
+        src.append('        __syncthreads();')
+    steady_first = 1 + sets
+    steady_end = max(steady_first, num_chunks - 1 - sets)
+    groups = (steady_end - steady_first) // sets
+    for k in range(0, min(steady_first, num_chunks)):
+        emit_step(k)
+    if groups:
+        src.append('        #pragma unroll 1')
+        src.append('        for (uint32_t k0 = %du; k0 < %du; k0 += %du) {' % (steady_first, steady_first + groups * sets, sets))
+        for d in range(sets):
+            regs = 'sets[%d]' % ((steady_first + d + 1) % sets)
+            src.append('            write_lds(k0 + %du, m, %s);' % (d + 1, regs))
+            src.append('            issue_loads(k0 + %du, m, %s);' % (d + 1 + sets, regs))
+            src.append('            store_chunk(k0 + %du - 1u, m);' % d)
+            src.append('            __syncthreads();')
+        src.append('        }')
+    for k in range(steady_first + groups * sets, num_chunks):
+        emit_step(k)
     src.append('        store_chunk(%du, m);' % (num_chunks - 1))
 
 
