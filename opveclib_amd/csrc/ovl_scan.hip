@@ -57,7 +57,9 @@ struct op_product {
 
 template <typename T, int VEC> struct vec_of { typedef T type __attribute__((ext_vector_type(VEC))); };
 
-// cols must be a multiple of 16 * VEC * WIDTH * DEPTH; x and out 16-byte aligned.
+// cols must be a multiple of 16 * VEC * WIDTH (a group) and at least DEPTH groups; x and out 16-byte aligned.  A row
+// whose number of groups is not a multiple of DEPTH ends in up to DEPTH - 1 single groups, requested at the start and
+// held in registers until then.
 template <typename T, typename OP, int VEC, int WIDTH, int DEPTH>
 __global__ void __launch_bounds__(BLOCK)
 skewed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, uint32_t cols) {
@@ -75,8 +77,22 @@ skewed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, 
     T* __restrict__ gout = out + (uint64_t)row * cols + part * RUN;
     const uint32_t num_batches = cols / BATCH_COLS;
     const uint32_t last_batch = num_batches - 1u;
+    const uint32_t num_groups = cols / GROUP_COLS;
+    const uint32_t tail = num_groups - num_batches * (uint32_t)DEPTH;      // 0 ... DEPTH - 1 groups after the batches
+    constexpr uint32_t TAIL_MAX = DEPTH > 1 ? DEPTH - 1 : 1;
 
     vec q[2][DEPTH][WIDTH];
+    // (a tail group that does not exist is requested as the row's last group once more and never used)
+    vec qt[TAIL_MAX][WIDTH];
+    if constexpr (DEPTH > 1) {
+#pragma unroll
+        for (uint32_t j = 0; j < TAIL_MAX; ++j) {
+            const uint32_t g = num_batches * (uint32_t)DEPTH + j < num_groups ? num_batches * (uint32_t)DEPTH + j : num_groups - 1u;
+#pragma unroll
+            for (uint32_t w = 0; w < (uint32_t)WIDTH; ++w)
+                qt[j][w] = *reinterpret_cast<const vec*>(gin + (uint64_t)g * GROUP_COLS + w * VEC);
+        }
+    }
 #pragma unroll
     for (uint32_t s = 0; s < 2u; ++s) {
         const uint32_t b = s < num_batches ? s : last_batch;
@@ -88,28 +104,33 @@ skewed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, 
     }
     T carry = OP::template start<T>();
 
+    // One group: in phase p every lane runs the recurrence over its columns from the carried state it holds and hands
+    // its final state to its right neighbour; after the last phase all lanes are exact and the last lane's state goes
+    // round to lane 0.
+    auto scan_group = [&](const vec (&in)[WIDTH], vec (&ov)[WIDTH]) {
+        T acc = carry;
+#pragma unroll
+        for (uint32_t phase = 0; phase < GROUP; ++phase) {
+            acc = carry;
+#pragma unroll
+            for (uint32_t w = 0; w < (uint32_t)WIDTH; ++w) {
+#pragma unroll
+                for (uint32_t u = 0; u < (uint32_t)VEC; ++u) {
+                    acc = OP::apply(acc, in[w][u]);
+                    ov[w][u] = acc;
+                }
+            }
+            carry = ovl_dpp_move<OVL_DPP_ROW_SHR1>(carry, acc);
+        }
+        carry = ovl_dpp_move<OVL_DPP_ROW_ROR1>(carry, acc);
+    };
+
     // One batch: scan the DEPTH groups held in register set s, store them, refill the set with batch b + 2.
     auto process = [&](auto set, uint32_t b) {
         constexpr uint32_t s = decltype(set)::value;
         vec ov[DEPTH][WIDTH];
 #pragma unroll
-        for (uint32_t j = 0; j < (uint32_t)DEPTH; ++j) {
-            T acc = carry;
-#pragma unroll
-            for (uint32_t phase = 0; phase < GROUP; ++phase) {
-                acc = carry;
-#pragma unroll
-                for (uint32_t w = 0; w < (uint32_t)WIDTH; ++w) {
-#pragma unroll
-                    for (uint32_t u = 0; u < (uint32_t)VEC; ++u) {
-                        acc = OP::apply(acc, q[s][j][w][u]);
-                        ov[j][w][u] = acc;
-                    }
-                }
-                carry = ovl_dpp_move<OVL_DPP_ROW_SHR1>(carry, acc);
-            }
-            carry = ovl_dpp_move<OVL_DPP_ROW_ROR1>(carry, acc);
-        }
+        for (uint32_t j = 0; j < (uint32_t)DEPTH; ++j) scan_group(q[s][j], ov[j]);
         // The scheduling fences keep the memory traffic of a batch together, after its arithmetic, and no load is
         // moved ahead of the last use of the registers it fills.
         __builtin_amdgcn_sched_barrier(0);
@@ -139,6 +160,20 @@ skewed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, 
         process(set1(), b0 + 1u);
     }
     if (b0 < num_batches) process(set0(), b0);
+    if constexpr (DEPTH > 1) {
+        // the single groups that end the row (the same number in every wavefront: the branches are uniform)
+#pragma unroll
+        for (uint32_t j = 0; j < TAIL_MAX; ++j) {
+            if (j < tail) {
+                vec ov[WIDTH];
+                scan_group(qt[j], ov);
+#pragma unroll
+                for (uint32_t w = 0; w < (uint32_t)WIDTH; ++w)
+                    __builtin_nontemporal_store(ov[w], reinterpret_cast<vec*>(
+                        gout + (uint64_t)(num_batches * (uint32_t)DEPTH + j) * GROUP_COLS + w * VEC));
+            }
+        }
+    }
 }
 
 // LDS-fed lane-skewed scan, for 8-byte elements: a scan of float64 rows runs at the latency of its recurrence, and in
@@ -325,7 +360,8 @@ int scan(const char* who, const T* x, uint32_t rows, uint32_t cols, T* out, void
     if (fed) {
     } else if (aligned && cols % GROUP_COLS == 0) {
         const dim3 grid((rows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK);
-        if (cols % (GROUP_COLS * DEPTH) == 0)
+        // (rows of fewer than DEPTH groups: one group per request)
+        if (cols >= GROUP_COLS * DEPTH)
             hipLaunchKernelGGL((skewed_scan_kernel<T, OP, VEC, WIDTH, DEPTH>), grid, block, 0, stream, x, out, rows, cols);
         else
             hipLaunchKernelGGL((skewed_scan_kernel<T, OP, VEC, WIDTH, 1>), grid, block, 0, stream, x, out, rows, cols);

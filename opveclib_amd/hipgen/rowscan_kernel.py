@@ -764,7 +764,7 @@ def _for_slot(text, slot):
     if slot == 0:
         return text
     suffix = '_r%d' % slot
-    text = re.sub(r'\b(carry_e\d+|e\d+|position|row_raw|row|gin|gout|q\d+|ov|xv|first_out|OVL_SCAN_STEP)\b',
+    text = re.sub(r'\b(carry_e\d+|e\d+|position|row_raw|row|gin|gout|q\d+|qt|ov|xv|first_out|OVL_SCAN_STEP)\b',
                   lambda m: m.group(1) + suffix, text)
     return text
 
@@ -799,8 +799,9 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
     if depth is None:
         # measured on MI355X: request bursts of 1 KiB per row are the fastest
         depth = max(1, 4 // width)
-    while num_groups % depth != 0:
-        depth //= 2
+    # (a row whose number of groups is not a multiple of the burst ends in one shorter burst; before, the burst was
+    # halved until it divided the row, and float32 [4096, 16448], 257 groups, took 177 us against 85 us for 16384)
+    depth = max(1, min(depth, num_groups))
 
     rank = len(info.workgroup_shape)
     pos_exprs = []
@@ -864,12 +865,14 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
     # on the loads only 90 us, on neither 102 us
     batch = depth
     num_batches = num_groups // batch
+    tail = num_groups % batch               # groups of the shorter burst that ends the row
     batch_cols = batch * group_cols
 
-    def request(regs, batch_expr):
-        """All loads of one batch, back to back: every row is read in runs of batch * 256 bytes."""
+    def request(regs, batch_expr, nb=None):
+        """All loads of one batch (of nb groups), back to back: every row is read in runs of batch * 256 bytes."""
+        nb = nb or batch
         lines = ['        #pragma unroll',
-                 '        for (uint32_t j = 0; j < %du; ++j)' % batch,
+                 '        for (uint32_t j = 0; j < %du; ++j)' % nb,
                  '            #pragma unroll',
                  '            for (uint32_t w = 0; w < %du; ++w)' % width]
         if 'l' in nt:
@@ -880,12 +883,13 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
                 regs, vname, batch_expr, batch_cols, group_cols, vec))
         emit(lines)
 
-    def process(regs, batch_expr, refill_expr):
+    def process(regs, batch_expr, refill_expr, nb=None):
+        nb = nb or batch
         src.append('        {')
         src.append('        const uint32_t b = %s;' % batch_expr)
-        emit(['        %s ov[%d][%d];' % (vname, batch, width)])
+        emit(['        %s ov[%d][%d];' % (vname, nb, width)])
         src.append('        #pragma unroll')
-        src.append('        for (uint32_t j = 0; j < %du; ++j) {' % batch)
+        src.append('        for (uint32_t j = 0; j < %du; ++j) {' % nb)
         src.append('            const uint32_t col0 = b * %du + j * %du + part * %du;' % (batch_cols, group_cols, vec * width))
         src.append('            const bool first_column = (j == 0u) && (b == 0u) && (part == 0u);')
         src.append('            #pragma unroll')
@@ -913,7 +917,7 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
         src.append('        // batch * 256 bytes per row, and no load is moved ahead of the last use of the registers it fills.')
         src.append('        __builtin_amdgcn_sched_barrier(0);')
         lines = ['        #pragma unroll',
-                 '        for (uint32_t j = 0; j < %du; ++j)' % batch,
+                 '        for (uint32_t j = 0; j < %du; ++j)' % nb,
                  '            #pragma unroll',
                  '            for (uint32_t w = 0; w < %du; ++w)' % width]
         if 's' in nt:
@@ -931,9 +935,14 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
     sets = max(2, min(sets or 2, num_batches)) if num_batches > 1 else 1
     src.append('    // %d register sets of %d groups each: one is consumed while the others are in flight' % (sets, batch))
     emit(['    %s %s;' % (vname, ', '.join('q%d[%d][%d]' % (k, batch, width) for k in range(sets)))])
+    if tail:
+        src.append('    // ... and the %d groups that end the row, requested now and held until the end' % tail)
+        emit(['    %s qt[%d][%d];' % (vname, tail, width)])
     src.append('    {')
-    for k in range(sets):
+    for k in range(sets if num_batches else 0):
         request('q%d' % k, '%du' % k)
+    if tail:
+        request('qt', '%du' % num_batches, tail)
     src.append('    }')
     src.append('    // first column: the statements the worker runs before its loop, in every lane')
     for slot in slots:
@@ -964,6 +973,10 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
     for k in range(num_batches % sets):
         src.append('    {')
         process('q%d' % k, '%du' % (rounds * sets + k), None)
+        src.append('    }')
+    if tail:
+        src.append('    {')
+        process('qt', '%du' % num_batches, None, tail)
         src.append('    }')
     for slot in slots:
         src.append('#undef %s' % _for_slot('OVL_SCAN_STEP', slot))

@@ -153,14 +153,19 @@ def c3_cumprod_f64(rng, shape=(24, 1024)):
 
 
 def c3_rowscan_shapes(rng):
-    """Row-scan template corner cases: partial last workgroup, several rows per workgroup, rank 3, int32, max."""
+    """Row-scan template corner cases: partial last workgroup, several rows per workgroup, rank 3, int32, max, rows that
+    end in a shorter burst."""
     outs = [cumsum(rng.standard_normal((515, 64), dtype=np.float32), axis=1)[0],
             cumprod(uniform(rng, 0.9, 1.1, (259, 128), np.float64), axis=1)[0],
             cumsum(rng.standard_normal((4, 70, 128), dtype=np.float32), axis=2)[0],
             cumsum(rng.integers(-1000, 1000, size=(20, 192)).astype(np.int32), axis=1)[0],
             accumulate(rng.standard_normal((7, 256), dtype=np.float32),
                        inner_fcn=lambda acc, x: ovl.maximum(acc, x), axis=1)[0],
-            cumsum(rng.standard_normal(4096, dtype=np.float32))[0]]
+            cumsum(rng.standard_normal(4096, dtype=np.float32))[0],
+            # rows whose number of groups is not a multiple of the request burst end in a shorter burst
+            cumsum(rng.standard_normal((9, 320), dtype=np.float32), axis=1)[0],
+            cumprod(uniform(rng, 0.9, 1.1, (5, 448), np.float32), axis=1)[0],
+            cumsum(rng.standard_normal((6, 320)), axis=1)[0]]
     return outs
 
 

@@ -16,7 +16,9 @@ from opveclib_amd.examples import cumsum, cumprod
 pytestmark = pytest.mark.gpu
 
 SHAPES = [(48, 1024), (7, 256), (5, 64), (3, 192), (515, 64), (259, 128), (4, 70, 128), (5, 70), (7, 3), (1, 1),
-          (2, 4096), (4096,), (6, 1536), (1027, 512), (3, 5, 2048)]
+          (2, 4096), (4096,), (6, 1536), (1027, 512), (3, 5, 2048),
+          # rows whose number of 64-column groups is not a multiple of the request burst: 1, 2 and 3 groups over
+          (9, 320), (70, 384), (33, 448), (130, 16448)]
 
 
 def _data(rng, shape, dtype, kind):
