@@ -128,7 +128,7 @@ def generate(expression_dag, function_name, options=None):
                                                      options.get('scan_batch'), options.get('scan_sets'))
     elif options.get('vec') is None and template in ('auto', 'transpose') and tile_kernel.applicable(info) is not None:
         kernel_src, launch = tile_kernel.generate(info, kernel_name, options.get('tile_i'), options.get('tile_j'),
-                                                  options.get('nt', 'ls'))
+                                                  options.get('nt'))
     else:
         kernel_src, launch = map_kernel.generate(info, kernel_name, options.get('vec'), options.get('nt'),
                                                  options.get('grid_cap'), options.get('per_thread'))

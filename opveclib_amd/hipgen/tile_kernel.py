@@ -67,7 +67,9 @@ def applicable(info):
     return vec
 
 
-def generate(info, kernel_name, tile_i=None, tile_j=None, nt='ls'):
+def generate(info, kernel_name, tile_i=None, tile_j=None, nt=None):
+    nt_given = nt is not None
+    nt = 'ls' if nt is None else nt
     load_fn = 'OVL_LOAD_NT' if 'l' in nt else 'OVL_LOAD_PLAIN'
     store_fn = 'OVL_STORE_NT' if 's' in nt else 'OVL_STORE_PLAIN'
     vec = applicable(info)
@@ -163,6 +165,7 @@ def generate(info, kernel_name, tile_i=None, tile_j=None, nt='ls'):
         src.append('    OVL_DECLARE_MATH_TABLES();')
     for acc in tstores.values():
         src.append('    __shared__ %s %s[%d][%d];' % (CTYPE[acc.tensor.dtype], acc.reg, tile_j, tile_i + 1))
+    blocks_needed = tiles_i * tiles_j
     src.append('    const uint32_t num_tiles = %du;' % (tiles_i * tiles_j))
     src.append('    for (uint32_t tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {')
     src.append('        const uint32_t i0 = (tile / %du) * %du;' % (tiles_j, tile_i))
@@ -200,7 +203,15 @@ def generate(info, kernel_name, tile_i=None, tile_j=None, nt='ls'):
     src.append('            }')
     src.append('        }')
     src.append('        __syncthreads();')
-    # phase 2: rows of the LDS tile are runs along i
+    # phase 2: rows of the LDS tile are runs along i.  A transposed output row that is not a whole number of 128-byte
+    # lines long puts the runs a tile stores across line boundaries, and the rest of each line belongs to the tile's
+    # neighbour along i; with the non-temporal hint the two parts reach memory as partial lines (float32
+    # [16380, 16384]: 1085 us against 484 us for [16384, 16384]), without it they meet in the L2 (603 us; giving the
+    # two neighbours to workgroups on one XCD at the same time made it slower, 744 us).  For whole lines the hint is
+    # the faster form (484 against 494 us).
+    tstore_fn = store_fn
+    if not nt_given and any((rows * ITEMSIZE[acc.tensor.dtype]) % 128 != 0 for acc in tstores.values()):
+        tstore_fn = 'OVL_STORE_PLAIN'
     src.append('        const uint32_t oi = (threadIdx.x %% %du) * %du;' % (threads_per_col, vec))
     src.append('        #pragma unroll 1')
     src.append('        for (uint32_t oj = threadIdx.x / %du; oj < %du; oj += %du) {' % (
@@ -216,7 +227,7 @@ def generate(info, kernel_name, tile_i=None, tile_j=None, nt='ls'):
         src.append('                for (uint32_t lane = 0; lane < %du; ++lane) v_%s[lane] = %s[oj][oi + lane];' % (
             vec, acc.reg, acc.reg))
         src.append('                %s(v_%s, reinterpret_cast<%s*>(out%d + (%s)));' % (
-            store_fn, acc.reg, vname, acc.tensor.io_index, _index_expr(acc.aff, pos_names, wide)))
+            tstore_fn, acc.reg, vname, acc.tensor.io_index, _index_expr(acc.aff, pos_names, wide)))
     src.append('            }')
     src.append('        }')
     src.append('        __syncthreads();')
@@ -235,7 +246,7 @@ def generate(info, kernel_name, tile_i=None, tile_j=None, nt='ls'):
         'template': 'transpose',
         'vec': vec,
         'block': BLOCK,
-        'blocks_needed': tiles_i * tiles_j,
+        'blocks_needed': blocks_needed,
         'align': align,
         'vector_loads': len(loads) + len(unaligned),
         'vector_stores': len(stores) + len(tstores),

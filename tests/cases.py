@@ -1023,6 +1023,8 @@ TEMPLATE_VARIANTS = [
     ('odd_sizes', {'grid_cap': 1}),
     ('pad_crop', {'grid_cap': 2}),
     ('c5_variants', {'grid_cap': 2}),
+    ('c5_variants', {'nt': 'l'}),
+    ('c5_variants', {'nt': 'ls'}),
     ('c5_variants', {'template': 'map', 'grid_cap': 5}),
 ]
 
