@@ -159,7 +159,7 @@ def generate(expression_dag, function_name, options=None):
     grid = launch['blocks_needed']
     if launch['template'] in ('map', 'transpose'):
         # these kernels stride over what the grid does not cover
-        grid = min(grid, options.get('grid_cap') or MAX_GRID, MAX_GRID)
+        grid = min(grid, launch.get('grid_cap') or options.get('grid_cap') or MAX_GRID, MAX_GRID)
     elif grid > MAX_GRID:
         raise ValueError('%d workgroups: the %s template launches at most %d' % (grid, launch['template'], MAX_GRID))
     src.append('    uint32_t grid = %du;' % grid)

@@ -27,6 +27,7 @@ BLOCK = 256
 # largest grid the generated entry points launch: 2^24 - 1 workgroups of 256 threads keep the number of threads of a
 # launch, and with it gridDim.x * 256 inside the kernels, below 2^32
 MAX_GRID = (1 << 24) - 1
+SCALAR_TABLE_GRID = 4096        # workgroups of a one-element-per-thread kernel that copies the math tables
 
 
 class Access(object):
@@ -239,6 +240,12 @@ def generate(info, kernel_name, vec=None, nt=None, grid_cap=None, per_thread=Non
     src.append('extern "C" __global__ void __launch_bounds__(%d)' % BLOCK)
     src.append(kernel_name + '(' + ', '.join(args) + ') {')
     blocks_needed = (num_vectors + BLOCK * per_thread - 1) // (BLOCK * per_thread)
+    # One element per thread (a last dimension that is not a multiple of the vector width) and the LDS math tables: a
+    # workgroup that covers 256 elements would copy the tables for 256 elements' worth of work.  Such kernels get a
+    # grid of SCALAR_TABLE_GRID workgroups that stride over the tensor (the 8-op chain on float32 [8191, 8191]: 'ulp2'
+    # 284 -> 159 us, 'exact' 318 -> 266 us; with four elements per thread and more the single pass is the faster one).
+    if grid_cap is None and vec == 1 and info.uses_math_tables() and blocks_needed > SCALAR_TABLE_GRID:
+        grid_cap = SCALAR_TABLE_GRID
     # When the grid covers every vector (always, unless the workgroup has more than 2^32 - 256 workers at VEC = 1 or
     # the caller caps the grid) a thread runs its vectors without a loop.  Kernels that use the LDS math tables then
     # request their operands first and copy the tables (with the barrier that implies) while they are in flight,
@@ -334,6 +341,7 @@ def generate(info, kernel_name, vec=None, nt=None, grid_cap=None, per_thread=Non
         'per_thread': per_thread,
         'block': BLOCK,
         'blocks_needed': blocks_needed,
+        'grid_cap': grid_cap,
         'align': align,
         'vector_loads': len(loads) + len(unaligned),
         'vector_stores': len(stores),

@@ -69,6 +69,12 @@ def c2_chain(rng, shape=(96, 256)):
     return [chain8(a, b, s)[-1][0]]
 
 
+def c2_chain_odd(rng):
+    """The chain on a last dimension that leaves one element per thread, with more than 4096 workgroups' worth of
+    elements: the kernel then strides over the tensor with the math tables copied once per workgroup."""
+    return c2_chain(rng, shape=(1025, 1027))
+
+
 def c2_chain_stages(rng, shape=(96, 256)):
     a = uniform(rng, -1, 1, shape)
     b = uniform(rng, -1, 1, shape)
@@ -649,6 +655,7 @@ CASES = [
     Case('c1_shift', c1_shift_only),
     Case('c1_shift_expm1_log1p', c1_shift_expm1_log1p),
     Case('c2_chain', c2_chain, seed=2),
+    Case('c2_chain_odd', c2_chain_odd, seed=2),
     Case('c2_chain_stages', c2_chain_stages, seed=2),
     Case('c2_chain_special', c2_chain_special, seed=2),
     Case('bounded_mix', bounded_mix, seed=2),
