@@ -212,7 +212,10 @@ def c5_variants(rng):
     """Gather index that provably never wraps (dword-aligned vector loads), ragged tile edges, float64 tiles."""
     return (c5_gather_transpose(rng, (192, 320), stride=3) + c5_gather_transpose(rng, (68, 100), stride=5) +
             c5_gather_transpose(rng, (130, 66), stride=7, dtype=np.float64) +
-            c5_gather_transpose(rng, (6, 10), stride=1))
+            c5_gather_transpose(rng, (6, 10), stride=1) +
+            # extents that leave two elements, or one, per access
+            c5_gather_transpose(rng, (70, 102), stride=11) + c5_gather_transpose(rng, (67, 101), stride=3) +
+            c5_gather_transpose(rng, (35, 129), stride=2, dtype=np.float64))
 
 
 # ----------------------------------------------------------------------------------------------------------------------
