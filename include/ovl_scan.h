@@ -20,8 +20,9 @@
  * after sixteen such phases the group is exact and the last lane's state is the carry into the next group.  float64
  * rows whose length is a multiple of 512 columns run the same recurrence fed from LDS (three wavefronts of the
  * workgroup stream four rows through LDS, the fourth scans them, a lane owning 16 columns per phase), which pays the
- * hand-over between lanes four times less often.  Column counts that are not a multiple of the group (64 columns) or
- * unaligned tensors take a plain kernel with one lane per row.  The result is the same bits whichever kernel runs.
+ * hand-over between lanes four times less often.  The columns after a row's last whole group (64 columns) are
+ * scanned by one lane; rows that do not start on 16-byte boundaries are moved with unaligned vectors; rows shorter than
+ * one group take a plain kernel with one lane per row.  The result is the same bits whichever kernel runs.
  *
  * Conventions: tensor memory belongs to the caller and must be device accessible; `out` may not overlap `x`; the
  * functions enqueue one kernel on `hip_stream` (a hipStream_t; NULL is the default stream), return without

@@ -57,10 +57,32 @@ struct op_product {
 
 template <typename T, int VEC> struct vec_of { typedef T type __attribute__((ext_vector_type(VEC))); };
 
-// cols must be a multiple of 16 * VEC * WIDTH (a group) and at least DEPTH groups; x and out 16-byte aligned.  A row
-// whose number of groups is not a multiple of DEPTH ends in up to DEPTH - 1 single groups, requested at the start and
-// held in registers until then.
-template <typename T, typename OP, int VEC, int WIDTH, int DEPTH>
+// A vector as it lies in memory: on a 16-byte boundary, or (ALIGNED = false) only aligned like its elements.  (The
+// alignment is stated on a typedef at the place of the access: as a template argument it would be dropped.)
+template <bool ALIGNED, typename V, typename T>
+static __device__ __forceinline__ V load_vector(const T* p) {
+    if constexpr (ALIGNED) {
+        return *reinterpret_cast<const V*>(p);
+    } else {
+        typedef V unaligned __attribute__((aligned(alignof(T))));
+        return *reinterpret_cast<const unaligned*>(p);
+    }
+}
+template <bool ALIGNED, typename V, typename T>
+static __device__ __forceinline__ void store_vector(V value, T* p) {
+    if constexpr (ALIGNED) {
+        __builtin_nontemporal_store(value, reinterpret_cast<V*>(p));
+    } else {
+        typedef V unaligned __attribute__((aligned(alignof(T))));
+        __builtin_nontemporal_store(value, reinterpret_cast<unaligned*>(p));
+    }
+}
+
+// cols must be at least DEPTH groups of 16 * VEC * WIDTH columns.  A row whose number of groups is not a multiple of
+// DEPTH ends in up to DEPTH - 1 single groups, requested at the start and held in registers until then; the columns
+// after the last whole group are scanned by lane 0 of the row's sixteen lanes, one at a time.  ALIGNED: every row of x
+// and out starts on a 16-byte boundary; otherwise vectors are moved with the alignment of their elements.
+template <typename T, typename OP, int VEC, int WIDTH, int DEPTH, bool ALIGNED>
 __global__ void __launch_bounds__(BLOCK)
 skewed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, uint32_t cols) {
     typedef typename vec_of<T, VEC>::type vec;
@@ -90,7 +112,7 @@ skewed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, 
             const uint32_t g = num_batches * (uint32_t)DEPTH + j < num_groups ? num_batches * (uint32_t)DEPTH + j : num_groups - 1u;
 #pragma unroll
             for (uint32_t w = 0; w < (uint32_t)WIDTH; ++w)
-                qt[j][w] = *reinterpret_cast<const vec*>(gin + (uint64_t)g * GROUP_COLS + w * VEC);
+                qt[j][w] = load_vector<ALIGNED, vec>(gin + (uint64_t)g * GROUP_COLS + w * VEC);
         }
     }
 #pragma unroll
@@ -100,7 +122,7 @@ skewed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, 
         for (uint32_t j = 0; j < (uint32_t)DEPTH; ++j)
 #pragma unroll
             for (uint32_t w = 0; w < (uint32_t)WIDTH; ++w)
-                q[s][j][w] = *reinterpret_cast<const vec*>(gin + (uint64_t)b * BATCH_COLS + j * GROUP_COLS + w * VEC);
+                q[s][j][w] = load_vector<ALIGNED, vec>(gin + (uint64_t)b * BATCH_COLS + j * GROUP_COLS + w * VEC);
     }
     T carry = OP::template start<T>();
 
@@ -138,15 +160,14 @@ skewed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, 
         for (uint32_t j = 0; j < (uint32_t)DEPTH; ++j)
 #pragma unroll
             for (uint32_t w = 0; w < (uint32_t)WIDTH; ++w)
-                __builtin_nontemporal_store(ov[j][w], reinterpret_cast<vec*>(
-                    gout + (uint64_t)b * BATCH_COLS + j * GROUP_COLS + w * VEC));
+                store_vector<ALIGNED, vec>(ov[j][w], gout + (uint64_t)b * BATCH_COLS + j * GROUP_COLS + w * VEC);
         // past the end a set is refilled with the last batch again, which keeps the loop free of branches
         const uint32_t next = b + 2u < num_batches ? b + 2u : last_batch;
 #pragma unroll
         for (uint32_t j = 0; j < (uint32_t)DEPTH; ++j)
 #pragma unroll
             for (uint32_t w = 0; w < (uint32_t)WIDTH; ++w)
-                q[s][j][w] = *reinterpret_cast<const vec*>(gin + (uint64_t)next * BATCH_COLS + j * GROUP_COLS + w * VEC);
+                q[s][j][w] = load_vector<ALIGNED, vec>(gin + (uint64_t)next * BATCH_COLS + j * GROUP_COLS + w * VEC);
         __builtin_amdgcn_sched_barrier(0);
     };
     typedef std::integral_constant<uint32_t, 0> set0;
@@ -169,9 +190,18 @@ skewed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, 
                 scan_group(qt[j], ov);
 #pragma unroll
                 for (uint32_t w = 0; w < (uint32_t)WIDTH; ++w)
-                    __builtin_nontemporal_store(ov[w], reinterpret_cast<vec*>(
-                        gout + (uint64_t)(num_batches * (uint32_t)DEPTH + j) * GROUP_COLS + w * VEC));
+                    store_vector<ALIGNED, vec>(ov[w], gout + (uint64_t)(num_batches * (uint32_t)DEPTH + j) * GROUP_COLS + w * VEC);
             }
+        }
+    }
+    // the columns after the last whole group: lane 0 of the row holds the state that leaves it (gin and gout of that
+    // lane are the row itself)
+    if (part == 0u) {
+        T acc = carry;
+#pragma unroll 1
+        for (uint32_t column = num_groups * GROUP_COLS; column < cols; ++column) {
+            acc = OP::apply(acc, gin[column]);
+            gout[column] = acc;
         }
     }
 }
@@ -319,7 +349,7 @@ fed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, uin
     }
 }
 
-// Any shape, any alignment: one lane per row.
+// Rows shorter than one group of the kernels above: one lane per row.
 template <typename T, typename OP>
 __global__ void __launch_bounds__(BLOCK)
 row_per_lane_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, uint32_t cols) {
@@ -347,6 +377,7 @@ int scan(const char* who, const T* x, uint32_t rows, uint32_t cols, T* out, void
     constexpr int VEC = 16 / sizeof(T), WIDTH = sizeof(T) == 8 ? 2 : 1, DEPTH = 4 / WIDTH;
     constexpr uint32_t GROUP_COLS = GROUP * VEC * WIDTH;
     const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+    const bool rows_aligned = aligned && cols % VEC == 0;      // every row starts on a 16-byte boundary
     const dim3 block(BLOCK);
     bool fed = false;
     if constexpr (sizeof(T) == 8) {
@@ -358,13 +389,20 @@ int scan(const char* who, const T* x, uint32_t rows, uint32_t cols, T* out, void
         }
     }
     if (fed) {
-    } else if (aligned && cols % GROUP_COLS == 0) {
+    } else if (cols >= GROUP_COLS) {
         const dim3 grid((rows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK);
         // (rows of fewer than DEPTH groups: one group per request)
-        if (cols >= GROUP_COLS * DEPTH)
-            hipLaunchKernelGGL((skewed_scan_kernel<T, OP, VEC, WIDTH, DEPTH>), grid, block, 0, stream, x, out, rows, cols);
-        else
-            hipLaunchKernelGGL((skewed_scan_kernel<T, OP, VEC, WIDTH, 1>), grid, block, 0, stream, x, out, rows, cols);
+        if (cols >= GROUP_COLS * DEPTH) {
+            if (rows_aligned)
+                hipLaunchKernelGGL((skewed_scan_kernel<T, OP, VEC, WIDTH, DEPTH, true>), grid, block, 0, stream, x, out, rows, cols);
+            else
+                hipLaunchKernelGGL((skewed_scan_kernel<T, OP, VEC, WIDTH, DEPTH, false>), grid, block, 0, stream, x, out, rows, cols);
+        } else {
+            if (rows_aligned)
+                hipLaunchKernelGGL((skewed_scan_kernel<T, OP, VEC, WIDTH, 1, true>), grid, block, 0, stream, x, out, rows, cols);
+            else
+                hipLaunchKernelGGL((skewed_scan_kernel<T, OP, VEC, WIDTH, 1, false>), grid, block, 0, stream, x, out, rows, cols);
+        }
     } else {
         // (a launch has fewer than 2^32 threads)
         if (rows > 0xffffffffu - BLOCK)

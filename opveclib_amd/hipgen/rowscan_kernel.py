@@ -45,8 +45,9 @@ class ScanPlan(object):
         self.chunk = chunk
 
 
-def plan(info, rows_per_block=None, chunk=None):
-    """A ScanPlan when the DAG is a last-axis row scan this template can run, else None."""
+def plan(info, rows_per_block=None, chunk=None, need_chunk=True):
+    """A ScanPlan when the DAG is a last-axis row scan this template can run, else None.  ``need_chunk``: the LDS
+    templates stream rows in chunks that divide them; the lane-skewed scan does not."""
     forced_rows, forced_chunk = rows_per_block, chunk
     if len(info.inputs) != 1 or len(info.outputs) != 1:
         return None
@@ -119,7 +120,7 @@ def plan(info, rows_per_block=None, chunk=None):
                 3 * rows_per_block * (cand + vec) * itemsize <= LDS_BUDGET:
             chunk = cand
             break
-    if chunk is None:
+    if chunk is None and need_chunk:
         return None
     return ScanPlan(loop, counter, length, rows, x, out, vec, rows_per_block, chunk)
 
@@ -402,8 +403,10 @@ def _carried_state(info, p):
 
 def skew_plan(info):
     """The structural plan when the lane-skewed variant can run this DAG, else None."""
-    p = plan(info)
-    if p is None or p.length % (GROUP_LANES * p.vec) != 0:
+    # (a row need not be a whole number of groups of 16 * VEC columns, nor aligned: what is left after the last whole
+    # group is scanned by one lane, and rows that do not start on 16-byte boundaries are moved with unaligned vectors)
+    p = plan(info, need_chunk=False)
+    if p is None or p.length < GROUP_LANES * p.vec:
         return None
     body_nodes = [n for n in info.nodes if info.in_loop[n.idx]]
     if len(body_nodes) > SKEW_MAX_BODY:
@@ -435,7 +438,7 @@ FED_ROWS = WAVE // GROUP_LANES      # rows per workgroup: one group of sixteen l
 def fed_plan(info, width=None, chunk=None):
     """(ScanPlan, width, chunk) when the LDS-fed lane-skewed variant can run this DAG, else None."""
     p = skew_plan(info)
-    if p is None:
+    if p is None or p.length % (GROUP_LANES * p.vec) != 0:
         return None
     itemsize = ITEMSIZE[p.x.dtype]
     width = width or 8
@@ -782,10 +785,13 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
     # memory, 85 us with one and 111 us with two)
     if width is None:
         width = 2 if vec == 2 else 1
-    while width > 1 and p.length % (GROUP_LANES * vec * width) != 0:
+    while width > 1 and (p.length < GROUP_LANES * vec * width or
+                         (p.length % (GROUP_LANES * vec) == 0 and p.length % (GROUP_LANES * vec * width) != 0)):
         width //= 2
     group_cols = GROUP_LANES * vec * width
     num_groups = p.length // group_cols
+    tail_cols = p.length % group_cols           # columns after the last whole group: scanned by one lane per row
+    aligned = (p.length * ITEMSIZE[p.x.dtype]) % 16 == 0
     # interleave = rows per group of sixteen lanes.  With few rows there are fewer wavefronts than SIMDs and each runs
     # at the latency of its one recurrence; a lane group that carries two rows has two independent recurrences whose
     # additions and hand-overs fill each other's wait states.
@@ -838,6 +844,11 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
                 src.append(_for_slot(line, slot))
 
     src.append('typedef %s %s __attribute__((ext_vector_type(%d)));' % (ctype, vname, vec))
+    mname = vname
+    if not aligned:
+        # rows start wherever the one before ends: vectors in memory are only aligned like their elements
+        mname = vname + '_u'
+        src.append('typedef %s %s __attribute__((aligned(%d)));' % (vname, mname, ITEMSIZE[p.x.dtype]))
     src.append('')
     src.append('extern "C" __global__ void __launch_bounds__(%d)' % BLOCK)
     src.append('%s(const %s* __restrict__ in%d, %s* __restrict__ out%d) {' % (
@@ -877,10 +888,10 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
                  '            for (uint32_t w = 0; w < %du; ++w)' % width]
         if 'l' in nt:
             lines.append('                %s[j][w] = __builtin_nontemporal_load(reinterpret_cast<const %s*>(gin + (%s) * %du + j * %du + w * %du));' % (
-                regs, vname, batch_expr, batch_cols, group_cols, vec))
+                regs, mname, batch_expr, batch_cols, group_cols, vec))
         else:
             lines.append('                %s[j][w] = *(reinterpret_cast<const %s*>(gin + (%s) * %du + j * %du + w * %du));' % (
-                regs, vname, batch_expr, batch_cols, group_cols, vec))
+                regs, mname, batch_expr, batch_cols, group_cols, vec))
         emit(lines)
 
     def process(regs, batch_expr, refill_expr, nb=None):
@@ -922,10 +933,10 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
                  '            for (uint32_t w = 0; w < %du; ++w)' % width]
         if 's' in nt:
             lines.append('                __builtin_nontemporal_store(ov[j][w], reinterpret_cast<%s*>(gout + b * %du + j * %du + w * %du));' % (
-                vname, batch_cols, group_cols, vec))
+                mname, batch_cols, group_cols, vec))
         else:
             lines.append('                *(reinterpret_cast<%s*>(gout + b * %du + j * %du + w * %du)) = ov[j][w];' % (
-                vname, batch_cols, group_cols, vec))
+                mname, batch_cols, group_cols, vec))
         emit(lines)
         if refill_expr is not None:
             request(regs, refill_expr)
@@ -978,18 +989,41 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
         src.append('    {')
         process('qt', '%du' % num_batches, None, tail)
         src.append('    }')
+    if tail_cols:
+        # The columns after the last whole group: lane 0 of the row's sixteen lanes holds the state that leaves the
+        # last group and runs the worker's loop over them, one column at a time (fewer than %d columns).
+        for slot in slots:
+            src.append('#undef OVL_SCAN_OUT_R%d' % slot)
+            src.append('#undef OVL_SCAN_IN_R%d' % slot)
+            src.append('#define OVL_SCAN_IN_R%d tail_in' % slot)
+            src.append('#define OVL_SCAN_OUT_R%d(value) tail_out = (value)' % slot)
+        src.append('    if (part == 0u) {')
+        for slot in slots:
+            one = lambda lines: src.extend(_for_slot(line, slot) for line in lines)
+            src.append('        {')
+            one(['        %s = carry_%s;' % (name, name) for name, _ in state])
+            src.append('        #pragma unroll 1')
+            src.append('        for (uint32_t column = %du; column < %du; ++column) {' % (num_groups * group_cols, p.length))
+            one(['            const %s tail_in = gin[column];' % ctype,
+                 '            %s tail_out;' % ctype,
+                 '            OVL_SCAN_STEP(column)',
+                 '            gout[column] = tail_out;'])
+            src.append('        }')
+            src.append('        }')
+        src.append('    }')
     for slot in slots:
         src.append('#undef %s' % _for_slot('OVL_SCAN_STEP', slot))
         src.append('#undef OVL_SCAN_OUT_R%d' % slot)
         src.append('#undef OVL_SCAN_IN_R%d' % slot)
     src.append('}')
 
+    row_align = 16 if aligned else ITEMSIZE[p.x.dtype]
     launch = {
         'template': 'skewscan',
         'vec': vec,
         'block': BLOCK,
         'blocks_needed': (p.rows + rows_per_block - 1) // rows_per_block,
-        'align': {('in', p.x.io_index): 16, ('out', p.out.io_index): 16},
+        'align': {('in', p.x.io_index): row_align, ('out', p.out.io_index): row_align},
         'vector_loads': 1,
         'vector_stores': 1,
     }

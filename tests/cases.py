@@ -171,7 +171,16 @@ def c3_rowscan_shapes(rng):
             # rows whose number of groups is not a multiple of the request burst end in a shorter burst
             cumsum(rng.standard_normal((9, 320), dtype=np.float32), axis=1)[0],
             cumprod(uniform(rng, 0.9, 1.1, (5, 448), np.float32), axis=1)[0],
-            cumsum(rng.standard_normal((6, 320)), axis=1)[0]]
+            cumsum(rng.standard_normal((6, 320)), axis=1)[0],
+            # rows that are not a whole number of groups, and rows that do not start on 16-byte boundaries: the columns
+            # after the last whole group are scanned by one lane, the vectors are moved unaligned
+            cumsum(rng.standard_normal((7, 100), dtype=np.float32), axis=1)[0],
+            cumsum(rng.standard_normal((5, 1000)), axis=1)[0],
+            cumprod(uniform(rng, 0.9, 1.1, (9, 333), np.float32), axis=1)[0],
+            cumsum(rng.standard_normal((4, 131)), axis=1)[0],
+            cumsum(rng.integers(-1000, 1000, size=(6, 70)).astype(np.int32), axis=1)[0],
+            accumulate(rng.standard_normal((3, 2, 203), dtype=np.float32),
+                       inner_fcn=lambda acc, x: ovl.maximum(acc, x), axis=2)[0]]
     return outs
 
 

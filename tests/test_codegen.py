@@ -85,8 +85,14 @@ def test_template_selection():
     lds = template(cumsum(np.zeros((48, 1024), np.float32), axis=1), {'template': 'rowscan'})
     assert lds['template'] == 'rowscan' and lds['blocks_needed'] == 48
     assert template(cumsum(np.zeros((48, 1024), np.float32), axis=1), {'template': 'map'})['template'] == 'map'
-    # rows that are not a multiple of 64 long, other axes, and loop bodies with branches use the general template
-    assert template(cumsum(np.zeros((48, 1000), np.float32), axis=1))['template'] == 'map'
+    # rows that are not a whole number of groups of 64 columns end in columns scanned by one lane; rows that do not
+    # start on 16-byte boundaries are moved with unaligned vectors; rows shorter than one group, other axes and loop
+    # bodies with branches use the general template
+    ragged = template(cumsum(np.zeros((48, 1000), np.float32), axis=1))
+    assert ragged['template'] == 'skewscan' and ragged['align'] == {('in', 0): 16, ('out', 0): 16}
+    unaligned = template(cumsum(np.zeros((48, 1001), np.float32), axis=1))
+    assert unaligned['template'] == 'skewscan' and unaligned['align'] == {('in', 0): 4, ('out', 0): 4}
+    assert template(cumsum(np.zeros((48, 63), np.float32), axis=1))['template'] == 'map'
     # along another axis: a short axis keeps one worker per thread, a long one with few lines gets strips of 64 lines
     assert template(cumsum(np.zeros((48, 1024), np.float32), axis=0))['template'] == 'map'
     # (up to 32768 lines: sixteen lanes per line, strips of 8 to 64 lines for about 256 workgroups)

@@ -18,7 +18,9 @@ pytestmark = pytest.mark.gpu
 SHAPES = [(48, 1024), (7, 256), (5, 64), (3, 192), (515, 64), (259, 128), (4, 70, 128), (5, 70), (7, 3), (1, 1),
           (2, 4096), (4096,), (6, 1536), (1027, 512), (3, 5, 2048),
           # rows whose number of 64-column groups is not a multiple of the request burst: 1, 2 and 3 groups over
-          (9, 320), (70, 384), (33, 448), (130, 16448)]
+          (9, 320), (70, 384), (33, 448), (130, 16448),
+          # rows that are not whole groups, rows that do not start on 16-byte boundaries
+          (50, 1000), (7, 333), (100, 16383), (3, 4, 131)]
 
 
 def _data(rng, shape, dtype, kind):
