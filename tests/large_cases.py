@@ -51,6 +51,12 @@ def cases(make):
     a = make((131088, 32832), np.int32)     # 2^32 + 2^23.3 elements, 131088 workers
     yield 'cumsum int32 [131088, 32832]', cumsum(a, axis=1), lambda: torch.cumsum(a, 1, dtype=torch.int32)
 
+    a = make((70, 2 ** 21 + 64), np.int32)  # more than two million lines along the scanned axis
+    yield 'cumsum int32 [70, 2^21 + 64] along axis 0', cumsum(a, axis=0), lambda: torch.cumsum(a, 0, dtype=torch.int32)
+
+    a = make((3000, 70001), np.int32)       # rows that are neither whole groups of 64 columns nor 16-byte aligned
+    yield 'cumsum int32 [3000, 70001]', cumsum(a, axis=1), lambda: torch.cumsum(a, 1, dtype=torch.int32)
+
     rows, cols = 65536, 32768 + 256         # 2^31 + 2^24 workers, transposed store
     a, flat = make((rows, cols), np.float32), make(rows * cols, np.float32)
 

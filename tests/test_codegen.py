@@ -107,7 +107,10 @@ def test_template_selection():
     assert wide['template'] == 'colskew' and wide['blocks_needed'] == 256 and wide['block'] == 1024
     many = template(cumsum(np.zeros((200, 65536), np.float32), axis=0))
     assert many['template'] == 'colscan' and many['blocks_needed'] == 1024 and many['block'] == 1024
-    assert template(cumsum(np.zeros((128, 1 << 17), np.float32), axis=0))['template'] == 'map'    # enough wavefronts
+    more = template(cumsum(np.zeros((100, 100000), np.float32), axis=0))
+    assert more['template'] == 'colscan' and more['blocks_needed'] == 1563
+    assert template(cumsum(np.zeros((128, 1 << 17), np.float32), axis=0))['template'] == 'colscan'    # however many lines
+    assert template(cumsum(np.zeros((32, 1 << 17), np.float32), axis=0))['template'] == 'map'         # a short axis
     assert template(cases.dot(np.zeros((16, 64)), np.zeros((16, 64))))['template'] == 'map'
     # transposed store of a rank-2 workgroup: LDS tiles; the gather is one dword-aligned 128-bit load per thread
     tr = template(gather_transpose(np.zeros((192, 320), np.float32), np.zeros(192 * 320, np.float32),
