@@ -197,6 +197,26 @@ def c3_colscan_shapes(rng):
             cumsum(rng.standard_normal((10, 33)), axis=0)[0]]
 
 
+@ovl.operator()
+def _swap_last_two(x, scale=None):
+    """A batched transpose with some arithmetic and a second, untransposed output: the dimensions before the last two
+    of the workgroup are batches of the tile template."""
+    shape = list(x.shape)
+    swapped = ovl.output(shape[:-2] + [shape[-1], shape[-2]], x.dtype)
+    plain = ovl.output_like(x)
+    pos = ovl.position_in(x.shape)
+    value = x[pos] * scale
+    swapped[tuple(pos[k] for k in range(len(shape) - 2)) + (pos[len(shape) - 1], pos[len(shape) - 2])] = value
+    plain[pos] = value + 1
+    return swapped, plain
+
+
+def batched_transposes(rng):
+    return (all_outputs(_swap_last_two(rng.standard_normal((3, 70, 100), dtype=np.float32), scale=0.5)) +
+            all_outputs(_swap_last_two(rng.standard_normal((2, 3, 66, 34)), scale=2.0)) +
+            all_outputs(_swap_last_two(rng.integers(-100, 100, size=(5, 33, 35)).astype(np.int32), scale=3)))
+
+
 def c4_lstm(rng, batch=32, units=128):
     concat = rng.standard_normal((batch, 4 * units), dtype=np.float32)
     c = rng.standard_normal((batch, units), dtype=np.float32)
@@ -681,6 +701,7 @@ CASES = [
     Case('c4_lstm_grad', c4_lstm_grad, seed=4),
     Case('c5_gather_transpose', c5_gather_transpose, seed=5),
     Case('c5_variants', c5_variants, seed=5),
+    Case('batched_transposes', batched_transposes, seed=5),
     _simple('store_order', _store_order),
     _simple('clip', lambda rng: [clip(rng.random(1000), threshold1=0.1, threshold2=0.9)[0]]),
     _simple('limits_f32', lambda rng: [set_limits(np.array([0], np.float32))[0]]),
@@ -1043,6 +1064,8 @@ TEMPLATE_VARIANTS = [
     ('pad_crop', {'grid_cap': 2}),
     ('c5_variants', {'grid_cap': 2}),
     ('c5_variants', {'nt': 'l'}),
+    ('batched_transposes', {'template': 'map'}),
+    ('batched_transposes', {'tile_i': 16, 'tile_j': 64}),
     ('c5_variants', {'nt': 'ls'}),
     ('c5_variants', {'template': 'map', 'grid_cap': 5}),
 ]
