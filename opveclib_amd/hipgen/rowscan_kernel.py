@@ -598,6 +598,287 @@ def generate_fed(info, kernel_name, width=None, chunk=None):
     return '\n'.join(src) + '\n', launch
 
 
+# ---------------------------------------------------------------------------------------------------------------------
+# Row reductions: a worker that walks the last axis of its inputs with a loop-carried state and stores nothing inside the
+# loop (a dot product, a sum, a norm, a running extremum: the reference's opveclib/test/test_dot_product.py:27-45).
+#
+# In the one-worker-per-thread template the lanes of a wavefront read addresses a whole row apart (float32
+# [4096, 16384]: 1.9 ms for a row sum).  The order of a floating point reduction is part of its result, so the rows are
+# walked exactly as in the lane-skewed scan above: sixteen lanes per row, a lane owns VEC * width consecutive columns of
+# a group, runs the loop body over them from the state it holds and hands its state to its right neighbour; after
+# sixteen phases the group is done and the last lane's state is the carry into the next.  There is nothing to store
+# per column; the statements after the loop run once per row, in the lane that holds the final state.
+# ---------------------------------------------------------------------------------------------------------------------
+class ReducePlan(object):
+    def __init__(self, loop_item, end_idx, counter, start, length, rows, tensors, vec):
+        self.loop_item = loop_item
+        self.end_idx = end_idx          # the node that closes the loop
+        self.counter = counter
+        self.start = start              # first column the loop visits: 0, or 1 when the worker sets up with column 0
+        self.length = length            # row length of the tensors read in the loop
+        self.rows = rows
+        self.tensors = tensors          # the INPUT nodes read in the loop
+        self.vec = vec
+
+
+def reduce_plan(info):
+    """A ReducePlan when the DAG is a reduction along the last axis that `generate_reduce` can run, else None."""
+    loops = [item for item in info.tree if item.kind == 'loop']
+    if len(loops) != 1 or any(item.kind == 'if' for item in info.tree):
+        return None
+    loop = loops[0]
+    if any(inner.kind != 'stmt' for inner in loop.body):
+        return None
+    range_node = info.nodes[loop.node]
+    counter = range_node.ops[0]
+    if counter not in info.loop_counters:
+        return None
+    start, stop, step = (info._literal_int(o) for o in range_node.ops[1:])
+    if start not in (0, 1) or step != 1 or stop is None:
+        return None
+    length = stop
+    closers = [n.idx for n in info.nodes if n.idx > loop.node and n.code == lang.ENDRANGE and not info.in_loop[n.idx]]
+    if not closers:
+        return None
+    end_idx = min(closers)
+
+    rows = info.num_workers
+    rank = len(info.workgroup_shape)
+    stride = 1
+    wg_stride = [1] * rank
+    for k in range(rank - 2, -1, -1):
+        stride *= info.workgroup_shape[k + 1]
+        wg_stride[k] = stride
+    in_loop = dict((('p', k), length * wg_stride[k]) for k in range(rank) if info.workgroup_shape[k] > 1)
+    in_loop[('v', counter)] = 1
+    sig_loop = (tuple(sorted(in_loop.items())), 0)
+
+    tensors = []
+    for node, tensor, aff in info.tensor_accesses():
+        if not info.in_loop[node.idx]:
+            continue                    # before and after the loop: ordinary code of one lane
+        if node.code != lang.READ_TENSOR or tensor.code != lang.INPUT or aff is None or aff.signature() != sig_loop:
+            return None
+        if tensor.size != rows * length or tensor.dtype not in CTYPE:
+            return None
+        if tensor not in tensors:
+            tensors.append(tensor)
+    if not tensors or len(tensors) > 4:
+        return None
+    itemsize = ITEMSIZE[tensors[0].dtype]
+    if itemsize not in (4, 8) or any(ITEMSIZE[t.dtype] != itemsize for t in tensors):
+        return None
+    vec = 16 // itemsize
+    # (short rows stay with one worker per thread: float32 [100000, 100] 18 us there, 26 us here)
+    if length < 4 * GROUP_LANES * vec:
+        return None
+    if len([n for n in info.nodes if info.in_loop[n.idx]]) > SKEW_MAX_BODY:
+        return None
+    p = ReducePlan(loop, end_idx, counter, start, length, rows, tensors, vec)
+    state = _carried_state(info, p)
+    if not state or any(info.nodes[idx].dtype not in CTYPE for idx in state):
+        return None
+    return p
+
+
+def generate_reduce(info, kernel_name, depth=None, width=None):
+    p = reduce_plan(info)
+    assert p is not None
+    vec = p.vec
+    itemsize = 16 // vec
+    if width is None:
+        width = 2 if vec == 2 else 1
+    while width > 1 and p.length < GROUP_LANES * vec * width:
+        width //= 2
+    group_cols = GROUP_LANES * vec * width
+    num_groups = p.length // group_cols
+    tail_cols = p.length % group_cols
+    aligned = (p.length * itemsize) % 16 == 0
+    depth = max(1, min(depth or max(1, 4 // width), num_groups))
+    rows_per_wave = WAVE // GROUP_LANES
+    waves = BLOCK // WAVE
+    rows_per_block = rows_per_wave * waves
+
+    rank = len(info.workgroup_shape)
+    pos_exprs = []
+    stride = 1
+    strides = [1] * rank
+    for k in range(rank - 2, -1, -1):
+        stride *= info.workgroup_shape[k + 1]
+        strides[k] = stride
+    for k in range(rank):
+        expr = 'row'
+        if k > 0:
+            expr = '(row % ' + str(strides[k - 1]) + 'u)'
+        pos_exprs.append(expr + ' / ' + str(strides[k]) + 'u')
+    loop_tensors = dict((t.idx, t) for t in p.tensors)
+
+    def read_hook(node, tensor, index_name):
+        if info.in_loop[node.idx] and tensor.idx in loop_tensors:
+            return 'OVL_REDUCE_IN%d' % tensor.io_index
+        return None
+    emitter = BodyEmitter(info, pos_exprs, read_hook=read_hook, store_hook=None)
+    tagged = emitter.emit_tagged()
+    range_idx = p.loop_item.node
+    prologue = [t for i, t in tagged if i < range_idx]
+    body = [t.strip() for i, t in tagged if range_idx < i < p.end_idx]
+    epilogue = [t for i, t in tagged if i > p.end_idx]
+    counter_name = 'e' + str(p.counter)
+    counter_type = CTYPE[info.nodes[p.counter].dtype]
+    state = [('e' + str(idx), CTYPE[info.nodes[idx].dtype]) for idx in _carried_state(info, p)]
+
+    src = []
+    vnames = {}
+    for t in p.tensors:
+        ctype = CTYPE[t.dtype]
+        if ctype not in vnames:
+            vname = 'ovl_reduce_' + ctype.replace(' ', '_') + 'x%d' % vec
+            vnames[ctype] = vname
+            src.append('typedef %s %s __attribute__((ext_vector_type(%d)));' % (ctype, vname, vec))
+            if not aligned:
+                # rows start wherever the one before ends: vectors in memory are only aligned like their elements
+                src.append('typedef %s %s_u __attribute__((aligned(%d)));' % (vname, vname, itemsize))
+    src.append('')
+    args = ['const %s* __restrict__ in%d' % (CTYPE[info.inputs[i].dtype], i) for i in range(len(info.inputs))]
+    args += ['%s* __restrict__ out%d' % (CTYPE[info.outputs[i].dtype], i) for i in range(len(info.outputs))]
+    src.append('extern "C" __global__ void __launch_bounds__(%d)' % BLOCK)
+    src.append('%s(%s) {' % (kernel_name, ', '.join(args)))
+    if info.uses_math_tables():
+        src.append('    OVL_DECLARE_MATH_TABLES();')
+    src.append('    const uint32_t lane = threadIdx.x %% %du;' % WAVE)
+    src.append('    const uint32_t part = lane %% %du;              // which columns of a group this lane holds' % GROUP_LANES)
+    src.append('    // A wavefront wholly past the last row leaves; single lanes past it shadow the last row instead (all lanes')
+    src.append('    // must stay active for the lane-to-lane moves): they load, compute and store exactly what its owners do.')
+    src.append('    if ((blockIdx.x * %du + threadIdx.x / %du) * %du >= %du) return;' % (waves, WAVE, rows_per_wave, p.rows))
+    src.append('    const uint32_t row_raw = (blockIdx.x * %du + threadIdx.x / %du) * %du + lane / %du;' % (
+        waves, WAVE, rows_per_wave, GROUP_LANES))
+    src.append('    const uint32_t row = row_raw < %du ? row_raw : %du;' % (p.rows, p.rows - 1))
+    for t in p.tensors:
+        src.append('    const %s* __restrict__ gin%d = in%d + (uint64_t)row * %dull + part * %du;' % (
+            CTYPE[t.dtype], t.io_index, t.io_index, p.length, vec * width))
+    batch = depth
+    num_batches = num_groups // batch
+    tail = num_groups % batch
+    batch_cols = batch * group_cols
+
+    def request(k, batch_expr, nb, suffix):
+        for t in p.tensors:
+            vname = vnames[CTYPE[t.dtype]]
+            mname = vname if aligned else vname + '_u'
+            src.append('        #pragma unroll')
+            src.append('        for (uint32_t j = 0; j < %du; ++j)' % nb)
+            src.append('            #pragma unroll')
+            src.append('            for (uint32_t w = 0; w < %du; ++w)' % width)
+            src.append('                q%d%s[j][w] = *reinterpret_cast<const %s*>(gin%d + (%s) * %du + j * %du + w * %du);' % (
+                t.io_index, suffix, mname, t.io_index, batch_expr, batch_cols, group_cols, vec))
+
+    def process(suffix, batch_expr, refill_expr, nb):
+        src.append('        {')
+        src.append('        const uint32_t b = %s;' % batch_expr)
+        src.append('        #pragma unroll')
+        src.append('        for (uint32_t j = 0; j < %du; ++j) {' % nb)
+        src.append('            const uint32_t col0 = b * %du + j * %du + part * %du;' % (batch_cols, group_cols, vec * width))
+        src.append('            #pragma unroll')
+        src.append('            for (uint32_t phase = 0; phase < %du; ++phase) {' % GROUP_LANES)
+        for name, _ in state:
+            src.append('                %s = carry_%s;' % (name, name))
+        src.append('                #pragma unroll')
+        src.append('                for (uint32_t w = 0; w < %du; ++w) {' % width)
+        for t in p.tensors:
+            src.append('                    const %s xv%d = q%d%s[j][w];' % (
+                vnames[CTYPE[t.dtype]], t.io_index, t.io_index, suffix))
+        src.append('                    #pragma unroll')
+        src.append('                    for (uint32_t u = 0; u < %du; ++u) {' % vec)
+        if p.start == 1:
+            src.append('                        if (col0 + w * %du + u == 0u) continue;     // column 0: done before the loop' % vec)
+        src.append('                        OVL_REDUCE_STEP(col0 + w * %du + u)' % vec)
+        src.append('                    }')
+        src.append('                }')
+        for name, _ in state:
+            src.append('                carry_%s = ovl_dpp_move<OVL_DPP_ROW_SHR1>(carry_%s, %s);' % (name, name, name))
+        src.append('            }')
+        src.append('            // the last lane of the group finished the group: its state is the carry into the next one')
+        for name, _ in state:
+            src.append('            carry_%s = ovl_dpp_move<OVL_DPP_ROW_ROR1>(carry_%s, %s);' % (name, name, name))
+        src.append('        }')
+        if refill_expr is not None:
+            src.append('        __builtin_amdgcn_sched_barrier(0);')
+            request(None, refill_expr, nb, suffix)
+            src.append('        __builtin_amdgcn_sched_barrier(0);')
+        src.append('        }')
+
+    sets = 2 if num_batches > 1 else 1
+    src.append('    // %d register sets of %d groups each per tensor: one is consumed while the other is in flight' % (sets, batch))
+    for t in p.tensors:
+        vname = vnames[CTYPE[t.dtype]]
+        src.append('    %s %s;' % (vname, ', '.join('q%d_%d[%d][%d]' % (t.io_index, k, batch, width) for k in range(sets))))
+        if tail:
+            src.append('    %s q%d_t[%d][%d];       // the groups that end the row, requested now and held until then' % (
+                vname, t.io_index, tail, width))
+    src.append('    {')
+    for k in range(sets):
+        request(k, '%du' % k, batch, '_%d' % k)
+    if tail:
+        request(None, '%du' % num_batches, tail, '_t')
+    src.append('    }')
+    src.append('    // the statements the worker runs before its loop, in every lane')
+    for stmt in prologue:
+        src.append('    ' + stmt)
+    for name, stype in state:
+        src.append('    %s carry_%s = %s;' % (stype, name, name))
+    for t in p.tensors:
+        src.append('#define OVL_REDUCE_IN%d xv%d[u]' % (t.io_index, t.io_index))
+    src.append('#define OVL_REDUCE_STEP(column) { %s = (%s)(column); %s }' % (counter_name, counter_type, ' '.join(body)))
+    rounds = num_batches // sets
+    last = num_batches - 1
+    if rounds:
+        src.append('    #pragma unroll 1')
+        src.append('    for (uint32_t b0 = 0; b0 < %du; b0 += %du) {' % (rounds * sets, sets))
+        # past the end a set is refilled with the last batch again, which keeps the loop free of branches
+        for k in range(sets):
+            process('_%d' % k, 'b0 + %du' % k, '(b0 + %du < %du ? b0 + %du : %du)' % (k + sets, num_batches, k + sets, last), batch)
+        src.append('    }')
+    for k in range(num_batches % sets):
+        src.append('    {')
+        process('_%d' % k, '%du' % (rounds * sets + k), None, batch)
+        src.append('    }')
+    if tail:
+        src.append('    {')
+        process('_t', '%du' % num_batches, None, tail)
+        src.append('    }')
+    for t in p.tensors:
+        src.append('#undef OVL_REDUCE_IN%d' % t.io_index)
+        src.append('#define OVL_REDUCE_IN%d gin%d[column]' % (t.io_index, t.io_index))
+    src.append('    // Lane 0 of the row holds the state that leaves the last group: it walks the columns after that group, one at a')
+    src.append('    // time, and runs the statements that follow the worker\'s loop.')
+    src.append('    if (part == 0u) {')
+    for name, _ in state:
+        src.append('        %s = carry_%s;' % (name, name))
+    if tail_cols:
+        src.append('        #pragma unroll 1')
+        src.append('        for (uint32_t column = %du; column < %du; ++column) OVL_REDUCE_STEP(column)' % (
+            num_groups * group_cols, p.length))
+    for stmt in epilogue:
+        src.append('        ' + stmt.strip())
+    src.append('    }')
+    for t in p.tensors:
+        src.append('#undef OVL_REDUCE_IN%d' % t.io_index)
+    src.append('#undef OVL_REDUCE_STEP')
+    src.append('}')
+
+    row_align = 16 if aligned else itemsize
+    launch = {
+        'template': 'rowreduce',
+        'vec': vec,
+        'block': BLOCK,
+        'blocks_needed': (p.rows + rows_per_block - 1) // rows_per_block,
+        'align': dict((('in', t.io_index), row_align) for t in p.tensors),
+        'vector_loads': len(p.tensors),
+        'vector_stores': 0,
+    }
+    return '\n'.join(src) + '\n', launch
+
+
 TREE_OPS = (lang.ADD, lang.MULTIPLY, lang.MIN, lang.MAX)
 
 

@@ -401,6 +401,67 @@ def dot(input0, input1):
 
 
 @ovl.operator()
+def _row_dot(a, b):
+    """A dot product per row, accumulated in float64, with a statement after the loop."""
+    shape = list(a.shape)
+    out = ovl.output(shape[:-1], ovl.float64)
+    pos = ovl.position_in(shape[:-1])
+    acc = ovl.variable(0.0, ovl.float64)
+    for j in ovl.arange(shape[-1]):
+        index = tuple(pos[k] for k in range(len(shape) - 1)) + (j,)
+        acc <<= acc + ovl.cast(a[index] * b[index], ovl.float64)
+    out[pos] = acc * 0.5
+    return out
+
+
+@ovl.operator()
+def _row_norm_and_max(x):
+    """Two carried states and two outputs: the square root of the sum of squares and the running maximum, which
+    starts from column 0 (the loop starts at 1)."""
+    rows, cols = x.shape
+    norm = ovl.output([rows], x.dtype)
+    largest = ovl.output([rows], x.dtype)
+    pos = ovl.position_in([rows])[0]
+    first = x[pos, 0]
+    total = ovl.variable(first * first, x.dtype)
+    top = ovl.variable(first, x.dtype)
+    for j in ovl.arange(1, cols):
+        v = x[pos, j]
+        total <<= total + v * v
+        top <<= ovl.maximum(top, v)
+    norm[pos] = ovl.sqrt(total)
+    largest[pos] = top
+    return norm, largest
+
+
+@ovl.operator()
+def _row_int_sum(x):
+    rows, cols = x.shape
+    out = ovl.output([rows], x.dtype)
+    pos = ovl.position_in([rows])[0]
+    acc = ovl.variable(0, x.dtype)
+    for j in ovl.arange(cols):
+        acc <<= acc + x[pos, j]
+    out[pos] = acc
+    return out
+
+
+def row_reductions(rng):
+    """Reductions along the last axis: rows of whole groups, rows with columns left over, rows that are not 16-byte
+    aligned, a rank-3 tensor, 4- and 8-byte elements, integers."""
+    a = rng.standard_normal((7, 256), dtype=np.float32)
+    b = rng.standard_normal((7, 256), dtype=np.float32)
+    c = rng.standard_normal((5, 333), dtype=np.float32)
+    d = rng.standard_normal((5, 333), dtype=np.float32)
+    e = rng.standard_normal((2, 3, 200))
+    f = rng.standard_normal((2, 3, 200))
+    return ([_row_dot(a, b), _row_dot(c, d), _row_dot(e, f)] +
+            all_outputs(_row_norm_and_max(rng.standard_normal((9, 131)))) + all_outputs(_row_norm_and_max(rng.standard_normal((9, 80)))) +
+            all_outputs(_row_norm_and_max(rng.standard_normal((70, 1000), dtype=np.float32))) +
+            [_row_int_sum(rng.integers(-50, 50, size=(6, 270)).astype(np.int32))])
+
+
+@ovl.operator()
 def multi_op(input0, input1, input2):
     pos = ovl.position_in(input0.shape)
     output0 = ovl.output_like(input0)
@@ -702,6 +763,7 @@ CASES = [
     Case('c5_gather_transpose', c5_gather_transpose, seed=5),
     Case('c5_variants', c5_variants, seed=5),
     Case('batched_transposes', batched_transposes, seed=5),
+    Case('row_reductions', row_reductions, seed=7),
     _simple('store_order', _store_order),
     _simple('clip', lambda rng: [clip(rng.random(1000), threshold1=0.1, threshold2=0.9)[0]]),
     _simple('limits_f32', lambda rng: [set_limits(np.array([0], np.float32))[0]]),
@@ -1065,6 +1127,9 @@ TEMPLATE_VARIANTS = [
     ('c5_variants', {'grid_cap': 2}),
     ('c5_variants', {'nt': 'l'}),
     ('batched_transposes', {'template': 'map'}),
+    ('row_reductions', {'template': 'map'}),
+    ('row_reductions', {'scan_depth': 1}),
+    ('row_reductions', {'scan_depth': 3, 'scan_width': 1}),
     ('batched_transposes', {'tile_i': 16, 'tile_j': 64}),
     ('c5_variants', {'nt': 'ls'}),
     ('c5_variants', {'template': 'map', 'grid_cap': 5}),
