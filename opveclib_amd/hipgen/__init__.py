@@ -62,7 +62,7 @@ def generate(expression_dag, function_name, options=None):
     """
     :param expression_dag: serialised expression DAG of one operator
     :param function_name: unique name of the operator (its content hash)
-    :param options: optional dict.  ``template``: 'auto' (default), 'map', 'transpose', 'rowscan', 'skewscan', 'fedscan', 'treescan', 'rowreduce', 'colscan' or 'colskew' restricts
+    :param options: optional dict.  ``template``: 'auto' (default), 'map', 'transpose', 'rowscan', 'skewscan', 'fedscan', 'treescan', 'rowreduce', 'colreduce', 'colscan' or 'colskew' restricts
         the choice of kernel template (a template that does not fit the DAG falls back to 'map'); ``vec`` forces the
         map template with that vector width, ``per_thread`` its vectors per thread (1 or 2); ``scan_movers`` the number of threads that only move data in the lane-skewed column scan (0: every wavefront scans and moves), ``scan_depth`` / ``scan_sets`` / ``scan_width`` / ``scan_interleave`` set the request burst (groups), the
         number of register sets, the 128-bit vectors per lane and phase and the rows per lane group of the lane-skewed scan; ``math``: 'exact'
@@ -130,6 +130,13 @@ def generate(expression_dag, function_name, options=None):
         # a loop-carried state over the last axis with nothing stored inside the loop: a dot product, a sum
         kernel_src, launch = rowscan_kernel.generate_reduce(info, kernel_name, options.get('scan_depth'),
                                                             options.get('scan_width'))
+    elif options.get('vec') is None and template in ('auto', 'colreduce') and \
+            colscan_kernel.reduce_plan(info, options.get('scan_rows'), options.get('scan_batch'),
+                                       options.get('scan_sets')) is not None and \
+            (template == 'colreduce' or colscan_kernel.worthwhile(info, colscan_kernel.reduce_plan(info))):
+        # a loop-carried state over an axis that is not the last, nothing stored inside the loop: a column sum
+        kernel_src, launch = colscan_kernel.generate(info, kernel_name, options.get('scan_rows'),
+                                                     options.get('scan_batch'), options.get('scan_sets'), reduce=True)
     elif options.get('vec') is None and template in ('auto', 'transpose') and tile_kernel.applicable(info) is not None:
         kernel_src, launch = tile_kernel.generate(info, kernel_name, options.get('tile_i'), options.get('tile_j'),
                                                   options.get('nt'))

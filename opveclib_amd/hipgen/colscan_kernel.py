@@ -57,6 +57,9 @@ class ColumnPlan(object):
         self.rows_per_chunk = rows_per_chunk
         self.batch = batch              # LDS accesses per register set of the scanning wavefront
         self.sets = sets                # register sets of the movers = chunks of loads in flight
+        self.reduce = False             # a reduction: nothing is stored inside the loop, `out` is None
+        self.start = 1                  # first row the loop visits
+        self.end_idx = None             # (reductions) the node that closes the loop
 
 
 def plan(info, rows_per_chunk=None, batch=None, sets=None):
@@ -142,14 +145,95 @@ def plan(info, rows_per_chunk=None, batch=None, sets=None):
     return p
 
 
+def reduce_plan(info, rows_per_chunk=None, batch=None, sets=None):
+    """A ColumnPlan (with ``reduce`` set) when the DAG is a reduction along a non-last axis of one input: a counted loop
+    with a loop-carried state that reads ``x[.., i, ..]`` and stores nothing inside the loop; else None."""
+    loops = [item for item in info.tree if item.kind == 'loop']
+    if len(loops) != 1 or any(item.kind == 'if' for item in info.tree):
+        return None
+    loop = loops[0]
+    if any(inner.kind != 'stmt' for inner in loop.body):
+        return None
+    range_node = info.nodes[loop.node]
+    counter = range_node.ops[0]
+    if counter not in info.loop_counters:
+        return None
+    start, stop, step = (info._literal_int(o) for o in range_node.ops[1:])
+    if start not in (0, 1) or step != 1 or stop is None or stop < 2:
+        return None
+    length = stop
+    closers = [n.idx for n in info.nodes if n.idx > loop.node and n.code == lang.ENDRANGE and not info.in_loop[n.idx]]
+    if not closers:
+        return None
+    x = None
+    in_loop_accesses = []
+    for node, tensor, aff in info.tensor_accesses():
+        if not info.in_loop[node.idx]:
+            continue                    # before and after the loop: ordinary code of the line's lane
+        if node.code != lang.READ_TENSOR or tensor.code != lang.INPUT or aff is None:
+            return None
+        if x is not None and tensor is not x:
+            return None
+        x = tensor
+        in_loop_accesses.append(aff)
+    if x is None or x.dtype not in CTYPE or ITEMSIZE[x.dtype] not in (4, 8):
+        return None
+    shape = list(x.shape)
+    rank = len(shape)
+    if rank < 2 or len(info.workgroup_shape) != rank - 1:
+        return None
+    axis = None
+    for k in range(rank - 1):
+        if shape[k] == length and shape[:k] + shape[k + 1:] == list(info.workgroup_shape):
+            axis = k
+            break
+    if axis is None:
+        return None
+    strides = [1] * rank
+    for k in range(rank - 2, -1, -1):
+        strides[k] = strides[k + 1] * shape[k + 1]
+    inner = strides[axis]
+    outer = 1
+    for d in shape[:axis]:
+        outer *= d
+    sig = {}
+    for j, dim in enumerate(d for d in range(rank) if d != axis):
+        if info.workgroup_shape[j] > 1:
+            sig[('p', j)] = strides[dim]
+    sig[('v', counter)] = inner
+    sig_loop = (tuple(sorted(sig.items())), 0)
+    if any(aff.signature() != sig_loop for aff in in_loop_accesses):
+        return None
+    per = 16 // ITEMSIZE[x.dtype]
+    rows_per_chunk = rows_per_chunk or 64
+    batch = batch or 8
+    while batch > 1 and (rows_per_chunk // per) % (2 * batch) != 0:
+        batch //= 2
+    if rows_per_chunk % per != 0 or (rows_per_chunk // per) % (2 * batch) != 0:
+        return None
+    if 3 * rows_per_chunk * STRIP * ITEMSIZE[x.dtype] > LDS_BUDGET:
+        return None
+    p = ColumnPlan(loop, counter, length, outer, inner, x, None, per, rows_per_chunk, batch,
+                   max(2, min(int(sets or SETS), 16)))
+    p.sets_forced = sets is not None
+    p.reduce = True
+    p.start = start
+    p.end_idx = min(closers)
+    from .rowscan_kernel import _carried_state
+    state = _carried_state(info, p)
+    if not state or any(info.nodes[idx].dtype not in CTYPE for idx in state):
+        return None
+    return p
+
+
 def worthwhile(info, p):
     """A long enough axis: there the one-worker-per-thread template is bound by the latency of its loads."""
     strips = (p.inner + STRIP - 1) // STRIP
     return p.length >= MIN_LENGTH and p.outer * strips <= MAX_BLOCKS
 
 
-def generate(info, kernel_name, rows_per_chunk=None, batch=None, sets=None):
-    p = plan(info, rows_per_chunk, batch, sets)
+def generate(info, kernel_name, rows_per_chunk=None, batch=None, sets=None, reduce=False):
+    p = (reduce_plan if reduce else plan)(info, rows_per_chunk, batch, sets)
     assert p is not None
     ctype = CTYPE[p.x.dtype]
     per, rc, batch = p.per, p.rows_per_chunk, p.batch
@@ -173,14 +257,21 @@ def generate(info, kernel_name, rows_per_chunk=None, batch=None, sets=None):
             expr = '(line % ' + str(wg_strides[k - 1]) + 'u)'
         pos_exprs.append(expr + ' / ' + str(wg_strides[k]) + 'u')
 
-    emitter = BodyEmitter(info, pos_exprs,
-                          read_hook=lambda node, tensor, idx: 'OVL_SCAN_IN',
-                          store_hook=lambda node, tensor, idx, value: 'OVL_SCAN_OUT(' + value + ');')
+    if p.reduce:
+        # only the reads inside the loop come out of the tile; what stands before and after the loop is ordinary code
+        emitter = BodyEmitter(info, pos_exprs,
+                              read_hook=lambda node, tensor, idx: 'OVL_SCAN_IN' if info.in_loop[node.idx] else None,
+                              store_hook=None)
+    else:
+        emitter = BodyEmitter(info, pos_exprs,
+                              read_hook=lambda node, tensor, idx: 'OVL_SCAN_IN',
+                              store_hook=lambda node, tensor, idx, value: 'OVL_SCAN_OUT(' + value + ');')
     tagged = emitter.emit_tagged()
     range_idx = p.loop_item.node
-    end_idx = max(i for i, _ in tagged)
+    end_idx = p.end_idx if p.reduce else max(i for i, _ in tagged)
     prologue = [t for i, t in tagged if i < range_idx]
     body = [t.strip() for i, t in tagged if range_idx < i < end_idx]
+    epilogue = [t.strip() for i, t in tagged if i > end_idx]
     counter_name = 'e' + str(p.counter)
     counter_type = CTYPE[info.nodes[p.counter].dtype]
 
@@ -190,8 +281,13 @@ def generate(info, kernel_name, rows_per_chunk=None, batch=None, sets=None):
     a('typedef %s %s __attribute__((ext_vector_type(%d)));' % (ctype, vname, per))
     a('')
     a('extern "C" __global__ void __launch_bounds__(%d)' % BLOCK)
-    a('%s(const %s* __restrict__ in%d, %s* __restrict__ out%d) {' % (
-        kernel_name, ctype, p.x.io_index, ctype, p.out.io_index))
+    if p.reduce:
+        args = ['const %s* __restrict__ in%d' % (CTYPE[info.inputs[i].dtype], i) for i in range(len(info.inputs))]
+        args += ['%s* __restrict__ out%d' % (CTYPE[info.outputs[i].dtype], i) for i in range(len(info.outputs))]
+        a('%s(%s) {' % (kernel_name, ', '.join(args)))
+    else:
+        a('%s(const %s* __restrict__ in%d, %s* __restrict__ out%d) {' % (
+            kernel_name, ctype, p.x.io_index, ctype, p.out.io_index))
     if info.uses_math_tables():
         a('    OVL_DECLARE_MATH_TABLES();')
     a('    // tile[buffer][rows / %d][line]: the %d consecutive rows of one line are one 128-bit word' % (per, per))
@@ -203,7 +299,8 @@ def generate(info, kernel_name, rows_per_chunk=None, batch=None, sets=None):
     a('    const uint64_t obase = (uint64_t)o * %dull + c0;      // element of row 0, first line of the strip' % (
         p.length * p.inner))
     a('    const %s* __restrict__ gin = in%d + obase;' % (ctype, p.x.io_index))
-    a('    %s* __restrict__ gout = out%d + obase;' % (ctype, p.out.io_index))
+    if not p.reduce:
+        a('    %s* __restrict__ gout = out%d + obase;' % (ctype, p.out.io_index))
     a('')
     a('    // Movers (threads 64 and up): a thread owns up to %d elements of each chunk, one row of the strip per' % ipt)
     a('    // wavefront and instruction (a wavefront covering %d rows of %d lines would write LDS without bank conflicts but' % (per, STRIP // per))
@@ -234,34 +331,40 @@ def generate(info, kernel_name, rows_per_chunk=None, batch=None, sets=None):
     a('            if (slot(k, m, i, r, c)) *lds_word(k, r, c) = regs.v[i];')
     a('        }')
     a('    };')
-    a('    auto store_chunk = [&](uint32_t k, uint32_t m) {')
-    a('        #pragma unroll')
-    a('        for (uint32_t i = 0; i < %du; ++i) {' % ipt)
-    a('            uint32_t r, c;')
-    a('            if (slot(k, m, i, r, c))')
-    a('                __builtin_nontemporal_store(*lds_word(k, r, c), gout + (uint64_t)(k * %du + r) * %dull + c);' % (
-        rc, p.inner))
-    a('        }')
-    a('    };')
+    if not p.reduce:
+        a('    auto store_chunk = [&](uint32_t k, uint32_t m) {')
+        a('        #pragma unroll')
+        a('        for (uint32_t i = 0; i < %du; ++i) {' % ipt)
+        a('            uint32_t r, c;')
+        a('            if (slot(k, m, i, r, c))')
+        a('                __builtin_nontemporal_store(*lds_word(k, r, c), gout + (uint64_t)(k * %du + r) * %dull + c);' % (
+            rc, p.inner))
+        a('        }')
+        a('    };')
     a('')
     sets = min(p.sets, max(2, num_chunks))
     if not p.sets_forced:
         # float64 [10000, 1000]: 8 sets spill (322 us), 4 sets 191 us
         sets = max(2, min(sets, SET_REGISTERS // (ipt * (ITEMSIZE[p.x.dtype] // 4))))
     a('    if (threadIdx.x >= %du) {' % WAVE)
-    _emit_movers(a, sets, num_chunks)
+    _emit_movers(a, sets, num_chunks, stores=not p.reduce)
     a('    } else {')
     a('        // The scanning wavefront: lane = line c0 + lane of the strip; a lane past the last line shadows it.')
     a('        const uint32_t c = (c0 + lane < %du) ? lane : %du - c0;' % (p.inner, p.inner - 1))
     a('        const uint32_t line = o * %du + c0 + c;' % p.inner)
-    a('        // first row: the statements the worker runs before its loop')
-    a('        %s first_out;' % ctype)
-    a('#define OVL_SCAN_IN (gin[c])')
-    a('#define OVL_SCAN_OUT(value) first_out = (value)')
-    for stmt in prologue:
-        a('        ' + stmt)
-    a('#undef OVL_SCAN_IN')
-    a('#undef OVL_SCAN_OUT')
+    if p.reduce:
+        a('        // the statements the worker runs before its loop')
+        for stmt in prologue:
+            a('        ' + stmt)
+    else:
+        a('        // first row: the statements the worker runs before its loop')
+        a('        %s first_out;' % ctype)
+        a('#define OVL_SCAN_IN (gin[c])')
+        a('#define OVL_SCAN_OUT(value) first_out = (value)')
+        for stmt in prologue:
+            a('        ' + stmt)
+        a('#undef OVL_SCAN_IN')
+        a('#undef OVL_SCAN_OUT')
     a('#define OVL_SCAN_IN xv[u]')
     a('#define OVL_SCAN_OUT(value) xv[u] = (value)')
     a('#define OVL_SCAN_STEP(row) { %s = (%s)(row); %s }' % (counter_name, counter_type, ' '.join(body)))
@@ -281,26 +384,39 @@ def generate(info, kernel_name, rows_per_chunk=None, batch=None, sets=None):
     a('                %s& xv = set[v];' % vname)
     a('                #pragma unroll')
     a('                for (uint32_t u = 0; u < %du; ++u) {' % per)
-    a('                    if (v == 0u && u == 0u && first) xv[0] = first_out;')
-    a('                    else OVL_SCAN_STEP(row0 + v * %du + u)' % per)
+    if p.reduce:
+        # (rows past the last one of the tensor hold copies of other rows: they must not reach the state)
+        skip_first = 'v == 0u && u == 0u && first' if p.start == 1 else 'false'
+        a('                    if (!(%s) && row0 + v * %du + u < %du) OVL_SCAN_STEP(row0 + v * %du + u)' % (
+            skip_first, per, p.length, per))
+    else:
+        a('                    if (v == 0u && u == 0u && first) xv[0] = first_out;')
+        a('                    else OVL_SCAN_STEP(row0 + v * %du + u)' % per)
     a('                }')
     a('            }')
     a('        };')
     a('        __syncthreads();')
     a('        for (uint32_t k = 0; k < %du; ++k) {' % num_chunks)
-    a('            %s* colp = &tile[k %% 3u][0][lane];' % vname)
+    # (a reduction's lanes past the last line store what its owner stores: they read the owner's rows too)
+    a('            %s* colp = &tile[k %% 3u][0][%s];' % (vname, 'c' if p.reduce else 'lane'))
     a('            fetch(set_a, colp);')
     a('            #pragma unroll 1')
     a('            for (uint32_t q = 0; q < %du; q += %du) {' % (reads_per_chunk, 2 * batch))
     a('                fetch(set_b, colp + (q + %du) * %du);' % (batch, STRIP))
     a('                run(set_a, k * %du + q * %du, k == 0u && q == 0u);' % (rc, per))
-    a('                put_back(set_a, colp + q * %du);' % STRIP)
+    if not p.reduce:
+        a('                put_back(set_a, colp + q * %du);' % STRIP)
     a('                if (q + %du < %du) fetch(set_a, colp + (q + %du) * %du);' % (2 * batch, reads_per_chunk, 2 * batch, STRIP))
     a('                run(set_b, k * %du + (q + %du) * %du, false);' % (rc, batch, per))
-    a('                put_back(set_b, colp + (q + %du) * %du);' % (batch, STRIP))
+    if not p.reduce:
+        a('                put_back(set_b, colp + (q + %du) * %du);' % (batch, STRIP))
     a('            }')
     a('            __syncthreads();')
     a('        }')
+    if p.reduce:
+        a('        // the statements after the worker\'s loop, once per line')
+        for stmt in epilogue:
+            a('        ' + stmt)
     a('#undef OVL_SCAN_STEP')
     a('#undef OVL_SCAN_IN')
     a('#undef OVL_SCAN_OUT')
@@ -309,18 +425,19 @@ def generate(info, kernel_name, rows_per_chunk=None, batch=None, sets=None):
 
     itemsize = ITEMSIZE[p.x.dtype]
     launch = {
-        'template': 'colscan',
+        'template': 'colreduce' if p.reduce else 'colscan',
         'vec': 1,
         'block': BLOCK,
         'blocks_needed': p.outer * strips,
-        'align': {('in', p.x.io_index): itemsize, ('out', p.out.io_index): itemsize},
+        'align': {('in', p.x.io_index): itemsize} if p.reduce else
+                 {('in', p.x.io_index): itemsize, ('out', p.out.io_index): itemsize},
         'vector_loads': 1,
         'vector_stores': 1,
     }
     return '\n'.join(src) + '\n', launch
 
 
-def _emit_movers(a, sets, num_chunks):
+def _emit_movers(a, sets, num_chunks, stores=True):
     a('        const uint32_t m = threadIdx.x - %du;' % WAVE)
     a('        // %d register sets keep %d chunks of loads in flight: chunk j travels through set j %% %d, is requested' % (
         sets, sets, sets))
@@ -337,7 +454,8 @@ def _emit_movers(a, sets, num_chunks):
     a('        auto step = [&](uint32_t k, MoverRegs& regs) {')
     a('            if (k + 1u < %du) write_lds(k + 1u, m, regs);' % num_chunks)
     a('            if (k + 1u + %du < %du) issue_loads(k + 1u + %du, m, regs);' % (sets, num_chunks, sets))
-    a('            if (k >= 1u) store_chunk(k - 1u, m);')
+    if stores:
+        a('            if (k >= 1u) store_chunk(k - 1u, m);')
     a('            __syncthreads();')
     a('        };')
     full = num_chunks // sets
@@ -349,7 +467,8 @@ def _emit_movers(a, sets, num_chunks):
         a('        }')
     for k in range(full * sets, num_chunks):
         a('        step(%du, sets[%d]);' % (k, (k + 1) % sets))
-    a('        store_chunk(%du, m);' % (num_chunks - 1))
+    if stores:
+        a('        store_chunk(%du, m);' % (num_chunks - 1))
 
 
 # ---------------------------------------------------------------------------------------------------------------------

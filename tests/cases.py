@@ -462,6 +462,53 @@ def row_reductions(rng):
 
 
 @ovl.operator()
+def _axis_mean_and_max(x, axis=None):
+    """Reductions along an axis that is not the last: the mean (a statement after the loop) and the maximum, which
+    starts from the first element (the loop starts at 1)."""
+    shape = list(x.shape)
+    rest = shape[:axis] + shape[axis + 1:]
+    mean = ovl.output(rest, x.dtype)
+    largest = ovl.output(rest, x.dtype)
+    pos = ovl.position_in(rest)
+
+    def at(i):
+        return tuple(pos[k] for k in range(axis)) + (i,) + tuple(pos[k] for k in range(axis, len(rest)))
+    first = x[at(0)]
+    total = ovl.variable(first, x.dtype)
+    top = ovl.variable(first, x.dtype)
+    for i in ovl.arange(1, shape[axis]):
+        v = x[at(i)]
+        total <<= total + v
+        top <<= ovl.maximum(top, v)
+    mean[pos] = total / shape[axis]
+    largest[pos] = top
+    return mean, largest
+
+
+@ovl.operator()
+def _column_sum(x):
+    rows, cols = x.shape
+    out = ovl.output([cols], x.dtype)
+    pos = ovl.position_in([cols])[0]
+    acc = ovl.variable(0, x.dtype)
+    for i in ovl.arange(rows):
+        acc <<= acc + x[i, pos]
+    out[pos] = acc
+    return out
+
+
+def col_reductions(rng):
+    """Reductions along an axis other than the last: partial strips, a partial last chunk of rows, dimensions before
+    the axis, 4- and 8-byte elements, integers, a loop from 0 and a loop from 1."""
+    return (all_outputs(_axis_mean_and_max(rng.standard_normal((200, 100)), axis=0)) +
+            all_outputs(_axis_mean_and_max(rng.standard_normal((130, 70), dtype=np.float32), axis=0)) +
+            all_outputs(_axis_mean_and_max(rng.standard_normal((3, 65, 40), dtype=np.float32), axis=1)) +
+            [_column_sum(rng.standard_normal((700, 30))),
+             _column_sum(rng.integers(-1000, 1000, size=(64, 5)).astype(np.int32)),
+             _column_sum(rng.standard_normal((1100, 20), dtype=np.float32))])
+
+
+@ovl.operator()
 def multi_op(input0, input1, input2):
     pos = ovl.position_in(input0.shape)
     output0 = ovl.output_like(input0)
@@ -764,6 +811,7 @@ CASES = [
     Case('c5_variants', c5_variants, seed=5),
     Case('batched_transposes', batched_transposes, seed=5),
     Case('row_reductions', row_reductions, seed=7),
+    Case('col_reductions', col_reductions, seed=8),
     _simple('store_order', _store_order),
     _simple('clip', lambda rng: [clip(rng.random(1000), threshold1=0.1, threshold2=0.9)[0]]),
     _simple('limits_f32', lambda rng: [set_limits(np.array([0], np.float32))[0]]),
@@ -1127,6 +1175,9 @@ TEMPLATE_VARIANTS = [
     ('c5_variants', {'grid_cap': 2}),
     ('c5_variants', {'nt': 'l'}),
     ('batched_transposes', {'template': 'map'}),
+    ('col_reductions', {'template': 'map'}),
+    ('col_reductions', {'scan_rows': 32, 'scan_batch': 2}),
+    ('col_reductions', {'scan_sets': 3}),
     ('row_reductions', {'template': 'map'}),
     ('row_reductions', {'scan_depth': 1}),
     ('row_reductions', {'scan_depth': 3, 'scan_width': 1}),

@@ -48,7 +48,7 @@ def test_loaded_operators_come_from_the_hip_extension():
     for compiled in runtime._loaded.values():
         assert compiled.so_path.endswith('_generic_hip.so')
         assert compiled.lib.info['template'] in ('map', 'transpose', 'rowscan', 'skewscan', 'fedscan', 'colscan', 'colskew', 'treescan',
-                                                'rowreduce')
+                                                'rowreduce', 'colreduce')
 
 
 def test_known_answer_fixtures_on_the_gpu():
