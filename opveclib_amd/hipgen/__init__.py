@@ -135,8 +135,16 @@ def generate(expression_dag, function_name, options=None):
                                        options.get('scan_sets')) is not None and \
             (template == 'colreduce' or colscan_kernel.worthwhile(info, colscan_kernel.reduce_plan(info))):
         # a loop-carried state over an axis that is not the last, nothing stored inside the loop: a column sum
-        kernel_src, launch = colscan_kernel.generate(info, kernel_name, options.get('scan_rows'),
-                                                     options.get('scan_batch'), options.get('scan_sets'), reduce=True)
+        if options.get('scan_skew', True) and options.get('scan_rows') is None and options.get('scan_batch') is None and \
+                colscan_kernel.prefers_skew(info, colscan_kernel.reduce_plan(info)):
+            # few lines: sixteen lanes per line, as for the scans
+            kernel_src, launch = colscan_kernel.generate_skewed(info, kernel_name, options.get('scan_sets'),
+                                                                options.get('scan_strip'), options.get('scan_width'),
+                                                                options.get('scan_movers'), reduce=True)
+        else:
+            kernel_src, launch = colscan_kernel.generate(info, kernel_name, options.get('scan_rows'),
+                                                         options.get('scan_batch'), options.get('scan_sets'),
+                                                         reduce=True)
     elif options.get('vec') is None and template in ('auto', 'transpose') and tile_kernel.applicable(info) is not None:
         kernel_src, launch = tile_kernel.generate(info, kernel_name, options.get('tile_i'), options.get('tile_j'),
                                                   options.get('nt'))

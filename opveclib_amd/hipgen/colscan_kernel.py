@@ -530,9 +530,9 @@ def prefers_skew(info, p):
     return all(info.nodes[idx].dtype in CTYPE for idx in _carried_state(info, p))
 
 
-def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, movers=None):
+def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, movers=None, reduce=False):
     from .rowscan_kernel import _carried_state
-    p = plan(info)
+    p = (reduce_plan if reduce else plan)(info)
     assert p is not None
     STRIP = strip or skew_strip(info, p)            # lines per workgroup
     SCAN_THREADS = STRIP * SKEW_GROUP               # sixteen lanes per line
@@ -582,14 +582,21 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
         if k > 0:
             expr = '(line % ' + str(wg_strides[k - 1]) + 'u)'
         pos_exprs.append(expr + ' / ' + str(wg_strides[k]) + 'u')
-    emitter = BodyEmitter(info, pos_exprs,
-                          read_hook=lambda node, tensor, idx: 'OVL_SCAN_IN',
-                          store_hook=lambda node, tensor, idx, value: 'OVL_SCAN_OUT(' + value + ');')
+    if p.reduce:
+        # only the reads inside the loop come out of the tile; what stands before and after the loop is ordinary code
+        emitter = BodyEmitter(info, pos_exprs,
+                              read_hook=lambda node, tensor, idx: 'OVL_SCAN_IN' if info.in_loop[node.idx] else None,
+                              store_hook=None)
+    else:
+        emitter = BodyEmitter(info, pos_exprs,
+                              read_hook=lambda node, tensor, idx: 'OVL_SCAN_IN',
+                              store_hook=lambda node, tensor, idx, value: 'OVL_SCAN_OUT(' + value + ');')
     tagged = emitter.emit_tagged()
     range_idx = p.loop_item.node
-    end_idx = max(i for i, _ in tagged)
+    end_idx = p.end_idx if p.reduce else max(i for i, _ in tagged)
     prologue = [t for i, t in tagged if i < range_idx]
     body = [t.strip() for i, t in tagged if range_idx < i < end_idx]
+    epilogue = [t.strip() for i, t in tagged if i > end_idx]
     counter_name = 'e' + str(p.counter)
     counter_type = CTYPE[info.nodes[p.counter].dtype]
     state = [('e' + str(idx), CTYPE[info.nodes[idx].dtype]) for idx in _carried_state(info, p)]
@@ -600,8 +607,13 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
     a('typedef %s %s __attribute__((ext_vector_type(%d)));' % (ctype, vname, per))
     a('')
     a('extern "C" __global__ void __launch_bounds__(%d)' % BLOCK)
-    a('%s(const %s* __restrict__ in%d, %s* __restrict__ out%d) {' % (
-        kernel_name, ctype, p.x.io_index, ctype, p.out.io_index))
+    if p.reduce:
+        args = ['const %s* __restrict__ in%d' % (CTYPE[info.inputs[i].dtype], i) for i in range(len(info.inputs))]
+        args += ['%s* __restrict__ out%d' % (CTYPE[info.outputs[i].dtype], i) for i in range(len(info.outputs))]
+        a('%s(%s) {' % (kernel_name, ', '.join(args)))
+    else:
+        a('%s(const %s* __restrict__ in%d, %s* __restrict__ out%d) {' % (
+            kernel_name, ctype, p.x.io_index, ctype, p.out.io_index))
     if info.uses_math_tables():
         a('    OVL_DECLARE_MATH_TABLES();')
     a('    // tile[buffer][line][row]: a line holds the %d rows of a chunk as 16 segments of %d rows, each followed by one' % (rc, seg))
@@ -627,7 +639,8 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
     a('    const uint64_t obase = (uint64_t)o * %dull + c0;      // element of row 0, first line of the strip' % (
         p.length * p.inner))
     a('    const %s* __restrict__ gin = in%d + obase;' % (ctype, p.x.io_index))
-    a('    %s* __restrict__ gout = out%d + obase;' % (ctype, p.out.io_index))
+    if not p.reduce:
+        a('    %s* __restrict__ gout = out%d + obase;' % (ctype, p.out.io_index))
     a('')
     if movers:
         a('    // Threads %d and up move data, the others scan.' % SCAN_THREADS)
@@ -671,33 +684,36 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
     a('        #pragma unroll')
     a('        for (uint32_t i = 0; i < %du; ++i) *lds_at(k, i) = regs.v[i];' % vpt)
     a('    };')
-    a('    auto store_chunk = [&](uint32_t k) {')
-    a('        // (a row past the chunk\'s last one is stored as that last row once more: its value comes from the word that')
-    a('        // holds the last row)')
-    a('        const uint32_t last = ((%du - k * %du < %du) ? %du - k * %du : %du) - 1u;' % (
-        p.length, rc, rc, p.length, rc, rc))
-    a('        MoverRegs regs;')
-    a('        #pragma unroll')
-    a('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
-    a('            const uint32_t word = mv + i * %du;' % rows_per_pass)
-    a('            const uint32_t r = (word < last / %du ? word : last / %du) * %du;' % (per, per, per))
-    a('            regs.v[i] = *reinterpret_cast<const %s*>(&tile[k %% %du][mc][(r / %du) * %du + r %% %du]);' % (
-        vname, NBUF, seg, seg_stride, seg))
-    a('        }')
-    a('        #pragma unroll')
-    a('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
-    a('            %s of_last = regs.v[i][0];' % ctype)
-    a('            #pragma unroll')
-    a('            for (uint32_t u = 1; u < %du; ++u) of_last = (last %% %du == u) ? regs.v[i][u] : of_last;' % (per, per))
-    a('            #pragma unroll')
-    a('            for (uint32_t u = 0; u < %du; ++u) {' % per)
-    a('                const uint32_t r = (mv + i * %du) * %du + u;' % (rows_per_pass, per))
-    a('                __builtin_nontemporal_store(r <= last ? regs.v[i][u] : of_last,')
-    a('                                            gout + (uint64_t)(k * %du + (r <= last ? r : last)) * %dull + mc);' % (
-        rc, p.inner))
-    a('            }')
-    a('        }')
-    a('    };')
+    if p.reduce:
+        a('    auto store_chunk = [&](uint32_t) {};      // a reduction stores nothing per row')
+    else:
+        a('    auto store_chunk = [&](uint32_t k) {')
+        a('        // (a row past the chunk\'s last one is stored as that last row once more: its value comes from the word that')
+        a('        // holds the last row)')
+        a('        const uint32_t last = ((%du - k * %du < %du) ? %du - k * %du : %du) - 1u;' % (
+            p.length, rc, rc, p.length, rc, rc))
+        a('        MoverRegs regs;')
+        a('        #pragma unroll')
+        a('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
+        a('            const uint32_t word = mv + i * %du;' % rows_per_pass)
+        a('            const uint32_t r = (word < last / %du ? word : last / %du) * %du;' % (per, per, per))
+        a('            regs.v[i] = *reinterpret_cast<const %s*>(&tile[k %% %du][mc][(r / %du) * %du + r %% %du]);' % (
+            vname, NBUF, seg, seg_stride, seg))
+        a('        }')
+        a('        #pragma unroll')
+        a('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
+        a('            %s of_last = regs.v[i][0];' % ctype)
+        a('            #pragma unroll')
+        a('            for (uint32_t u = 1; u < %du; ++u) of_last = (last %% %du == u) ? regs.v[i][u] : of_last;' % (per, per))
+        a('            #pragma unroll')
+        a('            for (uint32_t u = 0; u < %du; ++u) {' % per)
+        a('                const uint32_t r = (mv + i * %du) * %du + u;' % (rows_per_pass, per))
+        a('                __builtin_nontemporal_store(r <= last ? regs.v[i][u] : of_last,')
+        a('                                            gout + (uint64_t)(k * %du + (r <= last ? r : last)) * %dull + mc);' % (
+            rc, p.inner))
+        a('            }')
+        a('        }')
+        a('    };')
     a('')
     a('    // Scanning: wavefront w owns lines %d w ... %d w + %d of the strip, sixteen lanes each; lane `part` of a line owns' % (
         lines_per_wave, lines_per_wave, lines_per_wave - 1))
@@ -708,14 +724,19 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
         WAVE, lines_per_wave, SKEW_GROUP))
     a('    const uint32_t c = (c0 + sl < %du) ? sl : %du - c0;' % (p.inner, p.inner - 1))
     a('    const uint32_t line = o * %du + c0 + c;' % p.inner)
-    a('    // first row: the statements the worker runs before its loop, in every lane')
-    a('    %s first_out;' % ctype)
-    a('#define OVL_SCAN_IN (gin[c])')
-    a('#define OVL_SCAN_OUT(value) first_out = (value)')
-    for stmt in prologue:
-        a('    ' + stmt)
-    a('#undef OVL_SCAN_IN')
-    a('#undef OVL_SCAN_OUT')
+    if p.reduce:
+        a('    // the statements the worker runs before its loop, in every lane')
+        for stmt in prologue:
+            a('    ' + stmt)
+    else:
+        a('    // first row: the statements the worker runs before its loop, in every lane')
+        a('    %s first_out;' % ctype)
+        a('#define OVL_SCAN_IN (gin[c])')
+        a('#define OVL_SCAN_OUT(value) first_out = (value)')
+        for stmt in prologue:
+            a('    ' + stmt)
+        a('#undef OVL_SCAN_IN')
+        a('#undef OVL_SCAN_OUT')
     for name, stype in state:
         a('    %s carry_%s = %s;' % (stype, name, name))
     a('#define OVL_SCAN_IN xv[u]')
@@ -725,14 +746,16 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
     a('    // final state to its right neighbour; after phase p lanes 0..p are exact')
     a('    struct Segment { %s v[%d]; };' % (vname, seg_vectors))
     a('    auto fetch_segment = [&](uint32_t k, Segment& segment) {')
-    a('        const %s* segp = &tile[k %% %du][sl][part * %du];' % (ctype, NBUF, seg_stride))
+    # (a reduction's lanes past the last line store what its owner stores: they read the owner's rows too)
+    a('        const %s* segp = &tile[k %% %du][%s][part * %du];' % (ctype, NBUF, 'c' if p.reduce else 'sl', seg_stride))
     a('        #pragma unroll')
     a('        for (uint32_t w = 0; w < %du; ++w) segment.v[w] = *reinterpret_cast<const %s*>(segp + w * %du);' % (
         seg_vectors, vname, per))
     a('    };')
     a('    auto scan_segment = [&](uint32_t k, const Segment& segment) {')
-    a('        %s* segp = &tile[k %% %du][sl][part * %du];' % (ctype, NBUF, seg_stride))
-    a('        %s ov[%d];' % (vname, seg_vectors))
+    if not p.reduce:
+        a('        %s* segp = &tile[k %% %du][sl][part * %du];' % (ctype, NBUF, seg_stride))
+        a('        %s ov[%d];' % (vname, seg_vectors))
     a('        const uint32_t row0 = k * %du + part * %du;' % (rc, seg))
     a('        const bool first_row = k == 0u && part == 0u;')
     a('        #pragma unroll')
@@ -744,8 +767,14 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
     a('                const %s xv = segment.v[w];' % vname)
     a('                #pragma unroll')
     a('                for (uint32_t u = 0; u < %du; ++u) {' % per)
-    a('                    if (w == 0u && u == 0u && first_row) ov[0][0] = first_out;')
-    a('                    else OVL_SCAN_STEP(row0 + w * %du + u)' % per)
+    if p.reduce:
+        # (rows past the last one of the tensor hold copies of the last: they must not reach the state)
+        skip_first = 'w == 0u && u == 0u && first_row' if p.start == 1 else 'false'
+        a('                    if (!(%s) && row0 + w * %du + u < %du) OVL_SCAN_STEP(row0 + w * %du + u)' % (
+            skip_first, per, p.length, per))
+    else:
+        a('                    if (w == 0u && u == 0u && first_row) ov[0][0] = first_out;')
+        a('                    else OVL_SCAN_STEP(row0 + w * %du + u)' % per)
     a('                }')
     a('            }')
     for name, _ in state:
@@ -754,9 +783,10 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
     a('        // the last lane of the line finished the chunk: its state is the carry into the next one')
     for name, _ in state:
         a('        carry_%s = ovl_dpp_move<OVL_DPP_ROW_ROR1>(carry_%s, %s);' % (name, name, name))
-    a('        #pragma unroll')
-    a('        for (uint32_t w = 0; w < %du; ++w) *reinterpret_cast<%s*>(segp + w * %du) = ov[w];' % (
-        seg_vectors, vname, per))
+    if not p.reduce:
+        a('        #pragma unroll')
+        a('        for (uint32_t w = 0; w < %du; ++w) *reinterpret_cast<%s*>(segp + w * %du) = ov[w];' % (
+            seg_vectors, vname, per))
     a('    };')
     a('    auto scan_chunk = [&](uint32_t k) {')
     a('        Segment segment;')
@@ -848,6 +878,14 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
             a('    }')
         for k in range(full * sets, num_chunks):
             a('    step(%du, sets[%d]);' % (k, (k + 1) % sets))
+    if p.reduce:
+        a('    // the statements after the worker\'s loop, once per line: lane 0 of the line holds the final state')
+        a('    if (threadIdx.x < %du && part == 0u) {' % SCAN_THREADS)
+        for name, _ in state:
+            a('        %s = carry_%s;' % (name, name))
+        for stmt in epilogue:
+            a('        ' + stmt)
+        a('    }')
     a('#undef OVL_SCAN_STEP')
     a('#undef OVL_SCAN_IN')
     a('#undef OVL_SCAN_OUT')
@@ -855,11 +893,12 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
 
     itemsize = ITEMSIZE[p.x.dtype]
     launch = {
-        'template': 'colskew',
+        'template': 'colreduce' if p.reduce else 'colskew',
         'vec': 1,
         'block': BLOCK,
         'blocks_needed': p.outer * strips,
-        'align': {('in', p.x.io_index): itemsize, ('out', p.out.io_index): itemsize},
+        'align': {('in', p.x.io_index): itemsize} if p.reduce else
+                 {('in', p.x.io_index): itemsize, ('out', p.out.io_index): itemsize},
         'vector_loads': 1,
         'vector_stores': 1,
     }

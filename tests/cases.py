@@ -1178,6 +1178,11 @@ TEMPLATE_VARIANTS = [
     ('col_reductions', {'template': 'map'}),
     ('col_reductions', {'scan_rows': 32, 'scan_batch': 2}),
     ('col_reductions', {'scan_sets': 3}),
+    ('col_reductions', {'scan_skew': False}),
+    ('col_reductions', {'scan_movers': 0}),
+    ('col_reductions', {'scan_strip': 16, 'scan_movers': 0, 'scan_sets': 2}),
+    ('col_reductions', {'scan_strip': 64}),
+    ('col_reductions', {'scan_width': 4, 'scan_movers': 128}),
     ('row_reductions', {'template': 'map'}),
     ('row_reductions', {'scan_depth': 1}),
     ('row_reductions', {'scan_depth': 3, 'scan_width': 1}),
