@@ -160,6 +160,8 @@ class DagInfo(object):
         self.depth = {}             # node index -> nesting depth of control flow (0 = top level of the worker)
         self.in_loop = {}           # node index -> True when inside a counted loop
         self.tree = self._parse_blocks()
+        # variables that anything writes after their declaration (an assignment, or a loop that counts in them)
+        self.written_variables = set(n.ops[0] for n in self.nodes if n.code in (lang.ASSIGN_VARIABLE, lang.RANGE))
         self.loop_counters = self._find_loop_counters()
         self.ranges = {}
         for k, extent in enumerate(self.workgroup_shape):
@@ -245,9 +247,11 @@ class DagInfo(object):
         return counters
 
     def _literal_int(self, idx):
-        """Integer value of a literal or a cast chain ending in a literal, else None."""
+        """Integer value of a literal or a chain of casts and never-written variables ending in a literal (the
+        reference's dot-product test keeps its loop bound in a variable, opveclib/test/test_dot_product.py:34-36),
+        else None."""
         node = self.nodes[idx]
-        while node.code == lang.CAST:
+        while node.code == lang.CAST or (node.code == lang.VARIABLE and node.idx not in self.written_variables):
             if node.dtype not in INT_RANGE:
                 return None
             node = self.nodes[node.ops[0]]

@@ -455,7 +455,8 @@ def row_reductions(rng):
     d = rng.standard_normal((5, 333), dtype=np.float32)
     e = rng.standard_normal((2, 3, 200))
     f = rng.standard_normal((2, 3, 200))
-    return ([_row_dot(a, b), _row_dot(c, d), _row_dot(e, f)] +
+    # (the reference's own dot product keeps its loop bound in a variable that nothing writes)
+    return ([_row_dot(a, b), _row_dot(c, d), _row_dot(e, f), dot(rng.standard_normal((9, 300)), rng.standard_normal((9, 300)))] +
             all_outputs(_row_norm_and_max(rng.standard_normal((9, 131)))) + all_outputs(_row_norm_and_max(rng.standard_normal((9, 80)))) +
             all_outputs(_row_norm_and_max(rng.standard_normal((70, 1000), dtype=np.float32))) +
             [_row_int_sum(rng.integers(-50, 50, size=(6, 270)).astype(np.int32))])
