@@ -483,6 +483,8 @@ def main():
                                              full)
             cpu['gather'] = cpu_reference(gather_outputs(data['a5'], data['b5']), full, iters=2)
             cpu['cumsum_axis0'] = cpu_reference(cumsum_outputs(data['x0'], axis=0), full, iters=10)
+            cpu['dot'] = cpu_reference(workloads.dot_outputs(data['xs'], data['xp']), full)
+            cpu['column_sum'] = cpu_reference(workloads.column_sum_outputs(data['x0']), full, iters=10)
             for units in workloads.REFERENCE_LSTM_UNITS:
                 concat, c, dc, dh = data['lstm%d' % units]
                 cpu['lstm%d' % units] = cpu_reference(lstm_outputs(concat, c), full, iters=10)
@@ -665,6 +667,15 @@ def main():
         others.append(side_workload('reference timing: cumsum f64[10000,1000] along axis 0 '
                                     '(examples/test_perf_accumulate.py:35-47)', cumsum_outputs(data['x0'], axis=0),
                                     10, warm, reference=cpu.get('cumsum_axis0')))
+        # reductions in the worker's own order (the operator of the reference's dot-product test at C3's size, and
+        # the sum over the axis of the reference's accumulate timing)
+        others.append(side_workload('dot product per row f32[4096,16384] x f32[4096,16384] '
+                                    '(the operator of test/test_dot_product.py:27-45)',
+                                    workloads.dot_outputs(data['xs'], data['xp']), steps, warm,
+                                    reference=cpu.get('dot')))
+        others.append(side_workload('column sums f64[10000,1000] (sum along axis 0)',
+                                    workloads.column_sum_outputs(data['x0']), 10, warm,
+                                    reference=cpu.get('column_sum')))
         for units in workloads.REFERENCE_LSTM_UNITS:
             concat, c, dc, dh = data['lstm%d' % units]
             label = 'reference timing: lstm cell %%s, batch 20 x %d units (lstm/profile_lstm.py:41-51)' % units

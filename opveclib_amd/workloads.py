@@ -79,6 +79,44 @@ def lstm_grad_outputs(concat, c, dc, dh):
     return [op[0], op[1]]
 
 
+def dot_outputs(a, b):
+    """One dot product per row, accumulated in the order of the columns: the operator of the reference's dot-product
+    test (opveclib/test/test_dot_product.py:27-45), loop bound in a variable as there."""
+    import opveclib_amd as ovl
+
+    @ovl.operator()
+    def dot(input0, input1):
+        num_vectors = input0.shape[0]
+        dot_out = ovl.output(num_vectors, input0.dtype)
+        pos = ovl.position_in(num_vectors)[0]
+        accum = ovl.variable(0.0, input0.dtype)
+        num_elements = ovl.variable(input0.shape[1], ovl.uint32)
+        for i in ovl.arange(num_elements):
+            accum <<= accum + input0[pos, i] * input1[pos, i]
+        dot_out[pos] = accum
+        return dot_out
+
+    return [dot(a, b)]
+
+
+def column_sum_outputs(x):
+    """The sum of every column of a matrix, rows added in order."""
+    import opveclib_amd as ovl
+
+    @ovl.operator()
+    def column_sum(arg):
+        rows, cols = arg.shape
+        out = ovl.output([cols], arg.dtype)
+        pos = ovl.position_in([cols])[0]
+        acc = ovl.variable(0, arg.dtype)
+        for i in ovl.arange(rows):
+            acc <<= acc + arg[i, pos]
+        out[pos] = acc
+        return out
+
+    return [column_sum(x)]
+
+
 def gather_outputs(a, b_flat):
     from .examples import gather_transpose
     return [gather_transpose(a, b_flat, alpha=0.5, stride=7919)[0]]
@@ -107,6 +145,8 @@ def all_workload_outputs():
     yield lstm_grad_outputs(Spec((4096, 4096)), Spec((4096, 1024)), Spec((4096, 1024)), Spec((4096, 1024)))
     yield gather_outputs(Spec((16384, 16384)), Spec((16384 * 16384,)))
     yield cumsum_outputs(Spec(REFERENCE_CUMSUM_SHAPE, f64), axis=0)
+    yield dot_outputs(Spec((4096, 16384), f32), Spec((4096, 16384), f32))
+    yield column_sum_outputs(Spec(REFERENCE_CUMSUM_SHAPE, f64))
     for units in REFERENCE_LSTM_UNITS:
         batch = REFERENCE_LSTM_BATCH
         yield lstm_outputs(Spec((batch, 4 * units)), Spec((batch, units)))
