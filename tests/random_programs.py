@@ -262,11 +262,11 @@ INDEX_SEEDS = range(200, 224)
 # ----------------------------------------------------------------------------------------------------------------------
 # Random scan programs: one worker per row walks the last axis with loop-carried state.  The scan templates find the
 # carried state in the DAG, so the body can be any straight-line update: one or two state variables, sums, products,
-# running extrema, decayed sums, integer and floating point types; row lengths that do and do not fit the lane-skewed
-# template (a multiple of 16 vectors).
+# running extrema, decayed sums, integer and floating point types; row lengths that are whole groups of the lane-skewed
+# template (16 vectors), lengths with columns left over, lengths that leave rows unaligned, and rows too short for it.
 # ----------------------------------------------------------------------------------------------------------------------
 SCAN_DTYPES = [np.float32, np.float32, np.float64, np.int32, np.int64, np.int16]
-SCAN_LENGTHS = [64, 128, 192, 256, 320, 512, 1024, 32, 96, 100, 7, 2, 130]
+SCAN_LENGTHS = [64, 128, 192, 256, 320, 512, 1024, 32, 96, 100, 7, 2, 130, 70, 333, 517]
 SCAN_ROWS = [[1], [3], [4], [5], [16], [17], [67], [2, 3], [4, 9], [2, 2, 5]]
 
 
