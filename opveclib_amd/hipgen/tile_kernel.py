@@ -26,33 +26,57 @@ from .map_kernel import Access, _index_expr, _is_vector_access, contiguous_unali
 BLOCK = 256
 TILE_I_BYTES = 128        # extent of a tile along the workgroup dimension before the last, in bytes of the widest element
 TILE_J_BYTES = 1024       # extent along the last dimension
+MIN_TILE_EXTENT = 8       # tiles shrink to the workgroup's extents down to this many workers a side
 
 
-def _is_transposed_store(info, node, tensor, aff, vec):
-    """out[.., p_last*C + p_i + c] with i the workgroup dimension before the last: unit stride along it, vector
-    aligned (the dimensions before it are batch dimensions: any multiple of the vector width)."""
+def _tile_dim(info, aff):
+    """The workgroup dimension (not the last) along which this store has unit stride, or None."""
+    if aff is None:
+        return None
+    rank = len(info.workgroup_shape)
+    for k in range(rank - 2, -1, -1):
+        if info.workgroup_shape[k] > 1 and aff.coeff(('p', k)) == 1:
+            return k
+    return None
+
+
+def _is_transposed_store(info, node, tensor, aff, vec, dim):
+    """out[.., p_last*C + p_dim + c] with dim a workgroup dimension before the last: unit stride along it, vector
+    aligned (the other dimensions are batch dimensions: any multiple of the vector width)."""
     if aff is None or not aff.only_position() or info.in_loop[node.idx]:
         return False
     rank = len(info.workgroup_shape)
-    if aff.coeff(('p', rank - 2)) != 1:
+    if dim is None or aff.coeff(('p', dim)) != 1:
         return False
     c_last = aff.coeff(('p', rank - 1))
     if c_last == 0 or c_last % vec != 0 or aff.const % vec != 0:
         return False
     for sym, c in aff.coeffs.items():
-        if sym not in (('p', rank - 2), ('p', rank - 1)) and c % vec != 0:
+        if sym not in (('p', dim), ('p', rank - 1)) and c % vec != 0:
             return False
     if aff.lo < 0 or aff.hi >= tensor.size:
         return False
     return True
 
 
-def applicable(info):
-    """Vector width if the tile template fits this DAG, else None."""
-    if len(info.workgroup_shape) < 2:
+def _plan(info):
+    """(vector width, dimension that the tile spans beside the last), or None if the template does not fit.  The
+    dimension is the one along which the first position-indexed store outside loops has unit stride: [N, C, H, W]
+    stored as [N, H, W, C] takes C, a transposition of the last two dimensions takes the one before the last."""
+    rank = len(info.workgroup_shape)
+    if rank < 2:
         return None
-    rows, cols = info.workgroup_shape[-2:]
     accesses = info.tensor_accesses()
+    stores = [(n, t, a) for n, t, a in accesses if n.code == lang.ASSIGN_TENSOR]
+    dim = None
+    for n, t, a in stores:
+        if a is not None and a.only_position() and not info.in_loop[n.idx] and a.coeff(('p', rank - 1)) != 1:
+            dim = _tile_dim(info, a)
+            if dim is not None:
+                break
+    if dim is None:
+        return None
+    rows, cols = info.workgroup_shape[dim], info.workgroup_shape[-1]
     widest = 1
     for _, tensor, _ in accesses:
         widest = max(widest, ITEMSIZE[tensor.dtype])
@@ -62,14 +86,24 @@ def applicable(info):
     vec = max(1, 16 // widest)
     while vec > 1 and (rows % vec != 0 or cols % vec != 0):
         vec //= 2
+    return vec, dim
+
+
+def applicable(info):
+    """Vector width if the tile template fits this DAG, else None."""
+    planned = _plan(info)
+    if planned is None:
+        return None
+    vec, dim = planned
+    accesses = info.tensor_accesses()
     stores = [(n, t, a) for n, t, a in accesses if n.code == lang.ASSIGN_TENSOR]
-    keys = [(t.idx, a.signature()) for n, t, a in stores if _is_transposed_store(info, n, t, a, vec)]
+    keys = [(t.idx, a.signature()) for n, t, a in stores if _is_transposed_store(info, n, t, a, vec, dim)]
     if not keys:
         return None
     certain = info.definitely_stores(keys)
     bufferable = info.bufferable_outputs(
         lambda node, tensor, aff: (tensor.idx, aff.signature()) in certain and
-        _is_transposed_store(info, node, tensor, aff, vec))
+        _is_transposed_store(info, node, tensor, aff, vec, dim))
     certain = set(key for key in certain if key[0] in bufferable)
     if not certain:
         return None
@@ -82,23 +116,28 @@ def generate(info, kernel_name, tile_i=None, tile_j=None, nt=None):
     nt = 'ls' if nt is None else nt
     load_fn = 'OVL_LOAD_NT' if 'l' in nt else 'OVL_LOAD_PLAIN'
     store_fn = 'OVL_STORE_NT' if 's' in nt else 'OVL_STORE_PLAIN'
-    vec = applicable(info)
-    assert vec is not None
+    assert applicable(info) is not None
+    vec, dim = _plan(info)
     # Measured on MI355X (float32 [16384, 16384], gather + transposed store): 32 x 256 workers per tile, i.e. one
     # 128-byte line per transposed output row and 1 KiB runs along j, runs at the speed of a plain copy (480 us against
     # 570 us for 64 x 64 and 549 us for 128 x 128).
     rank = len(info.workgroup_shape)
-    rows, cols = info.workgroup_shape[-2:]      # the two dimensions that a tile spans; those before them are batches
-    batch_shape = list(info.workgroup_shape[:-2])
+    # the two dimensions that a tile spans; the others are batches
+    rows, cols = info.workgroup_shape[dim], info.workgroup_shape[-1]
+    batch_dims = [k for k in range(rank - 1) if k != dim]
     batches = 1
-    for extent in batch_shape:
-        batches *= extent
-    pi, pj = 'p%d' % (rank - 2), 'p%d' % (rank - 1)
+    for k in batch_dims:
+        batches *= info.workgroup_shape[k]
+    pi, pj = 'p%d' % dim, 'p%d' % (rank - 1)
     pos_names = ['p%d' % k for k in range(rank)]
     accesses = info.tensor_accesses()
     widest = max(ITEMSIZE[tensor.dtype] for _, tensor, _ in accesses)
     tile_i = tile_i or TILE_I_BYTES // widest
+    while tile_i // 2 >= max(rows, vec, MIN_TILE_EXTENT):     # short tile dimensions: no rows of idle threads
+        tile_i //= 2
     tile_j = tile_j or TILE_J_BYTES // widest
+    while tile_j // 2 >= max(cols, vec, MIN_TILE_EXTENT):
+        tile_j //= 2
 
     loads = {}
     unaligned = {}
@@ -117,12 +156,12 @@ def generate(info, kernel_name, tile_i=None, tile_j=None, nt=None):
         else:
             if _is_vector_access(info, node, tensor, aff, vec):
                 store_keys.append((tensor.idx, aff.signature()))
-            elif _is_transposed_store(info, node, tensor, aff, vec):
+            elif _is_transposed_store(info, node, tensor, aff, vec, dim):
                 tkeys.append((tensor.idx, aff.signature()))
     certain = info.definitely_stores(store_keys + tkeys)
     bufferable = info.bufferable_outputs(
         lambda node, tensor, aff: (tensor.idx, aff.signature()) in certain and
-        (_is_vector_access(info, node, tensor, aff, vec) or _is_transposed_store(info, node, tensor, aff, vec)))
+        (_is_vector_access(info, node, tensor, aff, vec) or _is_transposed_store(info, node, tensor, aff, vec, dim)))
     for node, tensor, aff in accesses:
         if node.code != lang.ASSIGN_TENSOR or aff is None or tensor.idx not in bufferable:
             continue
@@ -188,11 +227,11 @@ def generate(info, kernel_name, tile_i=None, tile_j=None, nt=None):
     src.append('    for (uint32_t tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {')
     src.append('        const uint32_t i0 = (tile / %du %% %du) * %du;' % (tiles_j, tiles_i, tile_i))
     src.append('        const uint32_t j0 = (tile %% %du) * %du;' % (tiles_j, tile_j))
-    # the dimensions before the tile's two: one tile grid after the other
+    # the dimensions beside the tile's two: one tile grid after the other
     stride = tiles_i * tiles_j
-    for k in range(rank - 3, -1, -1):
-        src.append('        const uint32_t p%d = tile / %du %% %du;' % (k, stride, batch_shape[k]))
-        stride *= batch_shape[k]
+    for k in reversed(batch_dims):
+        src.append('        const uint32_t p%d = tile / %du %% %du;' % (k, stride, info.workgroup_shape[k]))
+        stride *= info.workgroup_shape[k]
     src.append('        const uint32_t tj = (threadIdx.x %% %du) * %du;' % (threads_per_row, vec))
     src.append('        #pragma unroll 1')
     src.append('        for (uint32_t ti = threadIdx.x / %du; ti < %du; ti += %du) {' % (
@@ -232,7 +271,8 @@ def generate(info, kernel_name, tile_i=None, tile_j=None, nt=None):
     # two neighbours to workgroups on one XCD at the same time made it slower, 744 us).  For whole lines the hint is
     # the faster form (484 against 494 us).
     tstore_fn = store_fn
-    if not nt_given and any((rows * ITEMSIZE[acc.tensor.dtype]) % 128 != 0 for acc in tstores.values()):
+    if not nt_given and any((acc.aff.coeff(('p', rank - 1)) * ITEMSIZE[acc.tensor.dtype]) % 128 != 0
+                            for acc in tstores.values()):
         tstore_fn = 'OVL_STORE_PLAIN'
     src.append('        const uint32_t oi = (threadIdx.x %% %du) * %du;' % (threads_per_col, vec))
     src.append('        #pragma unroll 1')

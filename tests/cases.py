@@ -211,10 +211,30 @@ def _swap_last_two(x, scale=None):
     return swapped, plain
 
 
+@ovl.operator()
+def _move_axis_last(x, axis=None, bias=None):
+    """out[.., rest.., x.shape[axis]]: the given axis becomes the last one, the others keep their order ([N, C, H, W]
+    with axis 1 gives [N, H, W, C]).  The store has unit stride along a workgroup dimension that is neither the last nor
+    the one before it, which the tile template takes as its second dimension."""
+    shape = list(x.shape)
+    order = [k for k in range(len(shape)) if k != axis] + [axis]
+    moved = ovl.output([shape[k] for k in order], x.dtype)
+    pos = ovl.position_in(x.shape)
+    moved[tuple(pos[k] for k in order)] = x[pos] + bias
+    return moved
+
+
 def batched_transposes(rng):
     return (all_outputs(_swap_last_two(rng.standard_normal((3, 70, 100), dtype=np.float32), scale=0.5)) +
             all_outputs(_swap_last_two(rng.standard_normal((2, 3, 66, 34)), scale=2.0)) +
             all_outputs(_swap_last_two(rng.integers(-100, 100, size=(5, 33, 35)).astype(np.int32), scale=3)))
+
+
+def moved_axes(rng):
+    return (all_outputs(_move_axis_last(rng.standard_normal((2, 24, 5, 36), dtype=np.float32), axis=1, bias=1.0)) +
+            all_outputs(_move_axis_last(rng.standard_normal((3, 9, 4, 3, 10)), axis=1, bias=0.5)) +
+            all_outputs(_move_axis_last(rng.standard_normal((40, 3, 33), dtype=np.float32), axis=0, bias=2.0)) +
+            all_outputs(_move_axis_last(rng.integers(-9, 9, size=(2, 3, 7, 64)).astype(np.int32), axis=1, bias=1)))
 
 
 def c4_lstm(rng, batch=32, units=128):
@@ -811,6 +831,7 @@ CASES = [
     Case('c5_gather_transpose', c5_gather_transpose, seed=5),
     Case('c5_variants', c5_variants, seed=5),
     Case('batched_transposes', batched_transposes, seed=5),
+    Case('moved_axes', moved_axes, seed=6),
     Case('row_reductions', row_reductions, seed=7),
     Case('col_reductions', col_reductions, seed=8),
     _simple('store_order', _store_order),
@@ -1176,6 +1197,8 @@ TEMPLATE_VARIANTS = [
     ('c5_variants', {'grid_cap': 2}),
     ('c5_variants', {'nt': 'l'}),
     ('batched_transposes', {'template': 'map'}),
+    ('moved_axes', {'template': 'map'}),
+    ('moved_axes', {'tile_i': 16, 'tile_j': 64}),
     ('col_reductions', {'template': 'map'}),
     ('col_reductions', {'scan_rows': 32, 'scan_batch': 2}),
     ('col_reductions', {'scan_sets': 3}),
