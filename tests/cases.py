@@ -1314,6 +1314,10 @@ def prebuild_all(cases=None, workers=8, with_oracle=True):
             ops[program.SerializeToString()] = program
             oracle_ops[program.SerializeToString()] = program
             variants.append((program, {'math': 'fast'}))
+        for seed in random_programs.REDUCE_SEEDS:
+            program = random_programs.reduce_application(seed).expression_dag
+            ops[program.SerializeToString()] = program
+            oracle_ops[program.SerializeToString()] = program
         for seed in random_programs.DAG_SEEDS:
             outs = random_programs.random_dag(seed)
             for level in (0, 3):

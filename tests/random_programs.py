@@ -347,6 +347,107 @@ SCAN_SEEDS = range(300, 324)
 
 
 # ----------------------------------------------------------------------------------------------------------------------
+# Random reduction programs: one worker per line walks one axis with loop-carried state and stores only after the loop
+# (sums, dot products of two inputs, sums of squares, running extrema, decayed sums; one or two state variables, an
+# epilogue on the final state).  Along the last axis the lengths sit on both sides of what the row-reduction template
+# wants (four groups of 64 vectors) with columns left over and unaligned rows; along another axis the line counts run
+# from one to more than a strip.
+# ----------------------------------------------------------------------------------------------------------------------
+REDUCE_DTYPES = [np.float32, np.float32, np.float64, np.int32, np.int64]
+REDUCE_LAST = [([3], 1024), ([5], 1030), ([2, 3], 1100), ([4], 2049), ([7], 1537), ([2], 512), ([3], 700), ([1], 4096)]
+REDUCE_OTHER = [([], 64, 200), ([], 100, 7), ([2], 257, 64), ([], 1000, 33), ([3], 70, 129), ([], 300, 1), ([], 64, 1000)]
+
+
+def reduce_program_shape(seed):
+    """(shape, axis, element type)"""
+    rng = random.Random(seed * 7919 + 3)
+    dtype = rng.choice(REDUCE_DTYPES)
+    if rng.random() < 0.5:
+        outer, length = rng.choice(REDUCE_LAST)
+        return outer + [length], len(outer), dtype
+    outer, length, inner = rng.choice(REDUCE_OTHER)
+    return outer + [length, inner], len(outer), dtype
+
+
+def make_reduce_operator(seed):
+    shape, axis, dtype = reduce_program_shape(seed)
+    floating = np.dtype(dtype).kind == 'f'
+
+    @ovl.operator()
+    def reduce_program(x, y):
+        rng = random.Random(seed)
+        length = x.shape[axis]
+        line_shape = [extent for k, extent in enumerate(x.shape) if k != axis]
+        pos = ovl.position_in(line_shape)
+        first_out = ovl.output(line_shape, x.dtype)
+        second_out = ovl.output(line_shape, x.dtype)
+
+        def at(i):
+            index = [pos[k] for k in range(len(line_shape))]
+            index.insert(axis, i)
+            return index
+
+        use_y = rng.random() < 0.4
+
+        def update(state, other, element, partner):
+            form = rng.randrange(8)
+            if form == 0:
+                return state + element
+            if form == 1:
+                return state + element * partner if use_y else state + element * element
+            if form == 2:
+                return ovl.maximum(state, element)
+            if form == 3:
+                return ovl.minimum(state, element)
+            if form == 4:
+                return state + element * element
+            if form == 5:
+                return state * 0.5 + element if floating else state - element
+            if form == 6 and other is not None:
+                return ovl.maximum(state, other)
+            if form == 7 and other is not None:
+                return state + other
+            return element - state
+
+        two_states = rng.random() < 0.4
+        from_first = rng.random() < 0.5
+        s0 = ovl.variable(x[at(0)] if from_first else 0, x.dtype)
+        s1 = ovl.variable(0, x.dtype) if two_states else None
+        for i in ovl.arange(1 if from_first else 0, length):
+            element = x[at(i)]
+            partner = y[at(i)] if use_y else None
+            s0 <<= update(s0, None, element, partner)
+            if two_states:
+                s1 <<= update(s1, s0, element, partner)
+        epilogue = rng.randrange(3)
+        if epilogue == 0 or not floating:
+            first_out[pos] = s0
+        elif epilogue == 1:
+            first_out[pos] = s0 / length
+        else:
+            first_out[pos] = ovl.sqrt(ovl.absolute(s0))
+        second_out[pos] = s1 + s0 if two_states else s0 * 2
+        return first_out, second_out
+    return reduce_program
+
+
+def reduce_inputs(seed):
+    shape, axis, dtype = reduce_program_shape(seed)
+    rng = np.random.default_rng(seed)
+    if np.dtype(dtype).kind == 'f':
+        return [(rng.uniform(0.7, 1.3, shape) * rng.choice([-1.0, 1.0], shape, p=[0.3, 0.7])).astype(dtype)
+                for _ in range(2)]
+    return [rng.integers(-3, 4, shape).astype(dtype) for _ in range(2)]
+
+
+def reduce_application(seed):
+    return make_reduce_operator(seed)(*reduce_inputs(seed))
+
+
+REDUCE_SEEDS = range(500, 524)
+
+
+# ----------------------------------------------------------------------------------------------------------------------
 # Random typed programs: element-wise expressions over all ten element types with casts between them, integer
 # division and remainder (C truncation), comparisons that yield 0/1 in the operand type, small counted loops and
 # worker-local tensors.  Inputs are small integers, so that no signed arithmetic overflows (undefined in C, for the

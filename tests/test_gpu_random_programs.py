@@ -108,3 +108,21 @@ def test_random_typed_program_equals_the_oracle(seed):
     got = ovl.evaluate(outs, opt_level=3)
     for k, (g, r) in enumerate(zip(got, ref)):
         assert g.dtype == r.dtype and g.shape == r.shape and np.array_equal(g, r), 'seed %d output %d' % (seed, k)
+
+
+@pytest.mark.parametrize('seed', random_programs.REDUCE_SEEDS)
+def test_random_reduction_program_equals_the_oracle(seed):
+    """Reductions along the last or another axis with one or two loop-carried variables, one or two inputs and an
+    epilogue on the final state, through whichever template the generator picks (row reduction, column reduction, or
+    the map kernel for short lines): the order of the oracle's loop, hence its bits."""
+    op = random_programs.reduce_application(seed)
+    outs = [op[0], op[1]]
+    ref = oracle.evaluate(outs)
+    runtime.poison_outputs = True
+    try:
+        got = ovl.evaluate(outs, opt_level=3)
+    finally:
+        runtime.poison_outputs = False
+    for k, (g, r) in enumerate(zip(got, ref)):
+        assert g.dtype == r.dtype and g.shape == r.shape, 'seed %d output %d' % (seed, k)
+        assert np.array_equal(g, r, equal_nan=(r.dtype.kind == 'f')), 'seed %d output %d' % (seed, k)

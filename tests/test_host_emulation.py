@@ -95,6 +95,9 @@ def test_random_programs_emulated_on_the_host_equal_the_oracle():
         jobs.append(('index program %d' % seed, [op[0], op[1]], 3, None))
     for seed in random_programs.SCAN_SEEDS:
         jobs.append(('scan program %d' % seed, [random_programs.scan_application(seed)[0]], 3, None))
+    for seed in random_programs.REDUCE_SEEDS:
+        op = random_programs.reduce_application(seed)
+        jobs.append(('reduction program %d' % seed, [op[0], op[1]], 3, None))
     for seed in random_programs.TYPED_SEEDS:
         op = random_programs.typed_application(seed)
         jobs.append(('typed program %d' % seed, [op[0], op[1]], 3, None))
