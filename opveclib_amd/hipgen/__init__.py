@@ -147,7 +147,7 @@ def generate(expression_dag, function_name, options=None):
                                                          reduce=True)
     elif options.get('vec') is None and template in ('auto', 'transpose') and tile_kernel.applicable(info) is not None:
         kernel_src, launch = tile_kernel.generate(info, kernel_name, options.get('tile_i'), options.get('tile_j'),
-                                                  options.get('nt'))
+                                                  options.get('nt'), options.get('tile_order'))
     else:
         kernel_src, launch = map_kernel.generate(info, kernel_name, options.get('vec'), options.get('nt'),
                                                  options.get('grid_cap'), options.get('per_thread'))

@@ -111,7 +111,7 @@ def applicable(info):
     return vec
 
 
-def generate(info, kernel_name, tile_i=None, tile_j=None, nt=None):
+def generate(info, kernel_name, tile_i=None, tile_j=None, nt=None, tile_order=None):
     nt_given = nt is not None
     nt = 'ls' if nt is None else nt
     load_fn = 'OVL_LOAD_NT' if 'l' in nt else 'OVL_LOAD_PLAIN'
@@ -135,7 +135,11 @@ def generate(info, kernel_name, tile_i=None, tile_j=None, nt=None):
     tile_i = tile_i or TILE_I_BYTES // widest
     while tile_i // 2 >= max(rows, vec, MIN_TILE_EXTENT):     # short tile dimensions: no rows of idle threads
         tile_i //= 2
-    tile_j = tile_j or TILE_J_BYTES // widest
+    # Narrower vectors, shorter tiles: a thread then has fewer bytes in flight, and the smaller tile lets more
+    # workgroups share a compute unit's LDS (float32 [8191, 8191], one element per access: 209 us with 32 x 256
+    # workers, 133 us with 32 x 128; [16382, 16386], two per access: 539 -> 492 us).
+    full_vec = max(1, 16 // widest)
+    tile_j = tile_j or max(TILE_J_BYTES // widest * vec // full_vec, TILE_J_BYTES // 2 // widest)
     while tile_j // 2 >= max(cols, vec, MIN_TILE_EXTENT):
         tile_j //= 2
 
@@ -222,15 +226,54 @@ def generate(info, kernel_name, tile_i=None, tile_j=None, nt=None):
         src.append('    OVL_DECLARE_MATH_TABLES();')
     for acc in tstores.values():
         src.append('    __shared__ %s %s[%d][%d];' % (CTYPE[acc.tensor.dtype], acc.reg, tile_j, tile_i + 1))
+    misaligned = any((acc.aff.coeff(('p', rank - 1)) * ITEMSIZE[acc.tensor.dtype]) % 128 != 0
+                     for acc in tstores.values())
     blocks_needed = batches * tiles_i * tiles_j
+    stripes = batches * tiles_j                 # a stripe: the tiles_i tiles that follow one another along i
+    order = tile_order or ('xcd' if misaligned else 'plain')
     src.append('    const uint32_t num_tiles = %du;' % blocks_needed)
     src.append('    for (uint32_t tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {')
-    src.append('        const uint32_t i0 = (tile / %du %% %du) * %du;' % (tiles_j, tiles_i, tile_i))
-    src.append('        const uint32_t j0 = (tile %% %du) * %du;' % (tiles_j, tile_j))
+    if order == 'xcd':
+        # Transposed output rows that are not whole 128-byte lines: two tiles that follow one another along i share
+        # the line their runs meet in (see phase 2).  Workgroups go to the eight XCDs in turn, each with an L2 of its
+        # own, so the tiles are numbered 64 stripes abreast (the stripes left over eight abreast, and what is then
+        # left side by side): the two that share lines are a multiple of eight workgroups apart, on one XCD and at
+        # work at the same time, and the line leaves that L2 whole.  float32 [16380, 16388], 65 tiles along j:
+        # 783 -> 467 us.  (A workgroup that takes its neighbour's tile itself a moment later is too late:
+        # [16380, 16384] 447 -> 766 us; eight abreast throughout reads shorter runs of each row: 447 -> 532 us.)
+        segments = []           # (first tile, first stripe, stripes abreast, groups)
+        first_tile, first_stripe = 0, 0
+        for abreast in (64, 8, 1):
+            left = stripes - first_stripe
+            if abreast == 1:
+                abreast = left
+            if left == 0 or left < abreast:
+                continue
+            groups = left // abreast
+            segments.append((first_tile, first_stripe, abreast, groups))
+            first_tile += groups * abreast * tiles_i
+            first_stripe += groups * abreast
+        src.append('        uint32_t stripe, along_i;')
+        for k, (first_tile, first_stripe, abreast, groups) in enumerate(segments):
+            last = k == len(segments) - 1
+            head = '        ' + ('' if k == 0 else '} else ') + \
+                ('{' if last and k > 0 else 'if (tile < %du) {' % (first_tile + groups * abreast * tiles_i) if not last
+                 else '{')
+            src.append(head)
+            src.append('            const uint32_t t = tile - %du;' % first_tile)
+            src.append('            stripe = %du + t / %du * %du + t %% %du;' % (
+                first_stripe, abreast * tiles_i, abreast, abreast))
+            src.append('            along_i = t %% %du / %du;' % (abreast * tiles_i, abreast))
+        src.append('        }')
+    else:
+        src.append('        const uint32_t stripe = tile / %du * %du + tile %% %du;' % (tiles_i * tiles_j, tiles_j, tiles_j))
+        src.append('        const uint32_t along_i = tile / %du %% %du;' % (tiles_j, tiles_i))
+    src.append('        const uint32_t i0 = along_i * %du;' % tile_i)
+    src.append('        const uint32_t j0 = (stripe %% %du) * %du;' % (tiles_j, tile_j))
     # the dimensions beside the tile's two: one tile grid after the other
-    stride = tiles_i * tiles_j
+    stride = tiles_j
     for k in reversed(batch_dims):
-        src.append('        const uint32_t p%d = tile / %du %% %du;' % (k, stride, info.workgroup_shape[k]))
+        src.append('        const uint32_t p%d = stripe / %du %% %du;' % (k, stride, info.workgroup_shape[k]))
         stride *= info.workgroup_shape[k]
     src.append('        const uint32_t tj = (threadIdx.x %% %du) * %du;' % (threads_per_row, vec))
     src.append('        #pragma unroll 1')
@@ -271,8 +314,7 @@ def generate(info, kernel_name, tile_i=None, tile_j=None, nt=None):
     # two neighbours to workgroups on one XCD at the same time made it slower, 744 us).  For whole lines the hint is
     # the faster form (484 against 494 us).
     tstore_fn = store_fn
-    if not nt_given and any((acc.aff.coeff(('p', rank - 1)) * ITEMSIZE[acc.tensor.dtype]) % 128 != 0
-                            for acc in tstores.values()):
+    if not nt_given and misaligned:
         tstore_fn = 'OVL_STORE_PLAIN'
     src.append('        const uint32_t oi = (threadIdx.x %% %du) * %du;' % (threads_per_col, vec))
     src.append('        #pragma unroll 1')

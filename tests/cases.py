@@ -264,7 +264,9 @@ def c5_variants(rng):
             c5_gather_transpose(rng, (6, 10), stride=1) +
             # extents that leave two elements, or one, per access
             c5_gather_transpose(rng, (70, 102), stride=11) + c5_gather_transpose(rng, (67, 101), stride=3) +
-            c5_gather_transpose(rng, (35, 129), stride=2, dtype=np.float64))
+            c5_gather_transpose(rng, (35, 129), stride=2, dtype=np.float64) +
+            # (75 tiles along j once the tiles are forced down to 8 x 8)
+            c5_gather_transpose(rng, (24, 600), stride=13))
 
 
 # ----------------------------------------------------------------------------------------------------------------------
@@ -1199,6 +1201,10 @@ TEMPLATE_VARIANTS = [
     ('batched_transposes', {'template': 'map'}),
     ('moved_axes', {'template': 'map'}),
     ('moved_axes', {'tile_i': 16, 'tile_j': 64}),
+    ('moved_axes', {'tile_order': 'plain'}),
+    # (tiles of 8 x 8 workers: groups of 64 stripes, of eight, and stripes left over in one kernel)
+    ('c5_variants', {'tile_i': 8, 'tile_j': 8, 'tile_order': 'xcd'}),
+    ('batched_transposes', {'tile_i': 8, 'tile_j': 8, 'tile_order': 'xcd'}),
     ('col_reductions', {'template': 'map'}),
     ('col_reductions', {'scan_rows': 32, 'scan_batch': 2}),
     ('col_reductions', {'scan_sets': 3}),
