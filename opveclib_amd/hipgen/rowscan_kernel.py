@@ -649,20 +649,49 @@ def reduce_plan(info):
     for k in range(rank - 2, -1, -1):
         stride *= info.workgroup_shape[k + 1]
         wg_stride[k] = stride
-    in_loop = dict((('p', k), length * wg_stride[k]) for k in range(rank) if info.workgroup_shape[k] > 1)
-    in_loop[('v', counter)] = 1
-    sig_loop = (tuple(sorted(in_loop.items())), 0)
+    def layout_of(aff):
+        """(elements between the rows of two consecutive workers, offset of column 0) of an access that walks a
+        row with the loop counter: a matrix row (row stride = its row length, or more for a slice of wider rows) or
+        one vector that every worker reads (row stride 0)."""
+        if aff is None or aff.coeff(('v', counter)) != 1:
+            return None
+        row_stride = None
+        for sym, c in aff.coeffs.items():
+            if sym == ('v', counter):
+                continue
+            if sym[0] != 'p':
+                return None
+            k = sym[1]
+            if info.workgroup_shape[k] == 1:
+                continue
+            if c % wg_stride[k] != 0 or (row_stride is not None and c // wg_stride[k] != row_stride):
+                return None
+            row_stride = c // wg_stride[k]
+        moving = [k for k in range(rank) if info.workgroup_shape[k] > 1]
+        if row_stride is None:
+            row_stride = 0
+        elif any(aff.coeff(('p', k)) != row_stride * wg_stride[k] for k in moving):
+            return None
+        if row_stride < 0 or aff.const < 0:
+            return None
+        return row_stride, aff.const
 
     tensors = []
+    layouts = {}
     for node, tensor, aff in info.tensor_accesses():
         if not info.in_loop[node.idx]:
             continue                    # before and after the loop: ordinary code of one lane
-        if node.code != lang.READ_TENSOR or tensor.code != lang.INPUT or aff is None or aff.signature() != sig_loop:
+        if node.code != lang.READ_TENSOR or tensor.code != lang.INPUT or tensor.dtype not in CTYPE:
             return None
-        if tensor.size != rows * length or tensor.dtype not in CTYPE:
+        layout = layout_of(aff)
+        if layout is None or layouts.setdefault(tensor.idx, layout) != layout:
+            return None
+        if aff.lo < 0 or aff.hi >= tensor.size:
             return None
         if tensor not in tensors:
             tensors.append(tensor)
+    if all(layouts[t.idx][0] == 0 for t in tensors):
+        return None                     # no worker reads a row of its own
     if not tensors or len(tensors) > 4:
         return None
     itemsize = ITEMSIZE[tensors[0].dtype]
@@ -675,6 +704,7 @@ def reduce_plan(info):
     if len([n for n in info.nodes if info.in_loop[n.idx]]) > SKEW_MAX_BODY:
         return None
     p = ReducePlan(loop, end_idx, counter, start, length, rows, tensors, vec)
+    p.layouts = layouts
     state = _carried_state(info, p)
     if not state or any(info.nodes[idx].dtype not in CTYPE for idx in state):
         return None
@@ -693,7 +723,9 @@ def generate_reduce(info, kernel_name, depth=None, width=None):
     group_cols = GROUP_LANES * vec * width
     num_groups = p.length // group_cols
     tail_cols = p.length % group_cols
-    aligned = (p.length * itemsize) % 16 == 0
+    # rows that start wherever the one before ends: vectors in memory are then only aligned like their elements
+    aligned = dict((t.idx, (p.layouts[t.idx][0] * itemsize) % 16 == 0 and (p.layouts[t.idx][1] * itemsize) % 16 == 0)
+                   for t in p.tensors)
     depth = max(1, min(depth or max(1, 4 // width), num_groups))
     rows_per_wave = WAVE // GROUP_LANES
     waves = BLOCK // WAVE
@@ -735,9 +767,7 @@ def generate_reduce(info, kernel_name, depth=None, width=None):
             vname = 'ovl_reduce_' + ctype.replace(' ', '_') + 'x%d' % vec
             vnames[ctype] = vname
             src.append('typedef %s %s __attribute__((ext_vector_type(%d)));' % (ctype, vname, vec))
-            if not aligned:
-                # rows start wherever the one before ends: vectors in memory are only aligned like their elements
-                src.append('typedef %s %s_u __attribute__((aligned(%d)));' % (vname, vname, itemsize))
+            src.append('typedef %s %s_u __attribute__((aligned(%d)));' % (vname, vname, itemsize))
     src.append('')
     args = ['const %s* __restrict__ in%d' % (CTYPE[info.inputs[i].dtype], i) for i in range(len(info.inputs))]
     args += ['%s* __restrict__ out%d' % (CTYPE[info.outputs[i].dtype], i) for i in range(len(info.outputs))]
@@ -754,8 +784,8 @@ def generate_reduce(info, kernel_name, depth=None, width=None):
         waves, WAVE, rows_per_wave, GROUP_LANES))
     src.append('    const uint32_t row = row_raw < %du ? row_raw : %du;' % (p.rows, p.rows - 1))
     for t in p.tensors:
-        src.append('    const %s* __restrict__ gin%d = in%d + (uint64_t)row * %dull + part * %du;' % (
-            CTYPE[t.dtype], t.io_index, t.io_index, p.length, vec * width))
+        src.append('    const %s* __restrict__ gin%d = in%d + (uint64_t)row * %dull + %dull + part * %du;' % (
+            CTYPE[t.dtype], t.io_index, t.io_index, p.layouts[t.idx][0], p.layouts[t.idx][1], vec * width))
     batch = depth
     num_batches = num_groups // batch
     tail = num_groups % batch
@@ -764,7 +794,7 @@ def generate_reduce(info, kernel_name, depth=None, width=None):
     def request(k, batch_expr, nb, suffix):
         for t in p.tensors:
             vname = vnames[CTYPE[t.dtype]]
-            mname = vname if aligned else vname + '_u'
+            mname = vname if aligned[t.idx] else vname + '_u'
             src.append('        #pragma unroll')
             src.append('        for (uint32_t j = 0; j < %du; ++j)' % nb)
             src.append('            #pragma unroll')
@@ -866,13 +896,12 @@ def generate_reduce(info, kernel_name, depth=None, width=None):
     src.append('#undef OVL_REDUCE_STEP')
     src.append('}')
 
-    row_align = 16 if aligned else itemsize
     launch = {
         'template': 'rowreduce',
         'vec': vec,
         'block': BLOCK,
         'blocks_needed': (p.rows + rows_per_block - 1) // rows_per_block,
-        'align': dict((('in', t.io_index), row_align) for t in p.tensors),
+        'align': dict((('in', t.io_index), 16 if aligned[t.idx] else itemsize) for t in p.tensors),
         'vector_loads': len(p.tensors),
         'vector_stores': 0,
     }

@@ -468,6 +468,34 @@ def _row_int_sum(x):
     return out
 
 
+@ovl.operator()
+def _matrix_vector(m, v, first=None, count=None):
+    """y[.., r] = sum over columns first .. first+count-1 of m[.., r, c] * v[c - first]: every worker walks a slice
+    of its own matrix row and the one vector all workers share."""
+    shape = list(m.shape)
+    out = ovl.output(shape[:-1], m.dtype)
+    pos = ovl.position_in(shape[:-1])
+    acc = ovl.variable(0, m.dtype)
+    for j in ovl.arange(count):
+        index = tuple(pos[k] for k in range(len(shape) - 1)) + (j + first,)
+        acc <<= acc + m[index] * v[j]
+    out[pos] = acc
+    return out
+
+
+@ovl.operator()
+def _two_offsets(x):
+    """One tensor read at two offsets in the loop (a row's lag-1 products): not the row reduction's shape."""
+    rows, cols = x.shape
+    out = ovl.output([rows], x.dtype)
+    pos = ovl.position_in([rows])[0]
+    acc = ovl.variable(0, x.dtype)
+    for j in ovl.arange(cols - 1):
+        acc <<= acc + x[pos, j] * x[pos, j + 1]
+    out[pos] = acc
+    return out
+
+
 def row_reductions(rng):
     """Reductions along the last axis: rows of whole groups, rows with columns left over, rows that are not 16-byte
     aligned, a rank-3 tensor, 4- and 8-byte elements, integers."""
@@ -481,7 +509,14 @@ def row_reductions(rng):
     return ([_row_dot(a, b), _row_dot(c, d), _row_dot(e, f), dot(rng.standard_normal((9, 300)), rng.standard_normal((9, 300)))] +
             all_outputs(_row_norm_and_max(rng.standard_normal((9, 131)))) + all_outputs(_row_norm_and_max(rng.standard_normal((9, 80)))) +
             all_outputs(_row_norm_and_max(rng.standard_normal((70, 1000), dtype=np.float32))) +
-            [_row_int_sum(rng.integers(-50, 50, size=(6, 270)).astype(np.int32))])
+            [_row_int_sum(rng.integers(-50, 50, size=(6, 270)).astype(np.int32)),
+             # matrix times vector: whole rows, a slice that leaves the rows' vectors unaligned, rank 3
+             _matrix_vector(rng.standard_normal((9, 320), dtype=np.float32),
+                            rng.standard_normal(320, dtype=np.float32), first=0, count=320),
+             _matrix_vector(rng.standard_normal((5, 400)), rng.standard_normal(300), first=37, count=300),
+             _matrix_vector(rng.standard_normal((2, 3, 301), dtype=np.float32),
+                            rng.standard_normal(301, dtype=np.float32), first=0, count=301),
+             _two_offsets(rng.standard_normal((6, 300), dtype=np.float32))])
 
 
 @ovl.operator()
