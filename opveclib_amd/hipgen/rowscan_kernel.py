@@ -45,11 +45,13 @@ class ScanPlan(object):
         self.chunk = chunk
 
 
-def plan(info, rows_per_block=None, chunk=None, need_chunk=True):
+def plan(info, rows_per_block=None, chunk=None, need_chunk=True, multi=False):
     """A ScanPlan when the DAG is a last-axis row scan this template can run, else None.  ``need_chunk``: the LDS
-    templates stream rows in chunks that divide them; the lane-skewed scan does not."""
+    templates stream rows in chunks that divide them; the lane-skewed scan does not.  ``multi``: the body may read
+    several inputs of the output's shape and type (a gated recurrence ``h = a[r, i] * h + x[r, i]``); the lane-skewed
+    scan takes up to four, the other templates one."""
     forced_rows, forced_chunk = rows_per_block, chunk
-    if len(info.inputs) != 1 or len(info.outputs) != 1:
+    if not info.inputs or len(info.inputs) > (4 if multi else 1) or len(info.outputs) != 1:
         return None
     loops = [item for item in info.tree if item.kind == 'loop']
     if len(loops) != 1 or any(item.kind == 'if' for item in info.tree):
@@ -90,6 +92,7 @@ def plan(info, rows_per_block=None, chunk=None, need_chunk=True):
     sig_loop = (tuple(sorted(in_loop.items())), 0)
 
     x = out = None
+    xs = []
     for node, tensor, aff in info.tensor_accesses():
         if aff is None:
             return None
@@ -97,16 +100,18 @@ def plan(info, rows_per_block=None, chunk=None, need_chunk=True):
         if aff.signature() != expect:
             return None
         if node.code == lang.READ_TENSOR:
-            if x is not None and x is not tensor:
-                return None
-            x = tensor
+            if tensor not in xs:
+                xs.append(tensor)
+            x = xs[0]
         else:
             if out is not None and out is not tensor:
                 return None
             out = tensor
-    if x is None or out is None or x.dtype != out.dtype:
+    if x is None or out is None or len(xs) != len(info.inputs):
         return None
-    if x.size != rows * length or out.size != rows * length:
+    if any(t.code != lang.INPUT or t.dtype != out.dtype or t.size != rows * length for t in xs):
+        return None
+    if out.size != rows * length:
         return None
     itemsize = ITEMSIZE[x.dtype]
     if itemsize not in (4, 8) or x.dtype not in CTYPE:
@@ -122,7 +127,9 @@ def plan(info, rows_per_block=None, chunk=None, need_chunk=True):
             break
     if chunk is None and need_chunk:
         return None
-    return ScanPlan(loop, counter, length, rows, x, out, vec, rows_per_block, chunk)
+    p = ScanPlan(loop, counter, length, rows, x, out, vec, rows_per_block, chunk)
+    p.xs = xs           # every input the body reads, in the order of their first use; x is the first
+    return p
 
 
 def _emit_movers(src, p, ctype, vname, vec, chunk, rpb, num_chunks, lds_column=None):
@@ -405,7 +412,7 @@ def skew_plan(info):
     """The structural plan when the lane-skewed variant can run this DAG, else None."""
     # (a row need not be a whole number of groups of 16 * VEC columns, nor aligned: what is left after the last whole
     # group is scanned by one lane, and rows that do not start on 16-byte boundaries are moved with unaligned vectors)
-    p = plan(info, need_chunk=False)
+    p = plan(info, need_chunk=False, multi=True)
     if p is None or p.length < GROUP_LANES * p.vec:
         return None
     body_nodes = [n for n in info.nodes if info.in_loop[n.idx]]
@@ -438,7 +445,7 @@ FED_ROWS = WAVE // GROUP_LANES      # rows per workgroup: one group of sixteen l
 def fed_plan(info, width=None, chunk=None):
     """(ScanPlan, width, chunk) when the LDS-fed lane-skewed variant can run this DAG, else None."""
     p = skew_plan(info)
-    if p is None or p.length % (GROUP_LANES * p.vec) != 0:
+    if p is None or len(p.xs) != 1 or p.length % (GROUP_LANES * p.vec) != 0:
         return None
     itemsize = ITEMSIZE[p.x.dtype]
     width = width or 8
@@ -1077,7 +1084,7 @@ def _for_slot(text, slot):
     if slot == 0:
         return text
     suffix = '_r%d' % slot
-    text = re.sub(r'\b(carry_e\d+|e\d+|position|row_raw|row|gin|gout|q\d+|qt|ov|xv|first_out|OVL_SCAN_STEP)\b',
+    text = re.sub(r'\b(carry_e\d+|e\d+|position|row_raw|row|gin\d*|gout|q\d+|qt\d*|ov|xv\d*|first_out|OVL_SCAN_STEP)\b',
                   lambda m: m.group(1) + suffix, text)
     return text
 
@@ -1132,8 +1139,18 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
             expr = '(row % ' + str(strides[k - 1]) + 'u)'
         pos_exprs.append(expr + ' / ' + str(strides[k]) + 'u')
 
+    # the inputs the body reads, numbered in the order of their first use: each has its pointer, register sets and
+    # vector of the moment under a name with that number (the first without one)
+    number = dict((t.idx, k) for k, t in enumerate(p.xs))
+    tag = lambda k: '' if k == 0 else str(k)
+
+    def set_name(regs, k):
+        if k == 0:
+            return regs
+        return 'qt%d' % k if regs == 'qt' else 'q%d' % (int(regs[1:]) + 10 * k)
+
     emitter = BodyEmitter(info, pos_exprs,
-                          read_hook=lambda node, tensor, idx: 'OVL_SCAN_IN',
+                          read_hook=lambda node, tensor, idx: 'OVL_SCAN_IN_T%d' % number[tensor.idx],
                           store_hook=lambda node, tensor, idx, value: 'OVL_SCAN_OUT(' + value + ');')
     tagged = emitter.emit_tagged()
     range_idx = p.loop_item.node
@@ -1161,8 +1178,9 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
         src.append('typedef %s %s __attribute__((aligned(%d)));' % (vname, mname, ITEMSIZE[p.x.dtype]))
     src.append('')
     src.append('extern "C" __global__ void __launch_bounds__(%d)' % BLOCK)
-    src.append('%s(const %s* __restrict__ in%d, %s* __restrict__ out%d) {' % (
-        kernel_name, ctype, p.x.io_index, ctype, p.out.io_index))
+    src.append('%s(%s, %s* __restrict__ out%d) {' % (
+        kernel_name, ', '.join('const %s* __restrict__ in%d' % (CTYPE[info.inputs[i].dtype], i) for i in range(len(info.inputs))),
+        ctype, p.out.io_index))
     if info.uses_math_tables():
         src.append('    OVL_DECLARE_MATH_TABLES();')
     src.append('    const uint32_t lane = threadIdx.x %% %du;' % WAVE)
@@ -1177,11 +1195,11 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
             raw = '(blockIdx.x * %du + threadIdx.x / %du) * %du + (lane / %du) * %du + %du' % (
                 waves, WAVE, rows_per_wave, GROUP_LANES, interleave, slot)
         src.append(_for_slot('    const uint32_t row_raw = %s;' % raw, slot))
-    emit(['    const uint32_t row = row_raw < %du ? row_raw : %du;' % (p.rows, p.rows - 1),
-          '    const %s* __restrict__ gin = in%d + (uint64_t)row * %dull + part * %du;' % (
-              ctype, p.x.io_index, p.length, vec * width),
-          '    %s* __restrict__ gout = out%d + (uint64_t)row * %dull + part * %du;' % (
-              ctype, p.out.io_index, p.length, vec * width)])
+    emit(['    const uint32_t row = row_raw < %du ? row_raw : %du;' % (p.rows, p.rows - 1)] +
+         ['    const %s* __restrict__ gin%s = in%d + (uint64_t)row * %dull + part * %du;' % (
+             ctype, tag(k), t.io_index, p.length, vec * width) for k, t in enumerate(p.xs)] +
+         ['    %s* __restrict__ gout = out%d + (uint64_t)row * %dull + part * %du;' % (
+             ctype, p.out.io_index, p.length, vec * width)])
     # measured on MI355X (float32 [4096, 16384]): non-temporal stores with plain loads 85 us, hint on both 100 us,
     # on the loads only 90 us, on neither 102 us
     batch = depth
@@ -1192,17 +1210,18 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
     def request(regs, batch_expr, nb=None):
         """All loads of one batch (of nb groups), back to back: every row is read in runs of batch * 256 bytes."""
         nb = nb or batch
-        lines = ['        #pragma unroll',
-                 '        for (uint32_t j = 0; j < %du; ++j)' % nb,
-                 '            #pragma unroll',
-                 '            for (uint32_t w = 0; w < %du; ++w)' % width]
-        if 'l' in nt:
-            lines.append('                %s[j][w] = __builtin_nontemporal_load(reinterpret_cast<const %s*>(gin + (%s) * %du + j * %du + w * %du));' % (
-                regs, mname, batch_expr, batch_cols, group_cols, vec))
-        else:
-            lines.append('                %s[j][w] = *(reinterpret_cast<const %s*>(gin + (%s) * %du + j * %du + w * %du));' % (
-                regs, mname, batch_expr, batch_cols, group_cols, vec))
-        emit(lines)
+        for k in range(len(p.xs)):
+            lines = ['        #pragma unroll',
+                     '        for (uint32_t j = 0; j < %du; ++j)' % nb,
+                     '            #pragma unroll',
+                     '            for (uint32_t w = 0; w < %du; ++w)' % width]
+            if 'l' in nt:
+                lines.append('                %s[j][w] = __builtin_nontemporal_load(reinterpret_cast<const %s*>(gin%s + (%s) * %du + j * %du + w * %du));' % (
+                    set_name(regs, k), mname, tag(k), batch_expr, batch_cols, group_cols, vec))
+            else:
+                lines.append('                %s[j][w] = *(reinterpret_cast<const %s*>(gin%s + (%s) * %du + j * %du + w * %du));' % (
+                    set_name(regs, k), mname, tag(k), batch_expr, batch_cols, group_cols, vec))
+            emit(lines)
 
     def process(regs, batch_expr, refill_expr, nb=None):
         nb = nb or batch
@@ -1220,7 +1239,7 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
         emit(['                %s = carry_%s;' % (name, name) for name, _ in state])
         src.append('                #pragma unroll')
         src.append('                for (uint32_t w = 0; w < %du; ++w) {' % width)
-        emit(['                    const %s xv = %s[j][w];' % (vname, regs)])
+        emit(['                    const %s xv%s = %s[j][w];' % (vname, tag(k), set_name(regs, k)) for k in range(len(p.xs))])
         src.append('                    #pragma unroll')
         src.append('                    for (uint32_t u = 0; u < %du; ++u) {' % vec)
         emit(['                        if (w == 0u && u == 0u && first_column) ov[j][0][0] = first_out;',
@@ -1255,10 +1274,11 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
 
     sets = max(2, min(sets or 2, num_batches)) if num_batches > 1 else 1
     src.append('    // %d register sets of %d groups each: one is consumed while the others are in flight' % (sets, batch))
-    emit(['    %s %s;' % (vname, ', '.join('q%d[%d][%d]' % (k, batch, width) for k in range(sets)))])
+    emit(['    %s %s;' % (vname, ', '.join('%s[%d][%d]' % (set_name('q%d' % k, t), batch, width) for k in range(sets)))
+          for t in range(len(p.xs))])
     if tail:
         src.append('    // ... and the %d groups that end the row, requested now and held until the end' % tail)
-        emit(['    %s qt[%d][%d];' % (vname, tail, width)])
+        emit(['    %s %s[%d][%d];' % (vname, set_name('qt', t), tail, width) for t in range(len(p.xs))])
     src.append('    {')
     for k in range(sets if num_batches else 0):
         request('q%d' % k, '%du' % k)
@@ -1269,10 +1289,13 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
     for slot in slots:
         emit_one = lambda lines: src.extend(_for_slot(line, slot) for line in lines)
         emit_one(['    %s first_out;' % ctype])
-        src.append('#define OVL_SCAN_IN (in%d[(uint64_t)%s * %dull])' % (p.x.io_index, _for_slot('row', slot), p.length))
+        for k, t in enumerate(p.xs):
+            src.append('#define OVL_SCAN_IN_T%d (in%d[(uint64_t)%s * %dull])' % (
+                k, t.io_index, _for_slot('row', slot), p.length))
         src.append('#define OVL_SCAN_OUT(value) %s = (value)' % _for_slot('first_out', slot))
         emit_one(['    ' + stmt for stmt in prologue])
-        src.append('#undef OVL_SCAN_IN')
+        for k in range(len(p.xs)):
+            src.append('#undef OVL_SCAN_IN_T%d' % k)
         src.append('#undef OVL_SCAN_OUT')
         emit_one(['    %s carry_%s = %s;' % (stype, name, name) for name, stype in state])
     for slot in slots:
@@ -1280,7 +1303,8 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
         src.append(_for_slot('#define OVL_SCAN_STEP(column) { %s = (%s)(column); %s }' % (
             counter_name, counter_type, ' '.join(body)), slot).replace(
                 'OVL_SCAN_OUT(', 'OVL_SCAN_OUT_R%d(' % slot).replace('OVL_SCAN_IN', 'OVL_SCAN_IN_R%d' % slot))
-        src.append('#define OVL_SCAN_IN_R%d %s[u]' % (slot, _for_slot('xv', slot)))
+        for k in range(len(p.xs)):
+            src.append('#define OVL_SCAN_IN_R%d_T%d %s[u]' % (slot, k, _for_slot('xv' + tag(k), slot)))
         src.append('#define OVL_SCAN_OUT_R%d(value) %s[j][w][u] = (value)' % (slot, _for_slot('ov', slot)))
     rounds = num_batches // sets
     last = num_batches - 1
@@ -1304,8 +1328,9 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
         # last group and runs the worker's loop over them, one column at a time (fewer than %d columns).
         for slot in slots:
             src.append('#undef OVL_SCAN_OUT_R%d' % slot)
-            src.append('#undef OVL_SCAN_IN_R%d' % slot)
-            src.append('#define OVL_SCAN_IN_R%d tail_in' % slot)
+            for k in range(len(p.xs)):
+                src.append('#undef OVL_SCAN_IN_R%d_T%d' % (slot, k))
+                src.append('#define OVL_SCAN_IN_R%d_T%d tail_in%s' % (slot, k, tag(k)))
             src.append('#define OVL_SCAN_OUT_R%d(value) tail_out = (value)' % slot)
         src.append('    if (part == 0u) {')
         for slot in slots:
@@ -1314,8 +1339,8 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
             one(['        %s = carry_%s;' % (name, name) for name, _ in state])
             src.append('        #pragma unroll 1')
             src.append('        for (uint32_t column = %du; column < %du; ++column) {' % (num_groups * group_cols, p.length))
-            one(['            const %s tail_in = gin[column];' % ctype,
-                 '            %s tail_out;' % ctype,
+            one(['            const %s tail_in%s = gin%s[column];' % (ctype, tag(k), tag(k)) for k in range(len(p.xs))] +
+                ['            %s tail_out;' % ctype,
                  '            OVL_SCAN_STEP(column)',
                  '            gout[column] = tail_out;'])
             src.append('        }')
@@ -1324,7 +1349,8 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
     for slot in slots:
         src.append('#undef %s' % _for_slot('OVL_SCAN_STEP', slot))
         src.append('#undef OVL_SCAN_OUT_R%d' % slot)
-        src.append('#undef OVL_SCAN_IN_R%d' % slot)
+        for k in range(len(p.xs)):
+            src.append('#undef OVL_SCAN_IN_R%d_T%d' % (slot, k))
     src.append('}')
 
     row_align = 16 if aligned else ITEMSIZE[p.x.dtype]
@@ -1333,8 +1359,8 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
         'vec': vec,
         'block': BLOCK,
         'blocks_needed': (p.rows + rows_per_block - 1) // rows_per_block,
-        'align': {('in', p.x.io_index): row_align, ('out', p.out.io_index): row_align},
-        'vector_loads': 1,
+        'align': dict([(('in', t.io_index), row_align) for t in p.xs] + [(('out', p.out.io_index), row_align)]),
+        'vector_loads': len(p.xs),
         'vector_stores': 1,
     }
     return '\n'.join(src) + '\n', launch

@@ -496,6 +496,57 @@ def _two_offsets(x):
     return out
 
 
+def _gated_body(a, x, b):
+    shape = list(x.shape)
+    out = ovl.output_like(x)
+    pos = ovl.position_in(shape[:-1])
+
+    def at(i):
+        return tuple(pos[k] for k in range(len(shape) - 1)) + (i,)
+
+    h = ovl.variable(x[at(0)], x.dtype)
+    out[at(0)] = h
+    for i in ovl.arange(1, shape[-1]):
+        if b is None:
+            h <<= a[at(i)] * h + x[at(i)]
+        else:
+            h <<= a[at(i)] * h + x[at(i)] * b[at(i)]
+        out[at(i)] = h
+    return out
+
+
+@ovl.operator()
+def _gated_scan(a, x):
+    """A gated linear recurrence along the last axis, h = a[.., i] * h + x[.., i]: a row scan whose body reads two
+    inputs of the output's shape."""
+    return _gated_body(a, x, None)
+
+
+@ovl.operator()
+def _gated_scan3(a, x, b):
+    """h = a[.., i] * h + x[.., i] * b[.., i]: three inputs."""
+    return _gated_body(a, x, b)
+
+
+def gated_scans(rng):
+    """Row scans over several inputs: whole groups, columns left over, unaligned rows, rank 3, 8-byte elements, a row
+    shorter than one group (which stays on the general kernel)."""
+    def gate(shape, dtype):
+        return rng.uniform(0.5, 1.0, shape).astype(dtype)
+
+    def data(shape, dtype):
+        return rng.standard_normal(shape).astype(dtype)
+    outs = []
+    for shape, dtype, three in [((7, 256), np.float32, False), ((5, 333), np.float32, True), ((3, 131), np.float32, False),
+                                ((2, 3, 200), np.float64, True), ((9, 1024), np.float64, False),
+                                ((4, 40), np.float32, False), ((67, 640), np.float32, True)]:
+        if three:
+            outs.append(_gated_scan3(gate(shape, dtype), data(shape, dtype), data(shape, dtype)))
+        else:
+            outs.append(_gated_scan(gate(shape, dtype), data(shape, dtype)))
+    return outs
+
+
 def row_reductions(rng):
     """Reductions along the last axis: rows of whole groups, rows with columns left over, rows that are not 16-byte
     aligned, a rank-3 tensor, 4- and 8-byte elements, integers."""
@@ -870,6 +921,7 @@ CASES = [
     Case('batched_transposes', batched_transposes, seed=5),
     Case('moved_axes', moved_axes, seed=6),
     Case('row_reductions', row_reductions, seed=7),
+    Case('gated_scans', gated_scans, seed=8),
     Case('col_reductions', col_reductions, seed=8),
     _simple('store_order', _store_order),
     _simple('clip', lambda rng: [clip(rng.random(1000), threshold1=0.1, threshold2=0.9)[0]]),
@@ -1215,6 +1267,10 @@ TEMPLATE_VARIANTS = [
     ('c4_lstm_grad', {'per_thread': 2}),
     ('c4_lstm_grad', {'cse': False}),
     ('c3_rowscan_shapes', {'template': 'skewscan', 'scan_depth': 1, 'scan_sets': 3}),
+    ('gated_scans', {'scan_depth': 1, 'scan_sets': 3}),
+    ('gated_scans', {'scan_interleave': 2}),
+    ('gated_scans', {'scan_width': 2, 'scan_nt': 'l'}),
+    ('gated_scans', {'template': 'map'}),
     ('c3_cumsum_f32', {'template': 'skewscan', 'scan_depth': 2, 'scan_sets': 2}),
     ('c3_cumsum_f32', {'template': 'skewscan', 'scan_width': 2}),
     ('c3_cumprod_f64', {'template': 'skewscan', 'scan_width': 1}),
