@@ -129,7 +129,8 @@ def generate(expression_dag, function_name, options=None):
     elif options.get('vec') is None and template in ('auto', 'rowreduce') and rowscan_kernel.reduce_plan(info) is not None:
         # a loop-carried state over the last axis with nothing stored inside the loop: a dot product, a sum
         kernel_src, launch = rowscan_kernel.generate_reduce(info, kernel_name, options.get('scan_depth'),
-                                                            options.get('scan_width'))
+                                                            options.get('scan_width'), options.get('scan_sets'),
+                                                            options.get('scan_nt', ''))
     elif options.get('vec') is None and template in ('auto', 'colreduce') and \
             colscan_kernel.reduce_plan(info, options.get('scan_rows'), options.get('scan_batch'),
                                        options.get('scan_sets')) is not None and \

@@ -718,13 +718,20 @@ def reduce_plan(info):
     return p
 
 
-def generate_reduce(info, kernel_name, depth=None, width=None):
+def generate_reduce(info, kernel_name, depth=None, width=None, sets=None, nt=''):
     p = reduce_plan(info)
     assert p is not None
     vec = p.vec
     itemsize = 16 // vec
+    # width = 128-bit vectors per lane and phase.  With nothing to store, a reduction gains from wider lanes than a scan
+    # does: the hand-over between lanes comes once per VEC * width columns (measured on MI355X, [4096, 16384] float32,
+    # widths 1 / 2 / 4 / 8: row sum 58 / 46 / 44 / 45 us, dot product 98 / 93 / 91 / 104 us; float64 [1024, 16384] row
+    # sum 94 / 66 / 52 / 61 us).  The columns after the last whole group are walked by one lane, so a width is taken
+    # only if it leaves few of them.
     if width is None:
-        width = 2 if vec == 2 else 1
+        width = 4
+        while width > 1 and p.length % (GROUP_LANES * vec * width) >= max(GROUP_LANES * vec, p.length // 32):
+            width //= 2
     while width > 1 and p.length < GROUP_LANES * vec * width:
         width //= 2
     group_cols = GROUP_LANES * vec * width
@@ -733,7 +740,7 @@ def generate_reduce(info, kernel_name, depth=None, width=None):
     # rows that start wherever the one before ends: vectors in memory are then only aligned like their elements
     aligned = dict((t.idx, (p.layouts[t.idx][0] * itemsize) % 16 == 0 and (p.layouts[t.idx][1] * itemsize) % 16 == 0)
                    for t in p.tensors)
-    depth = max(1, min(depth or max(1, 4 // width), num_groups))
+    depth = max(1, min(depth or (2 if width == 4 else max(1, 4 // width)), num_groups))
     rows_per_wave = WAVE // GROUP_LANES
     waves = BLOCK // WAVE
     rows_per_block = rows_per_wave * waves
@@ -806,8 +813,9 @@ def generate_reduce(info, kernel_name, depth=None, width=None):
             src.append('        for (uint32_t j = 0; j < %du; ++j)' % nb)
             src.append('            #pragma unroll')
             src.append('            for (uint32_t w = 0; w < %du; ++w)' % width)
-            src.append('                q%d%s[j][w] = *reinterpret_cast<const %s*>(gin%d + (%s) * %du + j * %du + w * %du);' % (
-                t.io_index, suffix, mname, t.io_index, batch_expr, batch_cols, group_cols, vec))
+            src.append('                q%d%s[j][w] = %s(reinterpret_cast<const %s*>(gin%d + (%s) * %du + j * %du + w * %du));' % (
+                t.io_index, suffix, '__builtin_nontemporal_load' if 'l' in nt else '*', mname, t.io_index, batch_expr,
+                batch_cols, group_cols, vec))
 
     def process(suffix, batch_expr, refill_expr, nb):
         src.append('        {')
@@ -844,7 +852,7 @@ def generate_reduce(info, kernel_name, depth=None, width=None):
             src.append('        __builtin_amdgcn_sched_barrier(0);')
         src.append('        }')
 
-    sets = 2 if num_batches > 1 else 1
+    sets = max(2, min(sets or 2, num_batches)) if num_batches > 1 else 1
     src.append('    // %d register sets of %d groups each per tensor: one is consumed while the other is in flight' % (sets, batch))
     for t in p.tensors:
         vname = vnames[CTYPE[t.dtype]]

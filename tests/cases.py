@@ -1271,6 +1271,8 @@ TEMPLATE_VARIANTS = [
     ('gated_scans', {'scan_interleave': 2}),
     ('gated_scans', {'scan_width': 2, 'scan_nt': 'l'}),
     ('gated_scans', {'template': 'map'}),
+    ('row_reductions', {'scan_width': 1}),
+    ('row_reductions', {'scan_width': 2, 'scan_sets': 3, 'scan_nt': 'l'}),
     ('c3_cumsum_f32', {'template': 'skewscan', 'scan_depth': 2, 'scan_sets': 2}),
     ('c3_cumsum_f32', {'template': 'skewscan', 'scan_width': 2}),
     ('c3_cumprod_f64', {'template': 'skewscan', 'scan_width': 1}),
