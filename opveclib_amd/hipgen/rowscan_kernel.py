@@ -730,13 +730,21 @@ def generate_reduce(info, kernel_name, depth=None, width=None, sets=None, nt='')
     # only if it leaves few of them.
     if width is None:
         width = 4
-        while width > 1 and p.length % (GROUP_LANES * vec * width) >= max(GROUP_LANES * vec, p.length // 32):
-            width //= 2
     while width > 1 and p.length < GROUP_LANES * vec * width:
         width //= 2
     group_cols = GROUP_LANES * vec * width
     num_groups = p.length // group_cols
     tail_cols = p.length % group_cols
+    # What the wide groups leave over goes through the same lanes in groups of one vector per lane, requested at the
+    # start like the rest; only the fewer than 16 * VEC columns after those are walked by one lane (that walk costs:
+    # float32 [4096, 16448], 64 columns left over, 56 us against 44 us for 16384).
+    small = GROUP_LANES * vec
+    narrow0 = num_groups * group_cols           # first column of the narrow groups
+    narrow_groups = 0
+    if width > 1:
+        narrow_groups = tail_cols // small
+        tail_cols -= narrow_groups * small
+    tail0 = narrow0 + narrow_groups * small     # first column walked by one lane
     # rows that start wherever the one before ends: vectors in memory are then only aligned like their elements
     aligned = dict((t.idx, (p.layouts[t.idx][0] * itemsize) % 16 == 0 and (p.layouts[t.idx][1] * itemsize) % 16 == 0)
                    for t in p.tensors)
@@ -800,35 +808,45 @@ def generate_reduce(info, kernel_name, depth=None, width=None, sets=None, nt='')
     for t in p.tensors:
         src.append('    const %s* __restrict__ gin%d = in%d + (uint64_t)row * %dull + %dull + part * %du;' % (
             CTYPE[t.dtype], t.io_index, t.io_index, p.layouts[t.idx][0], p.layouts[t.idx][1], vec * width))
+        if narrow_groups:
+            src.append('    const %s* __restrict__ gs%d = in%d + (uint64_t)row * %dull + %dull + part * %du;' % (
+                CTYPE[t.dtype], t.io_index, t.io_index, p.layouts[t.idx][0], p.layouts[t.idx][1] + narrow0, vec))
     batch = depth
     num_batches = num_groups // batch
     tail = num_groups % batch
     batch_cols = batch * group_cols
 
-    def request(k, batch_expr, nb, suffix):
+    def request(k, batch_expr, nb, suffix, narrow=False):
         for t in p.tensors:
             vname = vnames[CTYPE[t.dtype]]
-            mname = vname if aligned[t.idx] else vname + '_u'
+            mname = vname if aligned[t.idx] and (not narrow or (narrow0 * itemsize) % 16 == 0) else vname + '_u'
+            load = '__builtin_nontemporal_load' if 'l' in nt else '*'
             src.append('        #pragma unroll')
             src.append('        for (uint32_t j = 0; j < %du; ++j)' % nb)
+            if narrow:
+                src.append('            q%d%s[j][0] = %s(reinterpret_cast<const %s*>(gs%d + j * %du));' % (
+                    t.io_index, suffix, load, mname, t.io_index, small))
+                continue
             src.append('            #pragma unroll')
             src.append('            for (uint32_t w = 0; w < %du; ++w)' % width)
             src.append('                q%d%s[j][w] = %s(reinterpret_cast<const %s*>(gin%d + (%s) * %du + j * %du + w * %du));' % (
-                t.io_index, suffix, '__builtin_nontemporal_load' if 'l' in nt else '*', mname, t.io_index, batch_expr,
-                batch_cols, group_cols, vec))
+                t.io_index, suffix, load, mname, t.io_index, batch_expr, batch_cols, group_cols, vec))
 
-    def process(suffix, batch_expr, refill_expr, nb):
+    def process(suffix, batch_expr, refill_expr, nb, narrow=False):
         src.append('        {')
         src.append('        const uint32_t b = %s;' % batch_expr)
         src.append('        #pragma unroll')
         src.append('        for (uint32_t j = 0; j < %du; ++j) {' % nb)
-        src.append('            const uint32_t col0 = b * %du + j * %du + part * %du;' % (batch_cols, group_cols, vec * width))
+        if narrow:
+            src.append('            const uint32_t col0 = %du + j * %du + part * %du;' % (narrow0, small, vec))
+        else:
+            src.append('            const uint32_t col0 = b * %du + j * %du + part * %du;' % (batch_cols, group_cols, vec * width))
         src.append('            #pragma unroll')
         src.append('            for (uint32_t phase = 0; phase < %du; ++phase) {' % GROUP_LANES)
         for name, _ in state:
             src.append('                %s = carry_%s;' % (name, name))
         src.append('                #pragma unroll')
-        src.append('                for (uint32_t w = 0; w < %du; ++w) {' % width)
+        src.append('                for (uint32_t w = 0; w < %du; ++w) {' % (1 if narrow else width))
         for t in p.tensors:
             src.append('                    const %s xv%d = q%d%s[j][w];' % (
                 vnames[CTYPE[t.dtype]], t.io_index, t.io_index, suffix))
@@ -860,11 +878,16 @@ def generate_reduce(info, kernel_name, depth=None, width=None, sets=None, nt='')
         if tail:
             src.append('    %s q%d_t[%d][%d];       // the groups that end the row, requested now and held until then' % (
                 vname, t.io_index, tail, width))
+        if narrow_groups:
+            src.append('    %s q%d_s[%d][1];       // ... and the groups of one vector per lane after those' % (
+                vname, t.io_index, narrow_groups))
     src.append('    {')
     for k in range(sets):
         request(k, '%du' % k, batch, '_%d' % k)
     if tail:
         request(None, '%du' % num_batches, tail, '_t')
+    if narrow_groups:
+        request(None, '0u', narrow_groups, '_s', narrow=True)
     src.append('    }')
     src.append('    // the statements the worker runs before its loop, in every lane')
     for stmt in prologue:
@@ -891,6 +914,10 @@ def generate_reduce(info, kernel_name, depth=None, width=None, sets=None, nt='')
         src.append('    {')
         process('_t', '%du' % num_batches, None, tail)
         src.append('    }')
+    if narrow_groups:
+        src.append('    {')
+        process('_s', '0u', None, narrow_groups, narrow=True)
+        src.append('    }')
     for t in p.tensors:
         src.append('#undef OVL_REDUCE_IN%d' % t.io_index)
         src.append('#define OVL_REDUCE_IN%d gin%d[column]' % (t.io_index, t.io_index))
@@ -902,7 +929,7 @@ def generate_reduce(info, kernel_name, depth=None, width=None, sets=None, nt='')
     if tail_cols:
         src.append('        #pragma unroll 1')
         src.append('        for (uint32_t column = %du; column < %du; ++column) OVL_REDUCE_STEP(column)' % (
-            num_groups * group_cols, p.length))
+            tail0, p.length))
     for stmt in epilogue:
         src.append('        ' + stmt.strip())
     src.append('    }')
