@@ -736,8 +736,10 @@ def generate_reduce(info, kernel_name, depth=None, width=None, sets=None, nt='')
     num_groups = p.length // group_cols
     tail_cols = p.length % group_cols
     # What the wide groups leave over goes through the same lanes in groups of one vector per lane, requested at the
-    # start like the rest; only the fewer than 16 * VEC columns after those are walked by one lane (that walk costs:
-    # float32 [4096, 16448], 64 columns left over, 56 us against 44 us for 16384).
+    # start like the rest, and the fewer than 16 * VEC columns after those as one more such group in which the
+    # columns past the end of the row are skipped (their loads read the row's last element instead).  A walk of one
+    # lane over the columns left over costs more: float32 [4096, 16448], 64 columns left over by groups of 256,
+    # 56 us that way against 44 us for 16384 columns.
     small = GROUP_LANES * vec
     narrow0 = num_groups * group_cols           # first column of the narrow groups
     narrow_groups = 0
@@ -811,10 +813,23 @@ def generate_reduce(info, kernel_name, depth=None, width=None, sets=None, nt='')
         if narrow_groups:
             src.append('    const %s* __restrict__ gs%d = in%d + (uint64_t)row * %dull + %dull + part * %du;' % (
                 CTYPE[t.dtype], t.io_index, t.io_index, p.layouts[t.idx][0], p.layouts[t.idx][1] + narrow0, vec))
+        if tail_cols:
+            src.append('    const %s* __restrict__ grow%d = in%d + (uint64_t)row * %dull + %dull;' % (
+                CTYPE[t.dtype], t.io_index, t.io_index, p.layouts[t.idx][0], p.layouts[t.idx][1]))
     batch = depth
     num_batches = num_groups // batch
     tail = num_groups % batch
     batch_cols = batch * group_cols
+
+    def request_partial():
+        # element by element: a vector may cross the end of the row, and of the tensor
+        for t in p.tensors:
+            src.append('        #pragma unroll')
+            src.append('        for (uint32_t u = 0; u < %du; ++u) {' % vec)
+            src.append('            const uint32_t column = %du + part * %du + u;' % (tail0, vec))
+            src.append('            q%d_z[0][0][u] = grow%d[column < %du ? column : %du];' % (
+                t.io_index, t.io_index, p.length, p.length - 1))
+            src.append('        }')
 
     def request(k, batch_expr, nb, suffix, narrow=False):
         for t in p.tensors:
@@ -832,12 +847,14 @@ def generate_reduce(info, kernel_name, depth=None, width=None, sets=None, nt='')
             src.append('                q%d%s[j][w] = %s(reinterpret_cast<const %s*>(gin%d + (%s) * %du + j * %du + w * %du));' % (
                 t.io_index, suffix, load, mname, t.io_index, batch_expr, batch_cols, group_cols, vec))
 
-    def process(suffix, batch_expr, refill_expr, nb, narrow=False):
+    def process(suffix, batch_expr, refill_expr, nb, narrow=False, partial=False):
         src.append('        {')
         src.append('        const uint32_t b = %s;' % batch_expr)
         src.append('        #pragma unroll')
         src.append('        for (uint32_t j = 0; j < %du; ++j) {' % nb)
-        if narrow:
+        if partial:
+            src.append('            const uint32_t col0 = %du + part * %du;' % (tail0, vec))
+        elif narrow:
             src.append('            const uint32_t col0 = %du + j * %du + part * %du;' % (narrow0, small, vec))
         else:
             src.append('            const uint32_t col0 = b * %du + j * %du + part * %du;' % (batch_cols, group_cols, vec * width))
@@ -854,6 +871,8 @@ def generate_reduce(info, kernel_name, depth=None, width=None, sets=None, nt='')
         src.append('                    for (uint32_t u = 0; u < %du; ++u) {' % vec)
         if p.start == 1:
             src.append('                        if (col0 + w * %du + u == 0u) continue;     // column 0: done before the loop' % vec)
+        if partial:
+            src.append('                        if (col0 + u >= %du) continue;              // past the end of the row' % p.length)
         src.append('                        OVL_REDUCE_STEP(col0 + w * %du + u)' % vec)
         src.append('                    }')
         src.append('                }')
@@ -881,6 +900,8 @@ def generate_reduce(info, kernel_name, depth=None, width=None, sets=None, nt='')
         if narrow_groups:
             src.append('    %s q%d_s[%d][1];       // ... and the groups of one vector per lane after those' % (
                 vname, t.io_index, narrow_groups))
+        if tail_cols:
+            src.append('    %s q%d_z[1][1];        // ... and the columns after the last whole group' % (vname, t.io_index))
     src.append('    {')
     for k in range(sets):
         request(k, '%du' % k, batch, '_%d' % k)
@@ -888,6 +909,8 @@ def generate_reduce(info, kernel_name, depth=None, width=None, sets=None, nt='')
         request(None, '%du' % num_batches, tail, '_t')
     if narrow_groups:
         request(None, '0u', narrow_groups, '_s', narrow=True)
+    if tail_cols:
+        request_partial()
     src.append('    }')
     src.append('    // the statements the worker runs before its loop, in every lane')
     for stmt in prologue:
@@ -918,18 +941,15 @@ def generate_reduce(info, kernel_name, depth=None, width=None, sets=None, nt='')
         src.append('    {')
         process('_s', '0u', None, narrow_groups, narrow=True)
         src.append('    }')
-    for t in p.tensors:
-        src.append('#undef OVL_REDUCE_IN%d' % t.io_index)
-        src.append('#define OVL_REDUCE_IN%d gin%d[column]' % (t.io_index, t.io_index))
-    src.append('    // Lane 0 of the row holds the state that leaves the last group: it walks the columns after that group, one at a')
-    src.append('    // time, and runs the statements that follow the worker\'s loop.')
+    if tail_cols:
+        src.append('    {')
+        process('_z', '0u', None, 1, narrow=True, partial=True)
+        src.append('    }')
+    src.append('    // Lane 0 of the row holds the state that leaves the last group: it runs the statements that follow the')
+    src.append('    // worker\'s loop.')
     src.append('    if (part == 0u) {')
     for name, _ in state:
         src.append('        %s = carry_%s;' % (name, name))
-    if tail_cols:
-        src.append('        #pragma unroll 1')
-        src.append('        for (uint32_t column = %du; column < %du; ++column) OVL_REDUCE_STEP(column)' % (
-            tail0, p.length))
     for stmt in epilogue:
         src.append('        ' + stmt.strip())
     src.append('    }')
