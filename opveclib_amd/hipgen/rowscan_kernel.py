@@ -1139,7 +1139,7 @@ def _for_slot(text, slot):
     if slot == 0:
         return text
     suffix = '_r%d' % slot
-    text = re.sub(r'\b(carry_e\d+|e\d+|position|row_raw|row|gin\d*|gout|q\d+|qt\d*|ov|xv\d*|first_out|OVL_SCAN_STEP)\b',
+    text = re.sub(r'\b(carry_e\d+|e\d+|position|row_raw|row|gin\d*|gout|grow\d*|orow|q\d+|qt\d*|qz\d*|ov|xv\d*|first_out|OVL_SCAN_STEP)\b',
                   lambda m: m.group(1) + suffix, text)
     return text
 
@@ -1254,7 +1254,11 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
          ['    const %s* __restrict__ gin%s = in%d + (uint64_t)row * %dull + part * %du;' % (
              ctype, tag(k), t.io_index, p.length, vec * width) for k, t in enumerate(p.xs)] +
          ['    %s* __restrict__ gout = out%d + (uint64_t)row * %dull + part * %du;' % (
-             ctype, p.out.io_index, p.length, vec * width)])
+             ctype, p.out.io_index, p.length, vec * width)] +
+         (['    const %s* __restrict__ grow%s = in%d + (uint64_t)row * %dull;' % (ctype, tag(k), t.io_index, p.length)
+           for k, t in enumerate(p.xs)] +
+          ['    %s* __restrict__ orow = out%d + (uint64_t)row * %dull;' % (ctype, p.out.io_index, p.length)]
+          if tail_cols else []))
     # measured on MI355X (float32 [4096, 16384]): non-temporal stores with plain loads 85 us, hint on both 100 us,
     # on the loads only 90 us, on neither 102 us
     batch = depth
@@ -1334,11 +1338,25 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
     if tail:
         src.append('    // ... and the %d groups that end the row, requested now and held until the end' % tail)
         emit(['    %s %s[%d][%d];' % (vname, set_name('qt', t), tail, width) for t in range(len(p.xs))])
+    tail0 = num_groups * group_cols
+    if tail_cols:
+        src.append('    // ... and the columns after the last whole group, element by element (a vector may cross the end of')
+        src.append('    // the row): they run as one more group in which the columns past the end are skipped')
+        emit(['    %s qz%s[%d];' % (vname, tag(t), width) for t in range(len(p.xs))])
     src.append('    {')
     for k in range(sets if num_batches else 0):
         request('q%d' % k, '%du' % k)
     if tail:
         request('qt', '%du' % num_batches, tail)
+    if tail_cols:
+        for k in range(len(p.xs)):
+            emit(['        #pragma unroll',
+                  '        for (uint32_t w = 0; w < %du; ++w)' % width,
+                  '            #pragma unroll',
+                  '            for (uint32_t u = 0; u < %du; ++u) {' % vec,
+                  '                const uint32_t column = %du + part * %du + w * %du + u;' % (tail0, vec * width, vec),
+                  '                qz%s[w][u] = grow%s[column < %du ? column : %du];' % (tag(k), tag(k), p.length, p.length - 1),
+                  '            }'])
     src.append('    }')
     src.append('    // first column: the statements the worker runs before its loop, in every lane')
     for slot in slots:
@@ -1379,27 +1397,33 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
         process('qt', '%du' % num_batches, None, tail)
         src.append('    }')
     if tail_cols:
-        # The columns after the last whole group: lane 0 of the row's sixteen lanes holds the state that leaves the
-        # last group and runs the worker's loop over them, one column at a time (fewer than %d columns).
-        for slot in slots:
-            src.append('#undef OVL_SCAN_OUT_R%d' % slot)
-            for k in range(len(p.xs)):
-                src.append('#undef OVL_SCAN_IN_R%d_T%d' % (slot, k))
-                src.append('#define OVL_SCAN_IN_R%d_T%d tail_in%s' % (slot, k, tag(k)))
-            src.append('#define OVL_SCAN_OUT_R%d(value) tail_out = (value)' % slot)
-        src.append('    if (part == 0u) {')
-        for slot in slots:
-            one = lambda lines: src.extend(_for_slot(line, slot) for line in lines)
-            src.append('        {')
-            one(['        %s = carry_%s;' % (name, name) for name, _ in state])
-            src.append('        #pragma unroll 1')
-            src.append('        for (uint32_t column = %du; column < %du; ++column) {' % (num_groups * group_cols, p.length))
-            one(['            const %s tail_in%s = gin%s[column];' % (ctype, tag(k), tag(k)) for k in range(len(p.xs))] +
-                ['            %s tail_out;' % ctype,
-                 '            OVL_SCAN_STEP(column)',
-                 '            gout[column] = tail_out;'])
-            src.append('        }')
-            src.append('        }')
+        # The columns after the last whole group (fewer than one lane group's worth): one more group of one vector per
+        # lane in which the columns past the end of the row are skipped, stored element by element.  (A walk of one
+        # lane over these columns waits for every load in turn: 0.2 us per column.)
+        src.append('    {')
+        emit(['        %s ov[1][%d];' % (vname, width)])
+        src.append('        const uint32_t col0 = %du + part * %du;' % (tail0, vec * width))
+        src.append('        const uint32_t j = 0u;')
+        src.append('        #pragma unroll')
+        src.append('        for (uint32_t phase = 0; phase < %du; ++phase) {' % GROUP_LANES)
+        emit(['            %s = carry_%s;' % (name, name) for name, _ in state])
+        src.append('            #pragma unroll')
+        src.append('            for (uint32_t w = 0; w < %du; ++w) {' % width)
+        emit(['                const %s xv%s = qz%s[w];' % (vname, tag(k), tag(k)) for k in range(len(p.xs))])
+        src.append('                #pragma unroll')
+        src.append('                for (uint32_t u = 0; u < %du; ++u) {' % vec)
+        src.append('                    if (col0 + w * %du + u >= %du) continue;' % (vec, p.length))
+        emit(['                    OVL_SCAN_STEP(col0 + w * %du + u)' % vec])
+        src.append('                }')
+        src.append('            }')
+        emit(['            carry_%s = ovl_dpp_move<OVL_DPP_ROW_SHR1>(carry_%s, %s);' % (name, name, name)
+              for name, _ in state])
+        src.append('        }')
+        emit(['        #pragma unroll',
+              '        for (uint32_t w = 0; w < %du; ++w)' % width,
+              '            #pragma unroll',
+              '            for (uint32_t u = 0; u < %du; ++u)' % vec,
+              '                if (col0 + w * %du + u < %du) orow[col0 + w * %du + u] = ov[0][w][u];' % (vec, p.length, vec)])
         src.append('    }')
     for slot in slots:
         src.append('#undef %s' % _for_slot('OVL_SCAN_STEP', slot))
