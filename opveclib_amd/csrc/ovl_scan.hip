@@ -124,6 +124,20 @@ skewed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, 
             for (uint32_t w = 0; w < (uint32_t)WIDTH; ++w)
                 q[s][j][w] = load_vector<ALIGNED, vec>(gin + (uint64_t)b * BATCH_COLS + j * GROUP_COLS + w * VEC);
     }
+    // ... and the columns after the last whole group, element by element (a vector may cross the end of the row; a
+    // column past it is read as the row's last element and never used)
+    const T* __restrict__ grow = gin - part * (uint32_t)(VEC * WIDTH);
+    T* __restrict__ orow = gout - part * (uint32_t)(VEC * WIDTH);
+    const uint32_t tail0 = num_groups * GROUP_COLS;
+    vec qz[WIDTH];
+#pragma unroll
+    for (uint32_t w = 0; w < (uint32_t)WIDTH; ++w) {
+#pragma unroll
+        for (uint32_t u = 0; u < (uint32_t)VEC; ++u) {
+            const uint32_t column = tail0 + part * (uint32_t)(VEC * WIDTH) + w * VEC + u;
+            qz[w][u] = grow[column < cols ? column : cols - 1u];
+        }
+    }
     T carry = OP::template start<T>();
 
     // One group: in phase p every lane runs the recurrence over its columns from the carried state it holds and hands
@@ -194,15 +208,32 @@ skewed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, 
             }
         }
     }
-    // the columns after the last whole group: lane 0 of the row holds the state that leaves it (gin and gout of that
-    // lane are the row itself)
-    if (part == 0u) {
+    // The columns after the last whole group (fewer than one group's worth) run as one more group in which the
+    // columns past the end of the row are skipped; they are stored element by element.  (A walk of one lane over them
+    // waits for each load in turn.)
+    if (tail0 < cols) {
+        const uint32_t col0 = tail0 + part * (uint32_t)(VEC * WIDTH);
+        vec ov[WIDTH] = {};
         T acc = carry;
-#pragma unroll 1
-        for (uint32_t column = num_groups * GROUP_COLS; column < cols; ++column) {
-            acc = OP::apply(acc, gin[column]);
-            gout[column] = acc;
+#pragma unroll
+        for (uint32_t phase = 0; phase < GROUP; ++phase) {
+            acc = carry;
+#pragma unroll
+            for (uint32_t w = 0; w < (uint32_t)WIDTH; ++w) {
+#pragma unroll
+                for (uint32_t u = 0; u < (uint32_t)VEC; ++u) {
+                    if (col0 + w * VEC + u >= cols) continue;
+                    acc = OP::apply(acc, qz[w][u]);
+                    ov[w][u] = acc;
+                }
+            }
+            carry = ovl_dpp_move<OVL_DPP_ROW_SHR1>(carry, acc);
         }
+#pragma unroll
+        for (uint32_t w = 0; w < (uint32_t)WIDTH; ++w)
+#pragma unroll
+            for (uint32_t u = 0; u < (uint32_t)VEC; ++u)
+                if (col0 + w * VEC + u < cols) orow[col0 + w * VEC + u] = ov[w][u];
     }
 }
 
