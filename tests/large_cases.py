@@ -23,6 +23,54 @@ def reverse(x):
     return out
 
 
+@ovl.operator()
+def channels_last(x):
+    """[N, C, H, W] stored as [N, H, W, C]: unit stride along a workgroup dimension that is not one of the last two."""
+    n, c, h, w = x.shape
+    out = ovl.output([n, h, w, c], x.dtype)
+    pos = ovl.position_in(x.shape)
+    out[pos[0], pos[2], pos[3], pos[1]] = x[pos]
+    return out
+
+
+@ovl.operator()
+def row_sum(x):
+    rows, cols = x.shape
+    out = ovl.output([rows], x.dtype)
+    r = ovl.position_in([rows])[0]
+    acc = ovl.variable(0, x.dtype)
+    for j in ovl.arange(cols):
+        acc <<= acc + x[r, j]
+    out[r] = acc
+    return out
+
+
+@ovl.operator()
+def column_sum(x):
+    rows, cols = x.shape
+    out = ovl.output([cols], x.dtype)
+    c = ovl.position_in([cols])[0]
+    acc = ovl.variable(0, x.dtype)
+    for i in ovl.arange(rows):
+        acc <<= acc + x[i, c]
+    out[c] = acc
+    return out
+
+
+@ovl.operator()
+def running_dot(a, b):
+    """out[r, i] = sum of a[r, k] * b[r, k] over k <= i: a row scan whose body reads two inputs."""
+    rows, cols = a.shape
+    out = ovl.output_like(a)
+    r = ovl.position_in([rows])[0]
+    acc = ovl.variable(a[r, 0] * b[r, 0], a.dtype)
+    out[r, 0] = acc
+    for i in ovl.arange(1, cols):
+        acc <<= acc + a[r, i] * b[r, i]
+        out[r, i] = acc
+    return out
+
+
 def placeholder(shape, dtype):
     """An array of the given shape that owns one element (every stride is zero): enough to trace an operator."""
     shape = shape if isinstance(shape, tuple) else (shape,)
@@ -56,6 +104,18 @@ def cases(make):
 
     a = make((3000, 70001), np.int32)       # rows that are neither whole groups of 64 columns nor 16-byte aligned
     yield 'cumsum int32 [3000, 70001]', cumsum(a, axis=1), lambda: torch.cumsum(a, 1, dtype=torch.int32)
+
+    a = make((48, 256, 168, 168), np.int32)   # the tile template over dimensions 1 and 3, 2016 batches
+    yield 'channels_last int32 [48, 256, 168, 168]', channels_last(a), lambda: a.permute(0, 2, 3, 1).contiguous()
+
+    a = make((8192, 70001), np.int32)       # row reduction: wide groups, narrow groups and a partial group
+    yield 'row_sum int32 [8192, 70001]', row_sum(a), lambda: torch.sum(a, 1, dtype=torch.int32)
+
+    a = make((70001, 4100), np.int32)       # column reduction with a last strip that is not full
+    yield 'column_sum int32 [70001, 4100]', column_sum(a), lambda: torch.sum(a, 0, dtype=torch.int32)
+
+    a, b = make((3000, 70001), np.int32), make((3000, 70001), np.int32)     # a scan over two inputs
+    yield 'running_dot int32 [3000, 70001]', running_dot(a, b), lambda: torch.cumsum(a * b, 1, dtype=torch.int32)
 
     rows, cols = 65536, 32768 + 256         # 2^31 + 2^24 workers, transposed store
     a, flat = make((rows, cols), np.float32), make(rows * cols, np.float32)
