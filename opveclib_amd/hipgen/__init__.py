@@ -110,7 +110,8 @@ def generate(expression_dag, function_name, options=None):
                                                          options.get('scan_chunk'))
     elif options.get('vec') is None and template in ('auto', 'skewscan') and rowscan_kernel.skew_plan(info) is not None:
         kernel_src, launch = rowscan_kernel.generate_skewed(info, kernel_name, options.get('scan_depth'), options.get('scan_sets'), options.get('scan_nt', 's'),
-                                                             options.get('scan_width'), options.get('scan_interleave'))
+                                                             options.get('scan_width'), options.get('scan_interleave'),
+                                                             options.get('scan_split'))
     elif options.get('vec') is None and template in ('auto', 'rowscan') and rowscan_kernel.plan(info) is not None:
         kernel_src, launch = rowscan_kernel.generate(info, kernel_name, options.get('scan_rows'),
                                                      options.get('scan_chunk'), options.get('scan_batch'))

@@ -51,7 +51,8 @@ def plan(info, rows_per_block=None, chunk=None, need_chunk=True, multi=False):
     several inputs of the output's shape and type (a gated recurrence ``h = a[r, i] * h + x[r, i]``); the lane-skewed
     scan takes up to four, the other templates one."""
     forced_rows, forced_chunk = rows_per_block, chunk
-    if not info.inputs or len(info.inputs) > (4 if multi else 1) or len(info.outputs) != 1:
+    if not info.inputs or len(info.inputs) > (4 if multi else 1) or not info.outputs or \
+            len(info.outputs) > (4 if multi else 1):
         return None
     loops = [item for item in info.tree if item.kind == 'loop']
     if len(loops) != 1 or any(item.kind == 'if' for item in info.tree):
@@ -64,7 +65,7 @@ def plan(info, rows_per_block=None, chunk=None, need_chunk=True, multi=False):
     stores_before = [item for item in info.tree[:-1] if item.kind == 'stmt' and
                      info.nodes[item.node].code == lang.ASSIGN_TENSOR and
                      info.nodes[info.nodes[item.node].ops[0]].code == lang.OUTPUT]
-    if len(stores_before) > 1:
+    if len(stores_before) > len(info.outputs):
         return None
     range_node = info.nodes[loop.node]
     counter = range_node.ops[0]
@@ -93,6 +94,7 @@ def plan(info, rows_per_block=None, chunk=None, need_chunk=True, multi=False):
 
     x = out = None
     xs = []
+    outs = []
     for node, tensor, aff in info.tensor_accesses():
         if aff is None:
             return None
@@ -104,15 +106,25 @@ def plan(info, rows_per_block=None, chunk=None, need_chunk=True, multi=False):
                 xs.append(tensor)
             x = xs[0]
         else:
-            if out is not None and out is not tensor:
-                return None
-            out = tensor
+            if tensor not in outs:
+                outs.append(tensor)
+            out = outs[0]
     if x is None or out is None or len(xs) != len(info.inputs):
         return None
     if any(t.code != lang.INPUT or t.dtype != out.dtype or t.size != rows * length for t in xs):
         return None
-    if out.size != rows * length:
+    if any(t.code != lang.OUTPUT or t.dtype != out.dtype or t.size != rows * length for t in outs):
         return None
+    if len(outs) != len(info.outputs):
+        return None
+    if len(outs) > 1:
+        # several outputs: each is stored exactly once before the loop (column 0) and once in it
+        for t in outs:
+            for inside in (False, True):
+                count = len([n for n, tensor, _ in info.tensor_accesses()
+                             if n.code == lang.ASSIGN_TENSOR and tensor is t and bool(info.in_loop[n.idx]) == inside])
+                if count != 1:
+                    return None
     itemsize = ITEMSIZE[x.dtype]
     if itemsize not in (4, 8) or x.dtype not in CTYPE:
         return None
@@ -129,6 +141,7 @@ def plan(info, rows_per_block=None, chunk=None, need_chunk=True, multi=False):
         return None
     p = ScanPlan(loop, counter, length, rows, x, out, vec, rows_per_block, chunk)
     p.xs = xs           # every input the body reads, in the order of their first use; x is the first
+    p.outs = outs       # every output the body stores, likewise; out is the first
     return p
 
 
@@ -393,7 +406,33 @@ def generate(info, kernel_name, rows_per_block=None, chunk=None, batch=None):
 # ---------------------------------------------------------------------------------------------------------------------
 
 GROUP_LANES = 16
-SKEW_MAX_BODY = 96
+SKEW_MAX_BODY = 64
+
+
+def _body_size(info):
+    """Nodes inside the loop, without the 64-bit index arithmetic of the tensor accesses (the templates address
+    the rows themselves, so those nodes leave no code): what is unrolled sixteen phases times a vector's elements."""
+    return len([n for n in info.nodes if info.in_loop[n.idx] and n.dtype != lang.UINT64])
+
+
+HEAVY_CODES = (lang.DIVIDE, lang.MODULO, lang.POW, lang.SQRT, lang.EXP, lang.LOG, lang.LOG10, lang.TANH, lang.SIN,
+               lang.COS, lang.TAN, lang.SINH, lang.COSH, lang.ASIN, lang.ACOS, lang.ATAN, lang.ATAN2)
+
+
+def _heavy_outside_recurrence(info, p):
+    """True when the loop body computes something costly (a division, a transcendental function) that the carried
+    state does not depend on: work for the outputs only, which need not be repeated in every phase of the skewed
+    recurrence."""
+    needed = set()
+    stack = [n.idx for n in info.nodes if info.in_loop[n.idx] and n.code == lang.ASSIGN_VARIABLE and
+             n.ops[0] != p.counter]
+    while stack:
+        idx = stack.pop()
+        if idx in needed:
+            continue
+        needed.add(idx)
+        stack.extend(info.nodes[idx].ops)
+    return any(info.in_loop[n.idx] and n.idx not in needed and n.code in HEAVY_CODES for n in info.nodes)
 
 
 def _carried_state(info, p):
@@ -415,8 +454,7 @@ def skew_plan(info):
     p = plan(info, need_chunk=False, multi=True)
     if p is None or p.length < GROUP_LANES * p.vec:
         return None
-    body_nodes = [n for n in info.nodes if info.in_loop[n.idx]]
-    if len(body_nodes) > SKEW_MAX_BODY:
+    if _body_size(info) > SKEW_MAX_BODY:
         return None
     for idx in _carried_state(info, p):
         if info.nodes[idx].dtype not in CTYPE:
@@ -445,7 +483,7 @@ FED_ROWS = WAVE // GROUP_LANES      # rows per workgroup: one group of sixteen l
 def fed_plan(info, width=None, chunk=None):
     """(ScanPlan, width, chunk) when the LDS-fed lane-skewed variant can run this DAG, else None."""
     p = skew_plan(info)
-    if p is None or len(p.xs) != 1 or p.length % (GROUP_LANES * p.vec) != 0:
+    if p is None or len(p.xs) != 1 or len(p.outs) != 1 or p.length % (GROUP_LANES * p.vec) != 0:
         return None
     itemsize = ITEMSIZE[p.x.dtype]
     width = width or 8
@@ -708,7 +746,7 @@ def reduce_plan(info):
     # (short rows stay with one worker per thread: float32 [100000, 100] 18 us there, 26 us here)
     if length < 4 * GROUP_LANES * vec:
         return None
-    if len([n for n in info.nodes if info.in_loop[n.idx]]) > SKEW_MAX_BODY:
+    if _body_size(info) > SKEW_MAX_BODY:
         return None
     p = ReducePlan(loop, end_idx, counter, start, length, rows, tensors, vec)
     p.layouts = layouts
@@ -1139,12 +1177,12 @@ def _for_slot(text, slot):
     if slot == 0:
         return text
     suffix = '_r%d' % slot
-    text = re.sub(r'\b(carry_e\d+|e\d+|position|row_raw|row|gin\d*|gout|grow\d*|orow|q\d+|qt\d*|qz\d*|ov|xv\d*|first_out|OVL_SCAN_STEP)\b',
+    text = re.sub(r'\b(carry_e\d+|e\d+|position|row_raw|row|gin\d*|gout\d*|grow\d*|orow\d*|q\d+|qt\d*|qz\d*|ov\d*|xv\d*|first_out\d*|OVL_SCAN_STEP_DRY|OVL_SCAN_STEP)\b',
                   lambda m: m.group(1) + suffix, text)
     return text
 
 
-def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None, interleave=None):
+def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None, interleave=None, split=None):
     p = skew_plan(info)
     assert p is not None
     ctype = CTYPE[p.x.dtype]
@@ -1196,7 +1234,12 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
 
     # the inputs the body reads, numbered in the order of their first use: each has its pointer, register sets and
     # vector of the moment under a name with that number (the first without one)
+    # Costly work that only the outputs need: the sixteen phases then run with the stores dropped (the compiler removes
+    # what only they used), and one more pass over the lane's columns, from the carried state that is exact by then,
+    # computes and stores the outputs (float32 [2048, 8192], c = f * c + i * g, h = o * tanh(c): 968 -> 313 us).
+    split = _heavy_outside_recurrence(info, p) if split is None else bool(split)
     number = dict((t.idx, k) for k, t in enumerate(p.xs))
+    out_number = dict((t.idx, k) for k, t in enumerate(p.outs))
     tag = lambda k: '' if k == 0 else str(k)
 
     def set_name(regs, k):
@@ -1206,7 +1249,7 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
 
     emitter = BodyEmitter(info, pos_exprs,
                           read_hook=lambda node, tensor, idx: 'OVL_SCAN_IN_T%d' % number[tensor.idx],
-                          store_hook=lambda node, tensor, idx, value: 'OVL_SCAN_OUT(' + value + ');')
+                          store_hook=lambda node, tensor, idx, value: 'OVL_SCAN_OUT_T%d(' % out_number[tensor.idx] + value + ');')
     tagged = emitter.emit_tagged()
     range_idx = p.loop_item.node
     end_idx = max(i for i, _ in tagged)
@@ -1233,9 +1276,9 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
         src.append('typedef %s %s __attribute__((aligned(%d)));' % (vname, mname, ITEMSIZE[p.x.dtype]))
     src.append('')
     src.append('extern "C" __global__ void __launch_bounds__(%d)' % BLOCK)
-    src.append('%s(%s, %s* __restrict__ out%d) {' % (
+    src.append('%s(%s, %s) {' % (
         kernel_name, ', '.join('const %s* __restrict__ in%d' % (CTYPE[info.inputs[i].dtype], i) for i in range(len(info.inputs))),
-        ctype, p.out.io_index))
+        ', '.join('%s* __restrict__ out%d' % (CTYPE[info.outputs[i].dtype], i) for i in range(len(info.outputs)))))
     if info.uses_math_tables():
         src.append('    OVL_DECLARE_MATH_TABLES();')
     src.append('    const uint32_t lane = threadIdx.x %% %du;' % WAVE)
@@ -1253,11 +1296,12 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
     emit(['    const uint32_t row = row_raw < %du ? row_raw : %du;' % (p.rows, p.rows - 1)] +
          ['    const %s* __restrict__ gin%s = in%d + (uint64_t)row * %dull + part * %du;' % (
              ctype, tag(k), t.io_index, p.length, vec * width) for k, t in enumerate(p.xs)] +
-         ['    %s* __restrict__ gout = out%d + (uint64_t)row * %dull + part * %du;' % (
-             ctype, p.out.io_index, p.length, vec * width)] +
+         ['    %s* __restrict__ gout%s = out%d + (uint64_t)row * %dull + part * %du;' % (
+             ctype, tag(k), t.io_index, p.length, vec * width) for k, t in enumerate(p.outs)] +
          (['    const %s* __restrict__ grow%s = in%d + (uint64_t)row * %dull;' % (ctype, tag(k), t.io_index, p.length)
            for k, t in enumerate(p.xs)] +
-          ['    %s* __restrict__ orow = out%d + (uint64_t)row * %dull;' % (ctype, p.out.io_index, p.length)]
+          ['    %s* __restrict__ orow%s = out%d + (uint64_t)row * %dull;' % (ctype, tag(k), t.io_index, p.length)
+           for k, t in enumerate(p.outs)]
           if tail_cols else []))
     # measured on MI355X (float32 [4096, 16384]): non-temporal stores with plain loads 85 us, hint on both 100 us,
     # on the loads only 90 us, on neither 102 us
@@ -1286,7 +1330,7 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
         nb = nb or batch
         src.append('        {')
         src.append('        const uint32_t b = %s;' % batch_expr)
-        emit(['        %s ov[%d][%d];' % (vname, nb, width)])
+        emit(['        %s ov%s[%d][%d];' % (vname, tag(k), nb, width) for k in range(len(p.outs))])
         src.append('        #pragma unroll')
         src.append('        for (uint32_t j = 0; j < %du; ++j) {' % nb)
         src.append('            const uint32_t col0 = b * %du + j * %du + part * %du;' % (batch_cols, group_cols, vec * width))
@@ -1301,13 +1345,31 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
         emit(['                    const %s xv%s = %s[j][w];' % (vname, tag(k), set_name(regs, k)) for k in range(len(p.xs))])
         src.append('                    #pragma unroll')
         src.append('                    for (uint32_t u = 0; u < %du; ++u) {' % vec)
-        emit(['                        if (w == 0u && u == 0u && first_column) ov[j][0][0] = first_out;',
-              '                        else OVL_SCAN_STEP(col0 + w * %du + u)' % vec])
+        if split:
+            emit(['                        if (w == 0u && u == 0u && first_column) continue;',
+                  '                        OVL_SCAN_STEP_DRY(col0 + w * %du + u)' % vec])
+        else:
+            emit(['                        if (w == 0u && u == 0u && first_column) { %s }' % ' '.join(
+                      'ov%s[j][0][0] = first_out%s;' % (tag(k), tag(k)) for k in range(len(p.outs))),
+                  '                        else OVL_SCAN_STEP(col0 + w * %du + u)' % vec])
         src.append('                    }')
         src.append('                }')
         emit(['                carry_%s = ovl_dpp_move<OVL_DPP_ROW_SHR1>(carry_%s, %s);' % (name, name, name)
               for name, _ in state])
         src.append('            }')
+        if split:
+            # every lane's carried state is exact now: one pass that computes and keeps the outputs
+            emit(['            %s = carry_%s;' % (name, name) for name, _ in state])
+            src.append('            #pragma unroll')
+            src.append('            for (uint32_t w = 0; w < %du; ++w) {' % width)
+            emit(['                const %s xv%s = %s[j][w];' % (vname, tag(k), set_name(regs, k)) for k in range(len(p.xs))])
+            src.append('                #pragma unroll')
+            src.append('                for (uint32_t u = 0; u < %du; ++u) {' % vec)
+            emit(['                    if (w == 0u && u == 0u && first_column) { %s }' % ' '.join(
+                      'ov%s[j][0][0] = first_out%s;' % (tag(k), tag(k)) for k in range(len(p.outs))),
+                  '                    else OVL_SCAN_STEP(col0 + w * %du + u)' % vec])
+            src.append('                }')
+            src.append('            }')
         src.append('            // the last lane of the group finished the group: its state is the carry into the next one')
         emit(['            carry_%s = ovl_dpp_move<OVL_DPP_ROW_ROR1>(carry_%s, %s);' % (name, name, name)
               for name, _ in state])
@@ -1315,17 +1377,18 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
         src.append('        // The scheduling fences keep the memory traffic of a batch together, after its arithmetic: runs of')
         src.append('        // batch * 256 bytes per row, and no load is moved ahead of the last use of the registers it fills.')
         src.append('        __builtin_amdgcn_sched_barrier(0);')
-        lines = ['        #pragma unroll',
-                 '        for (uint32_t j = 0; j < %du; ++j)' % nb,
-                 '            #pragma unroll',
-                 '            for (uint32_t w = 0; w < %du; ++w)' % width]
-        if 's' in nt:
-            lines.append('                __builtin_nontemporal_store(ov[j][w], reinterpret_cast<%s*>(gout + b * %du + j * %du + w * %du));' % (
-                mname, batch_cols, group_cols, vec))
-        else:
-            lines.append('                *(reinterpret_cast<%s*>(gout + b * %du + j * %du + w * %du)) = ov[j][w];' % (
-                mname, batch_cols, group_cols, vec))
-        emit(lines)
+        for k in range(len(p.outs)):
+            lines = ['        #pragma unroll',
+                     '        for (uint32_t j = 0; j < %du; ++j)' % nb,
+                     '            #pragma unroll',
+                     '            for (uint32_t w = 0; w < %du; ++w)' % width]
+            if 's' in nt:
+                lines.append('                __builtin_nontemporal_store(ov%s[j][w], reinterpret_cast<%s*>(gout%s + b * %du + j * %du + w * %du));' % (
+                    tag(k), mname, tag(k), batch_cols, group_cols, vec))
+            else:
+                lines.append('                *(reinterpret_cast<%s*>(gout%s + b * %du + j * %du + w * %du)) = ov%s[j][w];' % (
+                    mname, tag(k), batch_cols, group_cols, vec, tag(k)))
+            emit(lines)
         if refill_expr is not None:
             request(regs, refill_expr)
         src.append('        __builtin_amdgcn_sched_barrier(0);')
@@ -1361,24 +1424,34 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
     src.append('    // first column: the statements the worker runs before its loop, in every lane')
     for slot in slots:
         emit_one = lambda lines: src.extend(_for_slot(line, slot) for line in lines)
-        emit_one(['    %s first_out;' % ctype])
+        emit_one(['    %s first_out%s;' % (ctype, tag(k)) for k in range(len(p.outs))])
         for k, t in enumerate(p.xs):
             src.append('#define OVL_SCAN_IN_T%d (in%d[(uint64_t)%s * %dull])' % (
                 k, t.io_index, _for_slot('row', slot), p.length))
-        src.append('#define OVL_SCAN_OUT(value) %s = (value)' % _for_slot('first_out', slot))
+        for k in range(len(p.outs)):
+            src.append('#define OVL_SCAN_OUT_T%d(value) %s = (value)' % (k, _for_slot('first_out' + tag(k), slot)))
         emit_one(['    ' + stmt for stmt in prologue])
         for k in range(len(p.xs)):
             src.append('#undef OVL_SCAN_IN_T%d' % k)
-        src.append('#undef OVL_SCAN_OUT')
+        for k in range(len(p.outs)):
+            src.append('#undef OVL_SCAN_OUT_T%d' % k)
         emit_one(['    %s carry_%s = %s;' % (stype, name, name) for name, stype in state])
     for slot in slots:
         # (the output vector is named in the step macro itself, so that every row writes its own)
         src.append(_for_slot('#define OVL_SCAN_STEP(column) { %s = (%s)(column); %s }' % (
             counter_name, counter_type, ' '.join(body)), slot).replace(
-                'OVL_SCAN_OUT(', 'OVL_SCAN_OUT_R%d(' % slot).replace('OVL_SCAN_IN', 'OVL_SCAN_IN_R%d' % slot))
+                'OVL_SCAN_OUT_T', 'OVL_SCAN_OUT_R%d_T' % slot).replace('OVL_SCAN_IN', 'OVL_SCAN_IN_R%d' % slot))
+        if split:
+            src.append(_for_slot('#define OVL_SCAN_STEP_DRY(column) { %s = (%s)(column); %s }' % (
+                counter_name, counter_type, ' '.join(body)), slot).replace(
+                    'OVL_SCAN_OUT_T', 'OVL_SCAN_DROP_T').replace('OVL_SCAN_IN', 'OVL_SCAN_IN_R%d' % slot))
         for k in range(len(p.xs)):
             src.append('#define OVL_SCAN_IN_R%d_T%d %s[u]' % (slot, k, _for_slot('xv' + tag(k), slot)))
-        src.append('#define OVL_SCAN_OUT_R%d(value) %s[j][w][u] = (value)' % (slot, _for_slot('ov', slot)))
+        for k in range(len(p.outs)):
+            src.append('#define OVL_SCAN_OUT_R%d_T%d(value) %s[j][w][u] = (value)' % (
+                slot, k, _for_slot('ov' + tag(k), slot)))
+            if split and slot == 0:
+                src.append('#define OVL_SCAN_DROP_T%d(value) (void)(value)' % k)
     rounds = num_batches // sets
     last = num_batches - 1
     if rounds:
@@ -1401,7 +1474,7 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
         # lane in which the columns past the end of the row are skipped, stored element by element.  (A walk of one
         # lane over these columns waits for every load in turn: 0.2 us per column.)
         src.append('    {')
-        emit(['        %s ov[1][%d];' % (vname, width)])
+        emit(['        %s ov%s[1][%d];' % (vname, tag(k), width) for k in range(len(p.outs))])
         src.append('        const uint32_t col0 = %du + part * %du;' % (tail0, vec * width))
         src.append('        const uint32_t j = 0u;')
         src.append('        #pragma unroll')
@@ -1413,21 +1486,39 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
         src.append('                #pragma unroll')
         src.append('                for (uint32_t u = 0; u < %du; ++u) {' % vec)
         src.append('                    if (col0 + w * %du + u >= %du) continue;' % (vec, p.length))
-        emit(['                    OVL_SCAN_STEP(col0 + w * %du + u)' % vec])
+        emit(['                    %s(col0 + w * %du + u)' % ('OVL_SCAN_STEP_DRY' if split else 'OVL_SCAN_STEP', vec)])
         src.append('                }')
         src.append('            }')
         emit(['            carry_%s = ovl_dpp_move<OVL_DPP_ROW_SHR1>(carry_%s, %s);' % (name, name, name)
               for name, _ in state])
         src.append('        }')
-        emit(['        #pragma unroll',
-              '        for (uint32_t w = 0; w < %du; ++w)' % width,
-              '            #pragma unroll',
-              '            for (uint32_t u = 0; u < %du; ++u)' % vec,
-              '                if (col0 + w * %du + u < %du) orow[col0 + w * %du + u] = ov[0][w][u];' % (vec, p.length, vec)])
+        if split:
+            emit(['        %s = carry_%s;' % (name, name) for name, _ in state])
+            src.append('        #pragma unroll')
+            src.append('        for (uint32_t w = 0; w < %du; ++w) {' % width)
+            emit(['            const %s xv%s = qz%s[w];' % (vname, tag(k), tag(k)) for k in range(len(p.xs))])
+            src.append('            #pragma unroll')
+            src.append('            for (uint32_t u = 0; u < %du; ++u) {' % vec)
+            src.append('                if (col0 + w * %du + u >= %du) continue;' % (vec, p.length))
+            emit(['                OVL_SCAN_STEP(col0 + w * %du + u)' % vec])
+            src.append('            }')
+            src.append('        }')
+        for k in range(len(p.outs)):
+            emit(['        #pragma unroll',
+                  '        for (uint32_t w = 0; w < %du; ++w)' % width,
+                  '            #pragma unroll',
+                  '            for (uint32_t u = 0; u < %du; ++u)' % vec,
+                  '                if (col0 + w * %du + u < %du) orow%s[col0 + w * %du + u] = ov%s[0][w][u];' % (
+                      vec, p.length, tag(k), vec, tag(k))])
         src.append('    }')
     for slot in slots:
         src.append('#undef %s' % _for_slot('OVL_SCAN_STEP', slot))
-        src.append('#undef OVL_SCAN_OUT_R%d' % slot)
+        if split:
+            src.append('#undef %s' % _for_slot('OVL_SCAN_STEP_DRY', slot))
+        for k in range(len(p.outs)):
+            src.append('#undef OVL_SCAN_OUT_R%d_T%d' % (slot, k))
+            if split and slot == 0:
+                src.append('#undef OVL_SCAN_DROP_T%d' % k)
         for k in range(len(p.xs)):
             src.append('#undef OVL_SCAN_IN_R%d_T%d' % (slot, k))
     src.append('}')
@@ -1438,8 +1529,9 @@ def generate_skewed(info, kernel_name, depth=None, sets=None, nt='s', width=None
         'vec': vec,
         'block': BLOCK,
         'blocks_needed': (p.rows + rows_per_block - 1) // rows_per_block,
-        'align': dict([(('in', t.io_index), row_align) for t in p.xs] + [(('out', p.out.io_index), row_align)]),
+        'align': dict([(('in', t.io_index), row_align) for t in p.xs] +
+                      [(('out', t.io_index), row_align) for t in p.outs]),
         'vector_loads': len(p.xs),
-        'vector_stores': 1,
+        'vector_stores': len(p.outs),
     }
     return '\n'.join(src) + '\n', launch

@@ -528,6 +528,47 @@ def _gated_scan3(a, x, b):
     return _gated_body(a, x, b)
 
 
+@ovl.operator()
+def _cell_scan(f, i, g, o):
+    """An LSTM-like recurrence over the last axis with its matrix products taken out: c = f * c + i * g and
+    h = o * tanh(c), both stored for every column.  Four inputs, two outputs, one carried variable."""
+    shape = list(f.shape)
+    cs = ovl.output_like(f)
+    hs = ovl.output_like(f)
+    pos = ovl.position_in(shape[:-1])
+
+    def at(k):
+        return tuple(pos[d] for d in range(len(shape) - 1)) + (k,)
+
+    c = ovl.variable(i[at(0)] * g[at(0)], f.dtype)
+    cs[at(0)] = c
+    hs[at(0)] = o[at(0)] * ovl.tanh(c)
+    for k in ovl.arange(1, shape[-1]):
+        c <<= f[at(k)] * c + i[at(k)] * g[at(k)]
+        cs[at(k)] = c
+        hs[at(k)] = o[at(k)] * ovl.tanh(c)
+    return cs, hs
+
+
+@ovl.operator()
+def _sum_and_max(x):
+    """Running sum and running maximum of every row: two carried variables, two outputs."""
+    rows, cols = x.shape
+    sums = ovl.output_like(x)
+    tops = ovl.output_like(x)
+    r = ovl.position_in([rows])[0]
+    total = ovl.variable(x[r, 0], x.dtype)
+    top = ovl.variable(x[r, 0], x.dtype)
+    sums[r, 0] = total
+    tops[r, 0] = top
+    for k in ovl.arange(1, cols):
+        total <<= total + x[r, k]
+        top <<= ovl.maximum(top, x[r, k])
+        sums[r, k] = total
+        tops[r, k] = top
+    return sums, tops
+
+
 def gated_scans(rng):
     """Row scans over several inputs: whole groups, columns left over, unaligned rows, rank 3, 8-byte elements, a row
     shorter than one group (which stays on the general kernel)."""
@@ -544,6 +585,12 @@ def gated_scans(rng):
             outs.append(_gated_scan3(gate(shape, dtype), data(shape, dtype), data(shape, dtype)))
         else:
             outs.append(_gated_scan(gate(shape, dtype), data(shape, dtype)))
+    # several outputs
+    for shape, dtype in [((6, 256), np.float32), ((2, 3, 333), np.float32), ((5, 131), np.float32)]:
+        outs += all_outputs(_cell_scan(gate(shape, dtype), data(shape, dtype), data(shape, dtype), gate(shape, dtype)))
+    outs += all_outputs(_sum_and_max(data((9, 517), np.float32)))
+    outs += all_outputs(_sum_and_max(data((4, 200), np.float64)))
+    outs += all_outputs(_sum_and_max(rng.integers(-50, 50, size=(7, 320)).astype(np.int32)))
     return outs
 
 
@@ -1271,6 +1318,9 @@ TEMPLATE_VARIANTS = [
     ('gated_scans', {'scan_interleave': 2}),
     ('gated_scans', {'scan_width': 2, 'scan_nt': 'l'}),
     ('gated_scans', {'template': 'map'}),
+    ('gated_scans', {'scan_split': True}),
+    ('gated_scans', {'scan_split': False, 'scan_interleave': 2}),
+    ('c3_rowscan_shapes', {'template': 'skewscan', 'scan_split': True, 'scan_interleave': 2}),
     ('row_reductions', {'scan_width': 1}),
     ('row_reductions', {'scan_width': 2, 'scan_sets': 3, 'scan_nt': 'l'}),
     ('c3_cumsum_f32', {'template': 'skewscan', 'scan_depth': 2, 'scan_sets': 2}),
