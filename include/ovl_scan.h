@@ -17,12 +17,15 @@
  * Kernel: the lane-skewed order-preserving scan.  Sixteen neighbouring lanes share a row; a lane owns a run of
  * consecutive columns of the current group (one 128-bit access for float32, two for float64), runs the recurrence
  * over its run from the carried state it holds and hands its state to its right neighbour with a lane-to-lane move;
- * after sixteen such phases the group is exact and the last lane's state is the carry into the next group.  float64
- * rows whose length is a multiple of 512 columns run the same recurrence fed from LDS (three wavefronts of the
- * workgroup stream four rows through LDS, the fourth scans them, a lane owning 16 columns per phase), which pays the
- * hand-over between lanes four times less often.  The columns after a row's last whole group (64 columns) are
- * scanned by one lane; rows that do not start on 16-byte boundaries are moved with unaligned vectors; rows shorter than
- * one group take a plain kernel with one lane per row.  The result is the same bits whichever kernel runs.
+ * after sixteen such phases the group is exact and the last lane's state is the carry into the next group.  The
+ * columns after a row's last whole group run as one more, partial group across the same sixteen lanes (element-wise
+ * loads with the index clamped to the row's end, element-wise stores); rows that do not start on 16-byte boundaries
+ * are moved with unaligned vectors; rows shorter than one group take a plain kernel with one lane per row.
+ * float64 rows whose length is a multiple of 512 columns (and 16-byte aligned tensors) run the same recurrence fed
+ * from LDS by a workgroup of five wavefronts per four rows: two load chunks of 512 columns into LDS, one runs the
+ * recurrence with 32 columns per lane and phase and publishes only the exact state that enters each lane's segment,
+ * one recomputes the segments from those states (same order of operations, same bits) and one stores them.  The
+ * result is the same bits whichever kernel runs.
  *
  * Conventions: tensor memory belongs to the caller and must be device accessible; `out` may not overlap `x`; the
  * functions enqueue one kernel on `hip_stream` (a hipStream_t; NULL is the default stream), return without

@@ -170,7 +170,7 @@ def test_hand_written_lstm_cell_emulated_on_the_host_equals_the_oracle(batch, un
                                             (9, 64, 1), (6, 100, 0), (2, 7, 1), (70, 33, 0), (67, 512, 0), (1, 1024, 0),
                                             (6, 1536, 0), (5, 2048, 0), (3, 1024, 1), (3, 384, 0), (2, 448, 0), (5, 576, 0),
                                             (2, 832, 0), (3, 1000, 0), (5, 333, 0), (2, 131, 1), (4, 70, 0),
-                                            (3, 517, 1)])
+                                            (3, 517, 1), (3, 4608, 0), (2, 6144, 0), (9, 3584, 0)])
 def test_hand_written_row_scans_emulated_on_the_host_equal_numpy(rows, cols, skew):
     rng = np.random.default_rng(rows * 1000 + cols)
     dims = np.array([rows, cols, skew], np.uint32)
