@@ -22,10 +22,12 @@
  * loads with the index clamped to the row's end, element-wise stores); rows that do not start on 16-byte boundaries
  * are moved with unaligned vectors; rows shorter than one group take a plain kernel with one lane per row.
  * float64 rows whose length is a multiple of 512 columns (and 16-byte aligned tensors) run the same recurrence fed
- * from LDS by a workgroup of five wavefronts per four rows: two load chunks of 512 columns into LDS, one runs the
- * recurrence with 32 columns per lane and phase and publishes only the exact state that enters each lane's segment,
- * one recomputes the segments from those states (same order of operations, same bits) and one stores them.  The
- * result is the same bits whichever kernel runs.
+ * from LDS, four rows per workgroup.  When the tensor gives every compute unit at most one workgroup (or whole rounds
+ * of them with rows of 12288 columns and more) the workgroup has five wavefronts: two load chunks of 512 columns into
+ * LDS, one runs the recurrence with 32 columns per lane and phase and publishes only the exact state that enters each
+ * lane's segment, one recomputes the segments from those states (same order of operations, same bits) and one stores
+ * them.  Otherwise three wavefronts move the chunks and the fourth scans them in place, 16 columns per lane and phase.
+ * The result is the same bits whichever kernel runs.
  *
  * Conventions: tensor memory belongs to the caller and must be device accessible; `out` may not overlap `x`; the
  * functions enqueue one kernel on `hip_stream` (a hipStream_t; NULL is the default stream), return without

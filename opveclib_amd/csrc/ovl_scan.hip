@@ -240,47 +240,192 @@ skewed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, 
     }
 }
 
-// LDS-fed lane-skewed scan, for 8-byte elements: a scan of float64 rows runs at the latency of its recurrence (a
-// dependent float64 addition issues every 5 clocks), so everything that is not an addition is taken off the wavefront
-// that runs it.  A workgroup of five wavefronts owns four rows and streams them through six rotating LDS buffers in
-// chunks of FED_CHUNK = 16 * FED_SEG columns, one workgroup barrier per chunk:
+// LDS-fed lane-skewed scan, for 8-byte elements: a scan of float64 rows runs at the latency of its recurrence, and in
+// the kernel above the hand-over between lanes is paid once per RUN columns, where RUN is limited by the shape of the
+// memory requests (a lane that owns more than 32 consecutive bytes makes the wavefront's requests sparse).  Here the
+// requests are made by other wavefronts: wavefronts 1-3 of the workgroup stream its four rows through three rotating
+// LDS buffers of FED_CHUNK columns with dense 128-bit accesses (two chunks of loads in flight in registers), and
+// wavefront 0 runs the skewed recurrence out of LDS and in place, sixteen lanes per row, each lane owning FED_SEG
+// consecutive columns of every group of 16 * FED_SEG: the hand-over is paid once per FED_SEG additions.  Segments are
+// padded by one vector in LDS so that the sixteen lanes of a group read and write without bank conflicts.
+// cols must be a multiple of FED_CHUNK; x and out 16-byte aligned.  float64 [1024, 16384]: 59 us against 83 us.
+constexpr uint32_t FED_SEG = 16, FED_GROUP_COLS = GROUP * FED_SEG, FED_CHUNK = 2 * FED_GROUP_COLS;
+
+template <typename T, typename OP>
+__global__ void __launch_bounds__(BLOCK)
+fed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, uint32_t cols) {
+    constexpr uint32_t VEC = 16 / sizeof(T);
+    typedef typename vec_of<T, VEC>::type vec;
+    constexpr uint32_t W = FED_SEG / VEC;                          // vectors per lane and phase
+    constexpr uint32_t PADDED_SEG = FED_SEG + VEC;                 // a segment and its padding
+    constexpr uint32_t ROW_STRIDE = FED_CHUNK / FED_SEG * PADDED_SEG;
+    constexpr uint32_t MOVERS = BLOCK - WAVE;
+    constexpr uint32_t CHUNK_VECS = ROWS_PER_WAVE * FED_CHUNK / VEC;       // vectors of a chunk of the four rows
+    constexpr uint32_t PER_MOVER = (CHUNK_VECS + MOVERS - 1) / MOVERS;
+    __shared__ __attribute__((aligned(16))) T tile[3][ROWS_PER_WAVE][ROW_STRIDE];
+
+    const uint32_t row0 = blockIdx.x * ROWS_PER_WAVE;
+    const uint32_t num_chunks = cols / FED_CHUNK;
+
+    // Movers: thread m owns vectors m, m + 192, ... of every chunk.  A vector that does not exist (past the chunk or
+    // past the last row) is redirected to an existing one for loading and skipped when writing, so the loops are
+    // free of branches and all loads of a chunk are in flight together.
+    struct mover_regs { vec v[PER_MOVER]; };
+    auto slot = [&](uint32_t m, uint32_t i, uint32_t& r, uint32_t& c) -> bool {
+        const uint32_t v = m + i * MOVERS;
+        r = v / (FED_CHUNK / VEC);
+        c = (v % (FED_CHUNK / VEC)) * VEC;
+        return v < CHUNK_VECS && row0 + r < rows;
+    };
+    auto lds_at = [&](uint32_t k, uint32_t r, uint32_t c) -> vec* {
+        return reinterpret_cast<vec*>(&tile[k % 3u][r][c + (c / FED_SEG) * VEC]);
+    };
+    auto issue_loads = [&](uint32_t k, uint32_t m, mover_regs& regs) {
+#pragma unroll
+        for (uint32_t i = 0; i < PER_MOVER; ++i) {
+            uint32_t r, c;
+            if (!slot(m, i, r, c)) { r = 0; c = 0; }
+            // (plain loads: with the non-temporal hint on loads and stores the mixed stream runs a quarter slower)
+            regs.v[i] = *reinterpret_cast<const vec*>(x + (uint64_t)(row0 + r) * cols + (uint64_t)k * FED_CHUNK + c);
+        }
+    };
+    auto write_lds = [&](uint32_t k, uint32_t m, const mover_regs& regs) {
+#pragma unroll
+        for (uint32_t i = 0; i < PER_MOVER; ++i) {
+            uint32_t r, c;
+            if (slot(m, i, r, c)) *lds_at(k, r, c) = regs.v[i];
+        }
+    };
+    auto store_chunk = [&](uint32_t k, uint32_t m) {
+        mover_regs regs;
+#pragma unroll
+        for (uint32_t i = 0; i < PER_MOVER; ++i) {
+            uint32_t r, c;
+            if (!slot(m, i, r, c)) { r = 0; c = 0; }
+            regs.v[i] = *lds_at(k, r, c);
+        }
+#pragma unroll
+        for (uint32_t i = 0; i < PER_MOVER; ++i) {
+            uint32_t r, c;
+            if (slot(m, i, r, c))
+                __builtin_nontemporal_store(regs.v[i], reinterpret_cast<vec*>(
+                    out + (uint64_t)(row0 + r) * cols + (uint64_t)k * FED_CHUNK + c));
+        }
+    };
+
+    if (threadIdx.x >= WAVE) {
+        const uint32_t m = threadIdx.x - WAVE;
+        // chunk 0 and the even chunks travel through set_a, the odd ones through set_b: while chunk k is scanned,
+        // chunk k + 1 goes to LDS from the set requested two steps ago and chunk k + 3 is requested into that set
+        mover_regs set_a, set_b;
+        issue_loads(0u, m, set_a);
+        write_lds(0u, m, set_a);
+        if (1u < num_chunks) issue_loads(1u, m, set_b);
+        if (2u < num_chunks) issue_loads(2u, m, set_a);
+        __syncthreads();
+        auto step = [&](uint32_t k, mover_regs& regs) {
+            if (k + 1u < num_chunks) write_lds(k + 1u, m, regs);
+            if (k + 3u < num_chunks) issue_loads(k + 3u, m, regs);
+            if (k >= 1u) store_chunk(k - 1u, m);
+            __syncthreads();
+        };
+        uint32_t k = 0;
+#pragma unroll 1
+        for (; k + 1u < num_chunks; k += 2u) {
+            step(k, set_b);
+            step(k + 1u, set_a);
+        }
+        if (k < num_chunks) step(k, set_b);
+        store_chunk(num_chunks - 1u, m);
+    } else {
+        // The scanning wavefront.  A group of lanes whose row does not exist works on whatever its part of the tile
+        // holds: nobody stores it.
+        const uint32_t lane = threadIdx.x;
+        const uint32_t part = lane % GROUP, q = lane / GROUP;
+        T carry = OP::template start<T>();
+        vec set_a[W], set_b[W];
+        auto fetch = [&](vec (&set)[W], const T* from) {
+#pragma unroll
+            for (uint32_t w = 0; w < W; ++w) set[w] = *reinterpret_cast<const vec*>(from + w * VEC);
+        };
+        // one group of 16 * FED_SEG columns: in phase p every lane runs the recurrence over its segment from the
+        // state it holds and hands its final state to its right neighbour; after phase p lanes 0..p are exact
+        auto run = [&](vec (&set)[W], T* to) {
+            vec ov[W];
+            T acc = carry;
+#pragma unroll
+            for (uint32_t phase = 0; phase < GROUP; ++phase) {
+                acc = carry;
+#pragma unroll
+                for (uint32_t w = 0; w < W; ++w) {
+#pragma unroll
+                    for (uint32_t u = 0; u < VEC; ++u) {
+                        acc = OP::apply(acc, set[w][u]);
+                        ov[w][u] = acc;
+                    }
+                }
+                carry = ovl_dpp_move<OVL_DPP_ROW_SHR1>(carry, acc);
+            }
+            carry = ovl_dpp_move<OVL_DPP_ROW_ROR1>(carry, acc);
+#pragma unroll
+            for (uint32_t w = 0; w < W; ++w) *reinterpret_cast<vec*>(to + w * VEC) = ov[w];
+        };
+        constexpr uint32_t GROUP_STRIDE = GROUP * PADDED_SEG;         // distance between a lane's segments of two groups
+        __syncthreads();
+        for (uint32_t k = 0; k < num_chunks; ++k) {
+            T* here = &tile[k % 3u][q][part * PADDED_SEG];
+            fetch(set_a, here);
+            fetch(set_b, here + GROUP_STRIDE);
+            run(set_a, here);
+            run(set_b, here + GROUP_STRIDE);
+            __syncthreads();
+        }
+    }
+}
+
+// The same with the results taken off the scanning wavefront, for tensors that give every compute unit at most one
+// workgroup: a scan of float64 rows runs at the latency of its recurrence (a dependent float64 addition issues every
+// 5 clocks), so everything that is not an addition is taken off the wavefront that runs it.  A workgroup of five wavefronts owns four rows and streams them through six rotating LDS buffers in
+// chunks of CARRY_CHUNK = 16 * CARRY_SEG columns, one workgroup barrier per chunk:
 //
-//   loaders (wavefronts 3, 4)  global memory -> registers (FED_AHEAD chunks of requests in flight) -> LDS
+//   loaders (wavefronts 3, 4)  global memory -> registers (CARRY_AHEAD chunks of requests in flight) -> LDS
 //   scanner (wavefront 0)      reads its segments of the next chunk from LDS while it runs the skewed recurrence over
-//                              the current one: sixteen lanes per row, lane p owns FED_SEG consecutive columns, sixteen
-//                              phases of FED_SEG dependent operations and one hand-over (DPP row_shr:1) each.  It keeps
+//                              the current one: sixteen lanes per row, lane p owns CARRY_SEG consecutive columns, sixteen
+//                              phases of CARRY_SEG dependent operations and one hand-over (DPP row_shr:1) each.  It keeps
 //                              no results: after the last phase every lane holds the exact state that enters its
 //                              segment, and that one value per lane is all it writes to LDS (a 128-bit LDS write costs
 //                              the issuing wavefront about 25 clocks, five operations of the recurrence; a read 5)
-//   finisher (wavefront 1)     recomputes every segment from its exact entering state, one pass of FED_SEG operations
+//   finisher (wavefront 1)     recomputes every segment from its exact entering state, one pass of CARRY_SEG operations
 //                              in the same order, hence the same bits, and writes the results over the inputs in LDS
 //   storer (wavefront 2)       LDS -> global memory
 //
 // Chunk c is written to LDS in step c - 2, read by the scanner in step c - 1, scanned in step c, finished in step
 // c + 2 and stored in step c + 3; its buffer is written again in step c + 4.  Segments are padded by one vector in LDS
-// so that the sixteen lanes of a group read and write without bank conflicts.  cols must be a multiple of FED_CHUNK;
-// x and out 16-byte aligned.  float64 [1024, 16384]: 47 us against 59 us with the results written by the scanner.
-constexpr uint32_t FED_SEG = 32, FED_CHUNK = GROUP * FED_SEG, FED_BUFFERS = 6, FED_AHEAD = 4, FED_LOADER_WAVES = 2;
-constexpr uint32_t FED_BLOCK = (3 + FED_LOADER_WAVES) * WAVE;
+// so that the sixteen lanes of a group read and write without bank conflicts.  cols must be a multiple of CARRY_CHUNK;
+// x and out 16-byte aligned.  The workgroup holds 105 KiB of LDS, one workgroup per compute unit: float64 [1024, 16384]
+// 47 us against 58 us for the kernel above, [256, 65536] 154 against 192; with more workgroups than compute units the
+// kernel above, three workgroups of which share a compute unit, is the faster one ([4096, 4096] 46 against 59 us).
+constexpr uint32_t CARRY_SEG = 32, CARRY_CHUNK = GROUP * CARRY_SEG, CARRY_BUFFERS = 6, CARRY_AHEAD = 4, CARRY_LOADER_WAVES = 2;
+constexpr uint32_t CARRY_BLOCK = (3 + CARRY_LOADER_WAVES) * WAVE;
 // the phase of a group after which the scanner meets the others at the barrier: its LDS reads of the step are done
-constexpr uint32_t FED_SYNC_PHASE = 8;
+constexpr uint32_t CARRY_SYNC_PHASE = 8;
 
 template <typename T, typename OP>
-__global__ void __launch_bounds__(FED_BLOCK)
-fed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, uint32_t cols) {
+__global__ void __launch_bounds__(CARRY_BLOCK)
+carry_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, uint32_t cols) {
     constexpr uint32_t VEC = 16 / sizeof(T);
     typedef typename vec_of<T, VEC>::type vec;
-    constexpr uint32_t W = FED_SEG / VEC;                          // vectors per lane and chunk
-    constexpr uint32_t PADDED_SEG = FED_SEG + VEC;                 // a segment and its padding
+    constexpr uint32_t W = CARRY_SEG / VEC;                          // vectors per lane and chunk
+    constexpr uint32_t PADDED_SEG = CARRY_SEG + VEC;                 // a segment and its padding
     constexpr uint32_t ROW_STRIDE = GROUP * PADDED_SEG;
-    constexpr uint32_t CHUNK_VECS = ROWS_PER_WAVE * FED_CHUNK / VEC;       // vectors of a chunk of the four rows
-    constexpr uint32_t READS_PER_PHASE = W / FED_SYNC_PHASE;
-    static_assert(READS_PER_PHASE * FED_SYNC_PHASE == W, "the scanner's reads of a chunk fill the phases before the barrier");
-    __shared__ __attribute__((aligned(16))) T tile[FED_BUFFERS][ROWS_PER_WAVE][ROW_STRIDE];
-    __shared__ T entering[FED_BUFFERS][WAVE];
+    constexpr uint32_t CHUNK_VECS = ROWS_PER_WAVE * CARRY_CHUNK / VEC;       // vectors of a chunk of the four rows
+    constexpr uint32_t READS_PER_PHASE = W / CARRY_SYNC_PHASE;
+    static_assert(READS_PER_PHASE * CARRY_SYNC_PHASE == W, "the scanner's reads of a chunk fill the phases before the barrier");
+    __shared__ __attribute__((aligned(16))) T tile[CARRY_BUFFERS][ROWS_PER_WAVE][ROW_STRIDE];
+    __shared__ T entering[CARRY_BUFFERS][WAVE];
 
     const uint32_t row0 = blockIdx.x * ROWS_PER_WAVE;
-    const uint32_t n = cols / FED_CHUNK;                           // chunks, and steps 0 .. n + 2
+    const uint32_t n = cols / CARRY_CHUNK;                           // chunks, and steps 0 .. n + 2
     const uint32_t wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
     // Every wavefront passes the same n + 3 barriers: one after the first two chunks are in LDS, then one at the end
     // of each of the steps 0 .. n + 1.
@@ -312,7 +457,7 @@ fed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, uin
 #pragma unroll
                     for (uint32_t u = 0; u < VEC; ++u) acc = OP::apply(acc, in[cur][w][u]);
                 carry = ovl_dpp_move<OVL_DPP_ROW_SHR1>(carry, acc);
-                if (phase < FED_SYNC_PHASE) {
+                if (phase < CARRY_SYNC_PHASE) {
 #pragma unroll
                     for (uint32_t j = 0; j < READS_PER_PHASE; ++j) {
                         const uint32_t w = phase * READS_PER_PHASE + j;
@@ -321,7 +466,7 @@ fed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, uin
                 }
                 // (the fences keep each read in its phase and the barrier in its place)
                 __builtin_amdgcn_sched_barrier(0);
-                if (phase == FED_SYNC_PHASE) {
+                if (phase == CARRY_SYNC_PHASE) {
                     __syncthreads();
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -331,8 +476,8 @@ fed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, uin
             entering[slot][lane] = carry;
             // the last lane finished the chunk: its state is the carry into the next one
             carry = ovl_dpp_move<OVL_DPP_ROW_ROR1>(carry, acc);
-            next = next + 1u == FED_BUFFERS ? 0u : next + 1u;
-            slot = slot + 1u == FED_BUFFERS ? 0u : slot + 1u;
+            next = next + 1u == CARRY_BUFFERS ? 0u : next + 1u;
+            slot = slot + 1u == CARRY_BUFFERS ? 0u : slot + 1u;
             __builtin_amdgcn_sched_barrier(0);
         };
         typedef std::integral_constant<uint32_t, 0> set0;
@@ -353,7 +498,7 @@ fed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, uin
         __syncthreads();
         __syncthreads();
         for (uint32_t s = 2; s <= n + 1u; ++s) {
-            const uint32_t buffer = (s - 2u) % FED_BUFFERS;
+            const uint32_t buffer = (s - 2u) % CARRY_BUFFERS;
             T* mine = &tile[buffer][q][part * PADDED_SEG];
             vec v[W];
 #pragma unroll
@@ -374,14 +519,14 @@ fed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, uin
         // Loaders and storer: thread m of `movers` owns vectors m, m + movers, ... of every chunk.  A loader's vector
         // past the last row is a second copy of the last row's; the storer skips it.
         const bool storer = wave == 2;
-        constexpr uint32_t LOADERS = FED_LOADER_WAVES * WAVE;
+        constexpr uint32_t LOADERS = CARRY_LOADER_WAVES * WAVE;
         constexpr uint32_t PER_LOADER = CHUNK_VECS / LOADERS, PER_STORER = CHUNK_VECS / WAVE;
         static_assert(PER_LOADER * LOADERS == CHUNK_VECS && PER_STORER * WAVE == CHUNK_VECS, "whole vectors per thread");
         auto place = [&](uint32_t v, uint32_t& global_offset, uint32_t& lds_offset, bool& exists) {
-            const uint32_t r = v / (FED_CHUNK / VEC), c = (v % (FED_CHUNK / VEC)) * VEC;
+            const uint32_t r = v / (CARRY_CHUNK / VEC), c = (v % (CARRY_CHUNK / VEC)) * VEC;
             exists = row0 + r < rows;
             global_offset = (exists ? row0 + r : rows - 1u) * cols + c;           // rows * cols < 2^32
-            lds_offset = r * ROW_STRIDE + c + (c / FED_SEG) * VEC;
+            lds_offset = r * ROW_STRIDE + c + (c / CARRY_SEG) * VEC;
         };
         if (storer) {
             uint32_t global_offset[PER_STORER], lds_offset[PER_STORER];
@@ -389,14 +534,14 @@ fed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, uin
 #pragma unroll
             for (uint32_t i = 0; i < PER_STORER; ++i) place(lane + i * WAVE, global_offset[i], lds_offset[i], exists[i]);
             auto store_chunk = [&](uint32_t c) {
-                const T* buffer = &tile[c % FED_BUFFERS][0][0];
+                const T* buffer = &tile[c % CARRY_BUFFERS][0][0];
                 vec regs[PER_STORER];
 #pragma unroll
                 for (uint32_t i = 0; i < PER_STORER; ++i) regs[i] = *reinterpret_cast<const vec*>(buffer + lds_offset[i]);
 #pragma unroll
                 for (uint32_t i = 0; i < PER_STORER; ++i)
                     if (exists[i])
-                        __builtin_nontemporal_store(regs[i], reinterpret_cast<vec*>(out + global_offset[i] + c * FED_CHUNK));
+                        __builtin_nontemporal_store(regs[i], reinterpret_cast<vec*>(out + global_offset[i] + c * CARRY_CHUNK));
             };
             __syncthreads();
             __syncthreads();
@@ -423,40 +568,40 @@ fed_scan_kernel(const T* __restrict__ x, T* __restrict__ out, uint32_t rows, uin
                 const uint32_t cc = c < n ? c : n - 1u;
 #pragma unroll
                 for (uint32_t i = 0; i < PER_LOADER; ++i)
-                    regs[i] = *reinterpret_cast<const vec*>(x + global_offset[i] + cc * FED_CHUNK);
+                    regs[i] = *reinterpret_cast<const vec*>(x + global_offset[i] + cc * CARRY_CHUNK);
             };
             auto to_lds = [&](uint32_t c, const vec (&regs)[PER_LOADER]) {
-                T* buffer = &tile[c % FED_BUFFERS][0][0];
+                T* buffer = &tile[c % CARRY_BUFFERS][0][0];
 #pragma unroll
                 for (uint32_t i = 0; i < PER_LOADER; ++i) *reinterpret_cast<vec*>(buffer + lds_offset[i]) = regs[i];
             };
-            vec set[FED_AHEAD][PER_LOADER];
+            vec set[CARRY_AHEAD][PER_LOADER];
             {
                 vec first[2][PER_LOADER];
                 request(0u, first[0]);
                 request(1u, first[1]);
 #pragma unroll
-                for (uint32_t a = 0; a < FED_AHEAD; ++a) request(2u + a, set[(2u + a) % FED_AHEAD]);
+                for (uint32_t a = 0; a < CARRY_AHEAD; ++a) request(2u + a, set[(2u + a) % CARRY_AHEAD]);
                 to_lds(0u, first[0]);
                 to_lds(1u, first[1]);
             }
             __syncthreads();
-            // step s: chunk s + 2 goes to LDS from the register set requested FED_AHEAD steps ago, which is then
-            // requested again with chunk s + 2 + FED_AHEAD
+            // step s: chunk s + 2 goes to LDS from the register set requested CARRY_AHEAD steps ago, which is then
+            // requested again with chunk s + 2 + CARRY_AHEAD
             auto step = [&](uint32_t s, vec (&regs)[PER_LOADER]) {
                 to_lds(s + 2u, regs);
-                request(s + 2u + FED_AHEAD, regs);
+                request(s + 2u + CARRY_AHEAD, regs);
                 __syncthreads();
             };
             uint32_t s = 0;
 #pragma unroll 1
-            for (; s + FED_AHEAD <= n + 2u; s += FED_AHEAD) {
+            for (; s + CARRY_AHEAD <= n + 2u; s += CARRY_AHEAD) {
 #pragma unroll
-                for (uint32_t a = 0; a < FED_AHEAD; ++a) step(s + a, set[(2u + a) % FED_AHEAD]);
+                for (uint32_t a = 0; a < CARRY_AHEAD; ++a) step(s + a, set[(2u + a) % CARRY_AHEAD]);
             }
 #pragma unroll
-            for (uint32_t a = 0; a < FED_AHEAD; ++a)
-                if (s + a <= n + 1u) step(s + a, set[(2u + a) % FED_AHEAD]);
+            for (uint32_t a = 0; a < CARRY_AHEAD; ++a)
+                if (s + a <= n + 1u) step(s + a, set[(2u + a) % CARRY_AHEAD]);
         }
     }
 }
@@ -493,11 +638,20 @@ int scan(const char* who, const T* x, uint32_t rows, uint32_t cols, T* out, void
     const dim3 block(BLOCK);
     bool fed = false;
     if constexpr (sizeof(T) == 8) {
-        // 8-byte elements: the recurrence sets the pace, and the LDS-fed kernel pays fewer hand-overs
+        // 8-byte elements: the recurrence sets the pace, and the LDS-fed kernels pay fewer hand-overs
         if (aligned && cols % FED_CHUNK == 0) {
             fed = true;
-            const dim3 grid((rows + ROWS_PER_WAVE - 1) / ROWS_PER_WAVE);
-            hipLaunchKernelGGL((fed_scan_kernel<T, OP>), grid, dim3(FED_BLOCK), 0, stream, x, out, rows, cols);
+            const uint32_t groups = (rows + ROWS_PER_WAVE - 1) / ROWS_PER_WAVE;
+            // the kernel whose scanning wavefront keeps no results runs one workgroup per compute unit: it is chosen
+            // when the workgroups fit in one round, or fill their rounds and have rows long enough to pay for the
+            // start of its pipeline in each
+            const uint32_t rounds = (groups + OVL_NUM_CU - 1) / OVL_NUM_CU;
+            const bool one_round = groups <= OVL_NUM_CU;
+            const bool full_rounds = 10u * groups >= 9u * rounds * OVL_NUM_CU && cols / CARRY_CHUNK >= 24u;
+            if (cols % CARRY_CHUNK == 0 && (one_round || full_rounds))
+                hipLaunchKernelGGL((carry_scan_kernel<T, OP>), dim3(groups), dim3(CARRY_BLOCK), 0, stream, x, out, rows, cols);
+            else
+                hipLaunchKernelGGL((fed_scan_kernel<T, OP>), dim3(groups), block, 0, stream, x, out, rows, cols);
         }
     }
     if (fed) {
