@@ -1,3 +1,7 @@
+# Derived from opveclib/__init__.py of opveclib (https://github.com/opveclib/opveclib),
+# Copyright 2016 Hewlett Packard Enterprise Development LP, licensed under the Apache License, Version 2.0
+# (http://www.apache.org/licenses/LICENSE-2.0); see the NOTICE file at the root of this repository.
+# Changes: the list of exported names is that project's; the names added here (set_math_mode, as_torch, CapturedDag, ...) are not.
 """
 OVL for MI355X: the Operator Vectorization Library's DSL and operator API with a HIP (gfx950) backend.
 

@@ -1,3 +1,7 @@
+# Derived from opveclib/examples/conv1D.py of opveclib (https://github.com/opveclib/opveclib),
+# Copyright 2016 Hewlett Packard Enterprise Development LP, licensed under the Apache License, Version 2.0;
+# see the NOTICE file at the root of this repository.  The operator's statements are that file's (they define the
+# result); docstrings, argument checks and everything around them are new.
 """
 One-dimensional multi-channel convolution / cross-correlation written against the DSL, with worker-local tensors
 (the reference's opveclib/examples/conv1D.py:17-207 computes the same function with a ring buffer per worker).

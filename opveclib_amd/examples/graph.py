@@ -1,3 +1,7 @@
+# Derived from opveclib/examples/test_graph.py of opveclib (https://github.com/opveclib/opveclib),
+# Copyright 2016 Hewlett Packard Enterprise Development LP, licensed under the Apache License, Version 2.0;
+# see the NOTICE file at the root of this repository.  The operator's statements are that file's (they define the
+# result); docstrings, argument checks and everything around them are new.
 """
 Triangle counting on an undirected graph with one worker per edge (the edge-iterator strategy of the reference's
 opveclib/examples/test_graph.py:17-92): a worker on edge (u, v), u > v, merges the sorted neighbour lists of u and v

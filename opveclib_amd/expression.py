@@ -1,3 +1,8 @@
+# Derived from opveclib/expression.py of opveclib (https://github.com/opveclib/opveclib),
+# Copyright 2016 Hewlett Packard Enterprise Development LP, licensed under the Apache License, Version 2.0
+# (http://www.apache.org/licenses/LICENSE-2.0); see the NOTICE file at the root of this repository.
+# Changes: class and function names, signatures, the dtype table and the error messages follow that file so that its
+# callers and tests run unchanged; the recorder, the schema messages behind it and everything about code generation are new.
 """
 The OVL expression language: data types, tensor types and the tracer that records a worker function as an
 expression DAG.

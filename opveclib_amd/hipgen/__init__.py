@@ -8,8 +8,8 @@ CUDA text built around a one-thread-per-worker template.  Here the DAG is analys
 * :mod:`.map_kernel` - vectorised map (any DAG; vector width 1 is the general fallback);
 * :mod:`.tile_kernel` - rank-2 workgroups with transposed stores: LDS-tiled so reads and writes are both coalesced;
 * :mod:`.rowscan_kernel` - loop-carried accumulation along the last tensor axis: order-preserving row scans
-  (lane-skewed out of registers; lane-skewed or lane = row out of LDS, fed by dedicated data-moving wavefronts) and
-  the reassociating wavefront scan;
+  (lane-skewed out of registers; lane-skewed or lane = row out of LDS, fed by dedicated data-moving wavefronts, with
+  the results written by the scanning wavefront or recomputed by a second one) and the reassociating wavefront scan;
 * :mod:`.colscan_kernel` - the same accumulation along another axis: rows streamed through LDS, lane-skewed over
   sixteen lanes per line for tensors with up to 32768 lines ('colskew'), lane = line beyond ('colscan').
 
@@ -30,7 +30,7 @@ from . import rowscan_kernel
 from . import colscan_kernel
 
 #: bump when generated code changes for an unchanged DAG, so cached binaries are not reused
-CODEGEN_VERSION = 32
+CODEGEN_VERSION = 33
 
 
 
@@ -62,7 +62,7 @@ def generate(expression_dag, function_name, options=None):
     """
     :param expression_dag: serialised expression DAG of one operator
     :param function_name: unique name of the operator (its content hash)
-    :param options: optional dict.  ``template``: 'auto' (default), 'map', 'transpose', 'rowscan', 'skewscan', 'fedscan', 'treescan', 'rowreduce', 'colreduce', 'colscan' or 'colskew' restricts
+    :param options: optional dict.  ``template``: 'auto' (default), 'map', 'transpose', 'rowscan', 'skewscan', 'fedscan', 'carryscan', 'treescan', 'rowreduce', 'colreduce', 'colscan' or 'colskew' restricts
         the choice of kernel template (a template that does not fit the DAG falls back to 'map'); ``vec`` forces the
         map template with that vector width, ``per_thread`` its vectors per thread (1 or 2); ``scan_movers`` the number of threads that only move data in the lane-skewed column scan (0: every wavefront scans and moves), ``scan_depth`` / ``scan_sets`` / ``scan_width`` / ``scan_interleave`` set the request burst (groups), the
         number of register sets, the 128-bit vectors per lane and phase and the rows per lane group of the lane-skewed scan; ``math``: 'exact'
@@ -102,6 +102,13 @@ def generate(expression_dag, function_name, options=None):
     if tree is not None:
         # sums, products and running extrema whose order the caller has given up: the reassociating scan
         kernel_src, launch = rowscan_kernel.generate_tree(info, kernel_name, options.get('scan_ahead') or 8)
+    elif options.get('vec') is None and template in ('auto', 'carryscan') and \
+            rowscan_kernel.carry_plan(info, options.get('scan_width')) is not None and \
+            (template == 'carryscan' or (rowscan_kernel.carry_plan(info)[0].vec == 2 and
+                                         rowscan_kernel.carry_preferred(info))):
+        # 8-byte elements run at the latency of their recurrence: with at most one workgroup per compute unit the
+        # scanning wavefront does nothing but the recurrence, a second one recomputes and writes the results
+        kernel_src, launch = rowscan_kernel.generate_carry(info, kernel_name, options.get('scan_width'))
     elif options.get('vec') is None and template in ('auto', 'fedscan') and \
             rowscan_kernel.fed_plan(info, options.get('scan_width'), options.get('scan_chunk')) is not None and \
             (template == 'fedscan' or rowscan_kernel.fed_plan(info)[0].vec == 2):

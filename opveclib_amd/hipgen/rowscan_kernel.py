@@ -181,7 +181,8 @@ def _emit_movers(src, p, ctype, vname, vec, chunk, rpb, num_chunks, lds_column=N
     src.append('            uint32_t r, cv;')
     src.append('            slot(m, i, r, cv);')
     src.append('            const uint64_t g = (uint64_t)(row0 + r) * %dull + k * %du + cv;' % (p.length, chunk))
-    src.append('            regs.v[i] = __builtin_nontemporal_load(reinterpret_cast<const %s*>(gin + g));' % vname)
+    # (plain loads: with the non-temporal hint on loads and stores the mixed stream runs a quarter slower)
+    src.append('            regs.v[i] = *reinterpret_cast<const %s*>(gin + g);' % vname)
     src.append('        }')
     src.append('    };')
     src.append('    auto write_lds = [&](uint32_t k, uint32_t m, const MoverRegs& regs) {')
@@ -635,6 +636,351 @@ def generate_fed(info, kernel_name, width=None, chunk=None):
         'template': 'fedscan',
         'vec': vec,
         'block': BLOCK,
+        'blocks_needed': (p.rows + rpb - 1) // rpb,
+        'align': {('in', p.x.io_index): 16, ('out', p.out.io_index): 16},
+        'vector_loads': 1,
+        'vector_stores': 1,
+    }
+    return '\n'.join(src) + '\n', launch
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# The LDS-fed lane-skewed variant whose scanning wavefront keeps no results ('carryscan'), for tensors that give every
+# compute unit at most one workgroup.
+#
+# A scan of float64 rows runs at the latency of its recurrence (a dependent float64 addition issues every 5 clocks),
+# and in the variant above the scanning wavefront also writes every result to LDS: a 128-bit LDS write costs the
+# wavefront that issues it about 25 clocks, five steps of the recurrence, a read about 5.  Here the scanning wavefront
+# only reads: after the sixteenth phase of a chunk every lane holds the exact state that enters its segment, and that
+# state is all it writes (one value per lane and carried variable).  A second wavefront, the finisher, runs the loop
+# body once more over every segment from its entering state - the same operations in the same order, hence the same
+# bits - and writes the results over the inputs in LDS; a third stores them, two more load.  The workgroup streams its
+# four rows through six rotating LDS buffers in chunks of 16 * seg columns, one barrier per chunk; chunk c is written
+# to LDS in step c - 2, read by the scanning wavefront in step c - 1, scanned in step c, finished in step c + 2 and
+# stored in step c + 3.  float64 [1024, 16384]: 47 us against 58; the 105 KiB of LDS allow one workgroup per compute
+# unit, so tensors with more workgroups than compute units stay with the variant above unless they fill whole rounds
+# with long rows.
+# ---------------------------------------------------------------------------------------------------------------------
+CARRY_BUFFERS = 6
+CARRY_AHEAD = 4          # chunks of loads a loading thread keeps in flight
+CARRY_LOADER_WAVES = 2
+CARRY_BLOCK = (3 + CARRY_LOADER_WAVES) * WAVE
+CARRY_SYNC_PHASE = 8     # the scanning wavefront's LDS reads of a step fill the phases before this one
+
+
+def carry_plan(info, width=None):
+    """(ScanPlan, width) when the variant without results in the scanning wavefront can run this DAG, else None."""
+    p = skew_plan(info)
+    if p is None or len(p.xs) != 1 or len(p.outs) != 1:
+        return None
+    itemsize = ITEMSIZE[p.x.dtype]
+    width = width or 32 // p.vec
+    while width >= CARRY_SYNC_PHASE and p.length % (GROUP_LANES * p.vec * width) != 0:
+        width //= 2
+    # the scanning wavefront reads width vectors in CARRY_SYNC_PHASE phases; the movers own whole vectors
+    if width < CARRY_SYNC_PHASE or width % CARRY_SYNC_PHASE != 0 or p.length % (GROUP_LANES * p.vec * width) != 0:
+        return None
+    chunk_vectors = FED_ROWS * GROUP_LANES * width
+    if chunk_vectors % (CARRY_LOADER_WAVES * WAVE) != 0:
+        return None
+    padded = GROUP_LANES * (p.vec * width + p.vec)
+    if CARRY_BUFFERS * FED_ROWS * padded * itemsize > LDS_BUDGET:
+        return None
+    return p, width
+
+
+def carry_preferred(info):
+    """True when 'auto' should take the variant without results in the scanning wavefront: its workgroups fit in one
+    round over the compute units, or fill their rounds and have rows long enough to pay for the start of the pipeline
+    in each (measured, float64: [1024, 16384] 47 us against 58, [2048, 16384] 94 / 97, [256, 65536] 154 / 192, but
+    [4096, 4096] 59 / 41, [1500, 8192] 49 / 34, [16384, 512] 59 / 31)."""
+    planned = carry_plan(info)
+    if planned is None:
+        return False
+    p, width = planned
+    groups = (p.rows + FED_ROWS - 1) // FED_ROWS
+    rounds = (groups + NUM_CU - 1) // NUM_CU
+    chunks = p.length // (GROUP_LANES * p.vec * width)
+    return groups <= NUM_CU or (10 * groups >= 9 * rounds * NUM_CU and chunks >= 24)
+
+
+def generate_carry(info, kernel_name, width=None):
+    p, width = carry_plan(info, width)
+    ctype = CTYPE[p.x.dtype]
+    vec = p.vec
+    rpb = FED_ROWS
+    seg = vec * width                       # columns a lane owns per chunk
+    chunk = GROUP_LANES * seg
+    num_chunks = p.length // chunk
+    padded_seg = seg + vec
+    row_stride = GROUP_LANES * padded_seg
+    chunk_vectors = rpb * chunk // vec
+    per_loader = chunk_vectors // (CARRY_LOADER_WAVES * WAVE)
+    per_storer = chunk_vectors // WAVE
+    reads_per_phase = width // CARRY_SYNC_PHASE
+
+    rank = len(info.workgroup_shape)
+    pos_exprs = []
+    stride = 1
+    strides = [1] * rank
+    for k in range(rank - 2, -1, -1):
+        stride *= info.workgroup_shape[k + 1]
+        strides[k] = stride
+    for k in range(rank):
+        expr = 'row'
+        if k > 0:
+            expr = '(row % ' + str(strides[k - 1]) + 'u)'
+        pos_exprs.append(expr + ' / ' + str(strides[k]) + 'u')
+    emitter = BodyEmitter(info, pos_exprs,
+                          read_hook=lambda node, tensor, idx: 'OVL_SCAN_IN',
+                          store_hook=lambda node, tensor, idx, value: 'OVL_SCAN_OUT(' + value + ');')
+    tagged = emitter.emit_tagged()
+    range_idx = p.loop_item.node
+    end_idx = max(i for i, _ in tagged)
+    prologue = [t for i, t in tagged if i < range_idx]
+    body = [t.strip() for i, t in tagged if range_idx < i < end_idx]
+    counter_name = 'e' + str(p.counter)
+    counter_type = CTYPE[info.nodes[p.counter].dtype]
+    state = [('e' + str(idx), CTYPE[info.nodes[idx].dtype]) for idx in _carried_state(info, p)]
+
+    vname = 'ovl_scan_vec'
+    src = []
+    a = src.append
+    a('typedef %s %s __attribute__((ext_vector_type(%d)));' % (ctype, vname, vec))
+    a('struct ovl_scan_yes { static constexpr bool value = true; };')
+    a('struct ovl_scan_no { static constexpr bool value = false; };')
+    a('')
+    a('extern "C" __global__ void __launch_bounds__(%d)' % CARRY_BLOCK)
+    a('%s(const %s* __restrict__ in%d, %s* __restrict__ out%d) {' % (
+        kernel_name, ctype, p.x.io_index, ctype, p.out.io_index))
+    if info.uses_math_tables():
+        a('    OVL_DECLARE_MATH_TABLES();')
+    a('    __shared__ __attribute__((aligned(16))) %s tile[%d][%d][%d];' % (ctype, CARRY_BUFFERS, rpb, row_stride))
+    for name, stype in state:
+        a('    __shared__ %s entering_%s[%d][%d];' % (stype, name, CARRY_BUFFERS, WAVE))
+    a('    const uint32_t row0 = blockIdx.x * %du;' % rpb)
+    a('    const uint32_t wave = threadIdx.x / %du, lane = threadIdx.x %% %du;' % (WAVE, WAVE))
+    a('    const %s* __restrict__ gin = in%d;' % (ctype, p.x.io_index))
+    a('    %s* __restrict__ gout = out%d;' % (ctype, p.out.io_index))
+    a('    // Every wavefront passes the same %d barriers: one after the first two chunks are in LDS, then one at the end' % (num_chunks + 3))
+    a('    // of each of the steps 0 .. %d.' % (num_chunks + 1))
+    a('    if (wave < 2u) {')
+    a('        // Scanning wavefront (0) and finisher (1): sixteen lanes per row, lane `part` of a group owns columns')
+    a('        // [part * %d, part * %d + %d) of every chunk of %d columns.  A group past the last row shadows it.' % (
+        seg, seg, seg, chunk))
+    a('        const uint32_t part = lane %% %du;' % GROUP_LANES)
+    a('        const uint32_t q = lane / %du;' % GROUP_LANES)
+    a('        const uint32_t row = (row0 + q < %du) ? row0 + q : %du;' % (p.rows, p.rows - 1))
+    a('        %s* const mine = &tile[0][q][part * %du];' % (ctype, padded_seg))
+    a('        // first column: the statements the worker runs before its loop, in every lane')
+    a('        %s first_out;' % ctype)
+    a('#define OVL_SCAN_IN (in%d[(uint64_t)row * %dull])' % (p.x.io_index, p.length))
+    a('#define OVL_SCAN_OUT(value) first_out = (value)')
+    for stmt in prologue:
+        a('        ' + stmt)
+    a('#undef OVL_SCAN_IN')
+    a('#undef OVL_SCAN_OUT')
+    a('#define OVL_SCAN_IN xv[u]')
+    a('#define OVL_SCAN_STEP(column) { %s = (%s)(column); %s }' % (counter_name, counter_type, ' '.join(body)))
+    a('        if (wave == 0u) {')
+    for name, stype in state:
+        a('            %s carry_%s = %s;' % (stype, name, name))
+    a('#define OVL_SCAN_OUT(value) (void)(value)')
+    a('            %s set_a[%d], set_b[%d];' % (vname, width, width))
+    a('            __syncthreads();')
+    a('            #pragma unroll')
+    a('            for (uint32_t w = 0; w < %du; ++w) set_a[w] = *reinterpret_cast<const %s*>(mine + w * %du);' % (
+        width, vname, vec))
+    a('            uint32_t next = 1u, slot = 0u;        // buffer of the chunk after this one; this chunk\'s slot')
+    a('            // One chunk: in phase p every lane runs the recurrence over its segment from the state it holds and hands')
+    a('            // its final state to its right neighbour; after phase p lanes 0..p are exact.  Meanwhile the segments of')
+    a('            // the next chunk arrive in the other register set.  The results are not kept.')
+    a('            auto scan_chunk = [&](const %s (&set)[%d], %s (&other)[%d], uint32_t column0, auto first_chunk) {' % (
+        vname, width, vname, width))
+    a('                const %s* ahead = mine + next * %du;' % (ctype, rpb * row_stride))
+    a('                const uint32_t col0 = column0 + part * %du;' % seg)
+    a('                #pragma unroll')
+    a('                for (uint32_t phase = 0; phase < %du; ++phase) {' % GROUP_LANES)
+    for name, _ in state:
+        a('                    %s = carry_%s;' % (name, name))
+    a('                    #pragma unroll')
+    a('                    for (uint32_t w = 0; w < %du; ++w) {' % width)
+    a('                        const %s xv = set[w];' % vname)
+    a('                        #pragma unroll')
+    a('                        for (uint32_t u = 0; u < %du; ++u) {' % vec)
+    a('                            // (the row\'s first column is what the statements before the loop computed)')
+    a('                            if (decltype(first_chunk)::value && w == 0u && u == 0u) { if (part != 0u) OVL_SCAN_STEP(col0) }')
+    a('                            else OVL_SCAN_STEP(col0 + w * %du + u)' % vec)
+    a('                        }')
+    a('                    }')
+    for name, _ in state:
+        a('                    carry_%s = ovl_dpp_move<OVL_DPP_ROW_SHR1>(carry_%s, %s);' % (name, name, name))
+    a('                    if (phase < %du) {' % CARRY_SYNC_PHASE)
+    a('                        #pragma unroll')
+    a('                        for (uint32_t j = 0; j < %du; ++j)' % reads_per_phase)
+    a('                            other[phase * %du + j] = *reinterpret_cast<const %s*>(ahead + (phase * %du + j) * %du);' % (
+        reads_per_phase, vname, reads_per_phase, vec))
+    a('                    }')
+    a('                    // (the fences keep each read in its phase and the barrier in its place)')
+    a('                    __builtin_amdgcn_sched_barrier(0);')
+    a('                    if (phase == %du) {' % CARRY_SYNC_PHASE)
+    a('                        __syncthreads();')
+    a('                        __builtin_amdgcn_sched_barrier(0);')
+    a('                    }')
+    a('                }')
+    a('                // lanes 1..15 now hold their left neighbour\'s exact final state, lane 0 the state that entered the')
+    a('                // chunk: what enters each lane\'s segment')
+    for name, _ in state:
+        a('                entering_%s[slot][lane] = carry_%s;' % (name, name))
+    a('                // the last lane finished the chunk: its state is the carry into the next one')
+    for name, _ in state:
+        a('                carry_%s = ovl_dpp_move<OVL_DPP_ROW_ROR1>(carry_%s, %s);' % (name, name, name))
+    a('                next = next + 1u == %du ? 0u : next + 1u;' % CARRY_BUFFERS)
+    a('                slot = slot + 1u == %du ? 0u : slot + 1u;' % CARRY_BUFFERS)
+    a('                __builtin_amdgcn_sched_barrier(0);')
+    a('            };')
+    a('            scan_chunk(set_a, set_b, 0u, ovl_scan_yes());')
+    if num_chunks > 1:
+        a('            uint32_t g = 1u;')
+        a('            #pragma unroll 1')
+        a('            for (; g + 1u < %du; g += 2u) {' % num_chunks)
+        a('                scan_chunk(set_b, set_a, g * %du, ovl_scan_no());' % chunk)
+        a('                scan_chunk(set_a, set_b, (g + 1u) * %du, ovl_scan_no());' % chunk)
+        a('            }')
+        a('            if (g < %du) scan_chunk(set_b, set_a, g * %du, ovl_scan_no());' % (num_chunks, chunk))
+    a('            __syncthreads();       // the last two steps: the others finish and store')
+    a('            __syncthreads();')
+    a('#undef OVL_SCAN_OUT')
+    a('        } else {')
+    a('            // The finisher: chunk s - 2 in step s, every segment once more from the state that enters it.')
+    a('#define OVL_SCAN_OUT(value) v[w][u] = (value)')
+    a('            __syncthreads();')
+    a('            __syncthreads();')
+    a('            __syncthreads();')
+    a('            for (uint32_t s = 2u; s <= %du; ++s) {' % (num_chunks + 1))
+    a('                const uint32_t buffer = (s - 2u) %% %du;' % CARRY_BUFFERS)
+    a('                %s* here = mine + buffer * %du;' % (ctype, rpb * row_stride))
+    a('                const uint32_t col0 = (s - 2u) * %du + part * %du;' % (chunk, seg))
+    a('                %s v[%d];' % (vname, width))
+    a('                #pragma unroll')
+    a('                for (uint32_t w = 0; w < %du; ++w) v[w] = *reinterpret_cast<const %s*>(here + w * %du);' % (
+        width, vname, vec))
+    for name, _ in state:
+        a('                %s = entering_%s[buffer][lane];' % (name, name))
+    a('                #pragma unroll')
+    a('                for (uint32_t w = 0; w < %du; ++w) {' % width)
+    a('                    const %s xv = v[w];' % vname)
+    a('                    #pragma unroll')
+    a('                    for (uint32_t u = 0; u < %du; ++u) {' % vec)
+    a('                        if (w == 0u && u == 0u && col0 == 0u) v[0][0] = first_out;')
+    a('                        else OVL_SCAN_STEP(col0 + w * %du + u)' % vec)
+    a('                    }')
+    a('                }')
+    a('                #pragma unroll')
+    a('                for (uint32_t w = 0; w < %du; ++w) *reinterpret_cast<%s*>(here + w * %du) = v[w];' % (width, vname, vec))
+    a('                __syncthreads();')
+    a('            }')
+    a('#undef OVL_SCAN_OUT')
+    a('        }')
+    a('#undef OVL_SCAN_STEP')
+    a('#undef OVL_SCAN_IN')
+    a('    } else {')
+    a('        // Storer (wavefront 2) and loaders: thread m of its kind owns vectors m, m + <threads of the kind>, ... of')
+    a('        // every chunk.  A loader\'s vector past the last row is a second copy of the last row\'s; the storer skips it.')
+    a('        auto place = [&](uint32_t v, uint64_t& global_offset, uint32_t& lds_offset, bool& exists) {')
+    a('            const uint32_t r = v / %du, c = (v %% %du) * %du;' % (chunk // vec, chunk // vec, vec))
+    a('            exists = row0 + r < %du;' % p.rows)
+    a('            global_offset = (uint64_t)(exists ? row0 + r : %du) * %dull + c;' % (p.rows - 1, p.length))
+    a('            lds_offset = r * %du + c + (c / %du) * %du;' % (row_stride, seg, vec))
+    a('        };')
+    a('        if (wave == 2u) {')
+    a('            uint64_t global_offset[%d];' % per_storer)
+    a('            uint32_t lds_offset[%d];' % per_storer)
+    a('            bool exists[%d];' % per_storer)
+    a('            #pragma unroll')
+    a('            for (uint32_t i = 0; i < %du; ++i) place(lane + i * %du, global_offset[i], lds_offset[i], exists[i]);' % (
+        per_storer, WAVE))
+    a('            auto store_chunk = [&](uint32_t c) {')
+    a('                const %s* buffer = &tile[c %% %du][0][0];' % (ctype, CARRY_BUFFERS))
+    a('                %s regs[%d];' % (vname, per_storer))
+    a('                #pragma unroll')
+    a('                for (uint32_t i = 0; i < %du; ++i) regs[i] = *reinterpret_cast<const %s*>(buffer + lds_offset[i]);' % (
+        per_storer, vname))
+    a('                #pragma unroll')
+    a('                for (uint32_t i = 0; i < %du; ++i)' % per_storer)
+    a('                    if (exists[i])')
+    a('                        __builtin_nontemporal_store(regs[i], reinterpret_cast<%s*>(gout + global_offset[i] + c * %du));' % (
+        vname, chunk))
+    a('            };')
+    a('            __syncthreads();')
+    a('            __syncthreads();')
+    a('            __syncthreads();')
+    a('            __syncthreads();')
+    a('            for (uint32_t s = 3u; s <= %du; ++s) {' % (num_chunks + 1))
+    a('                store_chunk(s - 3u);')
+    a('                __syncthreads();')
+    a('            }')
+    a('            store_chunk(%du);' % (num_chunks - 1))
+    a('        } else {')
+    a('            const uint32_t m = threadIdx.x - %du;' % (3 * WAVE))
+    a('            uint64_t global_offset[%d];' % per_loader)
+    a('            uint32_t lds_offset[%d];' % per_loader)
+    a('            #pragma unroll')
+    a('            for (uint32_t i = 0; i < %du; ++i) {' % per_loader)
+    a('                bool exists;')
+    a('                place(m + i * %du, global_offset[i], lds_offset[i], exists);' % (CARRY_LOADER_WAVES * WAVE))
+    a('            }')
+    a('            // Plain loads (with the non-temporal hint on loads and stores the mixed stream runs a quarter slower).  A')
+    a('            // chunk past the end of the row is requested as the last chunk once more and lands in a buffer that')
+    a('            // nobody reads any more: the steps are free of conditions and the counts of requests in flight exact.')
+    a('            auto request = [&](uint32_t c, %s (&regs)[%d]) {' % (vname, per_loader))
+    a('                const uint32_t cc = c < %du ? c : %du;' % (num_chunks, num_chunks - 1))
+    a('                #pragma unroll')
+    a('                for (uint32_t i = 0; i < %du; ++i)' % per_loader)
+    a('                    regs[i] = *reinterpret_cast<const %s*>(gin + global_offset[i] + cc * %du);' % (vname, chunk))
+    a('            };')
+    a('            auto to_lds = [&](uint32_t c, const %s (&regs)[%d]) {' % (vname, per_loader))
+    a('                %s* buffer = &tile[c %% %du][0][0];' % (ctype, CARRY_BUFFERS))
+    a('                #pragma unroll')
+    a('                for (uint32_t i = 0; i < %du; ++i) *reinterpret_cast<%s*>(buffer + lds_offset[i]) = regs[i];' % (
+        per_loader, vname))
+    a('            };')
+    a('            %s set[%d][%d];' % (vname, CARRY_AHEAD, per_loader))
+    a('            {')
+    a('                %s first[2][%d];' % (vname, per_loader))
+    a('                request(0u, first[0]);')
+    a('                request(1u, first[1]);')
+    for k in range(CARRY_AHEAD):
+        a('                request(%du, set[%d]);' % (2 + k, (2 + k) % CARRY_AHEAD))
+    a('                to_lds(0u, first[0]);')
+    a('                to_lds(1u, first[1]);')
+    a('            }')
+    a('            __syncthreads();')
+    a('            // step s: chunk s + 2 goes to LDS from the register set requested %d steps ago, which is then requested' % CARRY_AHEAD)
+    a('            // again with chunk s + %d' % (2 + CARRY_AHEAD))
+    a('            auto step = [&](uint32_t s, %s (&regs)[%d]) {' % (vname, per_loader))
+    a('                to_lds(s + 2u, regs);')
+    a('                request(s + %du, regs);' % (2 + CARRY_AHEAD))
+    a('                __syncthreads();')
+    a('            };')
+    steps = num_chunks + 2
+    whole = steps // CARRY_AHEAD
+    if whole:
+        a('            #pragma unroll 1')
+        a('            for (uint32_t s = 0u; s < %du; s += %du) {' % (whole * CARRY_AHEAD, CARRY_AHEAD))
+        for k in range(CARRY_AHEAD):
+            a('                step(s + %du, set[%d]);' % (k, (2 + k) % CARRY_AHEAD))
+        a('            }')
+    for s_ in range(whole * CARRY_AHEAD, steps):
+        a('            step(%du, set[%d]);' % (s_, (2 + s_) % CARRY_AHEAD))
+    a('        }')
+    a('    }')
+    a('}')
+
+    launch = {
+        'template': 'carryscan',
+        'vec': vec,
+        'block': CARRY_BLOCK,
         'blocks_needed': (p.rows + rpb - 1) // rpb,
         'align': {('in', p.x.io_index): 16, ('out', p.out.io_index): 16},
         'vector_loads': 1,

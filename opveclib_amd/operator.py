@@ -1,3 +1,8 @@
+# Derived from opveclib/operator.py of opveclib (https://github.com/opveclib/opveclib),
+# Copyright 2016 Hewlett Packard Enterprise Development LP, licensed under the Apache License, Version 2.0
+# (http://www.apache.org/licenses/LICENSE-2.0); see the NOTICE file at the root of this repository.
+# Changes: the decorator, the lazy operator handles and the operator DAG builder follow that file's interface and error
+# messages; tracing caches, the re-binding check on current bytecode, evaluation on device tensors and the launcher are new.
 """
 Operator front-end: the ``@operator`` decorator, lazy operator handles, gradient registration, the operator-DAG
 builder and the ``evaluate``/``profile`` entry points that run a DAG of operators on the GPU.

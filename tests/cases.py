@@ -184,6 +184,20 @@ def c3_rowscan_shapes(rng):
     return outs
 
 
+def carry_scans(rng):
+    """Row scans of 8-byte elements (and, forced, 4-byte ones) whose rows are whole chunks of the LDS-fed variant that
+    keeps no results in its scanning wavefront: one to nine chunks per row (the six LDS buffers come round again),
+    partial last workgroup, rank 3, sums, products, extrema, integers."""
+    return [cumsum(rng.standard_normal((9, 1536)), axis=1)[0],
+            cumprod(uniform(rng, 0.9, 1.1, (4, 4096), np.float64), axis=1)[0],
+            cumsum(rng.standard_normal((2, 3, 512)), axis=2)[0],
+            cumsum(rng.integers(-2 ** 40, 2 ** 40, size=(6, 1024)).astype(np.int64), axis=1)[0],
+            accumulate(rng.standard_normal((3, 3584)), inner_fcn=lambda acc, x: ovl.maximum(acc, x), axis=1)[0],
+            cumsum(rng.standard_normal((5, 768)), axis=1)[0],
+            cumsum(rng.standard_normal((5, 4608), dtype=np.float32), axis=1)[0],
+            cumsum(rng.standard_normal((1, 2048)), axis=1)[0]]
+
+
 def c3_colscan_shapes(rng):
     """Scans along an axis other than the last: partial strips, a partial last chunk of rows, dimensions before the
     axis, 4- and 8-byte elements, a single short chunk, more chunks than register sets with and without a remainder."""
@@ -960,6 +974,7 @@ CASES = [
     Case('c3_cumsum_f64', c3_cumsum_f64, seed=3),
     Case('c3_cumprod_f64', c3_cumprod_f64, seed=3),
     Case('c3_rowscan_shapes', c3_rowscan_shapes, seed=3),
+    Case('carry_scans', carry_scans, seed=3),
     Case('c3_colscan_shapes', c3_colscan_shapes, seed=3),
     Case('c4_lstm', c4_lstm, seed=4),
     Case('c4_lstm_grad', c4_lstm_grad, seed=4),
@@ -1301,6 +1316,12 @@ TEMPLATE_VARIANTS = [
     ('c3_colscan_shapes', {'template': 'colscan', 'scan_sets': 3}),
     ('c3_colscan_shapes', {'template': 'map'}),
     ('c3_rowscan_shapes', {'template': 'fedscan'}),
+    ('carry_scans', {'template': 'carryscan'}),
+    ('carry_scans', {'template': 'carryscan', 'scan_width': 8}),
+    ('carry_scans', {'template': 'fedscan'}),
+    ('carry_scans', {'template': 'map'}),
+    ('c3_cumsum_f32', {'template': 'carryscan'}),
+    ('c3_cumprod_f64', {'template': 'carryscan', 'scan_width': 8}),
     ('c3_cumsum_f64', {'template': 'fedscan'}),
     ('c3_cumprod_f64', {'template': 'fedscan', 'scan_width': 2}),
     ('c3_cumsum_f32', {'template': 'fedscan', 'scan_width': 4, 'scan_chunk': 256}),

@@ -47,7 +47,7 @@ def test_loaded_operators_come_from_the_hip_extension():
     assert len(runtime._loaded) > 0
     for compiled in runtime._loaded.values():
         assert compiled.so_path.endswith('_generic_hip.so')
-        assert compiled.lib.info['template'] in ('map', 'transpose', 'rowscan', 'skewscan', 'fedscan', 'colscan', 'colskew', 'treescan',
+        assert compiled.lib.info['template'] in ('map', 'transpose', 'rowscan', 'skewscan', 'fedscan', 'carryscan', 'colscan', 'colskew', 'treescan',
                                                 'rowreduce', 'colreduce')
 
 
