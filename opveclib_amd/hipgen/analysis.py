@@ -251,12 +251,20 @@ class DagInfo(object):
         reference's dot-product test keeps its loop bound in a variable, opveclib/test/test_dot_product.py:34-36),
         else None."""
         node = self.nodes[idx]
+        chain = []
         while node.code == lang.CAST or (node.code == lang.VARIABLE and node.idx not in self.written_variables):
             if node.dtype not in INT_RANGE:
                 return None
+            chain.append(node.dtype)
             node = self.nodes[node.ops[0]]
         if node.code == lang.CONST_SCALAR and node.dtype in INT_RANGE:
-            return int(node.data[0])
+            value = int(node.data[0])
+            # a literal that does not fit a type on the way (variable(300, uint8)) is not the value the code sees
+            for dtype in chain + [node.dtype]:
+                lo, hi = INT_RANGE[dtype]
+                if not lo <= value <= hi:
+                    return None
+            return value
         return None
 
     # -- affine forms --------------------------------------------------------------------------------------------
@@ -321,12 +329,21 @@ class DagInfo(object):
         if mode in ('ulp2', 'fast'):
             # the call sites that keep the bit-compatible routine (none in 'fast' mode) and the once-rounded
             # log1p / expm1 that stand in for the reference's formulas
-            from . import accuracy, ranges
-            known = ranges.analyse(self) if getattr(self, 'value_ranges', True) else None
-            cheap = accuracy.cheap_sites(self, known)
+            from . import accuracy
+            cheap = accuracy.cheap_sites(self, self.known_ranges())
             calls = [] if mode == 'fast' else [n for n in calls if n.idx not in cheap]
             calls += [k for k in cheap.values() if k in ('log1p', 'expm1')]
         return bool(calls)
+
+    def known_ranges(self):
+        """The value-range analysis of this DAG (None when it is switched off), computed once per setting."""
+        enabled = (bool(getattr(self, 'value_ranges', True)), getattr(self, 'math', 'exact'))
+        cached = getattr(self, '_known_ranges', None)
+        if cached is None or cached[0] != enabled:
+            from . import ranges
+            cached = (enabled, ranges.analyse(self) if enabled[0] else None)
+            self._known_ranges = cached
+        return cached[1]
 
     def tensor_accesses(self):
         """[(node, tensor node, affine or None)] for reads of inputs and stores to outputs, in program order."""

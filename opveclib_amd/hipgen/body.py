@@ -239,7 +239,7 @@ class BodyEmitter(object):
         """[(index of the expression that produced it, statement text)] in program order."""
         info = self.info
         math_mode = getattr(info, 'math', 'exact')
-        known = value_ranges.analyse(info) if getattr(info, 'value_ranges', True) else None
+        known = info.known_ranges()
         cheap_sites = accuracy.cheap_sites(info, known)
 
         def site_mode(node):

@@ -117,14 +117,18 @@ def plan(info, rows_per_block=None, chunk=None, need_chunk=True, multi=False):
         return None
     if len(outs) != len(info.outputs):
         return None
-    if len(outs) > 1:
-        # several outputs: each is stored exactly once before the loop (column 0) and once in it
-        for t in outs:
-            for inside in (False, True):
-                count = len([n for n, tensor, _ in info.tensor_accesses()
-                             if n.code == lang.ASSIGN_TENSOR and tensor is t and bool(info.in_loop[n.idx]) == inside])
+    # every output is stored exactly once inside the loop (a worker that only stores before its loop is a reduction
+    # that writes one column: the scan templates would store registers nothing assigned over every column), and,
+    # when there are several outputs, exactly once before it (column 0); a single output at most once before it
+    for t in outs:
+        for inside in (False, True):
+            count = len([n for n, tensor, _ in info.tensor_accesses()
+                         if n.code == lang.ASSIGN_TENSOR and tensor is t and bool(info.in_loop[n.idx]) == inside])
+            if inside or len(outs) > 1:
                 if count != 1:
                     return None
+            elif count > 1:
+                return None
     itemsize = ITEMSIZE[x.dtype]
     if itemsize not in (4, 8) or x.dtype not in CTYPE:
         return None

@@ -240,6 +240,106 @@ def test_the_narrow_domain_limits_are_needed(sweep, kind, outside):
     assert int(out[2]) > accuracy.TOLERANCE
 
 
+FORMULA_PROGRAM = r"""
+#include <math.h>
+#include <stdio.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+static int32_t ordered(float f) { int32_t i; memcpy(&i, &f, 4); return i < 0 ? (int32_t)0x80000000 - i : i; }
+static float log1p_formula(float x) {
+    volatile float u = 1.0f + x; volatile float d = u - 1.0f;
+    if (isinf(x) && x > 0) return x;
+    if (d == 0) return x;
+    volatile float l = logf(u); volatile float p = l * x; return p / d;
+}
+static float expm1_formula(float x) {
+    volatile float e = expf(x);
+    if (isinf(x) && x > 0) return x;
+    if (e == 1.0f) return x;
+    volatile float em = e - 1.0f;
+    if (em == -1.0f) return -1.0f;
+    volatile float p = em * x; volatile float l = logf(e); return p / l;
+}
+static float sigmoid_formula(float x) { volatile float n = -x; volatile float e = expf(n); volatile float s = 1.0f + e; return 1.0f / s; }
+int main(int argc, char** argv) {
+    int which = atoi(argv[1]); float lo = strtof(argv[2], 0), hi = strtof(argv[3], 0); uint32_t step = atoi(argv[4]);
+    // every step-th float32 of [lo, hi] in increasing order, both ends included
+    int32_t a = ordered(lo), b = ordered(hi);
+    float least = INFINITY, most = -INFINITY; int worst = 0;
+    for (int64_t i = a; ; i += step) {
+        if (i > b) i = b;
+        int32_t o = (int32_t)i; int32_t bits = o < 0 ? (int32_t)0x80000000 - o : o; float x; memcpy(&x, &bits, 4);
+        float got = which == 0 ? log1p_formula(x) : which == 1 ? expm1_formula(x) : sigmoid_formula(x);
+        double exact = which == 0 ? log1p((double)x) : which == 1 ? expm1((double)x) : 1.0 / (1.0 + exp(-(double)x));
+        int d = abs(ordered(got) - ordered((float)exact));
+        if (d > worst) worst = d;
+        if (got < least) least = got;
+        if (got > most) most = got;
+        if (i == b) break;
+    }
+    printf("%d %.9g %.9g\n", worst, least, most);
+    return 0;
+}
+"""
+
+
+@pytest.fixture(scope='module')
+def formula_sweep(tmp_path_factory):
+    directory = tmp_path_factory.mktemp('formulas')
+    src = directory / 'formulas.cpp'
+    src.write_text(FORMULA_PROGRAM)
+    exe = directory / 'formulas'
+    subprocess.check_call(['g++', '-O2', '-ffp-contract=off', '-std=c++17', str(src), '-o', str(exe)])
+    return exe
+
+
+def _formula_division_range(kind, lo, hi):
+    """The value range the analysis gives the division that ends the formula of ``kind`` on arguments in [lo, hi]."""
+    @ovl.operator()
+    def clipped(x, lo=None, hi=None):
+        out = ovl.output_like(x)
+        pos = ovl.position_in(x.shape)
+        out[pos] = ovl.minimum(ovl.maximum(x[pos], lo), hi)
+        return out
+
+    formula = {'log1p': log1p, 'expm1': expm1, 'sigmoid': stdops.sigmoid}[kind]
+    op, = workloads.fused_operators([formula(clipped(Spec((1024,)), lo=lo, hi=hi))[0]])
+    info = DagInfo(op)
+    known = ranges.analyse(info)
+    quotients = [n for n in info.nodes if n.code == lang.DIVIDE and accuracy.match_idiom(info, known, n)]
+    assert len(quotients) == 1, kind
+    return known.ranges[quotients[0].idx]
+
+
+@pytest.mark.parametrize('kind', ['log1p', 'expm1', 'sigmoid'])
+def test_formula_values_stay_inside_the_range_the_analysis_narrows_them_to(formula_sweep, kind):
+    """The analysis bounds the division that ends a recognised formula by the image of the function itself, widened
+    by ranges._SLACK_ULPS float32 steps, in every math mode (guards are pruned and in-range routines chosen from
+    it).  That is sound only while the formula evaluated with the host library stays within that many steps of the
+    function on the whole compared domain: measured here on a sweep of each domain with both ends, and the narrowed
+    range of several sub-intervals is compared with the least and greatest value the formula takes on them."""
+    assert ranges._SLACK_ULPS >= 7          # "in every math mode within seven" (ranges.RangeInfo._formula_image)
+    which = {'log1p': '0', 'expm1': '1', 'sigmoid': '2'}[kind]
+    lo, hi = accuracy.IDIOM_DOMAIN[kind]
+    worst, _, _ = subprocess.check_output([str(formula_sweep), which, repr(lo), repr(hi), '61'],
+                                          universal_newlines=True).split()
+    assert int(worst) <= 3                  # "within three float32 steps of the function itself"
+    intervals = {'log1p': [(lo, hi), (lo, 2.0 ** -9), (0.25, 0.75), (0.2689, 0.7311), (1.0, 1.0e19), (2.0 ** 63, hi)],
+                 'expm1': [(lo, hi), (lo, 2.0 ** -11), (0.2384, 0.5489), (1.0, 10.0), (60.0, hi)],
+                 'sigmoid': [(lo, hi), (lo, -15.0), (-1.0, 1.0), (-0.7616, 0.7616), (20.0, hi)]}[kind]
+    for a, b in intervals:
+        a32, b32 = float(np.float32(a)), float(np.float32(b))
+        if a32 < lo:
+            a32 = float(np.nextafter(np.float32(a32), np.float32(np.inf)))
+        if b32 > hi:
+            b32 = float(np.nextafter(np.float32(b32), np.float32(-np.inf)))
+        r = _formula_division_range(kind, a32, b32)
+        _, least, most = subprocess.check_output([str(formula_sweep), which, repr(a32), repr(b32), '17'],
+                                                 universal_newlines=True).split()
+        assert r.lo <= float(least) and float(most) <= r.hi, (kind, a, b, r.lo, r.hi, least, most)
+
+
 @pytest.mark.parametrize('kind,outside', [('log1p', (8e37, 3e38)), ('expm1', (70.0, 88.0))])
 def test_the_domain_limits_are_needed(sweep, kind, outside):
     """Towards overflow the reference's formulas (whose 1 + x and exp(x) become infinite early) leave the once-rounded

@@ -78,9 +78,18 @@ def test_template_selection():
     # last-axis accumulation with a chunkable row length: the order-preserving row scan
     scan = template(cumsum(np.zeros((48, 1024), np.float32), axis=1))
     assert scan['template'] == 'skewscan' and scan['blocks_needed'] == 3       # 16 rows per workgroup
-    # 8-byte elements: the lane-skewed recurrence fed from LDS, four rows per workgroup
-    fed = template(cumsum(np.zeros((1024, 16384), np.float64), axis=1))
-    assert fed['template'] == 'fedscan' and fed['blocks_needed'] == 256
+    # 8-byte elements: the lane-skewed recurrence fed from LDS, four rows per workgroup.  With at most one workgroup
+    # per compute unit (or whole rounds of them and long rows) the scanning wavefront keeps no results and a second
+    # wavefront recomputes them; with more, three of the lockstep variant's workgroups share a compute unit
+    carry = template(cumsum(np.zeros((1024, 16384), np.float64), axis=1))
+    assert carry['template'] == 'carryscan' and carry['blocks_needed'] == 256 and carry['block'] == 320
+    assert template(cumsum(np.zeros((2048, 16384), np.float64), axis=1))['template'] == 'carryscan'
+    fed = template(cumsum(np.zeros((4096, 4096), np.float64), axis=1))
+    assert fed['template'] == 'fedscan' and fed['blocks_needed'] == 1024
+    assert template(cumsum(np.zeros((1500, 8192), np.float64), axis=1))['template'] == 'fedscan'
+    assert template(cumsum(np.zeros((1024, 16384), np.float64), axis=1), {'template': 'fedscan'})['template'] == 'fedscan'
+    # (rows that are not whole chunks of at least 128 columns keep the lockstep variant or the register-fed scan)
+    assert template(cumsum(np.zeros((64, 1088), np.float64), axis=1))['template'] == 'fedscan'
     assert template(cumsum(np.zeros((1024, 16384), np.float64), axis=1), {'template': 'skewscan'})['blocks_needed'] == 64
     lds = template(cumsum(np.zeros((48, 1024), np.float32), axis=1), {'template': 'rowscan'})
     assert lds['template'] == 'rowscan' and lds['blocks_needed'] == 48
@@ -123,6 +132,29 @@ def test_template_selection():
     odd = template(gather_transpose(np.zeros((6, 9), np.float32), np.zeros(54, np.float32), alpha=0.5, stride=1))
     # (extents that no vector width divides still go through the tile, one element per access)
     assert odd['template'] == 'transpose' and odd['vec'] == 1
+
+
+def test_a_row_sum_into_one_column_of_a_full_size_output_is_not_taken_for_a_scan():
+    """A worker that stores only before its loop (a row sum kept in column 0 of an output as large as the input) has
+    the loop shape of a scan but nothing to store per column: the scan templates would write registers that nothing
+    assigned over the whole output.  It must go to a template that stores what the worker stores."""
+    @ovl.operator()
+    def sum_into_first_column(x):
+        rows, cols = x.shape
+        row = ovl.position_in([rows])[0]
+        out = ovl.output_like(x)
+        acc = ovl.variable(0, x.dtype)
+        acc <<= x[row, 0]
+        out[row, 0] = acc
+        for i in ovl.arange(1, cols):
+            acc <<= acc + x[row, i]
+        return out
+
+    generated = hipgen.generate(sum_into_first_column(np.zeros((48, 1024), np.float32)).expression_dag, 'f' + '5' * 56)
+    assert generated.launch['template'] not in ('skewscan', 'fedscan', 'carryscan', 'rowscan', 'treescan')
+    from opveclib_amd.hipgen import rowscan_kernel
+    info = DagInfo(sum_into_first_column(np.zeros((48, 1024), np.float32)).expression_dag)
+    assert rowscan_kernel.plan(info, need_chunk=False, multi=True) is None
 
 
 def test_chain8_kernel_shape():
