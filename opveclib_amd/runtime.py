@@ -41,11 +41,25 @@ def _io_types(op):
 codegen_options = {}
 
 
+#: the operations whose code the 'ulp2' math mode can change (float32 only)
+_MATH_SENSITIVE = (lang.EXP, lang.LOG, lang.TANH, lang.DIVIDE)
+
+
+def effective_options(op, options):
+    """``options`` without a 'ulp2' math mode that cannot change this operator's code (no float32 exp, log, tanh or
+    division in it): such an operator is the 'exact' kernel, and is generated, compiled and cached as that."""
+    if options and options.get('math') == 'ulp2' and not any(
+            e.code in _MATH_SENSITIVE and e.dtype == lang.FLOAT32 for e in op.expressions):
+        options = dict((k, v) for k, v in options.items() if k != 'math')
+    return options or None
+
+
 def build_operator(op, options=None):
     """Generate HIP for one operator and make sure its library exists on disk.  Needs hipcc, not a GPU.
 
     :return: (GeneratedOperator, library path)
     """
+    options = effective_options(op, options)
     name = _op_hash(op)
     key = (name, repr(sorted((options or {}).items())))
     with _lock:
@@ -107,6 +121,7 @@ class CompiledOperator(object):
 def load_operator(op, options=None):
     if codegen_options:
         options = dict(codegen_options, **(options or {}))
+    options = effective_options(op, options)
     name = _op_hash(op)
     key = (name, repr(sorted((options or {}).items())))
     with _lock:
@@ -130,10 +145,10 @@ def _build_missing(operators, options):
     """
     if codegen_options:
         options = dict(codegen_options, **(options or {}))
-    option_key = repr(sorted((options or {}).items()))
     missing = {}
     for op in operators:
         name = _op_hash(op)
+        option_key = repr(sorted((effective_options(op, options) or {}).items()))
         with _lock:
             known = (name, option_key) in _loaded or (name, option_key) in _generated
         if not known:

@@ -1542,7 +1542,7 @@ def run_case_on_gpu(case, opt_level):
     import oracle
     outs = case.outputs()
     ref = oracle.profile(outs, 1, 0)[0]
-    got = ovl.evaluate(outs, target_language='hip', opt_level=opt_level)
+    got = ovl.evaluate(outs, target_language='hip', opt_level=opt_level, math_mode='exact')
     got = got if isinstance(got, list) else [got]
     assert len(got) == len(ref)
     for n, (g, r) in enumerate(zip(got, ref)):

@@ -231,6 +231,51 @@ def test_evaluate_rejects_other_targets():
         ovl.profile(stdops.add(np.zeros(3), np.zeros(3)), 'hip', 0, 3)
 
 
+@pytest.fixture
+def unpinned_math_mode(monkeypatch):
+    """The math mode as a fresh process finds it (this suite pins 'exact' in conftest.py)."""
+    import importlib
+    ovl_operator = importlib.import_module('opveclib_amd.operator')
+    monkeypatch.setattr(ovl_operator, '_default_math_mode', [None])
+    monkeypatch.delenv('OPVECLIB_MATH', raising=False)
+    return monkeypatch
+
+
+def test_the_default_math_mode_is_ulp2_and_the_environment_overrides_it(unpinned_math_mode):
+    """An unchanged reference-style call (`evaluate(outputs)`, opveclib/operator.py:2099-2117: no math argument) runs
+    in the mode the task states as the float32 tolerance; the bit-exact mode is one switch away."""
+    import importlib
+    ovl_operator = importlib.import_module('opveclib_amd.operator')
+    assert ovl.get_math_mode() == 'ulp2' == ovl_operator.DEFAULT_MATH_MODE
+    ovl_operator._default_math_mode[0] = None
+    unpinned_math_mode.setenv('OPVECLIB_MATH', 'exact')
+    assert ovl.get_math_mode() == 'exact'
+    ovl.set_math_mode('fast')
+    assert ovl.get_math_mode() == 'fast'
+    ovl_operator._default_math_mode[0] = None
+    unpinned_math_mode.setenv('OPVECLIB_MATH', 'sloppy')
+    with pytest.raises(ValueError):
+        ovl.get_math_mode()
+
+
+def test_a_math_mode_that_cannot_change_an_operator_selects_the_exact_kernel():
+    """'ulp2' only concerns float32 exp, log, tanh and division: operators without them (data movement, integer and
+    float64 arithmetic, accumulations) are generated, compiled and cached once, as the bit-exact kernel."""
+    from opveclib_amd import runtime, workloads
+    from opveclib_amd.workloads import Spec
+    plain, = workloads.fused_operators([stdops.add(Spec((64,)), Spec((64,)))[0]])
+    assert runtime.effective_options(plain, {'math': 'ulp2'}) is None
+    assert runtime.effective_options(plain, {'math': 'ulp2', 'vec': 2}) == {'vec': 2}
+    assert runtime.effective_options(plain, {'math': 'fast'}) == {'math': 'fast'}
+    f64, = workloads.fused_operators([stdops.tanh(Spec((64,), np.float64))[0]])
+    assert runtime.effective_options(f64, {'math': 'ulp2'}) is None
+    scan, = workloads.fused_operators([cumsum(Spec((8, 64)), axis=1)[0]])
+    assert runtime.effective_options(scan, {'math': 'ulp2'}) is None
+    f32, = workloads.fused_operators([stdops.tanh(Spec((64,)))[0]])
+    assert runtime.effective_options(f32, {'math': 'ulp2'}) == {'math': 'ulp2'}
+    assert runtime.effective_options(f32, None) is None
+
+
 # ----------------------------------------------------------------------------------------------------------------------
 # gradients
 # ----------------------------------------------------------------------------------------------------------------------

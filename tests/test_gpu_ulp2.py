@@ -166,3 +166,45 @@ def test_lstm_keeps_the_oracle_bits_in_ulp2_mode():
         got = ovl.evaluate(outs, opt_level=3, math_mode='ulp2')
         for g, r in zip(got, ref):
             assert np.array_equal(g, r, equal_nan=True), name
+
+
+def test_an_unmodified_reference_style_call_runs_the_ulp2_kernel(monkeypatch):
+    """`ovl.evaluate(outputs)` as the reference's callers write it (opveclib/operator.py:2099-2117: no math argument),
+    in a process that has chosen no mode: the 'ulp2' kernel runs, also when the environment says OPVECLIB_MATH=ulp2,
+    and OPVECLIB_MATH=exact selects the bit-exact one."""
+    import torch
+    import importlib
+    from opveclib_amd import runtime
+    ovl_operator = importlib.import_module('opveclib_amd.operator')
+    case = cases.CASE_BY_NAME['c2_chain']
+    outs = case.outputs()
+    dag, _ = __import__('opveclib_amd.fusion', fromlist=['_merge_op_dag'])._merge_op_dag(
+        ovl_operator._build_op_dag(*outs).proto_dag, None)
+    assert len(dag.operators) == 1
+
+    def kernel_of_an_unqualified_call():
+        before = set(runtime._loaded)
+        got = ovl.evaluate(outs)
+        key = [k for k in runtime._loaded if k[0] == ovl_operator._op_hash(dag.operators[0])]
+        used = [k for k in key if k not in before] or key
+        return got, [runtime._loaded[k].lib.info['kernel'] for k in used]
+
+    exact = ovl.evaluate(outs, math_mode='exact')
+    for setting, suffix in ((None, '_ulp2'), ('ulp2', '_ulp2')):
+        monkeypatch.setattr(ovl_operator, '_default_math_mode', [None])
+        if setting is None:
+            monkeypatch.delenv('OPVECLIB_MATH', raising=False)
+        else:
+            monkeypatch.setenv('OPVECLIB_MATH', setting)
+        runtime._loaded.clear()
+        got, kernels = kernel_of_an_unqualified_call()
+        assert ovl.get_math_mode() == 'ulp2'
+        assert len(kernels) == 1 and kernels[0].endswith(suffix), kernels
+        # close to the bit-exact result (the chain ends in a subtraction, so the bound is absolute)
+        assert np.abs(np.asarray(got, np.float64) - np.asarray(exact, np.float64)).max() < 1e-6
+    monkeypatch.setattr(ovl_operator, '_default_math_mode', [None])
+    monkeypatch.setenv('OPVECLIB_MATH', 'exact')
+    runtime._loaded.clear()
+    got, kernels = kernel_of_an_unqualified_call()
+    assert len(kernels) == 1 and not kernels[0].endswith('_ulp2') and not kernels[0].endswith('_fast')
+    assert np.array_equal(np.asarray(got), np.asarray(exact))
