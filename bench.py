@@ -9,12 +9,15 @@ one launch of the fused kernel on inputs that are already resident in HBM.  The 
 in GB/s counted on algorithmic bytes (each input element read once, each output element written once:
 3 * 2^26 * 4 + 4 bytes per launch).
 
-Math mode of the headline: 'ulp2' - every operator of the chain returns values within two float32 units in the last
-place of what the reference's generated C++ computes from the same operator inputs (the tolerance the task states for
-transcendental operators).  The benchmark checks exactly that on the full tensors before it reports the mode (each
-transcendental stage of the fused kernel against the bit-exact operator applied to the same stage input) and falls
-back to the bit-exact 'exact' mode as headline if the check fails.  The 'exact' mode's own line, compared bit for bit
-with the CPU oracle on the full tensors, is always reported under `others`.
+Math mode of the headline: 'ulp2', the package's default - every operator of the chain returns values within two
+float32 units in the last place of what the reference's generated C++ computes from the same operator inputs (the
+tolerance the task states for transcendental operators).  The benchmark checks exactly that on the full tensors
+before it reports the mode, two ways: each transcendental stage of the fused kernel against the bit-exact operator
+applied to the same stage input, and each transcendental operator on its own, fed the CPU oracle's stage input,
+against the CPU oracle's stage output (all 2^26 elements); it falls back to the bit-exact 'exact' mode as headline if
+a check fails.  The fused chain is NOT within 2 ulp end to end (its last stages subtract nearly equal numbers); the
+end-to-end distance is reported.  The 'exact' mode is always timed too and compared bit for bit with the CPU oracle
+on the full tensors; its bandwidth stands next to the headline's in `config`.
 
 Order of work: everything that runs on the host (the CPU oracle: compiling where no built library exists, timing,
 reference results) happens first, before the process touches the GPU, so that no child process is started afterwards.
@@ -56,9 +59,12 @@ from opveclib_amd.workloads import (uniform, chain8_outputs, chain8_stage_output
 
 HBM_PEAK_GBPS = 8000.0
 
-# HBM bytes per launch of the chain8 kernel from rocprofv3 counters (FETCH_SIZE, WRITE_SIZE, each scaled by the same
-# counter's reading for the copy kernel of known size).  Source: profiles/bench_all_kernels_hbm_traffic_counters.md
-CHAIN8_TRAFFIC_BYTES = {'exact': 805167788, 'ulp2': 805168674}
+# HBM bytes per launch of the chain8 kernels from rocprofv3 counters (FETCH_SIZE, WRITE_SIZE, each scaled by the same
+# counter's reading for the copy kernel of known size), by the name of the kernel they were measured on: a kernel
+# the generator has changed since has another name and reports no traffic until it is measured again.
+# Source: profiles/bench_all_kernels_hbm_traffic_counters.md
+CHAIN8_TRAFFIC_BYTES = {'ovl_add_mul_tanh_sigmoid_log1p_expm1_sub_absolute_b1b47766': 805167788,
+                        'ovl_add_mul_tanh_sigmoid_log1p_expm1_sub_absolute_b1b47766_ulp2': 805168674}
 
 CHAIN8_STAGES = ('add', 'mul', 'tanh', 'sigmoid', 'log1p', 'expm1', 'sub', 'abs')
 
@@ -275,10 +281,12 @@ class HandWrittenScan(object):
         self.out = torch.empty_like(self.x)
         self.rows, self.cols = self.x.shape
         self.algorithmic_bytes = 2 * self.x.numel() * self.x.element_size()
-        # (8-byte rows of a multiple of 512 columns take the LDS-fed kernel, include/ovl_scan.h)
+        # (8-byte rows of a multiple of 512 columns take the LDS-fed kernels, include/ovl_scan.h: with at most one
+        # workgroup of four rows per compute unit the one whose scanning wavefront keeps no results)
         fed = self.x.element_size() == 8 and self.cols % 512 == 0
+        carry = fed and (self.rows + 3) // 4 <= 256
         self.kernels = [{'kernel': 'reassociated_scan_kernel' if entry.endswith('_reassociated')
-                         else 'fed_scan_kernel' if fed else 'skewed_scan_kernel'}]
+                         else 'carry_scan_kernel' if carry else 'fed_scan_kernel' if fed else 'skewed_scan_kernel'}]
 
     def launch(self, stream):
         if self.entry(self.x.data_ptr(), self.rows, self.cols, self.out.data_ptr(), stream) != 0:
@@ -288,9 +296,15 @@ class HandWrittenScan(object):
         return [self.out]
 
 
+ONLY = [None]           # --only
+
+
 def side_workload(name, outputs, steps, warmup, options=None, reference=None, sustained=False):
     """Time one workload; with ``reference`` (a cpu_reference record) also compare the results with the oracle's;
-    ``sustained``: after a second and a half of continuous work (for kernels at the power limit)."""
+    ``sustained``: after a second and a half of continuous work (for kernels at the power limit).  None for a
+    workload that --only leaves out."""
+    if ONLY[0] is not None and ONLY[0] not in name:
+        return None
     handwritten = isinstance(outputs, (HandWrittenLstm, HandWrittenScan))
     prepared = outputs if handwritten else Prepared(outputs, options)
     settle(prepared)
@@ -402,6 +416,50 @@ def chain8_stagewise(a, b, s, mode):
     return worst
 
 
+def chain8_single_operators_vs_oracle(oracle_stages, mode):
+    """
+    Every transcendental operator of the chain on its own in ``mode``, fed the CPU oracle's stage input and compared
+    with the CPU oracle's stage output on the full tensors.  Returns {stage: largest distance in float32 units in the
+    last place}.
+    """
+    import torch
+    import opveclib_amd as ovl
+    from opveclib_amd import stdops
+    from opveclib_amd.examples import log1p, expm1
+    single = {'tanh': stdops.tanh, 'sigmoid': stdops.sigmoid, 'log1p': log1p, 'expm1': expm1}
+    worst = {}
+    for k, name in enumerate(CHAIN8_STAGES):
+        if name in single:
+            x = torch.from_numpy(oracle_stages[k - 1]).cuda()
+            got = ovl.evaluate(single[name](x)[0], opt_level=0, math_mode=mode)
+            want = torch.from_numpy(oracle_stages[k]).cuda()
+            worst[name] = int(ulp_distance(got, want).max())
+            del x, got, want
+    torch.cuda.empty_cache()
+    return worst
+
+
+def stdops_lstm_stagewise(concat, c, mode):
+    """The promise of a math mode on the LSTM cell composed of library operators at full size: the fused kernel with
+    every operator's output requested, each sigmoid and tanh against the bit-exact operator applied to the kernel's
+    own value of that operator's input.  Returns {operator: largest distance in float32 ulp}."""
+    import torch
+    import opveclib_amd as ovl
+    from opveclib_amd import stdops
+    got = dict(zip(workloads.STDOPS_LSTM_STAGES,
+                   ovl.evaluate(workloads.stdops_lstm_stage_outputs(concat, c), opt_level=3, math_mode=mode)))
+    worst = {}
+    for name, fcn, arg in (('sigmoid_f', stdops.sigmoid, 'f'), ('sigmoid_i', stdops.sigmoid, 'i'),
+                           ('tanh_j', stdops.tanh, 'j'), ('tanh_new_c', stdops.tanh, 'new_c'),
+                           ('sigmoid_o', stdops.sigmoid, 'o')):
+        ref = ovl.evaluate(fcn(got[arg])[0], opt_level=0, math_mode='exact')
+        worst[name] = int(ulp_distance(got[name], ref).max())
+        del ref
+    del got
+    torch.cuda.empty_cache()
+    return worst
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument('--gpus', type=int, default=1)
@@ -413,11 +471,18 @@ def main():
     parser.add_argument('--settle-ms', type=float, default=40.0,
                         help='kernel time spent on untimed launches before each warm-up so that the clocks settle; '
                              '0 skips them (for counter collection, where every launch is slow and only counted)')
+    parser.add_argument('--only', default=None,
+                        help='time only the side workloads whose name contains this text (to profile one kernel): '
+                             'no CPU oracle, no parity checks of the headline; "row stride" adds float32 scans of '
+                             'rows of 16384, 16448 and 16640 columns')
     parser.add_argument('--sustain-ms', type=float, default=1500.0,
                         help='continuous work before a kernel that reaches the power limit is timed (steady state)')
     args = parser.parse_args()
     SETTLE_MS[0] = args.settle_ms
     SUSTAIN_MS[0] = args.sustain_ms
+    ONLY[0] = args.only
+    if args.only is not None:
+        args.no_cpu = True
     if args.gpus != 1:
         sys.exit('bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)' % args.gpus)
 
@@ -447,6 +512,7 @@ def main():
         g = np.random.default_rng(5)
         data['a5'] = g.standard_normal((16384, 16384), dtype=np.float32)
         data['b5'] = g.standard_normal(16384 * 16384, dtype=np.float32)
+        data['conv1d'] = workloads.conv1d_reference_inputs()
         g = np.random.default_rng(6)
         data['x0'] = g.standard_normal(workloads.REFERENCE_CUMSUM_SHAPE)
         for units in workloads.REFERENCE_LSTM_UNITS:
@@ -470,8 +536,9 @@ def main():
             'sample': 'the full chain8 inputs (float32 [8192, 8192]); reference-shaped fused C++ (g++, no -O flag as '
                       'in the reference), std::thread block split, thread create/join inside the timed region, '
                       'best of 3'}
-        # the operators as written (eight generated functions): the reference result for the bit-exact check
-        cpu['chain8'] = cpu_reference(chain8_outputs(a, b, s), 'the full tensors', iters=1)
+        # the operators as written (eight generated functions), every stage kept: the reference results for the
+        # bit-exact check of the last stage and for the per-operator check of the 'ulp2' mode
+        cpu['chain8'] = cpu_reference(chain8_stage_outputs(a, b, s), 'the full tensors', iters=1)
         if with_others:
             full = 'the full tensors'
             cpu['c1'] = cpu_reference(c1_outputs(data['c1']), full)
@@ -481,6 +548,8 @@ def main():
             cpu['lstm'] = cpu_reference(lstm_outputs(data['concat'], data['c']), full)
             cpu['lstm_grad'] = cpu_reference(lstm_grad_outputs(data['concat'], data['c'], data['dc'], data['dh']),
                                              full)
+            cpu['stdops_lstm'] = cpu_reference(workloads.stdops_lstm_outputs(data['concat'], data['c']), full)
+            cpu['conv1d'] = cpu_reference(workloads.conv1d_outputs(*data['conv1d']), full, iters=10)
             cpu['gather'] = cpu_reference(gather_outputs(data['a5'], data['b5']), full, iters=2)
             cpu['cumsum_axis0'] = cpu_reference(cumsum_outputs(data['x0'], axis=0), full, iters=10)
             cpu['dot'] = cpu_reference(workloads.dot_outputs(data['xs'], data['xp']), full)
@@ -503,17 +572,55 @@ def main():
     leaves = exact.leaves
     nbytes = exact.algorithmic_bytes
 
-    stagewise = chain8_stagewise(leaves[0], leaves[1], leaves[2], 'ulp2')
-    mode = 'ulp2' if max(stagewise.values()) <= 2 else 'exact'
+    quick = args.only is not None       # profiling one side workload: the headline is launched, not examined
+    stagewise = {'not_checked': 0} if quick else chain8_stagewise(leaves[0], leaves[1], leaves[2], 'ulp2')
+    against_oracle = None
+    if 'chain8' in cpu:
+        against_oracle = chain8_single_operators_vs_oracle(cpu['chain8']['results'], 'ulp2')
+        # only the last stage is needed from here on (the bit-exact check of the exact mode)
+        cpu['chain8']['results'] = cpu['chain8']['results'][-1:]
+    promised = max(stagewise.values()) <= 2 and (against_oracle is None or max(against_oracle.values()) <= 2)
+    mode = 'ulp2' if promised else 'exact'
     chain = Prepared(chain8_outputs(*leaves), {'math': 'ulp2'}) if mode == 'ulp2' else exact
     assert len(chain.ops) == 1
 
     settled_after = settle(chain)
-    sustain(chain)
+    if not quick:
+        sustain(chain)
     wall_ms, event_ms, min_ms = measure(chain, args.steps, args.warmup)
     value = nbytes / (wall_ms * 1e-3) / 1e9
     achieved = nbytes / (event_ms * 1e-3) / 1e9
+    headline_clocks = None if quick else clocks_under_load(chain)
 
+    # the bit-exact mode of the same workload, always: what a caller gets who asks for the reference's bits
+    settle(exact)
+    if not quick:
+        sustain(exact)
+    exact_wall_ms, exact_ms, exact_min = measure(exact, 3 if quick else max(10, min(args.steps, 40)), args.warmup)
+    exact_gbps = nbytes / (exact_ms * 1e-3) / 1e9
+
+    # parity of the headline: stage-wise distances of the ulp2 mode, end-to-end statistics against the exact mode,
+    # and the exact mode against the CPU oracle bit for bit on the full tensors
+    torch.cuda.synchronize()
+    parity = {'ulp2_stagewise_max_ulp': stagewise, 'ulp2_single_operators_vs_cpu_oracle_max_ulp': against_oracle}
+    end_to_end = None
+    if mode == 'ulp2':
+        exact_y, y = exact.results()[0], chain.results()[0]
+        ulps = ulp_distance(y, exact_y)
+        end_to_end = parity['ulp2_end_to_end_vs_exact'] = {
+            'max_abs_err': float((y.double() - exact_y.double()).abs().max()),
+            'frac_bit_equal': float((ulps == 0).double().mean()),
+            'frac_within_2ulp': float((ulps <= 2).double().mean()),
+            'note': 'the fused chain is NOT within 2 ulp end to end: the last stages subtract nearly equal numbers, so '
+                    'distances in ulp of the small difference are unbounded in any mode that is not bit-exact; the '
+                    'absolute error is a few ulp of the O(1) intermediates'}
+        del ulps
+    exact_bits = None
+    if 'chain8' in cpu:
+        exact_bits = same_bits(exact.results(), cpu['chain8']['results'])
+        parity['exact_mode_vs_cpu_oracle'] = {'elements_checked': int(a.size), 'bit_exact': exact_bits}
+
+    kernel_name = chain.kernels[0]['kernel']
     result = {
         'metric': 'achieved HBM bandwidth on the fused 8-op chain (algorithmic bytes / time)',
         'value': round(value, 1), 'unit': 'GB/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
@@ -522,80 +629,74 @@ def main():
         'config': {'workload': 'chain8: add, mul 1.0001, tanh, sigmoid, log1p, expm1, sub, abs fused into one kernel; '
                                'A, B float32 [8192, 8192] uniform[-1, 1], numpy default_rng(2)',
                    'math_mode': mode,
-                   'math_mode_promise': 'every operator output within 2 float32 ulp of the reference code on the '
-                                        'same operator inputs' if mode == 'ulp2' else 'bit-exact',
-                   'algorithmic_bytes': nbytes, 'kernel': chain.kernels[0]['kernel'],
+                   'math_mode_promise': 'the default mode of evaluate(): every operator output within 2 float32 ulp of '
+                                        'the reference code on the same operator inputs; not end to end'
+                                        if mode == 'ulp2' else 'bit-exact',
+                   'algorithmic_bytes': nbytes, 'kernel': kernel_name,
                    'pct_of_hbm_peak': round(100.0 * value / HBM_PEAK_GBPS, 2),
+                   # short scalars of the parity record (the whole record: `parity`)
+                   'parity_ulp2_stagewise_max_ulp': max(stagewise.values()),
+                   'parity_ulp2_single_operators_vs_cpu_oracle_max_ulp':
+                       None if against_oracle is None else max(against_oracle.values()),
+                   'parity_ulp2_elements_checked_per_stage': int(a.size),
+                   'parity_ulp2_end_to_end_max_abs_err': None if end_to_end is None else end_to_end['max_abs_err'],
+                   'parity_ulp2_end_to_end_frac_within_2ulp':
+                       None if end_to_end is None else round(end_to_end['frac_within_2ulp'], 4),
+                   'parity_exact_mode_bit_exact_vs_cpu_oracle': exact_bits,
+                   # the same workload in the bit-exact mode (math_mode='exact' / OPVECLIB_MATH=exact)
+                   'exact_mode_GBps': round(exact_gbps, 1),
+                   'exact_mode_frac_of_hbm_peak': round(exact_gbps / HBM_PEAK_GBPS, 4),
+                   'exact_mode_kernel_us': round(exact_ms * 1e3, 2),
                    'clock_settling_launches_before_warmup': settled_after,
-                   'clocks_under_load': clocks_under_load(chain)},
+                   'clocks_under_load': headline_clocks},
         'roofline': {'bound': 'hbm', 'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
-                     'frac': round(achieved / HBM_PEAK_GBPS, 4), 'traffic': CHAIN8_TRAFFIC_BYTES[mode],
+                     'frac': round(achieved / HBM_PEAK_GBPS, 4), 'traffic': CHAIN8_TRAFFIC_BYTES.get(kernel_name),
+                     'traffic_measured_on_kernel': kernel_name if kernel_name in CHAIN8_TRAFFIC_BYTES else None,
                      'kernel_us': round(event_ms * 1e3, 2), 'kernel_min_us': round(min_ms * 1e3, 2)},
         'cpu_baseline': cpu_baseline,
     }
-
-    # parity of the headline: stage-wise distances of the ulp2 mode, end-to-end statistics against the exact mode,
-    # and the exact mode against the CPU oracle bit for bit on the full tensors
-    exact.launch(torch.cuda.current_stream().cuda_stream)
-    torch.cuda.synchronize()
-    parity = {'ulp2_stagewise_max_ulp': stagewise}
-    if mode == 'ulp2':
-        exact_y, y = exact.results()[0], chain.results()[0]
-        ulps = ulp_distance(y, exact_y)
-        parity['ulp2_end_to_end_vs_exact'] = {
-            'max_abs_err': float((y.double() - exact_y.double()).abs().max()),
-            'frac_bit_equal': float((ulps == 0).double().mean()),
-            'frac_within_2ulp': float((ulps <= 2).double().mean()),
-            'note': 'the last stages subtract nearly equal numbers, so distances in ulp of the small difference are '
-                    'unbounded in any mode that is not bit-exact; the absolute error is a few ulp of the O(1) '
-                    'intermediates'}
-        del ulps
-    if 'chain8' in cpu:
-        parity['exact_mode_vs_cpu_oracle'] = {'elements_checked': int(a.size),
-                                              'bit_exact': same_bits(exact.results(), cpu['chain8']['results'])}
     result['parity'] = parity
 
     if with_others:
         others = []
         steps = max(5, min(args.steps, 20))
         warm = args.warmup
-        # the bit-exact mode of the headline workload
-        settle(exact)
-        sustain(exact)
-        _, exact_ms, exact_min = measure(exact, 2 * steps, warm)
-        gbps = nbytes / (exact_ms * 1e-3) / 1e9
-        others.append({'workload': "chain8 in the bit-exact 'exact' math mode", 'us': round(exact_ms * 1e3, 2),
-                       'min_us': round(exact_min * 1e3, 2), 'GB/s': round(gbps, 1),
-                       'frac': round(gbps / HBM_PEAK_GBPS, 4), 'algorithmic_bytes': nbytes,
-                       'kernels': [k['kernel'] for k in exact.kernels],
-                       'cpu_reference': None if 'chain8' not in cpu else {
-                           'ms': cpu['chain8']['ms'], 'cores': cpu['chain8']['cores'],
-                           'sample': cpu['chain8']['sample'],
-                           'bit_exact': parity['exact_mode_vs_cpu_oracle']['bit_exact']},
-                       'clocks_under_load': clocks_under_load(exact, seconds=2.5)})
-        # The 'fast' math mode (hardware-based routines everywhere): no promise per operator beyond 4 ulp, reported
-        # with its distance from the exact result.
-        fast = Prepared(chain8_outputs(*leaves), {'math': 'fast'})
-        settle(fast)
-        sustain(fast)
-        _, fast_ms, fast_min = measure(fast, 2 * steps, warm)
-        exact_y, fast_y = exact.results()[0], fast.results()[0]
-        ulps = ulp_distance(fast_y, exact_y)
-        fast_gbps = nbytes / (fast_ms * 1e-3) / 1e9
-        others.append({'workload': "chain8 in the optional 'fast' math mode (not a parity path)",
-                       'us': round(fast_ms * 1e3, 2), 'min_us': round(fast_min * 1e3, 2),
-                       'GB/s': round(fast_gbps, 1), 'frac': round(fast_gbps / HBM_PEAK_GBPS, 4),
-                       'algorithmic_bytes': nbytes, 'kernels': [k['kernel'] for k in fast.kernels],
-                       'stagewise_max_ulp': chain8_stagewise(leaves[0], leaves[1], leaves[2], 'fast'),
-                       'vs_exact': {'max_abs_err': float((fast_y.double() - exact_y.double()).abs().max()),
-                                    'frac_bit_equal': float((ulps == 0).double().mean()),
-                                    'frac_within_2ulp': float((ulps <= 2).double().mean())}})
-        del fast, exact_y, fast_y, ulps
+        if not quick:
+            # the bit-exact mode of the headline workload (timed above)
+            gbps = exact_gbps
+            others.append({'workload': "chain8 in the bit-exact 'exact' math mode", 'us': round(exact_ms * 1e3, 2),
+                           'min_us': round(exact_min * 1e3, 2), 'GB/s': round(gbps, 1),
+                           'frac': round(gbps / HBM_PEAK_GBPS, 4), 'algorithmic_bytes': nbytes,
+                           'kernels': [k['kernel'] for k in exact.kernels],
+                           'cpu_reference': None if 'chain8' not in cpu else {
+                               'ms': cpu['chain8']['ms'], 'cores': cpu['chain8']['cores'],
+                               'sample': cpu['chain8']['sample'],
+                               'bit_exact': parity['exact_mode_vs_cpu_oracle']['bit_exact']},
+                           'clocks_under_load': clocks_under_load(exact, seconds=2.5)})
+            # The 'fast' math mode (hardware-based routines everywhere): no promise per operator beyond 4 ulp, reported
+            # with its distance from the exact result.
+            fast = Prepared(chain8_outputs(*leaves), {'math': 'fast'})
+            settle(fast)
+            sustain(fast)
+            _, fast_ms, fast_min = measure(fast, 2 * steps, warm)
+            exact_y, fast_y = exact.results()[0], fast.results()[0]
+            ulps = ulp_distance(fast_y, exact_y)
+            fast_gbps = nbytes / (fast_ms * 1e-3) / 1e9
+            others.append({'workload': "chain8 in the optional 'fast' math mode (not a parity path)",
+                           'us': round(fast_ms * 1e3, 2), 'min_us': round(fast_min * 1e3, 2),
+                           'GB/s': round(fast_gbps, 1), 'frac': round(fast_gbps / HBM_PEAK_GBPS, 4),
+                           'algorithmic_bytes': nbytes, 'kernels': [k['kernel'] for k in fast.kernels],
+                           'stagewise_max_ulp': chain8_stagewise(leaves[0], leaves[1], leaves[2], 'fast'),
+                           'vs_exact': {'max_abs_err': float((fast_y.double() - exact_y.double()).abs().max()),
+                                        'frac_bit_equal': float((ulps == 0).double().mean()),
+                                        'frac_within_2ulp': float((ulps <= 2).double().mean())}})
+            del fast, exact_y, fast_y, ulps
         others.append(side_workload('copy f32[8192,8192] (counter calibration, plain copy bandwidth)',
                                     copy_outputs(leaves[0]), steps, warm))
         # the same readings under a kernel that only moves data: what the clocks and the board power are when the
         # arithmetic is absent
-        others[-1]['clocks_under_load'] = clocks_under_load(Prepared(copy_outputs(leaves[0])), seconds=2.5)
+        if others[-1]:
+            others[-1]['clocks_under_load'] = clocks_under_load(Prepared(copy_outputs(leaves[0])), seconds=2.5)
         others.append(side_workload('launch floor: copy of 1024 floats, one workgroup (what the clock around a launch '
                                     'reads for a kernel with nothing to do)',
                                     copy_outputs(np.zeros(1024, np.float32)), steps, warm))
@@ -623,6 +724,8 @@ def main():
             tree = HandWrittenScan(x, entry + '_reassociated')
             others.append(side_workload('c3 cumsum %s, reassociating wavefront scan (not the parity path)' % label,
                                         tree, steps, warm))
+            if not others[-1]:
+                continue
             sequential = HandWrittenScan(x, entry)
             sequential.launch(torch.cuda.current_stream().cuda_stream)
             torch.cuda.synchronize()
@@ -644,9 +747,11 @@ def main():
         others.append(side_workload('c4 lstm cell gradient [4096, 4x1024]', lstm_grad_outputs(concat, c, dc, dh),
                                     steps, warm, reference=cpu.get('lstm_grad'), sustained=True))
         # these two also run at the board's power limit: the readings say so
-        others[-2]['clocks_under_load'] = clocks_under_load(Prepared(lstm_outputs(concat, c)), seconds=2.5)
-        others[-1]['clocks_under_load'] = clocks_under_load(Prepared(lstm_grad_outputs(concat, c, dc, dh)),
-                                                            seconds=2.5)
+        if others[-2]:
+            others[-2]['clocks_under_load'] = clocks_under_load(Prepared(lstm_outputs(concat, c)), seconds=2.5)
+        if others[-1]:
+            others[-1]['clocks_under_load'] = clocks_under_load(Prepared(lstm_grad_outputs(concat, c, dc, dh)),
+                                                                seconds=2.5)
         others.append(side_workload('c4 lstm cell forward, hand-written kernel (run-time shape, same bits)',
                                     HandWrittenLstm(concat, c), steps, warm, reference=cpu.get('lstm'),
                                     sustained=True))
@@ -657,6 +762,20 @@ def main():
                                     steps, warm, {'math': 'fast'}))
         others.append(side_workload("c4 lstm cell gradient in the optional 'fast' math mode",
                                     lstm_grad_outputs(concat, c, dc, dh), steps, warm, {'math': 'fast'}))
+        # the cell composed of library operators (opveclib/test/test_operator_merge.py:311-321) at the same size,
+        # fused by the optimizer: every sigmoid and tanh is an operator of its own, so the 'ulp2' promise applies to
+        # each given its own input
+        concat_d, c_d = torch.from_numpy(concat).cuda(), torch.from_numpy(c).cuda()
+        others.append(side_workload("c4 lstm cell composed of library operators, fused, 'exact' math mode",
+                                    workloads.stdops_lstm_outputs(concat_d, c_d), steps, warm,
+                                    reference=cpu.get('stdops_lstm'), sustained=True))
+        others.append(side_workload("c4 lstm cell composed of library operators, fused, 'ulp2' math mode (the default)",
+                                    workloads.stdops_lstm_outputs(concat_d, c_d), steps, warm, {'math': 'ulp2'},
+                                    sustained=True))
+        if others[-1]:
+            others[-1]['ulp2_stagewise_max_ulp'] = stdops_lstm_stagewise(concat_d, c_d, 'ulp2')
+        del concat_d, c_d
+        cpu.pop('stdops_lstm', None)
         torch.cuda.empty_cache()
         others.append(side_workload('c5 gather + transposed scatter f32[16384,16384], numpy default_rng(5)',
                                     gather_outputs(data['a5'], data['b5']), max(3, steps // 4), 2,
@@ -667,6 +786,9 @@ def main():
         others.append(side_workload('reference timing: cumsum f64[10000,1000] along axis 0 '
                                     '(examples/test_perf_accumulate.py:35-47)', cumsum_outputs(data['x0'], axis=0),
                                     10, warm, reference=cpu.get('cumsum_axis0')))
+        others.append(side_workload('reference timing: conv1D f64 [5,1000,3] x [10,13,3], mode same, NEC '
+                                    '(examples/conv1D.py:323-340)', workloads.conv1d_outputs(*data['conv1d']), steps,
+                                    warm, reference=cpu.get('conv1d')))
         # reductions in the worker's own order (the operator of the reference's dot-product test at C3's size, and
         # the sum over the axis of the reference's accumulate timing)
         others.append(side_workload('dot product per row f32[4096,16384] x f32[4096,16384] '
@@ -689,7 +811,14 @@ def main():
                                         reference=cpu.get('lstm%d' % units)))
             others.append(side_workload(label % 'gradient, generated', lstm_grad_outputs(concat, c, dc, dh), steps,
                                         warm, reference=cpu.get('lstm_grad%d' % units)))
-        result['others'] = others
+        if args.only is not None and 'row stride' in args.only:
+            # float32 scans whose rows are 64 KiB, 64 KiB + 256 B and 65 KiB long (for counter collection)
+            g = np.random.default_rng(7)
+            for cols in (16384, 16448, 16640):
+                others.append(side_workload('row stride probe: cumsum f32[4096,%d] last axis' % cols,
+                                            cumsum_outputs(g.standard_normal((4096, cols), dtype=np.float32)),
+                                            steps, warm))
+        result['others'] = [line for line in others if line]
 
     print(json.dumps(result))
     sys.stdout.flush()

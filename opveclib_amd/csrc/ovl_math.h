@@ -65,6 +65,8 @@
 // selects: no execution-mask juggling on the common path, and identical calls in one kernel can be merged by the
 // compiler because the common path is not nested in a condition.
 #define OVL_ANY(cond) (__builtin_amdgcn_ballot_w64(cond) != 0)
+// True when the condition holds in every active lane of the wavefront (also wave-uniform).
+#define OVL_ALL(cond) (__builtin_amdgcn_ballot_w64(!(cond)) == 0)
 // OVL_RARE() as first statement of such a block keeps the compiler from turning the block into unconditional code
 // with selects, which it does when it judges the block cheap.  That is welcome for the few selects of the routines in
 // this file (measured: faster without the marker) and unwelcome for blocks that call a library routine
@@ -74,6 +76,7 @@
 #define OVL_HD static inline
 #define OVL_TABLE static const
 #define OVL_ANY(cond) (cond)
+#define OVL_ALL(cond) (cond)
 #define OVL_RARE() ((void)0)
 #endif
 

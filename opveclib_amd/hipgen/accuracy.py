@@ -58,13 +58,27 @@ STAGE_VARIABLE = 1
 #: division: from the correctly rounded quotient), and of the once-rounded log1p / expm1 of csrc/ovl_math.h from the
 #: reference's formulas evaluated with the host C library over every argument of `IDIOM_DOMAIN`; asserted by
 #: tests/test_gpu_math_exhaustive.py
-ROUTINE_ULPS = {lang.TANH: 2, lang.EXP: 1, lang.LOG: 2, lang.DIVIDE: 1, 'sigmoid': 2, 'log1p': 2, 'expm1': 2}
+ROUTINE_ULPS = {lang.TANH: 2, lang.EXP: 1, lang.LOG: 2, lang.DIVIDE: 1, 'sigmoid': 2, 'log1p': 2, 'expm1': 2,
+                'sigmoid_guarded': 2, 'log1p_guarded': 2, 'expm1_guarded': 2}
 
 #: what a site saves when it may use the cheap routine (issue clocks per element, measured); orders the repairs
-_GAIN = {lang.TANH: 225, lang.EXP: 60, lang.LOG: 50, lang.DIVIDE: 19, 'sigmoid': 60, 'log1p': 25, 'expm1': 100}
+_GAIN = {lang.TANH: 225, lang.EXP: 60, lang.LOG: 50, lang.DIVIDE: 19, 'sigmoid': 60, 'log1p': 25, 'expm1': 100,
+         'sigmoid_guarded': 50, 'log1p_guarded': 15, 'expm1_guarded': 90}
 
 #: argument ranges on which the once-rounded routines were compared with the reference's formulas
 IDIOM_DOMAIN = {'sigmoid': (-16.0, 64.0), 'log1p': (2.0 ** -10, 2.0 ** 64), 'expm1': (2.0 ** -12, 64.0)}
+
+#: A formula whose argument's range is not known to lie in `IDIOM_DOMAIN` (it comes straight from a tensor: every
+#: sigmoid of an LSTM cell, opveclib/stdops/math.py:91-93) is replaced behind a test at run time: when every lane of
+#: the wavefront holds an argument inside these intervals the once-rounded routine runs, otherwise the wavefront
+#: evaluates the formula itself with the bit-compatible routines.  Either way the value is within `TOLERANCE` of the
+#: reference's.  The intervals are those on which the routines were compared with the formulas on every float32
+#: argument: `IDIOM_DOMAIN`, and for log1p also the negative arguments down to the last float32 above -1.
+GUARD_DOMAIN = {'sigmoid': ((-16.0, 64.0),),
+                'log1p': ((-(1.0 - 2.0 ** -24), -(2.0 ** -10)), (2.0 ** -10, 2.0 ** 64)),
+                'expm1': ((2.0 ** -12, 64.0),)}
+#: kind of a guarded call site -> the formula it stands for
+GUARDED = {'sigmoid_guarded': 'sigmoid', 'log1p_guarded': 'log1p', 'expm1_guarded': 'expm1'}
 
 #: narrower argument ranges on which shorter forms of the once-rounded routines hold the same bound (also compared
 #: with the formulas on every argument): for 2^-4 <= x < 1 the sum 1 + x has a known exponent (`ovl_log1p_unit`), up
@@ -105,23 +119,34 @@ def _is_one(info, idx):
     return node.code == lang.CONST_SCALAR and len(node.data) == 1 and float(node.data[0]) == 1.0
 
 
-def match_idiom(info, known, node):
-    """
-    Recognise, at the division that ends them, the reference's formulas for the logistic function
-    (opveclib/stdops/math.py:93) and its numerically careful ones for log(1 + x) and exp(x) - 1
-    (opveclib/examples/test_log1p.py:55-60, test_expm1.py:57-61):
+def _same_value(info, a, b, depth=12):
+    """Two expressions certainly hold the same value: the same node, or pure expressions of the same operation on
+    operands that hold the same values (a worker that writes ``x[pos]`` twice reads the tensor twice; inputs are
+    never written, and positions do not change)."""
+    if a == b:
+        return True
+    if depth == 0:
+        return False
+    na, nb = info.nodes[a], info.nodes[b]
+    if na.code != nb.code or na.dtype != nb.dtype or len(na.ops) != len(nb.ops):
+        return False
+    if na.code == lang.CONST_SCALAR:
+        return list(na.data) == list(nb.data)
+    if na.code in (lang.INPUT, lang.POSITION):
+        return False                    # (the same tensor is the same node)
+    if na.code == lang.READ_TENSOR:
+        if info.nodes[na.ops[0]].code not in (lang.INPUT, lang.POSITION) or info.in_loop.get(a) or info.in_loop.get(b):
+            return False
+    elif na.code not in (lang.CAST, lang.ADD, lang.SUBTRACT, lang.MULTIPLY, lang.NEGATE):
+        return False
+    return all(_same_value(info, x, y, depth - 1) for x, y in zip(na.ops, nb.ops))
 
-        sigmoid:  1 / (1 + exp(-x))
-        log1p:    log(u) * x / (u - 1)   with u = 1 + x
-        expm1:    (e - 1) * x / log(e)   with e = exp(x)
 
-    Returns (kind, index of x, value range of x there) when ``node`` is such a division in float32 and the range lies
-    inside the domain on which the once-rounded routine was compared with the formula, else None.  (The formulas exist to avoid
-    the rounding of ``1 + x`` and the cancellation in ``e - 1``; a routine that forms the result in double precision
-    and rounds it once has neither problem.)
-    """
+def _match_formula(info, node):
+    """The structure of `match_idiom` without the condition on the argument's range: (kind, index of x, index of the
+    expression that takes x, which of its operands x is) or None."""
     nodes = info.nodes
-    if node.code != lang.DIVIDE or node.dtype != lang.FLOAT32 or known is None:
+    if node.code != lang.DIVIDE or node.dtype != lang.FLOAT32:
         return None
     product, divisor = nodes[node.ops[0]], nodes[node.ops[1]]
 
@@ -144,11 +169,7 @@ def match_idiom(info, known, node):
             return None
         if info.in_loop.get(node.idx):
             return None
-        lo, hi = IDIOM_DOMAIN[kind]
-        seen = known.operand(user, operand)
-        if seen is None or not seen.within(lo, hi):
-            return None
-        return kind, x, seen
+        return kind, x, user, operand
 
     if _is_one(info, node.ops[0]):
         inner = one_plus(divisor.idx)
@@ -164,11 +185,12 @@ def match_idiom(info, known, node):
     for first, x in ((product.ops[0], product.ops[1]), (product.ops[1], product.ops[0])):
         factor = nodes[first]
         if factor.code == lang.LOG and divisor.code == lang.SUBTRACT and divisor.ops[0] == factor.ops[0] and \
-                _is_one(info, divisor.ops[1]) and one_plus(factor.ops[0]) == x:
+                _is_one(info, divisor.ops[1]) and one_plus(factor.ops[0]) is not None and \
+                _same_value(info, one_plus(factor.ops[0]), x):
             found = ('log1p', x, (factor.ops[0],))
         elif factor.code == lang.SUBTRACT and _is_one(info, factor.ops[1]) and divisor.code == lang.LOG and \
                 divisor.ops[0] == factor.ops[0] and nodes[factor.ops[0]].code == lang.EXP and \
-                nodes[factor.ops[0]].ops[0] == x:
+                _same_value(info, nodes[factor.ops[0]].ops[0], x):
             found = ('expm1', x, (factor.ops[0],))
         if found:
             break
@@ -176,6 +198,44 @@ def match_idiom(info, known, node):
         return None
     kind, x, parts = found
     return finish(kind, x, product.idx, 0 if product.ops[0] == x else 1, parts + (product.idx, divisor.idx))
+
+
+def match_idiom(info, known, node):
+    """
+    Recognise, at the division that ends them, the reference's formulas for the logistic function
+    (opveclib/stdops/math.py:93) and its numerically careful ones for log(1 + x) and exp(x) - 1
+    (opveclib/examples/test_log1p.py:55-60, test_expm1.py:57-61):
+
+        sigmoid:  1 / (1 + exp(-x))
+        log1p:    log(u) * x / (u - 1)   with u = 1 + x
+        expm1:    (e - 1) * x / log(e)   with e = exp(x)
+
+    Returns (kind, index of x, value range of x there) when ``node`` is such a division in float32 and the range lies
+    inside the domain on which the once-rounded routine was compared with the formula, else None.  (The formulas exist to avoid
+    the rounding of ``1 + x`` and the cancellation in ``e - 1``; a routine that forms the result in double precision
+    and rounds it once has neither problem.)
+    """
+    if known is None:
+        return None
+    found = _match_formula(info, node)
+    if found is None:
+        return None
+    kind, x, user, operand = found
+    lo, hi = IDIOM_DOMAIN[kind]
+    seen = known.operand(user, operand)
+    if seen is None or not seen.within(lo, hi):
+        return None
+    return kind, x, seen
+
+
+def match_guarded(info, known, node):
+    """(kind, index of x) when ``node`` is the division that ends one of the formulas of `match_idiom` and the range
+    of x is not known to lie in the compared domain: the replacement then happens behind a test of the arguments at
+    run time (`GUARD_DOMAIN`).  None for a formula `match_idiom` already takes, and for anything else."""
+    found = _match_formula(info, node)
+    if found is None or match_idiom(info, known, node) is not None:
+        return None
+    return found[0], found[1]
 
 
 def site_kind(info, known, node):
@@ -188,6 +248,9 @@ def site_kind(info, known, node):
         idiom = match_idiom(info, known, node)
         if idiom is not None:
             return idiom[0]
+        guarded = match_guarded(info, known, node)
+        if guarded is not None:
+            return guarded[0] + '_guarded'
         if _is_one(info, node.ops[0]):
             return None
     return node.code
@@ -344,6 +407,14 @@ class _Interpreter(object):
                     lang.MAX_VALUE, lang.EPSILON, lang.RANGE, lang.ENDRANGE, lang.IF, lang.ELSEIF, lang.ELSE,
                     lang.ENDIF):
             return
+        if self.kinds.get(node.idx) in GUARDED and node.idx in self.cheap:
+            # the once-rounded routine where the arguments allow it, else the formula with the bit-compatible
+            # routines: within the routine's distance of the reference either way, given an exact x
+            kind, x = match_guarded(self.info, self.known, node)
+            bound = self._get(x, env)
+            sites = bound.sites | frozenset([node.idx])
+            self.value[node.idx] = _Bound(INF if bound.ulps else ROUTINE_ULPS[kind], sites)
+            return
         if self.kinds.get(node.idx) in IDIOM_DOMAIN and node.idx in self.cheap:
             # the once-rounded routine takes x itself: nothing of the formula's parts enters
             kind, x, seen = match_idiom(self.info, self.known, node)
@@ -450,10 +521,11 @@ def candidate_sites(info, known):
 
 
 def formula_sites(info, known):
-    """{node index: kind} of the divisions that end a recognised sigmoid / log1p / expm1 formula whose argument lies
-    in the compared domain.  The 'fast' math mode replaces these too: the one routine is both closer to the reference
-    and shorter than the formula composed of cheap routines."""
-    return dict((idx, kind) for idx, kind in candidate_sites(info, known).items() if kind in IDIOM_DOMAIN)
+    """{node index: kind} of the divisions that end a recognised sigmoid / log1p / expm1 formula (kind + '_guarded'
+    when the argument is not known to lie in the compared domain).  The 'fast' math mode replaces these too: the one
+    routine is both closer to the reference and shorter than the formula composed of cheap routines."""
+    return dict((idx, kind) for idx, kind in candidate_sites(info, known).items()
+                if kind in IDIOM_DOMAIN or kind in GUARDED)
 
 
 def cheap_sites(info, known):

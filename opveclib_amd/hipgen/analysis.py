@@ -332,7 +332,11 @@ class DagInfo(object):
             from . import accuracy
             cheap = accuracy.cheap_sites(self, self.known_ranges())
             calls = [] if mode == 'fast' else [n for n in calls if n.idx not in cheap]
-            calls += [k for k in cheap.values() if k in ('log1p', 'expm1')]
+            calls += [k for k in cheap.values() if k in ('log1p', 'expm1', 'log1p_guarded', 'expm1_guarded')]
+            # a formula replaced behind a run-time test of its argument keeps the formula itself as the other branch,
+            # evaluated with the bit-compatible exp and log in the 'ulp2' mode
+            if mode == 'ulp2':
+                calls += [k for k in cheap.values() if k == 'sigmoid_guarded']
         return bool(calls)
 
     def known_ranges(self):

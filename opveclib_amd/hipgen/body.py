@@ -396,6 +396,30 @@ class BodyEmitter(object):
                     elif code == lang.LOG and value_ranges.log_in_range(x):
                         fcn = IN_RANGE[mode]['log nan' if x.nan else code]
                 put(CTYPE[node.dtype] + ' ' + name + ' = ' + fcn + '(' + names[ops[0]] + ');')
+            elif code == lang.DIVIDE and cheap_sites.get(node.idx) in accuracy.GUARDED:
+                # the same formula with an argument of unknown range: the routine when every lane of the wavefront
+                # holds an argument of the compared domain, else the formula itself (with the routines the other
+                # call sites of this mode use: the bit-compatible ones in 'ulp2')
+                kind, x = accuracy.match_guarded(info, known, node)
+                arg = names[x]
+                fallback = 'fast' if math_mode == 'fast' else 'exact'
+                exp_fn = MATH_MODES[fallback].get(lang.EXP, UNARY[lang.EXP][lang.FLOAT32])
+                log_fn = MATH_MODES[fallback].get(lang.LOG, UNARY[lang.LOG][lang.FLOAT32])
+                quotient = (lambda a, b: MATH_MODES[fallback][lang.DIVIDE] + '(' + a + ', ' + b + ')') \
+                    if lang.DIVIDE in MATH_MODES[fallback] else (lambda a, b: '(' + a + ' / ' + b + ')')
+                routine = {'sigmoid': 'ovl_sigmoid_ulp2', 'log1p': 'ovl_log1p_direct', 'expm1': 'ovl_expm1_direct'}[kind]
+                if kind == 'sigmoid':
+                    formula = 'ovl_recipf(1.0f + ' + exp_fn + '(-' + arg + '))'
+                elif kind == 'log1p':
+                    formula = quotient('(' + log_fn + '(1.0f + ' + arg + ') * ' + arg + ')', '((1.0f + ' + arg + ') - 1.0f)')
+                else:
+                    formula = quotient('((' + exp_fn + '(' + arg + ') - 1.0f) * ' + arg + ')',
+                                       log_fn + '(' + exp_fn + '(' + arg + '))')
+                inside = ' || '.join('(%s >= %s && %s <= %s)' % (arg, literal(lo) + 'f', arg, literal(hi) + 'f')
+                                     for lo, hi in accuracy.GUARD_DOMAIN[kind])
+                put('float ' + name + ';')
+                put('if (OVL_ALL(' + inside + ')) { ' + name + ' = ' + routine + '(' + arg + '); } else { ' +
+                    name + ' = ' + formula + '; }')
             elif code == lang.DIVIDE and cheap_sites.get(node.idx) in accuracy.IDIOM_DOMAIN:
                 # the division that ends the reference's sigmoid / log1p / expm1 formula: one routine on x instead
                 kind, x, seen = accuracy.match_idiom(info, known, node)

@@ -73,6 +73,56 @@ def lstm_outputs(concat, c):
     return [op[0], op[1]]
 
 
+def stdops_lstm_outputs(concat, c):
+    """The LSTM cell composed of library operators as the reference's merge test writes it
+    (opveclib/test/test_operator_merge.py:311-321; no forget bias there): new_c and new_h.  The optimizer fuses the
+    ten operators into one kernel."""
+    from . import stdops
+    parts = stdops.split(concat, split_dim=1, num_split=4)
+    i, j, f, o = (parts[k] for k in range(4))
+    new_c = stdops.mul(c, stdops.sigmoid(f)) + stdops.sigmoid(i) * stdops.tanh(j)
+    new_h = stdops.tanh(new_c) * stdops.sigmoid(o)
+    return [new_c[0], new_h[0]]
+
+
+#: names of the stages `stdops_lstm_stage_outputs` returns, in its order
+STDOPS_LSTM_STAGES = ('i', 'j', 'f', 'o', 'sigmoid_f', 'sigmoid_i', 'tanh_j', 'c_sigmoid_f', 'sigmoid_i_tanh_j', 'new_c',
+                      'tanh_new_c', 'sigmoid_o', 'new_h')
+
+
+def stdops_lstm_stage_outputs(concat, c):
+    """Every operator output of the composed cell as a requested output, in the order of `STDOPS_LSTM_STAGES` (the
+    optimizer still fuses the operators into one kernel, which then also stores the intermediates)."""
+    from . import stdops
+    parts = stdops.split(concat, split_dim=1, num_split=4)
+    i, j, f, o = (parts[k] for k in range(4))
+    sigmoid_f, sigmoid_i, tanh_j = stdops.sigmoid(f), stdops.sigmoid(i), stdops.tanh(j)
+    left, right = stdops.mul(c, sigmoid_f), sigmoid_i * tanh_j
+    new_c = left + right
+    tanh_new_c, sigmoid_o = stdops.tanh(new_c), stdops.sigmoid(o)
+    new_h = tanh_new_c * sigmoid_o
+    return [i, j, f, o, sigmoid_f[0], sigmoid_i[0], tanh_j[0], left[0], right[0], new_c[0], tanh_new_c[0], sigmoid_o[0],
+            new_h[0]]
+
+
+def conv1d_reference_inputs():
+    """The tensors of the reference's conv1D timing run (opveclib/examples/conv1D.py:279-319): TensorFlow sizes
+    [5, 1, 1000, 3] and [1, 13, 3, 10] filled with 1, 2, 3, ... as float64, in the 'NEC' layout of the OVL operator:
+    input [5 batches, 1000 elements, 3 channels], filters [10 filters, 13 taps, 3 channels]."""
+    batches, elements, channels, taps, filters = 5, 1000, 3, 13, 10
+    x = np.arange(1, batches * elements * channels + 1, dtype=np.float64).reshape(batches, elements, channels)
+    flat = np.arange(1, taps * channels * filters + 1, dtype=np.float64)
+    # TensorFlow's filter layout is [tap, channel, filter]; OVL's 'NEC' layout is [filter, tap, channel]
+    v = np.ascontiguousarray(flat.reshape(taps, channels, filters).transpose(2, 0, 1))
+    return x, v
+
+
+def conv1d_outputs(x, v):
+    """The convolution of that run: mode 'same', filters as they are, 'NEC' layout (conv1D.py:327)."""
+    from .examples import conv_1d
+    return [conv_1d(x, v, mode='same', kernel_orientation='as-is', data_format='NEC')[0]]
+
+
 def lstm_grad_outputs(concat, c, dc, dh):
     from .lstm import lstm_grad
     op = lstm_grad(concat, c, dc, dh, forget_bias=1.0)
@@ -144,6 +194,8 @@ def all_workload_outputs():
     yield lstm_outputs(Spec((4096, 4096)), Spec((4096, 1024)))
     yield lstm_grad_outputs(Spec((4096, 4096)), Spec((4096, 1024)), Spec((4096, 1024)), Spec((4096, 1024)))
     yield gather_outputs(Spec((16384, 16384)), Spec((16384 * 16384,)))
+    yield stdops_lstm_outputs(Spec((4096, 4096)), Spec((4096, 1024)))
+    yield conv1d_outputs(Spec((5, 1000, 3), f64), Spec((10, 13, 3), f64))
     yield cumsum_outputs(Spec(REFERENCE_CUMSUM_SHAPE, f64), axis=0)
     yield dot_outputs(Spec((4096, 16384), f32), Spec((4096, 16384), f32))
     yield column_sum_outputs(Spec(REFERENCE_CUMSUM_SHAPE, f64))
@@ -191,6 +243,15 @@ def prebuild(force=False, workers=8):
     # the single operators of the chain at full size, bit-exact: what the benchmark compares each stage with
     headline = chain8_stage_outputs(Spec((8192, 8192)), Spec((8192, 8192)), Spec((1,)))
     for op in unfused_operators(headline):
+        jobs[(op.SerializeToString(), 'exact')] = (op, None)
+        # ... and each operator on its own in the default mode, compared with the CPU oracle's stages
+        jobs[(op.SerializeToString(), 'ulp2')] = (op, {'math': 'ulp2'})
+    # the composed LSTM cell: the fused kernel that stores every operator's output, and the single bit-exact
+    # operators its stages are compared with
+    cell = stdops_lstm_stage_outputs(Spec((4096, 4096)), Spec((4096, 1024)))
+    for op in fused_operators(cell):
+        jobs[(op.SerializeToString(), 'ulp2')] = (op, {'math': 'ulp2'})
+    for op in unfused_operators(cell):
         jobs[(op.SerializeToString(), 'exact')] = (op, None)
     previous = compiler.prebuild_mode, compiler.force_rebuild
     compiler.prebuild_mode, compiler.force_rebuild = True, bool(force)

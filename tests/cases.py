@@ -1252,15 +1252,15 @@ def chain8_single_stage(name, x, with_range=False):
 
 
 #: (formula, lower and upper end of the clip in front of it, the routine the 'ulp2' mode must choose): the general
-#: once-rounded routines on wide ranges, their shorter forms on narrow ones, the formula itself where the range leaves
-#: the compared domain
+#: once-rounded routines on wide ranges, their shorter forms on narrow ones, the test at run time (with the formula as
+#: its other branch) where the range leaves the compared domain
 ULP2_CLIPPED_FORMULAS = [
     ('log1p', 2.0 ** -9, 1.0e6, 'ovl_log1p_direct'),
     ('log1p', 0.0625, 0.999, 'ovl_log1p_unit'),
-    ('log1p', 1.0e-5, 0.5, 'ovl_logf_inrange'),
+    ('log1p', 1.0e-5, 0.5, 'OVL_ALL'),
     ('expm1', 0.001, 50.0, 'ovl_expm1_direct'),
     ('expm1', 0.001, 0.68, 'ovl_expm1_small'),
-    ('expm1', -1.0, 0.5, 'ovl_expf_inrange'),
+    ('expm1', -1.0, 0.5, 'OVL_ALL'),
     ('sigmoid', -15.0, 60.0, 'ovl_sigmoid_ulp2'),
     ('sigmoid', -1.0, 60.0, 'ovl_sigmoid_small'),
 ]
@@ -1286,6 +1286,46 @@ def ulp2_clipped_arguments(lo, hi):
     return x.astype(np.float32)
 
 
+#: rows of the band on which the full-size 'ulp2' tests run the oracle itself
+ORACLE_BAND_ROWS = 1024
+
+
+def _special_float32_values():
+    return np.array([np.nan, np.inf, -np.inf, 0.0, -0.0, 1e30, -1e30, 100.0, -100.0, 88.7, -88.7, 64.0, -16.0, 17.0,
+                     -17.0, 1e-30, -1e-30, 1e-45, 2.0 ** -10, -(2.0 ** -10), 2.0 ** -12, -1.0, -0.99999994, -2.0,
+                     2.0 ** -24, 2.0 ** -25, 709.0, -709.0], np.float32)
+
+
+def stdops_lstm_full_size_inputs():
+    """concat [4096, 4 x 1024] and c [4096, 1024], N(0, 1) from default_rng(4) (the benchmark's C4 tensors), with
+    special values planted in the first rows of every gate and of c."""
+    rng = np.random.default_rng(4)
+    concat = rng.standard_normal((4096, 4096), dtype=np.float32)
+    c = rng.standard_normal((4096, 1024), dtype=np.float32)
+    special = _special_float32_values()
+    for gate in range(4):
+        for row in range(4):
+            concat[row, gate * 1024 + 7 * row:gate * 1024 + 7 * row + special.size] = np.roll(special, gate + row)
+    c[1, 5:5 + special.size] = special
+    return concat, c
+
+
+def guarded_formula_arguments():
+    """float32 [1 << 20]: N(0, 1), a logarithmic sweep of both signs over 2^-30 .. 2^7, positive values, and the
+    special values (each planted into an otherwise ordinary stretch, so that single wavefronts leave the compared
+    domain)."""
+    rng = np.random.default_rng(11)
+    n = 1 << 20
+    x = rng.standard_normal(n, dtype=np.float32)
+    sweep = np.exp2(rng.uniform(-30.0, 7.0, n // 4)).astype(np.float32) * rng.choice([-1.0, 1.0], n // 4).astype(np.float32)
+    x[n // 2:n // 2 + n // 4] = sweep
+    # (a stretch of positive arguments inside every domain: whole wavefronts that take the routines)
+    x[3 * n // 4:] = np.abs(x[3 * n // 4:]) + np.float32(2.0 ** -9)
+    special = _special_float32_values()
+    x[1000:1000 + special.size * 4096:4096][:special.size] = special
+    return x
+
+
 def ulp2_full_size_operators():
     """[(operator, options)] of tests/test_gpu_ulp2.py that the benchmark's own prebuild step does not cover."""
     from opveclib_amd import workloads
@@ -1298,6 +1338,20 @@ def ulp2_full_size_operators():
         for op in _operators_of([ulp2_clipped_formula(kind, lo, hi, workloads.Spec((ULP2_CLIPPED_COUNT,)))], 3):
             jobs.append((op, {'math': 'ulp2'}))
             jobs.append((op, None))
+    # the composed LSTM cell at full size: the fused kernel that stores every stage, the single operators it is
+    # compared with, the fused cell in the exact mode
+    concat, c = workloads.Spec((4096, 4096)), workloads.Spec((4096, 1024))
+    for op in _operators_of(workloads.stdops_lstm_stage_outputs(concat, c), 3):
+        jobs.append((op, {'math': 'ulp2'}))
+    for op in _operators_of(workloads.stdops_lstm_outputs(concat, c), 3):
+        jobs.append((op, None))
+    for out in (stdops.sigmoid(c)[0], stdops.tanh(c)[0], stdops.mul(c, c)[0], stdops.add(c, c)[0]):
+        for op in _operators_of([out], 0):
+            jobs.append((op, None))
+    x = workloads.Spec((1 << 20,))
+    for out in (stdops.sigmoid(x)[0], log1p(x)[0], expm1(x)[0]):
+        for op in _operators_of([out], 0):
+            jobs.append((op, {'math': 'ulp2'}))
     return jobs
 
 
@@ -1456,8 +1510,11 @@ def prebuild_all(cases=None, workers=8, with_oracle=True):
                 oracle_ops[op.SerializeToString()] = op
         # tests/test_gpu_ulp2.py: the oracle on slices of 64 rows of the full-size chain and on the small chain's stages
         rows = np.zeros((64, CHAIN8_SHAPE[1]), np.float32)
+        band = np.zeros((ORACLE_BAND_ROWS, CHAIN8_SHAPE[1]), np.float32)
         small = np.zeros((96, 256), np.float32)
-        for x in (rows, small):
+        lstm_band = np.zeros((ORACLE_BAND_ROWS, 1024), np.float32)
+        guarded = np.zeros(1 << 20, np.float32)
+        for x in (rows, small, band, lstm_band, guarded):
             for name in ('tanh', 'sigmoid', 'log1p', 'expm1'):
                 for op in _operators_of([chain8_single_stage(name, x)], 0):
                     oracle_ops[op.SerializeToString()] = op

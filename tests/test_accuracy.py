@@ -14,7 +14,7 @@ import pytest
 
 import opveclib_amd as ovl
 from opveclib_amd import language as lang
-from opveclib_amd import stdops, workloads
+from opveclib_amd import hipgen, stdops, workloads
 from opveclib_amd.examples import log1p, expm1
 from opveclib_amd.hipgen import accuracy, ranges
 from opveclib_amd.hipgen.analysis import DagInfo
@@ -44,25 +44,55 @@ def test_fused_chain_uses_cheap_routines_where_two_ulp_are_proved():
     assert [kind for kind, is_cheap in chosen if kind in accuracy.IDIOM_DOMAIN and not is_cheap] == []
 
 
-def test_unfused_formulas_keep_the_bit_compatible_log_and_exp():
-    """Without a known argument range the formulas are not replaced; their log and exp feed a product and a quotient,
-    which can double an error twice, so they stay exact, while the final division (1 ulp) may be the cheap one."""
+def test_formulas_on_arguments_of_unknown_range_are_replaced_behind_a_run_time_test():
+    """Without a known argument range the formula cannot be replaced outright; it is replaced behind a test of the
+    arguments at run time, whose other branch is the formula itself with the bit-compatible routines.  The formula's
+    own exp / log no longer reach the stored value (a cheap one among them is dead code); an exp that also decides a
+    branch of the operator (expm1's ``e == 1``) stays the bit-compatible one."""
     x = Spec((1024,))
     chosen = dict(selection(workloads.unfused_operators([log1p(x)[0]])[0]))
-    assert chosen[lang.LOG] is False and chosen[lang.DIVIDE] is True
+    assert chosen['log1p_guarded'] is True
     chosen = dict(selection(workloads.unfused_operators([expm1(x)[0]])[0]))
-    assert chosen[lang.EXP] is False and chosen[lang.LOG] is False and chosen[lang.DIVIDE] is True
+    assert chosen['expm1_guarded'] is True and chosen[lang.EXP] is False
+    chosen = dict(selection(workloads.unfused_operators([stdops.sigmoid(x)[0]])[0]))
+    assert chosen['sigmoid_guarded'] is True
+    for op, kind in ((log1p, 'log1p'), (expm1, 'expm1'), (stdops.sigmoid, 'sigmoid')):
+        operator_dag, = workloads.unfused_operators([op(x)[0]])
+        text = hipgen.generate(operator_dag, 'f' + '7' * 56, {'math': 'ulp2'}).source
+        guards = [line for line in text.split('\n') if 'OVL_ALL(' in line]
+        assert guards and all('else' in line for line in guards), kind
+        routine = {'log1p': 'ovl_log1p_direct(', 'expm1': 'ovl_expm1_direct(', 'sigmoid': 'ovl_sigmoid_ulp2('}[kind]
+        exact = {'log1p': 'ovl_logf(', 'expm1': 'ovl_expf(', 'sigmoid': 'ovl_expf('}[kind]
+        assert all(routine in line and exact in line for line in guards), kind
+        assert 'OVL_DECLARE_MATH_TABLES' in text        # the other branch needs the tables of the exact exp / log
+        for lo, hi in accuracy.GUARD_DOMAIN[kind]:
+            assert all(repr(float(lo)) + 'f' in line and repr(float(hi)) + 'f' in line for line in guards)
+        # the bit-exact mode has no such test
+        assert 'OVL_ALL(' not in hipgen.generate(operator_dag, 'f' + '7' * 56, None).source
 
 
 def test_single_calls_are_cheap_and_cancelling_sums_are_not():
     x = Spec((1024,))
     assert selection(workloads.unfused_operators([stdops.tanh(x)[0]])[0]) == [(lang.TANH, True)]
-    # 1 / (1 + e): an inexact e loses a step in the sum and up to twice that in the reciprocal; without a known
-    # argument range the formula is not replaced either
-    assert selection(workloads.unfused_operators([stdops.sigmoid(x)[0]])[0]) == [(lang.EXP, False)]
     # the LSTM cell adds products of either sign: a distance in the operands is unbounded in ulp of the sum
     outs = workloads.lstm_outputs(Spec((8, 64)), Spec((8, 16)))
     assert all(not is_cheap for _, is_cheap in selection(workloads.fused_operators(outs)[0]))
+    outs = workloads.lstm_grad_outputs(Spec((8, 64)), Spec((8, 16)), Spec((8, 16)), Spec((8, 16)))
+    assert all(not is_cheap for _, is_cheap in selection(workloads.fused_operators(outs)[0]))
+
+
+def test_the_lstm_cell_composed_of_library_operators_gets_cheap_routines_per_operator():
+    """The cell of opveclib/test/test_operator_merge.py:311-321: every sigmoid and tanh is an operator of its own, so
+    the promise applies to each of them given its own input (which the fused kernel holds exactly), and the sums of
+    products that follow are exact operations on those results."""
+    outs = workloads.stdops_lstm_outputs(Spec((8, 64)), Spec((8, 16)))
+    op, = workloads.fused_operators(outs)
+    chosen = selection(op)
+    assert [kind for kind, cheap in chosen if cheap and kind == 'sigmoid_guarded'] == ['sigmoid_guarded'] * 3
+    assert [kind for kind, cheap in chosen if cheap and kind == lang.TANH] == [lang.TANH] * 2
+    text = hipgen.generate(op, 'f' + '7' * 56, {'math': 'ulp2'}).source
+    # (one test per sigmoid and vector element of the thread)
+    assert text.count('OVL_ALL(') % 3 == 0 and text.count('OVL_ALL(') >= 3 and 'ovl_fast_tanhf' in text
 
 
 def test_an_inexact_value_never_decides_a_branch_or_an_index():
@@ -208,14 +238,19 @@ def sweep(tmp_path_factory):
 
 @pytest.mark.parametrize('kind', ['log1p', 'expm1'])
 def test_once_rounded_routines_within_two_ulp_of_the_reference_formulas_on_the_host(sweep, kind):
-    lo, hi = accuracy.IDIOM_DOMAIN[kind]
-    out = subprocess.check_output([str(sweep), '01'[kind == 'expm1'], repr(lo), repr(hi), '31'],
-                                  universal_newlines=True).split()
-    total, differing, worst, nan_kept = (int(v) for v in out)
-    assert total > 4 << 20
-    assert worst <= accuracy.ROUTINE_ULPS[kind] == accuracy.TOLERANCE
-    assert 0 < differing < total // 2
-    assert nan_kept == 1
+    """Every 31st argument of the domains the generator replaces the formulas on: the one a value range must prove
+    (IDIOM_DOMAIN) and the intervals tested at run time (GUARD_DOMAIN: for log1p also the negative arguments)."""
+    assert accuracy.IDIOM_DOMAIN[kind] in accuracy.GUARD_DOMAIN[kind]
+    for lo, hi in accuracy.GUARD_DOMAIN[kind]:
+        if hi < 0:
+            lo, hi = hi, lo             # the program walks bit patterns upwards: away from zero
+        out = subprocess.check_output([str(sweep), '01'[kind == 'expm1'], repr(lo), repr(hi), '31'],
+                                      universal_newlines=True).split()
+        total, differing, worst, nan_kept = (int(v) for v in out)
+        assert total > (4 << 20 if lo > 0 else 2 << 20)
+        assert worst <= accuracy.ROUTINE_ULPS[kind] == accuracy.TOLERANCE
+        assert 0 < differing < total // 2
+        assert nan_kept == 1
 
 
 @pytest.mark.parametrize('kind', ['log1p', 'expm1'])

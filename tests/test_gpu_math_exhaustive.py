@@ -121,10 +121,19 @@ def test_formula_routines_within_two_ulp_of_the_reference_formulas(lib, kind):
     lib.ovl_exh_ulp_in_range.argtypes = [ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32] + \
         [ctypes.POINTER(ctypes.c_uint64)] * 3 + [ctypes.POINTER(ctypes.c_uint32)] * 2
     narrow = {'log1p_unit': 'log1p', 'expm1_small': 'expm1', 'sigmoid_small': 'sigmoid'}.get(kind)
-    lo, hi = accuracy.NARROW_DOMAIN[narrow] if narrow else accuracy.IDIOM_DOMAIN[kind]
+    # (the intervals tested at run time include the one a value range must prove, IDIOM_DOMAIN)
+    intervals = [accuracy.NARROW_DOMAIN[narrow]] if narrow else list(accuracy.GUARD_DOMAIN[kind])
+    assert narrow or accuracy.IDIOM_DOMAIN[kind] in intervals
     bound = accuracy.TOLERANCE if narrow else accuracy.ROUTINE_ULPS[kind]
     # ranges of bit patterns of one sign each: consecutive patterns are consecutive floats
-    spans = [(_bits(lo), _bits(hi))] if lo > 0 else [(_bits(-0.0), _bits(lo)), (_bits(0.0), _bits(hi))]
+    spans = []
+    for lo, hi in intervals:
+        if lo > 0:
+            spans.append((_bits(lo), _bits(hi)))
+        elif hi < 0:
+            spans.append((_bits(hi), _bits(lo)))
+        else:
+            spans += [(_bits(-0.0), _bits(lo)), (_bits(0.0), _bits(hi))]
     total = total_differing = 0
     for first, last in spans:
         compared, differing, beyond = ctypes.c_uint64(0), ctypes.c_uint64(0), ctypes.c_uint64(0)

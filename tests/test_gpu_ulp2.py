@@ -67,8 +67,8 @@ def test_every_stage_of_the_fused_chain_at_full_size(chain_inputs):
             ref = ovl.evaluate(exact_ops[name](prev)[0], opt_level=0, math_mode='exact')
             assert torch.equal(stages[k], ref), 'stage %s is not exact' % name
         del ref
-    # the oracle itself on a slice of rows of every transcendental stage
-    rows = slice(4000, 4064)
+    # the oracle itself on a band of 1024 rows, all 8192 columns, of every transcendental stage
+    rows = slice(4000, 4000 + cases.ORACLE_BAND_ROWS)
     for k, name in enumerate(cases.CHAIN8_STAGES):
         if name in MATH_STAGES:
             x = stages[k - 1][rows].cpu().numpy()
@@ -156,6 +156,88 @@ def test_small_chain_stagewise_against_the_oracle():
         if name in MATH_STAGES:
             want = oracle.evaluate(cases.chain8_single_stage(name, stages[k - 1]))
             assert cases.ulp_distance(stages[k], want).max() <= TOLERANCE, name
+
+
+def _ulps_nan_equal(x, y):
+    """Float32 steps between two device tensors, 0 where both are NaN."""
+    import torch
+    d = _ulps(x, y)
+    return torch.where(torch.isnan(x) & torch.isnan(y), torch.zeros_like(d), d)
+
+
+def test_lstm_cell_composed_of_library_operators_at_full_size():
+    """The cell of opveclib/test/test_operator_merge.py:311-321 at [4096, 4 x 1024], fused into one 'ulp2' kernel that
+    also stores every operator's output.  Inputs are N(0, 1) with NaN, infinities, zeros of both signs, huge and tiny
+    values planted in the first rows.  Every sigmoid and tanh is compared with the bit-exact operator applied to the
+    kernel's own value of that operator's input (at most 2 ulp); split, the products and the sum must be exact; and
+    on a band of rows that holds the planted values every transcendental operator is compared with the oracle."""
+    import torch
+    from opveclib_amd import runtime
+    concat, c = cases.stdops_lstm_full_size_inputs()
+    concat_d, c_d = torch.from_numpy(concat).cuda(), torch.from_numpy(c).cuda()
+    outs = workloads.stdops_lstm_stage_outputs(concat_d, c_d)
+    fused = workloads.fused_operators(outs)
+    assert len(fused) == 1
+    got = dict(zip(workloads.STDOPS_LSTM_STAGES, ovl.evaluate(outs, opt_level=3, math_mode='ulp2')))
+    source = runtime.load_operator(fused[0], {'math': 'ulp2'}).gen.source
+    assert 'ovl_sigmoid_ulp2(' in source and 'OVL_ALL(' in source and 'ovl_fast_tanhf(' in source
+    units = c.shape[1]
+    for k, name in enumerate('ijfo'):
+        assert torch.equal(got[name].view(torch.int32), concat_d[:, k * units:(k + 1) * units].contiguous().view(torch.int32))
+    stdops = cases.stdops
+    for name, fcn, arg in (('sigmoid_f', stdops.sigmoid, 'f'), ('sigmoid_i', stdops.sigmoid, 'i'),
+                           ('tanh_j', stdops.tanh, 'j'), ('tanh_new_c', stdops.tanh, 'new_c'),
+                           ('sigmoid_o', stdops.sigmoid, 'o')):
+        ref = ovl.evaluate(fcn(got[arg])[0], opt_level=0, math_mode='exact')
+        worst = int(_ulps_nan_equal(got[name], ref).max())
+        assert worst <= TOLERANCE, '%s: %d ulp' % (name, worst)
+        assert torch.equal(torch.isnan(got[name]), torch.isnan(ref)), name
+        # the oracle on the band that holds the planted values
+        band = slice(0, cases.ORACLE_BAND_ROWS)
+        want = oracle.evaluate(fcn(got[arg][band].cpu().numpy())[0])
+        mine = got[name][band].cpu().numpy()
+        both_nan = np.isnan(want) & np.isnan(mine)
+        assert np.array_equal(np.isnan(want), np.isnan(mine)), name
+        distance = cases.ulp_distance(np.where(both_nan, 0, mine), np.where(both_nan, 0, want))
+        assert distance.max() <= TOLERANCE, '%s against the oracle: %d ulp' % (name, int(distance.max()))
+        del ref
+    for name, fcn, args in (('c_sigmoid_f', stdops.mul, (c_d, got['sigmoid_f'])),
+                            ('sigmoid_i_tanh_j', stdops.mul, (got['sigmoid_i'], got['tanh_j'])),
+                            ('new_c', stdops.add, (got['c_sigmoid_f'], got['sigmoid_i_tanh_j'])),
+                            ('new_h', stdops.mul, (got['tanh_new_c'], got['sigmoid_o']))):
+        ref = ovl.evaluate(fcn(*args)[0], opt_level=0, math_mode='exact')
+        same = (got[name].view(torch.int32) == ref.view(torch.int32)) | (torch.isnan(got[name]) & torch.isnan(ref))
+        assert bool(same.all()), name + ' is not exact'
+        del ref
+    # end to end against the bit-exact mode: a few ulp of the O(1) intermediates where nothing is NaN or infinite
+    exact_c, exact_h = ovl.evaluate(workloads.stdops_lstm_outputs(concat_d, c_d), opt_level=3, math_mode='exact')
+    for mine, ref in ((got['new_c'], exact_c), (got['new_h'], exact_h)):
+        finite = torch.isfinite(ref)
+        assert torch.equal(torch.isfinite(mine), finite)
+        scale = float(ref[finite].abs().max())
+        assert float((mine[finite].double() - ref[finite].double()).abs().max()) <= 8 * np.finfo(np.float32).eps * max(1.0, scale)
+
+
+def test_guarded_formulas_on_arguments_straight_from_a_tensor():
+    """sigmoid, log1p and expm1 as single operators on a tensor of unknown range (N(0, 1), a wide sweep, the planted
+    special values): the kernel tests its arguments at run time, wavefronts whose arguments all lie in the compared
+    domain take the once-rounded routine, the others the formula.  Against the oracle: at most 2 ulp, NaN where it has
+    NaN."""
+    from opveclib_amd import runtime
+    x = cases.guarded_formula_arguments()
+    for name, fcn in (('sigmoid', cases.stdops.sigmoid), ('log1p', cases.log1p), ('expm1', cases.expm1)):
+        out = fcn(x)[0]
+        want = oracle.evaluate(out)
+        got = ovl.evaluate(out, opt_level=0, math_mode='ulp2')
+        assert np.array_equal(np.isnan(want), np.isnan(got)), name
+        both_nan = np.isnan(want)
+        distance = cases.ulp_distance(np.where(both_nan, 0, got), np.where(both_nan, 0, want))
+        assert distance.max() <= TOLERANCE, '%s: %d ulp' % (name, int(distance.max()))
+        # both branches ran: some wavefronts took the routine (results that differ from the formula's bits exist)
+        # and the planted values took the formula
+        assert (distance > 0).any(), name + ': no result differs from the formula, the routine never ran'
+    sources = [c.gen.source for key, c in runtime._loaded.items() if "'math', 'ulp2'" in key[1]]
+    assert sum('OVL_ALL(' in text for text in sources) >= 3
 
 
 def test_lstm_keeps_the_oracle_bits_in_ulp2_mode():
