@@ -179,6 +179,11 @@ REFERENCE_LSTM_UNITS = (200, 650, 1500)
 REFERENCE_CUMSUM_SHAPE = (10000, 1000)
 
 
+#: row lengths of the float32 scans that `bench.py --only "row stride"` times for counter collection: rows of 64 KiB,
+#: 64 KiB + 256 bytes and 65 KiB
+ROW_STRIDE_PROBE_COLUMNS = (16384, 16448, 16640)
+
+
 def all_workload_outputs():
     """Operator outputs of every benchmark workload at full size, built from shape specs."""
     f32, f64 = np.float32, np.float64
@@ -197,6 +202,8 @@ def all_workload_outputs():
     yield stdops_lstm_outputs(Spec((4096, 4096)), Spec((4096, 1024)))
     yield conv1d_outputs(Spec((5, 1000, 3), f64), Spec((10, 13, 3), f64))
     yield cumsum_outputs(Spec(REFERENCE_CUMSUM_SHAPE, f64), axis=0)
+    for cols in ROW_STRIDE_PROBE_COLUMNS:           # bench.py --only "row stride"
+        yield cumsum_outputs(Spec((4096, cols), f32))
     yield dot_outputs(Spec((4096, 16384), f32), Spec((4096, 16384), f32))
     yield column_sum_outputs(Spec(REFERENCE_CUMSUM_SHAPE, f64))
     for units in REFERENCE_LSTM_UNITS:
