@@ -296,6 +296,30 @@ class HandWrittenScan(object):
         return [self.out]
 
 
+class StripCopy(object):
+    """The measurement aid ovl_strip_copy_f64 (include/ovl_scan.h): a float64 [rows, cols] tensor moved by one workgroup
+    per strip of ``lines`` columns, without scanning; ``mode`` 1 loads, 2 stores, 3 copies."""
+
+    def __init__(self, x, lines, mode):
+        import torch
+        from opveclib_amd import row_scan
+        self.lib = row_scan.library()
+        self.x = torch.from_numpy(np.ascontiguousarray(x)).cuda()
+        self.out = torch.empty_like(self.x)
+        self.rows, self.cols = self.x.shape
+        self.lines, self.mode = lines, mode
+        self.algorithmic_bytes = (1 if mode < 3 else 2) * self.x.numel() * self.x.element_size()
+        self.kernels = [{'kernel': 'strip_copy_kernel'}]
+
+    def launch(self, stream):
+        if self.lib.ovl_strip_copy_f64(self.x.data_ptr(), self.rows, self.cols, self.out.data_ptr(), self.lines,
+                                       self.mode, stream) != 0:
+            raise RuntimeError(self.lib.ovl_scan_last_error().decode())
+
+    def results(self):
+        return [self.out]
+
+
 ONLY = [None]           # --only
 
 
@@ -305,7 +329,7 @@ def side_workload(name, outputs, steps, warmup, options=None, reference=None, su
     workload that --only leaves out."""
     if ONLY[0] is not None and ONLY[0] not in name:
         return None
-    handwritten = isinstance(outputs, (HandWrittenLstm, HandWrittenScan))
+    handwritten = isinstance(outputs, (HandWrittenLstm, HandWrittenScan, StripCopy))
     prepared = outputs if handwritten else Prepared(outputs, options)
     settle(prepared)
     if sustained:
@@ -742,9 +766,9 @@ def main():
         for key in ('cumsum32', 'cumprod32', 'cumsum64'):
             cpu.pop(key, None)
         concat, c, dh, dc = data['concat'], data['c'], data['dh'], data['dc']
-        others.append(side_workload('c4 lstm cell forward [4096, 4x1024]', lstm_outputs(concat, c), steps, warm,
+        others.append(side_workload("c4 lstm cell forward [4096, 4x1024], 'exact' math mode", lstm_outputs(concat, c), steps, warm,
                                     reference=cpu.get('lstm'), sustained=True))
-        others.append(side_workload('c4 lstm cell gradient [4096, 4x1024]', lstm_grad_outputs(concat, c, dc, dh),
+        others.append(side_workload("c4 lstm cell gradient [4096, 4x1024], 'exact' math mode", lstm_grad_outputs(concat, c, dc, dh),
                                     steps, warm, reference=cpu.get('lstm_grad'), sustained=True))
         # these two also run at the board's power limit: the readings say so
         if others[-2]:
@@ -757,6 +781,15 @@ def main():
                                     sustained=True))
         others.append(side_workload('c4 lstm cell gradient, hand-written kernel (run-time shape, same bits)',
                                     HandWrittenLstm(concat, c, dc, dh), steps, warm,
+                                    reference=cpu.get('lstm_grad'), sustained=True))
+        # what an unchanged caller's evaluate() runs on the hand-fused cell: in the default 'ulp2' mode no routine of
+        # it is replaced (the operator's own outputs are sums that cancel, so 2 ulp of them leaves no room), the bits
+        # stay the oracle's; the cell composed of library operators below is where the mode acts
+        others.append(side_workload("c4 lstm cell forward in the default 'ulp2' math mode (nothing replaced: same bits)",
+                                    lstm_outputs(concat, c), steps, warm, {'math': 'ulp2'},
+                                    reference=cpu.get('lstm'), sustained=True))
+        others.append(side_workload("c4 lstm cell gradient in the default 'ulp2' math mode (nothing replaced: same bits)",
+                                    lstm_grad_outputs(concat, c, dc, dh), steps, warm, {'math': 'ulp2'},
                                     reference=cpu.get('lstm_grad'), sustained=True))
         others.append(side_workload("c4 lstm cell forward in the optional 'fast' math mode", lstm_outputs(concat, c),
                                     steps, warm, {'math': 'fast'}))
@@ -786,6 +819,12 @@ def main():
         others.append(side_workload('reference timing: cumsum f64[10000,1000] along axis 0 '
                                     '(examples/test_perf_accumulate.py:35-47)', cumsum_outputs(data['x0'], axis=0),
                                     10, warm, reference=cpu.get('cumsum_axis0')))
+        # the same tensor only moved, in the strips the scan along axis 0 uses (8 columns per workgroup) and in the
+        # neighbouring choices: what the access pattern costs without the recurrence
+        for lines, mode, what in ((8, 3, 'copied'), (8, 1, 'loaded'), (8, 2, 'stored'), (16, 3, 'copied'),
+                                  (4, 3, 'copied')):
+            others.append(side_workload('strip copy: f64[10000,1000] %s, one workgroup per %d columns (no scan)'
+                                        % (what, lines), StripCopy(data['x0'], lines, mode), 10, warm))
         others.append(side_workload('reference timing: conv1D f64 [5,1000,3] x [10,13,3], mode same, NEC '
                                     '(examples/conv1D.py:323-340)', workloads.conv1d_outputs(*data['conv1d']), steps,
                                     warm, reference=cpu.get('conv1d')))

@@ -62,6 +62,17 @@ int ovl_cumprod_f32_reassociated(const float* x, uint32_t rows, uint32_t cols, f
 int ovl_cumsum_f64_reassociated(const double* x, uint32_t rows, uint32_t cols, double* out, void* hip_stream);
 int ovl_cumprod_f64_reassociated(const double* x, uint32_t rows, uint32_t cols, double* out, void* hip_stream);
 
+/*
+ * Measurement aid with no counterpart in the reference: moves a dense [rows, cols] float64 tensor the way the
+ * generated kernels that scan along the FIRST axis do, without scanning.  One workgroup owns `lines` (4, 8 or 16)
+ * neighbouring columns and walks down the rows, so every row contributes `lines` * 8 consecutive bytes to it.
+ * `mode` 1 only loads x, 2 only stores (the row index) to out, 3 copies x to out.  Timed beside a scan along the first
+ * axis it says how much of that scan's time is the access pattern and how much the recurrence.  Same conventions and
+ * status codes as the functions above.
+ */
+int ovl_strip_copy_f64(const double* x, uint32_t rows, uint32_t cols, double* out, uint32_t lines, uint32_t mode,
+                       void* hip_stream);
+
 /* Text of the last error on the calling thread ("" if none). */
 const char* ovl_scan_last_error(void);
 

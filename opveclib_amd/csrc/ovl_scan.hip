@@ -772,11 +772,101 @@ int reassociated_scan(const char* who, const T* x, uint32_t rows, uint32_t cols,
     return OVL_OK;
 }
 
+// ---------------------------------------------------------------------------------------------------------------------
+// Measurement aid: what moving a [rows, cols] float64 tensor costs when one workgroup owns a strip of LINES neighbouring
+// lines (columns) and walks down the rows, as the kernels that scan along the first axis do (hipgen/colscan_kernel.py).
+// Every load instruction of a wavefront reads 64 / LINES rows, LINES * 8 bytes of each; eight rows per thread are in
+// flight.  MODE 1 only loads (the values are added up and the sum is stored where no run reaches), 2 only stores
+// (the row index), 3 copies.
+// ---------------------------------------------------------------------------------------------------------------------
+constexpr int STRIP_THREADS = 256, STRIP_IN_FLIGHT = 8;
+
+template <int LINES, int MODE>
+__global__ __launch_bounds__(STRIP_THREADS) void strip_copy_kernel(const double* __restrict__ x, double* __restrict__ out,
+                                                                   uint32_t rows, uint32_t cols) {
+    constexpr uint32_t ROWS_PER_PASS = STRIP_THREADS / LINES, ROWS_PER_STEP = ROWS_PER_PASS * STRIP_IN_FLIGHT;
+    // Strips narrower than a 128-byte line share lines with their neighbours; as in the generated scans, the
+    // workgroups of one XCD (every eighth) take the strips that share: groups of SHARE neighbours when every row
+    // starts on a line boundary, else one contiguous range per XCD.
+    constexpr uint32_t SHARE = 128 / (LINES * 8) > 1 ? 128 / (LINES * 8) : 1;
+    const uint32_t total = gridDim.x;
+    uint32_t strip = blockIdx.x;
+    if (SHARE > 1 && (cols * 8u) % 128u == 0u && total >= 8u * SHARE) {
+        const uint32_t whole = total / (8u * SHARE) * (8u * SHARE);
+        if (blockIdx.x < whole)
+            strip = blockIdx.x / (8u * SHARE) * (8u * SHARE) + blockIdx.x % 8u * SHARE + blockIdx.x / 8u % SHARE;
+    } else if (SHARE > 1 && total >= 16u) {
+        const uint32_t q = total / 8u, r = total % 8u, xcd = blockIdx.x % 8u;
+        strip = xcd * q + (xcd < r ? xcd : r) + blockIdx.x / 8u;
+    }
+    uint32_t c = strip * LINES + threadIdx.x % LINES;
+    const bool line_exists = c < cols;
+    if (!line_exists) c = cols - 1u;          // a thread past the last line loads that line once more and stores nothing
+    const uint32_t r0 = threadIdx.x / LINES;
+    const double* p = x + (uint64_t)r0 * cols + c;
+    double* q = out + (uint64_t)r0 * cols + c;
+    const uint64_t pass_stride = (uint64_t)ROWS_PER_PASS * cols;
+    double sum = 0.0;
+    uint32_t base = 0;
+    // steps all of whose rows exist: no conditions around the loads
+    for (; base + ROWS_PER_STEP <= rows; base += ROWS_PER_STEP) {
+        double v[STRIP_IN_FLIGHT];
+        #pragma unroll
+        for (uint32_t u = 0; u < STRIP_IN_FLIGHT; ++u) v[u] = (MODE & 1) ? p[u * pass_stride] : (double)(base + u * ROWS_PER_PASS + r0);
+        if (MODE & 2) {
+            if (line_exists) {
+                #pragma unroll
+                for (uint32_t u = 0; u < STRIP_IN_FLIGHT; ++u) __builtin_nontemporal_store(v[u], &q[u * pass_stride]);
+            }
+        } else {
+            #pragma unroll
+            for (uint32_t u = 0; u < STRIP_IN_FLIGHT; ++u) sum += v[u];
+        }
+        p += STRIP_IN_FLIGHT * pass_stride;
+        q += STRIP_IN_FLIGHT * pass_stride;
+    }
+    // the last rows
+    for (uint32_t r = base + r0; r < rows; r += ROWS_PER_PASS) {
+        const double v = (MODE & 1) ? x[(uint64_t)r * cols + c] : (double)r;
+        if (MODE & 2) {
+            if (line_exists) __builtin_nontemporal_store(v, &out[(uint64_t)r * cols + c]);
+        } else {
+            sum += v;
+        }
+    }
+    if (!(MODE & 2) && sum == -1.2345e300) out[0] = sum;
+}
+
+template <int LINES>
+void launch_strip_copy(int mode, const double* x, double* out, uint32_t rows, uint32_t cols, hipStream_t stream) {
+    const dim3 grid((cols + LINES - 1) / LINES), block(STRIP_THREADS);
+    if (mode == 1) hipLaunchKernelGGL((strip_copy_kernel<LINES, 1>), grid, block, 0, stream, x, out, rows, cols);
+    else if (mode == 2) hipLaunchKernelGGL((strip_copy_kernel<LINES, 2>), grid, block, 0, stream, x, out, rows, cols);
+    else hipLaunchKernelGGL((strip_copy_kernel<LINES, 3>), grid, block, 0, stream, x, out, rows, cols);
+}
+
 }  // namespace
 
 extern "C" {
 
 const char* ovl_scan_last_error(void) { return g_last_error.c_str(); }
+
+int ovl_strip_copy_f64(const double* x, uint32_t rows, uint32_t cols, double* out, uint32_t lines, uint32_t mode,
+                       void* hip_stream) {
+    const char* who = "ovl_strip_copy_f64";
+    if (x == nullptr || out == nullptr) return fail(OVL_EINVAL, std::string(who) + ": null tensor");
+    if (rows == 0 || cols == 0) return fail(OVL_EINVAL, std::string(who) + ": rows and cols must be positive");
+    if ((uint64_t)rows * cols >= (1ull << 32)) return fail(OVL_EINVAL, std::string(who) + ": rows * cols must be below 2^32");
+    if (mode < 1 || mode > 3) return fail(OVL_EINVAL, std::string(who) + ": mode is 1 (load), 2 (store) or 3 (copy)");
+    hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    if (lines == 4) launch_strip_copy<4>((int)mode, x, out, rows, cols, stream);
+    else if (lines == 8) launch_strip_copy<8>((int)mode, x, out, rows, cols, stream);
+    else if (lines == 16) launch_strip_copy<16>((int)mode, x, out, rows, cols, stream);
+    else return fail(OVL_EINVAL, std::string(who) + ": 4, 8 or 16 lines per workgroup");
+    const hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return fail(OVL_EHIP, std::string(who) + ": " + hipGetErrorString(err));
+    return OVL_OK;
+}
 
 int ovl_cumsum_f32_reassociated(const float* x, uint32_t rows, uint32_t cols, float* out, void* hip_stream) {
     return reassociated_scan<float, op_sum>("ovl_cumsum_f32_reassociated", x, rows, cols, out, hip_stream);

@@ -30,7 +30,7 @@ from . import rowscan_kernel
 from . import colscan_kernel
 
 #: bump when generated code changes for an unchanged DAG, so cached binaries are not reused
-CODEGEN_VERSION = 33
+CODEGEN_VERSION = 37
 
 
 
@@ -64,7 +64,7 @@ def generate(expression_dag, function_name, options=None):
     :param function_name: unique name of the operator (its content hash)
     :param options: optional dict.  ``template``: 'auto' (default), 'map', 'transpose', 'rowscan', 'skewscan', 'fedscan', 'carryscan', 'treescan', 'rowreduce', 'colreduce', 'colscan' or 'colskew' restricts
         the choice of kernel template (a template that does not fit the DAG falls back to 'map'); ``vec`` forces the
-        map template with that vector width, ``per_thread`` its vectors per thread (1 or 2); ``scan_movers`` the number of threads that only move data in the lane-skewed column scan (0: every wavefront scans and moves), ``scan_depth`` / ``scan_sets`` / ``scan_width`` / ``scan_interleave`` set the request burst (groups), the
+        map template with that vector width, ``per_thread`` its vectors per thread (1 or 2); ``scan_movers`` the number of threads that only move data in the lane-skewed column scan (0: every wavefront scans and moves), ``scan_carry`` False keeps the results in its scanning wavefronts instead of recomputing them in finishing ones, ``scan_depth`` / ``scan_sets`` / ``scan_width`` / ``scan_interleave`` set the request burst (groups), the
         number of register sets, the 128-bit vectors per lane and phase and the rows per lane group of the lane-skewed scan; ``math``: 'exact'
         or 'fast'; ``if_conversion`` / ``value_ranges`` / ``cse``: False switches that transformation off; ``scan_rows`` / ``scan_chunk`` the LDS tile of the row scan, ``scan_batch`` the vectors per register set of its scanning wavefront; ``nt`` /
         ``scan_nt`` which vector accesses carry the non-temporal hint ('l' loads, 's' stores, 'ls', ''); ``grid_cap``
@@ -127,7 +127,8 @@ def generate(expression_dag, function_name, options=None):
                                        colscan_kernel.prefers_skew(info, colscan_kernel.plan(info)))):
         kernel_src, launch = colscan_kernel.generate_skewed(info, kernel_name, options.get('scan_sets'),
                                                             options.get('scan_strip'), options.get('scan_width'),
-                                                            options.get('scan_movers'))
+                                                            options.get('scan_movers'), carry=options.get('scan_carry'),
+                                                            nt=options.get('scan_nt'))
     elif options.get('vec') is None and template in ('auto', 'colscan') and \
             colscan_kernel.plan(info, options.get('scan_rows'), options.get('scan_batch'),
                                 options.get('scan_sets')) is not None and \

@@ -530,7 +530,8 @@ def prefers_skew(info, p):
     return all(info.nodes[idx].dtype in CTYPE for idx in _carried_state(info, p))
 
 
-def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, movers=None, reduce=False):
+def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, movers=None, reduce=False, carry=None,
+                    nt=None):
     from .rowscan_kernel import _carried_state
     p = (reduce_plan if reduce else plan)(info)
     assert p is not None
@@ -545,6 +546,11 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
         # [10000, 1000] without separate movers: 79 us with 32 bytes, 65 with 64, 59 with 128; with wider strips the
         # longer segments lose: float64 [4096, 4096] 41 -> 45 us)
         seg_vectors = SKEW_SEG_VECTORS_NARROW if narrow else SKEW_SEG_VECTORS
+        if narrow and reduce and per == 2 and p.length >= 8192:
+            # a reduction over a long axis of 8-byte elements keeps nothing per row, so twice the segment costs only
+            # registers: column sums float64 [10000, 1000] 37.0 -> 34.6 us, [20000, 512] 66.9 -> 60.1 (float32, and
+            # float64 [4096, 2048], lose 1 to 2 us)
+            seg_vectors = 2 * SKEW_SEG_VECTORS_NARROW
     seg = seg_vectors * per                         # rows a lane owns per phase
     rc = SKEW_GROUP * seg                           # rows per chunk
     if movers is None:
@@ -558,9 +564,24 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
         # the workgroups run ahead of each other the more often a line is fetched twice); without them the narrow
         # strips take four
         sets = 2 if movers else 4 if narrow else SKEW_SETS
-    BLOCK = SCAN_THREADS + movers
+    # With separate movers, a scan (not a reduction) of 8-byte elements also takes its results off the scanning
+    # wavefronts: they keep none, publish the exact state that enters each lane's segment, and as many finishing
+    # wavefronts recompute the segments from those states and write them to LDS (see `rowscan_kernel.generate_carry`:
+    # a 128-bit LDS write costs the wavefront that issues it five steps of a float64 recurrence).  The scanning
+    # wavefronts then also read the next chunk's segments during the phases of the current one.  Measured: float64
+    # [10000, 1000] along axis 0 41.4 -> 38.5 us, [5000, 300] 23.5 -> 21.6; float32 [10000, 1000] 33.9 -> 34.3 (not
+    # chosen there).  What is left is moving the data: a kernel that only copies the tensor in the same strips (one
+    # workgroup per 8 lines, 64 bytes of every row) takes 36 us, one that only loads it 24 us; 16 lines per workgroup
+    # copy in 45 us on half as many compute units and 4 lines (32 bytes per row) in 86 us.
+    if carry is None:
+        carry = per == 2
+    carry = bool(carry and movers and not p.reduce and seg_vectors in (1, 2, 4, 8, 16, 32))
+    FINISH_THREADS = SCAN_THREADS if carry else 0
+    BLOCK = SCAN_THREADS + FINISH_THREADS + movers
+    if BLOCK > 1024:
+        carry, FINISH_THREADS, BLOCK = False, 0, SCAN_THREADS + movers
     MOVE = movers or BLOCK                          # threads that move data
-    NBUF = 3 if movers else 2
+    NBUF = 6 if carry else 3 if movers else 2
     seg_stride = seg + per                          # a segment and its padding vector (bank conflicts)
     line_stride = SKEW_GROUP * seg_stride + per     # a line and its padding vector
     num_chunks = (p.length + rc - 1) // rc
@@ -605,6 +626,9 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
     src = []
     a = src.append
     a('typedef %s %s __attribute__((ext_vector_type(%d)));' % (ctype, vname, per))
+    if carry:
+        a('struct ovl_scan_yes { static constexpr bool value = true; };')
+        a('struct ovl_scan_no { static constexpr bool value = false; };')
     a('')
     a('extern "C" __global__ void __launch_bounds__(%d)' % BLOCK)
     if p.reduce:
@@ -619,20 +643,47 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
     a('    // tile[buffer][line][row]: a line holds the %d rows of a chunk as 16 segments of %d rows, each followed by one' % (rc, seg))
     a('    // spare vector, and one more at its end')
     a('    __shared__ __attribute__((aligned(16))) %s tile[%d][%d][%d];' % (ctype, NBUF, STRIP, line_stride))
+    if carry:
+        for name, stype in state:
+            a('    __shared__ %s entering_%s[%d][%d];' % (stype, name, NBUF, SCAN_THREADS))
     # A strip narrower than a 128-byte line shares the lines of every row with its neighbours.  Workgroups go to the
-    # eight XCDs (each with its own L2) in turn, so neighbouring strips are given to workgroups 8 apart: they land on
-    # one XCD at about the same time and the line is fetched from memory once (float64 [10000, 1000] in strips of 8
-    # lines read its input twice).
+    # eight XCDs (each with its own L2) in turn, so the strips that share lines are given to workgroups a multiple of
+    # 8 apart: they run on one XCD at the same time and a line is fetched from memory once.
+    #  * Row pitch a multiple of 128 bytes: the same 128 / (strip bytes) strips share a line in every row; they go to
+    #    one XCD, the next such group to the next XCD (the pieces an XCD reads are spread over the whole row).
+    #  * Any other pitch: which neighbours share depends on the row (float64 rows of 1000 columns: even rows pair a
+    #    strip with one side, odd rows with the other), so every XCD is given one contiguous range of strips.  float64
+    #    [10000, 1000] in strips of 8 lines reads its input 2.0 times with neighbouring strips on neighbouring XCDs,
+    #    1.55 times with pairs of strips per XCD, 1.07 times with ranges (38.5 -> 37.5 us; float32 34 -> 31 us).
+    #    (With a pitch that is a multiple of 128 bytes ranges lose: an XCD then reads one narrow column of the tensor
+    #    at a power-of-two pitch; float32 [4096, 2048] 18 -> 23 us.)
     share = max(1, 128 // (STRIP * ITEMSIZE[p.x.dtype]))
     total = p.outer * strips
-    if share > 1 and total >= 8 * share:
+    if share > 1 and (p.inner * ITEMSIZE[p.x.dtype]) % 128 == 0 and total >= 8 * share:
         whole = total // (8 * share) * (8 * share)
-        a('    // workgroups b and b + 8 (same XCD) take neighbouring strips, which share the cache lines of every row')
+        a('    // workgroups b, b + 8, ... (one XCD) take the %d neighbouring strips that share the cache lines of every row' % share)
         a('    const uint32_t wg = blockIdx.x < %du' % whole)
         a('        ? blockIdx.x / %du * %du + blockIdx.x %% 8u * %du + blockIdx.x / 8u %% %du : blockIdx.x;' % (
             8 * share, 8 * share, share, share))
+    elif share > 1 and total >= 16:
+        q, r = divmod(total, 8)
+        a('    // workgroups b, b + 8, b + 16, ... (one XCD) take a contiguous range of strips, which share cache lines')
+        a('    const uint32_t xcd = blockIdx.x % 8u, slot = blockIdx.x / 8u;')
+        a('    const uint32_t wg = xcd * %du + (xcd < %du ? xcd : %du) + slot;' % (q, r, r))
     else:
         a('    const uint32_t wg = blockIdx.x;')
+    if nt is None:
+        # Stores carry the non-temporal hint (the results are not read again), except where the same neighbouring strips
+        # share every line: there plain stores let the L2 put a line's parts together before it is written back
+        # (float64 [4096, 2048]: 29.0 -> 24.7 us).  Where the sharing neighbours change from row to row plain stores
+        # bring the written bytes from 1.25 times the tensor to 1.0 but take 1 us longer (float64 [10000, 1000]:
+        # 37.7 -> 38.9 us), so the hint stays.
+        nt = '' if share > 1 and (p.inner * ITEMSIZE[p.x.dtype]) % 128 == 0 else 's'
+    if not p.reduce:
+        if 's' in nt:
+            a('#define OVL_SCAN_STORE(value, address) __builtin_nontemporal_store(value, address)')
+        else:
+            a('#define OVL_SCAN_STORE(value, address) (*(address) = (value))')
     a('    const uint32_t strip = wg %% %du;' % strips)
     a('    const uint32_t o = wg / %du;                         // index over the dimensions before the scanned axis' % strips)
     a('    const uint32_t c0 = strip * %du;                      // first line of the strip within its row' % STRIP)
@@ -642,8 +693,18 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
     if not p.reduce:
         a('    %s* __restrict__ gout = out%d + obase;' % (ctype, p.out.io_index))
     a('')
-    if movers:
+    if carry:
+        # (A compute unit places the wavefronts of a workgroup on its four SIMDs in turn, wavefronts w and w + 4 share
+        # one.  Which roles share a SIMD made no difference to the time: scanning with finishing, scanning with
+        # moving, or the scanning wavefronts alone beside two wavefronts of movers.)
+        a('    // Threads 0..%d scan, %d..%d finish, %d and up move data.' % (
+            SCAN_THREADS - 1, SCAN_THREADS, SCAN_THREADS + FINISH_THREADS - 1, SCAN_THREADS + FINISH_THREADS))
+        a('    const uint32_t vt = threadIdx.x;')
+        a('    const bool is_mover = vt >= %du;' % (SCAN_THREADS + FINISH_THREADS))
+        a('    const uint32_t mt = vt - %du;' % (SCAN_THREADS + FINISH_THREADS))
+    elif movers:
         a('    // Threads %d and up move data, the others scan.' % SCAN_THREADS)
+        a('    const bool is_mover = threadIdx.x >= %du;' % SCAN_THREADS)
         a('    const uint32_t mt = threadIdx.x - %du;' % SCAN_THREADS)
     else:
         a('    const uint32_t mt = threadIdx.x;')
@@ -684,6 +745,46 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
     a('        #pragma unroll')
     a('        for (uint32_t i = 0; i < %du; ++i) *lds_at(k, i) = regs.v[i];' % vpt)
     a('    };')
+    # The same for a chunk all of whose rows exist (every chunk but the last), without the clamps: byte offsets and
+    # LDS positions of a thread's elements are computed once, a chunk's base address is uniform.  (With the clamps and
+    # the 64-bit index arithmetic per element a moving wavefront issued some 250 vector instructions per chunk; a
+    # wavefront that shares a SIMD with a scanning one costs it about four clocks per instruction.)
+    a('    uint32_t element_offset[%d], lds_offset[%d];' % (vpt * per, vpt))
+    a('    #pragma unroll')
+    a('    for (uint32_t i = 0; i < %du; ++i) {' % vpt)
+    a('        const uint32_t r = (mv + i * %du) * %du;' % (rows_per_pass, per))
+    a('        lds_offset[i] = mc * %du + (r / %du) * %du + r %% %du;' % (line_stride, seg, seg_stride, seg))
+    a('        #pragma unroll')
+    a('        for (uint32_t u = 0; u < %du; ++u) element_offset[i * %du + u] = ((r + u) * %du + mc) * %du;' % (
+        per, per, p.inner, ITEMSIZE[p.x.dtype]))
+    a('    }')
+    a('    auto issue_loads_full = [&](uint32_t k, MoverRegs& regs) {')
+    a('        const char* base = reinterpret_cast<const char*>(gin + (uint64_t)k * %dull);' % (rc * p.inner))
+    a('        #pragma unroll')
+    a('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
+    a('            #pragma unroll')
+    a('            for (uint32_t u = 0; u < %du; ++u)' % per)
+    a('                regs.v[i][u] = *reinterpret_cast<const %s*>(base + element_offset[i * %du + u]);' % (ctype, per))
+    a('        }')
+    a('    };')
+    if not p.reduce:
+        a('    auto store_chunk_full = [&](uint32_t k) {')
+        a('        const %s* buffer = &tile[k %% %du][0][0];' % (ctype, NBUF))
+        a('        char* base = reinterpret_cast<char*>(gout + (uint64_t)k * %dull);' % (rc * p.inner))
+        a('        MoverRegs regs;')
+        a('        #pragma unroll')
+        a('        for (uint32_t i = 0; i < %du; ++i) regs.v[i] = *reinterpret_cast<const %s*>(buffer + lds_offset[i]);' % (
+            vpt, vname))
+        a('        #pragma unroll')
+        a('        for (uint32_t i = 0; i < %du; ++i) {' % vpt)
+        a('            #pragma unroll')
+        a('            for (uint32_t u = 0; u < %du; ++u)' % per)
+        a('                OVL_SCAN_STORE(regs.v[i][u], reinterpret_cast<%s*>(base + element_offset[i * %du + u]));' % (
+            ctype, per))
+        a('        }')
+        a('    };')
+    else:
+        a('    auto store_chunk_full = [&](uint32_t) {};')
     if p.reduce:
         a('    auto store_chunk = [&](uint32_t) {};      // a reduction stores nothing per row')
     else:
@@ -708,8 +809,8 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
         a('            #pragma unroll')
         a('            for (uint32_t u = 0; u < %du; ++u) {' % per)
         a('                const uint32_t r = (mv + i * %du) * %du + u;' % (rows_per_pass, per))
-        a('                __builtin_nontemporal_store(r <= last ? regs.v[i][u] : of_last,')
-        a('                                            gout + (uint64_t)(k * %du + (r <= last ? r : last)) * %dull + mc);' % (
+        a('                OVL_SCAN_STORE(r <= last ? regs.v[i][u] : of_last,')
+        a('                               gout + (uint64_t)(k * %du + (r <= last ? r : last)) * %dull + mc);' % (
             rc, p.inner))
         a('            }')
         a('        }')
@@ -720,8 +821,14 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
     a('    // rows [part * %d, part * %d + %d) of every chunk.  A line past the last one shadows it.' % (seg, seg, seg))
     a('    const uint32_t lane = threadIdx.x %% %du;' % WAVE)
     a('    const uint32_t part = lane %% %du;' % SKEW_GROUP)
-    a('    const uint32_t sl = threadIdx.x / %du * %du + lane / %du;      // line of the strip' % (
-        WAVE, lines_per_wave, SKEW_GROUP))
+    if carry:
+        a('    // scanning and finishing threads map to lines alike')
+        a('    const uint32_t st = vt %% %du;' % SCAN_THREADS)
+        a('    const uint32_t sl = st / %du * %du + lane / %du;      // line of the strip' % (
+            WAVE, lines_per_wave, SKEW_GROUP))
+    else:
+        a('    const uint32_t sl = threadIdx.x / %du * %du + lane / %du;      // line of the strip' % (
+            WAVE, lines_per_wave, SKEW_GROUP))
     a('    const uint32_t c = (c0 + sl < %du) ? sl : %du - c0;' % (p.inner, p.inner - 1))
     a('    const uint32_t line = o * %du + c0 + c;' % p.inner)
     if p.reduce:
@@ -797,20 +904,157 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
     a('    // %d register sets keep %d chunks of loads in flight: chunk j travels through set j %% %d' % (sets, sets, sets))
     a('    MoverRegs sets[%d];' % sets)
     full = num_chunks // sets
-    if movers:
+    if carry:
+        n = num_chunks
+        read_phases = min(8, seg_vectors)              # the phases in which the next chunk's segments are read
+        reads_per_phase = seg_vectors // read_phases
+        a('    // Six buffers rotate, one barrier per step.  Step s: the movers bring chunk s + 2 into LDS and take the')
+        a('    // results of chunk s - 3 out; the scanning wavefronts run the recurrence over chunk s and read their segments')
+        a('    // of chunk s + 1 meanwhile; the finishing wavefronts recompute chunk s - 2 from the states that enter its')
+        a('    // segments.  Every thread passes the same %d barriers.' % (n + 3))
+        a('    if (is_mover) {')
+        for j in range(2):
+            a('        issue_loads%s(%du, sets[%d]);' % ('_full' if j < n - 1 else '', min(j, n - 1), j % sets))
+        # chunks 0 and 1 go to LDS before the first barrier; chunks 2 .. 1 + sets are requested behind them
+        a('        write_lds(0u, sets[0]);')
+        if n > 1:
+            a('        write_lds(1u, sets[1 %% %du]);' % sets)
+        for j in range(sets):
+            if 2 + j < n:
+                a('        issue_loads%s(%du, sets[%d]);' % ('_full' if 2 + j < n - 1 else '', 2 + j, (2 + j) % sets))
+        a('        __syncthreads();')
+
+        def emit_step(k):
+            regs = 'sets[%d]' % ((k + 2) % sets)
+            if k + 2 < n:
+                a('        write_lds(%du, %s);' % (k + 2, regs))
+            if k + 2 + sets < n:
+                a('        issue_loads%s(%du, %s);' % ('_full' if k + 2 + sets < n - 1 else '', k + 2 + sets, regs))
+            if k >= 3:
+                a('        store_chunk_full(%du);' % (k - 3))
+            a('        __syncthreads();')
+        steps = n + 2                                   # steps 0 .. n + 1
+        steady_first = ((3 + sets - 1) // sets + 1) * sets      # a multiple of `sets` past the first stores
+        # steps [steady_first, steady_end) do all three things, on chunks all of whose rows exist
+        steady_end = max(steady_first, n - 3 - sets)
+        groups = (steady_end - steady_first) // sets
+        for k in range(0, min(steady_first, steps)):
+            emit_step(k)
+        if groups:
+            a('        #pragma unroll 1')
+            a('        for (uint32_t k0 = %du; k0 < %du; k0 += %du) {' % (steady_first, steady_first + groups * sets, sets))
+            for d in range(sets):
+                a('            write_lds(k0 + %du, sets[%d]);' % (d + 2, (steady_first + d + 2) % sets))
+                a('            issue_loads_full(k0 + %du, sets[%d]);' % (d + 2 + sets, (steady_first + d + 2) % sets))
+                a('            store_chunk_full(k0 + %du - 3u);' % d)
+                a('            __syncthreads();')
+            a('        }')
+        for k in range(max(steady_first + groups * sets, min(steady_first, steps)), steps):
+            emit_step(k)
+        a('        store_chunk(%du);' % (n - 1))
+        a('    } else if (vt < %du) {' % SCAN_THREADS)
+        a('        // scanning wavefronts: no results kept; the next chunk\'s segments arrive during the first eight phases')
+        a('#undef OVL_SCAN_OUT')
+        a('#define OVL_SCAN_OUT(value) (void)(value)')
+        a('        Segment set_a, set_b;')
+        a('        __syncthreads();')
+        a('        fetch_segment(0u, set_a);')
+        a('        auto scan_only = [&](uint32_t k, const Segment& segment, Segment& other, auto first_chunk) {')
+        a('            const %s* ahead = &tile[(k + 1u) %% %du][sl][part * %du];' % (ctype, NBUF, seg_stride))
+        a('            const uint32_t row0 = k * %du + part * %du;' % (rc, seg))
+        a('            #pragma unroll')
+        a('            for (uint32_t phase = 0; phase < %du; ++phase) {' % SKEW_GROUP)
+        for name, _ in state:
+            a('                %s = carry_%s;' % (name, name))
+        a('                #pragma unroll')
+        a('                for (uint32_t w = 0; w < %du; ++w) {' % seg_vectors)
+        a('                    const %s xv = segment.v[w];' % vname)
+        a('                    #pragma unroll')
+        a('                    for (uint32_t u = 0; u < %du; ++u) {' % per)
+        a('                        // (the first row is what the statements before the loop computed)')
+        a('                        if (decltype(first_chunk)::value && w == 0u && u == 0u) { if (part != 0u) OVL_SCAN_STEP(row0) }')
+        a('                        else OVL_SCAN_STEP(row0 + w * %du + u)' % per)
+        a('                    }')
+        a('                }')
+        for name, _ in state:
+            a('                carry_%s = ovl_dpp_move<OVL_DPP_ROW_SHR1>(carry_%s, %s);' % (name, name, name))
+        a('                if (phase < %du) {' % read_phases)
+        a('                    #pragma unroll')
+        a('                    for (uint32_t j = 0; j < %du; ++j)' % reads_per_phase)
+        a('                        other.v[phase * %du + j] = *reinterpret_cast<const %s*>(ahead + (phase * %du + j) * %du);' % (
+            reads_per_phase, vname, reads_per_phase, per))
+        a('                }')
+        a('                __builtin_amdgcn_sched_barrier(0);')
+        a('                if (phase == 8u) {')
+        a('                    __syncthreads();')
+        a('                    __builtin_amdgcn_sched_barrier(0);')
+        a('                }')
+        a('            }')
+        a('            // lanes 1..15 hold their left neighbour\'s exact final state, lane 0 the state that entered the chunk')
+        for name, _ in state:
+            a('            entering_%s[k %% %du][st] = carry_%s;' % (name, NBUF, name))
+        for name, _ in state:
+            a('            carry_%s = ovl_dpp_move<OVL_DPP_ROW_ROR1>(carry_%s, %s);' % (name, name, name))
+        a('            __builtin_amdgcn_sched_barrier(0);')
+        a('        };')
+        a('        scan_only(0u, set_a, set_b, ovl_scan_yes());')
+        if n > 1:
+            a('        uint32_t k = 1u;')
+            a('        #pragma unroll 1')
+            a('        for (; k + 1u < %du; k += 2u) {' % n)
+            a('            scan_only(k, set_b, set_a, ovl_scan_no());')
+            a('            scan_only(k + 1u, set_a, set_b, ovl_scan_no());')
+            a('        }')
+            a('        if (k < %du) scan_only(k, set_b, set_a, ovl_scan_no());' % n)
+        a('        __syncthreads();')
+        a('        __syncthreads();')
+        a('#undef OVL_SCAN_OUT')
+        a('#define OVL_SCAN_OUT(value) ov[w][u] = (value)')
+        a('    } else {')
+        a('        // finishing wavefronts: chunk s - 2 in step s, every segment once more from the state that enters it')
+        a('        __syncthreads();')
+        a('        __syncthreads();')
+        a('        __syncthreads();')
+        a('        #pragma unroll 1')
+        a('        for (uint32_t s = 2u; s <= %du; ++s) {' % (n + 1))
+        a('            const uint32_t k = s - 2u;')
+        a('            Segment segment;')
+        a('            fetch_segment(k, segment);')
+        a('            %s* segp = &tile[k %% %du][sl][part * %du];' % (ctype, NBUF, seg_stride))
+        a('            %s ov[%d];' % (vname, seg_vectors))
+        a('            const uint32_t row0 = k * %du + part * %du;' % (rc, seg))
+        for name, _ in state:
+            a('            %s = entering_%s[k %% %du][st];' % (name, name, NBUF))
+        a('            #pragma unroll')
+        a('            for (uint32_t w = 0; w < %du; ++w) {' % seg_vectors)
+        a('                const %s xv = segment.v[w];' % vname)
+        a('                #pragma unroll')
+        a('                for (uint32_t u = 0; u < %du; ++u) {' % per)
+        a('                    if (w == 0u && u == 0u && row0 == 0u) ov[0][0] = first_out;')
+        a('                    else OVL_SCAN_STEP(row0 + w * %du + u)' % per)
+        a('                }')
+        a('            }')
+        a('            #pragma unroll')
+        a('            for (uint32_t w = 0; w < %du; ++w) *reinterpret_cast<%s*>(segp + w * %du) = ov[w];' % (
+            seg_vectors, vname, per))
+        a('            __syncthreads();')
+        a('        }')
+        a('    }')
+    elif movers:
         # Three buffers rotate: while chunk k is scanned in place, the movers bring chunk k + 1 into the next buffer and
         # take the results of chunk k - 1 out of the one before; one barrier per chunk.  (A fourth buffer, the movers one
         # chunk further ahead and the scanning wavefronts reading the segments of chunk k + 1 into a second register
         # set before they start on chunk k gained 0.4 us of 40 on float64 [10000, 1000]: not kept.)
         ahead = 1
         a('    if (threadIdx.x >= %du) {' % SCAN_THREADS)
+        full_tag = lambda k: '_full' if k < num_chunks - 1 else ''
         for j in range(min(sets, num_chunks)):
-            a('        issue_loads(%du, sets[%d]);' % (j, j))
+            a('        issue_loads%s(%du, sets[%d]);' % (full_tag(j), j, j))
         for j in range(ahead):
             if j < num_chunks:
                 a('        write_lds(%du, sets[%d]);' % (j, j % sets))
                 if j + sets < num_chunks:
-                    a('        issue_loads(%du, sets[%d]);' % (j + sets, j % sets))
+                    a('        issue_loads%s(%du, sets[%d]);' % (full_tag(j + sets), j + sets, j % sets))
             a('        __syncthreads();')
         # Step k: chunk k + ahead goes to LDS, its register set is refilled with chunk k + ahead + sets, chunk k - 1 goes
         # out.  The steps in which all three happen run in a loop without conditions; the first steps and the last ones
@@ -823,14 +1067,15 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
             if k + ahead < num_chunks:
                 a('        write_lds(%du, %s);' % (k + ahead, regs))
             if k + ahead + sets < num_chunks:
-                a('        issue_loads(%du, %s);' % (k + ahead + sets, regs))
+                a('        issue_loads%s(%du, %s);' % (full_tag(k + ahead + sets), k + ahead + sets, regs))
             if k >= 1:
-                a('        store_chunk(%du);' % (k - 1))
+                a('        store_chunk%s(%du);' % (full_tag(k - 1), k - 1))
             a('        __syncthreads();')
         # (the loop is entered after one full round of complete steps, so that the requests outstanding at its entry are
         # those outstanding at its end: otherwise the compiler counts with the fewer of the two)
         steady_first = 1 + sets
-        steady_end = max(steady_first, num_chunks - ahead - sets)       # steps [steady_first, steady_end) are complete
+        # steps [steady_first, steady_end) are complete, on chunks all of whose rows exist
+        steady_end = max(steady_first, num_chunks - ahead - sets - 1)
         groups = (steady_end - steady_first) // sets
         for k in range(0, min(steady_first, num_chunks)):
             emit_step(k)
@@ -839,8 +1084,8 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
             a('        for (uint32_t k0 = %du; k0 < %du; k0 += %du) {' % (steady_first, steady_first + groups * sets, sets))
             for d in range(sets):
                 a('            write_lds(k0 + %du, sets[%d]);' % (d + ahead, (steady_first + d + ahead) % sets))
-                a('            issue_loads(k0 + %du, sets[%d]);' % (d + ahead + sets, (steady_first + d + ahead) % sets))
-                a('            store_chunk(k0 + %du - 1u);' % d)
+                a('            issue_loads_full(k0 + %du, sets[%d]);' % (d + ahead + sets, (steady_first + d + ahead) % sets))
+                a('            store_chunk_full(k0 + %du - 1u);' % d)
                 a('            __syncthreads();')
             a('        }')
         for k in range(steady_first + groups * sets, num_chunks):
@@ -887,6 +1132,8 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
             a('        ' + stmt)
         a('    }')
     a('#undef OVL_SCAN_STEP')
+    if not p.reduce:
+        a('#undef OVL_SCAN_STORE')
     a('#undef OVL_SCAN_IN')
     a('#undef OVL_SCAN_OUT')
     a('}')

@@ -21,7 +21,7 @@ include_directory = os.path.normpath(os.path.join(local.csrc_directory, '..', '.
 SCAN_SYMBOLS = ('ovl_cumsum_f32', 'ovl_cumprod_f32', 'ovl_cumsum_f64', 'ovl_cumprod_f64',
                 'ovl_cumsum_f32_reassociated', 'ovl_cumprod_f32_reassociated',
                 'ovl_cumsum_f64_reassociated', 'ovl_cumprod_f64_reassociated')
-EXPORTED_SYMBOLS = SCAN_SYMBOLS + ('ovl_scan_last_error',)
+EXPORTED_SYMBOLS = SCAN_SYMBOLS + ('ovl_strip_copy_f64', 'ovl_scan_last_error')
 
 
 def build(force=False):
@@ -58,6 +58,9 @@ def library():
         fn = getattr(lib, name)
         fn.argtypes = [ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_void_p]
         fn.restype = ctypes.c_int
+    lib.ovl_strip_copy_f64.argtypes = [ctypes.c_void_p, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p,
+                                       ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p]
+    lib.ovl_strip_copy_f64.restype = ctypes.c_int
     lib.ovl_scan_last_error.restype = ctypes.c_char_p
     _lib = lib
     return lib

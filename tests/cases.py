@@ -211,6 +211,16 @@ def c3_colscan_shapes(rng):
             cumsum(rng.standard_normal((10, 33)), axis=0)[0]]
 
 
+def c3_colscan_placements(rng):
+    """Scans along the first axis with sixteen strips and more, where strips are placed by XCD: a row pitch that is
+    not a multiple of 128 bytes (one contiguous range of strips per XCD), pitches that are (groups of two and of four
+    strips that share every line, with left-over strips), and a dimension before the axis."""
+    return [cumsum(rng.standard_normal((300, 200)), axis=0)[0],
+            cumsum(rng.standard_normal((300, 160)), axis=0)[0],
+            cumsum(rng.standard_normal((280, 288), dtype=np.float32), axis=0)[0],
+            cumsum(rng.standard_normal((2, 270, 72)), axis=1)[0]]
+
+
 @ovl.operator()
 def _swap_last_two(x, scale=None):
     """A batched transpose with some arithmetic and a second, untransposed output: the dimensions before the last two
@@ -669,13 +679,15 @@ def _column_sum(x):
 
 def col_reductions(rng):
     """Reductions along an axis other than the last: partial strips, a partial last chunk of rows, dimensions before
-    the axis, 4- and 8-byte elements, integers, a loop from 0 and a loop from 1."""
+    the axis, 4- and 8-byte elements, integers, a loop from 0 and a loop from 1, a long axis."""
     return (all_outputs(_axis_mean_and_max(rng.standard_normal((200, 100)), axis=0)) +
             all_outputs(_axis_mean_and_max(rng.standard_normal((130, 70), dtype=np.float32), axis=0)) +
             all_outputs(_axis_mean_and_max(rng.standard_normal((3, 65, 40), dtype=np.float32), axis=1)) +
             [_column_sum(rng.standard_normal((700, 30))),
              _column_sum(rng.integers(-1000, 1000, size=(64, 5)).astype(np.int32)),
-             _column_sum(rng.standard_normal((1100, 20), dtype=np.float32))])
+             _column_sum(rng.standard_normal((1100, 20), dtype=np.float32)),
+             # (a long axis of 8-byte elements: segments of 32 rows per lane)
+             _column_sum(rng.standard_normal((8200, 11)))])
 
 
 @ovl.operator()
@@ -975,6 +987,7 @@ CASES = [
     Case('c3_cumprod_f64', c3_cumprod_f64, seed=3),
     Case('c3_rowscan_shapes', c3_rowscan_shapes, seed=3),
     Case('carry_scans', carry_scans, seed=3),
+    Case('c3_colscan_placements', c3_colscan_placements, seed=12),
     Case('c3_colscan_shapes', c3_colscan_shapes, seed=3),
     Case('c4_lstm', c4_lstm, seed=4),
     Case('c4_lstm_grad', c4_lstm_grad, seed=4),
@@ -1362,9 +1375,13 @@ TEMPLATE_VARIANTS = [
     ('c3_colscan_shapes', {'template': 'colskew', 'scan_strip': 16, 'scan_sets': 2}),
     ('c3_colscan_shapes', {'template': 'colskew', 'scan_width': 4, 'scan_sets': 5}),
     ('c3_colscan_shapes', {'template': 'colskew', 'scan_movers': 0}),
+    ('c3_colscan_shapes', {'template': 'colskew', 'scan_carry': False}),
+    ('c3_colscan_shapes', {'template': 'colskew', 'scan_carry': False, 'scan_sets': 3}),
     ('c3_colscan_shapes', {'template': 'colskew', 'scan_movers': 512, 'scan_sets': 3}),
     ('c3_colscan_shapes', {'template': 'colskew', 'scan_sets': 5}),
     ('c3_colscan_shapes', {'template': 'colskew', 'scan_movers': 128, 'scan_strip': 16}),
+    ('c3_colscan_placements', {'scan_nt': 's'}),
+    ('c3_colscan_placements', {'scan_nt': '', 'scan_carry': False}),
     ('c3_colscan_shapes', {'template': 'colscan'}),
     ('c3_colscan_shapes', {'template': 'colscan', 'scan_rows': 32, 'scan_batch': 2}),
     ('c3_colscan_shapes', {'template': 'colscan', 'scan_sets': 3}),

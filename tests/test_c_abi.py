@@ -166,6 +166,16 @@ def test_scan_header_binding_and_argument_errors():
         assert entry(p, 4, 0, p, None) == launcher.OVL_EINVAL
         assert entry(p, 1 << 16, 1 << 16, p, None) == launcher.OVL_EINVAL
         assert b'2^32' in L.ovl_scan_last_error()
+    # the measurement aid: strips of 4, 8 or 16 lines; load, store or copy
+    assert L.ovl_strip_copy_f64(None, 4, 8, p, 8, 3, None) == launcher.OVL_EINVAL
+    assert L.ovl_strip_copy_f64(p, 4, 8, None, 8, 3, None) == launcher.OVL_EINVAL
+    assert L.ovl_strip_copy_f64(p, 0, 8, p, 8, 3, None) == launcher.OVL_EINVAL
+    assert L.ovl_strip_copy_f64(p, 1 << 16, 1 << 16, p, 8, 3, None) == launcher.OVL_EINVAL
+    assert L.ovl_strip_copy_f64(p, 4, 8, p, 5, 3, None) == launcher.OVL_EINVAL
+    assert b'lines per workgroup' in L.ovl_scan_last_error()
+    assert L.ovl_strip_copy_f64(p, 4, 8, p, 8, 0, None) == launcher.OVL_EINVAL
+    assert L.ovl_strip_copy_f64(p, 4, 8, p, 8, 4, None) == launcher.OVL_EINVAL
+    assert b'mode' in L.ovl_scan_last_error()
 
 
 def test_scan_python_wrapper_validates_its_arguments():

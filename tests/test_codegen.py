@@ -106,7 +106,9 @@ def test_template_selection():
     assert template(cumsum(np.zeros((48, 1024), np.float32), axis=0))['template'] == 'map'
     # (up to 32768 lines: sixteen lanes per line, strips of 8 to 64 lines for about 256 workgroups)
     col = template(cumsum(np.zeros((1000, 200), np.float64), axis=0))
-    # (strips of 8 lines: two scanning wavefronts and four that only move data)
+    # (strips of 8 lines: two scanning wavefronts and four that only move data; 8-byte elements add two finishing ones)
+    assert col['template'] == 'colskew' and col['blocks_needed'] == 25 and col['block'] == 128 + 128 + 256
+    col = template(cumsum(np.zeros((1000, 200), np.float64), axis=0), {'scan_carry': False})
     assert col['template'] == 'colskew' and col['blocks_needed'] == 25 and col['block'] == 128 + 256
     old = template(cumsum(np.zeros((1000, 200), np.float64), axis=0), {'scan_movers': 0})
     assert old['template'] == 'colskew' and old['block'] == 128

@@ -110,3 +110,30 @@ def test_reassociated_scans_at_full_size_and_their_distance_from_the_sequential_
     xp = (0.99 + 0.02 * torch.rand((1024, 16384), device='cuda', generator=g, dtype=torch.float64))
     seq, tree = row_scan.cumprod(xp), row_scan.cumprod(xp, reassociate=True)
     assert float(((seq - tree) / seq).abs().max()) <= 1e-11
+
+
+@pytest.mark.parametrize('lines', [4, 8, 16])
+@pytest.mark.parametrize('shape', [(1000, 200), (517, 37), (3, 5), (2048, 64)], ids=str)
+def test_strip_copy_measurement_aid_moves_exactly_the_tensor(shape, lines):
+    """ovl_strip_copy_f64 (include/ovl_scan.h): mode 3 copies the tensor, mode 2 writes every element's row index,
+    mode 1 writes nothing; nothing outside the tensor is touched (guard values either side)."""
+    lib = row_scan.library()
+    rows, cols = shape
+    g = torch.Generator(device='cuda')
+    g.manual_seed(11)
+    x = torch.randn(shape, device='cuda', generator=g, dtype=torch.float64)
+    guard = 64
+    for mode in (3, 2, 1):
+        buffer = torch.full((rows * cols + 2 * guard,), -7.0, device='cuda', dtype=torch.float64)
+        out = buffer[guard:guard + rows * cols].view(rows, cols)
+        status = lib.ovl_strip_copy_f64(x.data_ptr(), rows, cols, out.data_ptr(), lines, mode, None)
+        assert status == 0, lib.ovl_scan_last_error()
+        torch.cuda.synchronize()
+        assert bool((buffer[:guard] == -7.0).all()) and bool((buffer[guard + rows * cols:] == -7.0).all())
+        if mode == 3:
+            assert torch.equal(out, x)
+        elif mode == 2:
+            want = torch.arange(rows, device='cuda', dtype=torch.float64)[:, None].expand(rows, cols)
+            assert torch.equal(out, want)
+        else:
+            assert bool((out == -7.0).all())
