@@ -216,6 +216,12 @@ def c3_colscan_placements(rng):
     not a multiple of 128 bytes (one contiguous range of strips per XCD), pitches that are (groups of two and of four
     strips that share every line, with left-over strips), and a dimension before the axis."""
     return [cumsum(rng.standard_normal((300, 200)), axis=0)[0],
+            # (long axes: the movers' loop over whole chunks runs, with 2 and with 3 chunks of loads in flight; 8-byte
+            # integers wrap around like the oracle's; exactly 4 and 5 chunks of 256 rows)
+            cumsum(rng.standard_normal((3400, 9)), axis=0)[0],
+            cumsum(rng.integers(-2 ** 62, 2 ** 62, size=(3700, 5)), axis=0)[0],
+            cumprod(uniform(rng, 0.99, 1.01, (1024, 12), np.float64), axis=0)[0],
+            cumsum(rng.standard_normal((1280, 3)), axis=0)[0],
             cumsum(rng.standard_normal((300, 160)), axis=0)[0],
             cumsum(rng.standard_normal((280, 288), dtype=np.float32), axis=0)[0],
             cumsum(rng.standard_normal((2, 270, 72)), axis=1)[0]]
@@ -1381,6 +1387,7 @@ TEMPLATE_VARIANTS = [
     ('c3_colscan_shapes', {'template': 'colskew', 'scan_sets': 5}),
     ('c3_colscan_shapes', {'template': 'colskew', 'scan_movers': 128, 'scan_strip': 16}),
     ('c3_colscan_placements', {'scan_nt': 's'}),
+    ('c3_colscan_placements', {'scan_sets': 3}),
     ('c3_colscan_placements', {'scan_nt': '', 'scan_carry': False}),
     ('c3_colscan_shapes', {'template': 'colscan'}),
     ('c3_colscan_shapes', {'template': 'colscan', 'scan_rows': 32, 'scan_batch': 2}),
