@@ -724,8 +724,10 @@ def main():
         others.append(side_workload('launch floor: copy of 1024 floats, one workgroup (what the clock around a launch '
                                     'reads for a kernel with nothing to do)',
                                     copy_outputs(np.zeros(1024, np.float32)), steps, warm))
-        others.append(side_workload('c1 shift_cyclic -> expm1 -> log1p, f32[2^20]', c1_outputs(data['c1']), steps,
-                                    warm, reference=cpu.get('c1')))
+        others.append(side_workload("c1 shift_cyclic -> expm1 -> log1p, f32[2^20], 'exact' math mode",
+                                    c1_outputs(data['c1']), steps, warm, reference=cpu.get('c1')))
+        others.append(side_workload("c1 shift_cyclic -> expm1 -> log1p, f32[2^20], default 'ulp2' math mode",
+                                    c1_outputs(data['c1']), steps, warm, {'math': 'ulp2'}))
         del chain, exact, leaves
         cpu.pop('chain8', None)
         torch.cuda.empty_cache()

@@ -102,6 +102,10 @@ def contiguous_unaligned(info, node, tensor, aff, vec):
     return not _is_vector_access(info, node, tensor, aff, vec)
 
 
+#: several vectors per thread are chosen only while the grid keeps this many workgroups (eight per compute unit)
+MIN_BLOCKS_PER_THREAD_VECTORS = 2048
+
+
 def _arithmetic_weight(info):
     """Rough count of expensive float operations per worker (transcendental calls and divisions)."""
     heavy = (lang.EXP, lang.LOG, lang.TANH, lang.DIVIDE, lang.SIN, lang.COS, lang.TAN, lang.POW, lang.SQRT,
@@ -191,7 +195,11 @@ def generate(info, kernel_name, vec=None, nt=None, grid_cap=None, per_thread=Non
         few_streams = len(loads) + len(unaligned) + len(stores) <= 3
         per_thread = 4 if (vec > 1 and few_streams and _arithmetic_weight(info) >= 4 and
                            getattr(info, 'math', 'exact') != 'exact') else 1
-        while per_thread > 1 and num_vectors % (BLOCK * per_thread) != 0:
+        # (a small tensor keeps one vector per thread: its time is latency, and fewer, longer threads only add to it.
+        # The reference's README pipeline on 2^20 floats in the 'ulp2' mode: 10 us with four vectors per thread and
+        # 256 workgroups, 6 us with one and 1024)
+        while per_thread > 1 and (num_vectors % (BLOCK * per_thread) != 0 or
+                                  num_vectors // (BLOCK * per_thread) < MIN_BLOCKS_PER_THREAD_VECTORS):
             per_thread //= 2
     if per_thread > 1 and not (single_grid and num_vectors % (BLOCK * per_thread) == 0 and
                                not any(info.in_loop.values())):

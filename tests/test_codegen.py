@@ -381,3 +381,21 @@ def test_repeated_subexpressions_are_evaluated_once():
     text = hipgen.generate(guarded(Spec((256,))).expression_dag, 'f' + '1' * 56,
                            {'if_conversion': False, 'per_thread': 1}).source
     assert text.count('ovl_expf') == 2
+
+
+def test_vectors_per_thread_follow_the_size_of_the_grid():
+    """Outside the 'exact' mode a thread of a body with few streams and some arithmetic takes four vectors, but only
+    while the grid keeps eight workgroups per compute unit: a small tensor's time is latency."""
+    from opveclib_amd import workloads
+    from opveclib_amd.workloads import Spec
+
+    def launch(outputs, mode):
+        op, = workloads.fused_operators(outputs)
+        return hipgen.generate(op, 'f' + '5' * 56, {'math': mode}).launch
+
+    big = [Spec((8192, 8192), np.float32), Spec((8192, 8192), np.float32), Spec((1,), np.float32)]
+    assert launch(workloads.chain8_outputs(*big), 'ulp2')['per_thread'] == 4
+    assert launch(workloads.chain8_outputs(*big), 'exact')['per_thread'] == 1
+    assert launch(workloads.c1_outputs(Spec((1 << 20,), np.float32)), 'ulp2')['per_thread'] == 1
+    assert launch(workloads.c1_outputs(Spec((1 << 23,), np.float32)), 'ulp2')['per_thread'] == 4
+    assert launch(workloads.c1_outputs(Spec((1 << 22,), np.float32)), 'ulp2')['per_thread'] == 2
