@@ -239,7 +239,7 @@ def sweep(tmp_path_factory):
 @pytest.mark.parametrize('kind', ['log1p', 'expm1'])
 def test_once_rounded_routines_within_two_ulp_of_the_reference_formulas_on_the_host(sweep, kind):
     """Every 31st argument of the domains the generator replaces the formulas on: the one a value range must prove
-    (IDIOM_DOMAIN) and the intervals tested at run time (GUARD_DOMAIN: for log1p also the negative arguments)."""
+    (IDIOM_DOMAIN) and the intervals tested at run time (GUARD_DOMAIN: also negative arguments)."""
     assert accuracy.IDIOM_DOMAIN[kind] in accuracy.GUARD_DOMAIN[kind]
     for lo, hi in accuracy.GUARD_DOMAIN[kind]:
         if hi < 0:
