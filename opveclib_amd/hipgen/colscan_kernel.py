@@ -492,8 +492,13 @@ def _emit_movers(a, sets, num_chunks, stores=True):
 # there four more wavefronts of the workgroup do nothing but move data through three rotating buffers (one barrier per
 # chunk) and the scanning wavefronts only read their segments, run the recurrence and write them back (float64
 # [10000, 1000] 58 -> 40 us, float32 47 -> 33 us, float64 [5000, 300] 32 -> 23 us; in strips of 16 lines the extra
-# wavefronts lose: float64 [4096, 4096] 41 -> 45 us).  What is left there is the recurrence: 0.86 us per chunk of 256
-# rows, of which the sixteen phases of sixteen dependent float64 additions and a hand-over are 0.70.
+# wavefronts lose: float64 [4096, 4096] 41 -> 45 us).  For 8-byte elements the scanning wavefronts of those strips do
+# not write results either: they publish the state that enters each lane's segment and as many finishing wavefronts
+# recompute the segments (six buffers; see `generate_skewed`).  Strips narrower than a cache line are placed on the
+# XCDs so that the strips that share lines share an L2.  With all of it float64 [10000, 1000] takes 36 us; a kernel
+# that only copies the tensor in the same strips takes 31 us (`ovl_strip_copy_f64`, csrc/ovl_scan.hip), and the
+# scanning wavefront's own instruction stream 23.5 us (sixteen phases of sixteen dependent float64 additions and a
+# hand-over: 5.6 clocks per row).
 # ---------------------------------------------------------------------------------------------------------------------
 SKEW_GROUP = 16                 # lanes per line
 SKEW_SEG_VECTORS = 2            # 128-bit vectors a lane owns per phase (32 bytes: 4 float64 or 8 float32 rows)
