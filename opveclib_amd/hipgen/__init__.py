@@ -30,7 +30,7 @@ from . import rowscan_kernel
 from . import colscan_kernel
 
 #: bump when generated code changes for an unchanged DAG, so cached binaries are not reused
-CODEGEN_VERSION = 39
+CODEGEN_VERSION = 43
 
 
 

@@ -279,6 +279,8 @@ def generate(info, kernel_name, rows_per_chunk=None, batch=None, sets=None, redu
     src = []
     a = src.append
     a('typedef %s %s __attribute__((ext_vector_type(%d)));' % (ctype, vname, per))
+    a('struct ovl_scan_yes { static constexpr bool value = true; };')
+    a('struct ovl_scan_no { static constexpr bool value = false; };')
     a('')
     a('extern "C" __global__ void __launch_bounds__(%d)' % BLOCK)
     if p.reduce:
@@ -378,17 +380,19 @@ def generate(info, kernel_name, rows_per_chunk=None, batch=None, sets=None, redu
     a('            for (uint32_t v = 0; v < %du; ++v) to[v * %du] = set[v];' % (batch, STRIP))
     a('        };')
     a('        // the recurrence over one register set; the tensor\'s first row was done above')
-    a('        auto run = [&](%s (&set)[%d], uint32_t row0, bool first) {' % (vname, batch))
+    a('        auto run = [&](%s (&set)[%d], uint32_t row0, bool first, auto last_chunk) {' % (vname, batch))
     a('            #pragma unroll')
     a('            for (uint32_t v = 0; v < %du; ++v) {' % batch)
     a('                %s& xv = set[v];' % vname)
     a('                #pragma unroll')
     a('                for (uint32_t u = 0; u < %du; ++u) {' % per)
     if p.reduce:
-        # (rows past the last one of the tensor hold copies of other rows: they must not reach the state)
+        # (rows past the last one of the tensor hold copies of other rows: they must not reach the state; only the
+        # last chunk has such rows, so only its instantiation tests for them)
         skip_first = 'v == 0u && u == 0u && first' if p.start == 1 else 'false'
-        a('                    if (!(%s) && row0 + v * %du + u < %du) OVL_SCAN_STEP(row0 + v * %du + u)' % (
-            skip_first, per, p.length, per))
+        in_tensor = 'true' if p.length % rc == 0 else \
+            '(!decltype(last_chunk)::value || row0 + v * %du + u < %du)' % (per, p.length)
+        a('                    if (!(%s) && %s) OVL_SCAN_STEP(row0 + v * %du + u)' % (skip_first, in_tensor, per))
     else:
         a('                    if (v == 0u && u == 0u && first) xv[0] = first_out;')
         a('                    else OVL_SCAN_STEP(row0 + v * %du + u)' % per)
@@ -396,23 +400,26 @@ def generate(info, kernel_name, rows_per_chunk=None, batch=None, sets=None, redu
     a('            }')
     a('        };')
     a('        __syncthreads();')
-    a('        for (uint32_t k = 0; k < %du; ++k) {' % num_chunks)
+    a('        auto chunk = [&](uint32_t k, auto last_chunk) {')
     # (a reduction's lanes past the last line store what its owner stores: they read the owner's rows too)
     a('            %s* colp = &tile[k %% 3u][0][%s];' % (vname, 'c' if p.reduce else 'lane'))
     a('            fetch(set_a, colp);')
     a('            #pragma unroll 1')
     a('            for (uint32_t q = 0; q < %du; q += %du) {' % (reads_per_chunk, 2 * batch))
     a('                fetch(set_b, colp + (q + %du) * %du);' % (batch, STRIP))
-    a('                run(set_a, k * %du + q * %du, k == 0u && q == 0u);' % (rc, per))
+    a('                run(set_a, k * %du + q * %du, k == 0u && q == 0u, last_chunk);' % (rc, per))
     if not p.reduce:
         a('                put_back(set_a, colp + q * %du);' % STRIP)
     a('                if (q + %du < %du) fetch(set_a, colp + (q + %du) * %du);' % (2 * batch, reads_per_chunk, 2 * batch, STRIP))
-    a('                run(set_b, k * %du + (q + %du) * %du, false);' % (rc, batch, per))
+    a('                run(set_b, k * %du + (q + %du) * %du, false, last_chunk);' % (rc, batch, per))
     if not p.reduce:
         a('                put_back(set_b, colp + (q + %du) * %du);' % (batch, STRIP))
     a('            }')
     a('            __syncthreads();')
-    a('        }')
+    a('        };')
+    a('        #pragma unroll 1')
+    a('        for (uint32_t k = 0; k < %du; ++k) chunk(k, ovl_scan_no());' % (num_chunks - 1))
+    a('        chunk(%du, ovl_scan_yes());' % (num_chunks - 1))
     if p.reduce:
         a('        // the statements after the worker\'s loop, once per line')
         for stmt in epilogue:
@@ -551,11 +558,6 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
         # [10000, 1000] without separate movers: 79 us with 32 bytes, 65 with 64, 59 with 128; with wider strips the
         # longer segments lose: float64 [4096, 4096] 41 -> 45 us)
         seg_vectors = SKEW_SEG_VECTORS_NARROW if narrow else SKEW_SEG_VECTORS
-        if narrow and reduce and per == 2 and p.length >= 8192:
-            # a reduction over a long axis of 8-byte elements keeps nothing per row, so twice the segment costs only
-            # registers: column sums float64 [10000, 1000] 37.0 -> 34.6 us, [20000, 512] 66.9 -> 60.1 (float32, and
-            # float64 [4096, 2048], lose 1 to 2 us)
-            seg_vectors = 2 * SKEW_SEG_VECTORS_NARROW
     seg = seg_vectors * per                         # rows a lane owns per phase
     rc = SKEW_GROUP * seg                           # rows per chunk
     if movers is None:
@@ -631,9 +633,8 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
     src = []
     a = src.append
     a('typedef %s %s __attribute__((ext_vector_type(%d)));' % (ctype, vname, per))
-    if carry:
-        a('struct ovl_scan_yes { static constexpr bool value = true; };')
-        a('struct ovl_scan_no { static constexpr bool value = false; };')
+    a('struct ovl_scan_yes { static constexpr bool value = true; };')
+    a('struct ovl_scan_no { static constexpr bool value = false; };')
     a('')
     a('extern "C" __global__ void __launch_bounds__(%d)' % BLOCK)
     if p.reduce:
@@ -864,7 +865,7 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
     a('        for (uint32_t w = 0; w < %du; ++w) segment.v[w] = *reinterpret_cast<const %s*>(segp + w * %du);' % (
         seg_vectors, vname, per))
     a('    };')
-    a('    auto scan_segment = [&](uint32_t k, const Segment& segment) {')
+    a('    auto scan_segment = [&](uint32_t k, const Segment& segment, auto last_chunk) {')
     if not p.reduce:
         a('        %s* segp = &tile[k %% %du][sl][part * %du];' % (ctype, NBUF, seg_stride))
         a('        %s ov[%d];' % (vname, seg_vectors))
@@ -880,10 +881,14 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
     a('                #pragma unroll')
     a('                for (uint32_t u = 0; u < %du; ++u) {' % per)
     if p.reduce:
-        # (rows past the last one of the tensor hold copies of the last: they must not reach the state)
+        # (rows past the last one of the tensor hold copies of the last: they must not reach the state.  Only the last
+        # chunk has such rows, and only when the axis is not a whole number of chunks: the test stands in that chunk's
+        # instantiation alone.  In every step of every chunk it cost the recurrence more than the additions did: column
+        # sums float64 [10000, 1000] 34.6 -> 31.6 us, float32 29.0 -> 26.9)
         skip_first = 'w == 0u && u == 0u && first_row' if p.start == 1 else 'false'
-        a('                    if (!(%s) && row0 + w * %du + u < %du) OVL_SCAN_STEP(row0 + w * %du + u)' % (
-            skip_first, per, p.length, per))
+        in_tensor = 'true' if p.length % rc == 0 else \
+            '(!decltype(last_chunk)::value || row0 + w * %du + u < %du)' % (per, p.length)
+        a('                    if (!(%s) && %s) OVL_SCAN_STEP(row0 + w * %du + u)' % (skip_first, in_tensor, per))
     else:
         a('                    if (w == 0u && u == 0u && first_row) ov[0][0] = first_out;')
         a('                    else OVL_SCAN_STEP(row0 + w * %du + u)' % per)
@@ -900,10 +905,10 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
         a('        for (uint32_t w = 0; w < %du; ++w) *reinterpret_cast<%s*>(segp + w * %du) = ov[w];' % (
             seg_vectors, vname, per))
     a('    };')
-    a('    auto scan_chunk = [&](uint32_t k) {')
+    a('    auto scan_chunk = [&](uint32_t k, auto last_chunk) {')
     a('        Segment segment;')
     a('        fetch_segment(k, segment);')
-    a('        scan_segment(k, segment);')
+    a('        scan_segment(k, segment, last_chunk);')
     a('    };')
     a('')
     a('    // %d register sets keep %d chunks of loads in flight: chunk j travels through set j %% %d' % (sets, sets, sets))
@@ -1049,7 +1054,9 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
         # Three buffers rotate: while chunk k is scanned in place, the movers bring chunk k + 1 into the next buffer and
         # take the results of chunk k - 1 out of the one before; one barrier per chunk.  (A fourth buffer, the movers one
         # chunk further ahead and the scanning wavefronts reading the segments of chunk k + 1 into a second register
-        # set before they start on chunk k gained 0.4 us of 40 on float64 [10000, 1000]: not kept.)
+        # set before they start on chunk k gained 0.4 us of 40 on float64 [10000, 1000]: not kept.  Movers two to six
+        # chunks ahead of a reduction's scanning wavefronts lose 0.5 to 2 us of 32, like more chunks of loads in flight:
+        # workgroups that drift apart no longer meet their neighbours' lines in the L2.)
         ahead = 1
         a('    if (threadIdx.x >= %du) {' % SCAN_THREADS)
         full_tag = lambda k: '_full' if k < num_chunks - 1 else ''
@@ -1099,10 +1106,12 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
         a('    } else {')
         a('        __syncthreads();')
         a('        #pragma unroll 1')
-        a('        for (uint32_t k = 0; k < %du; ++k) {' % num_chunks)
-        a('            scan_chunk(k);')
+        a('        for (uint32_t k = 0; k < %du; ++k) {' % (num_chunks - 1))
+        a('            scan_chunk(k, ovl_scan_no());')
         a('            __syncthreads();')
         a('        }')
+        a('        scan_chunk(%du, ovl_scan_yes());' % (num_chunks - 1))
+        a('        __syncthreads();')
         a('    }')
     else:
         for j in range(min(sets, num_chunks)):
@@ -1112,22 +1121,23 @@ def generate_skewed(info, kernel_name, sets=None, strip=None, seg_vectors=None, 
             a('    issue_loads(%du, sets[0]);' % sets)
         a('    __syncthreads();')
         a('    // step k: chunk k is scanned in place; then its results go out while chunk k + 1 comes into the other buffer')
-        a('    auto step = [&](uint32_t k, MoverRegs& regs) {')
-        a('        scan_chunk(k);')
+        a('    auto step = [&](uint32_t k, MoverRegs& regs, auto last_chunk) {')
+        a('        scan_chunk(k, last_chunk);')
         a('        __syncthreads();')
         a('        store_chunk(k);')
         a('        if (k + 1u < %du) write_lds(k + 1u, regs);' % num_chunks)
         a('        if (k + 1u + %du < %du) issue_loads(k + 1u + %du, regs);' % (sets, num_chunks, sets))
         a('        __syncthreads();')
         a('    };')
+        full = (num_chunks - 1) // sets                 # whole rounds of the register sets before the last chunk
         if full:
             a('    #pragma unroll 1')
             a('    for (uint32_t k0 = 0; k0 < %du; k0 += %du) {' % (full * sets, sets))
             for d in range(sets):
-                a('        step(k0 + %du, sets[%d]);' % (d, (d + 1) % sets))
+                a('        step(k0 + %du, sets[%d], ovl_scan_no());' % (d, (d + 1) % sets))
             a('    }')
         for k in range(full * sets, num_chunks):
-            a('    step(%du, sets[%d]);' % (k, (k + 1) % sets))
+            a('    step(%du, sets[%d], ovl_scan_%s());' % (k, (k + 1) % sets, 'yes' if k == num_chunks - 1 else 'no'))
     if p.reduce:
         a('    // the statements after the worker\'s loop, once per line: lane 0 of the line holds the final state')
         a('    if (threadIdx.x < %du && part == 0u) {' % SCAN_THREADS)

@@ -692,7 +692,7 @@ def col_reductions(rng):
             [_column_sum(rng.standard_normal((700, 30))),
              _column_sum(rng.integers(-1000, 1000, size=(64, 5)).astype(np.int32)),
              _column_sum(rng.standard_normal((1100, 20), dtype=np.float32)),
-             # (a long axis of 8-byte elements: segments of 32 rows per lane)
+             # (a long axis: the steps of the last, partial chunk alone test their rows against its end)
              _column_sum(rng.standard_normal((8200, 11)))])
 
 
